@@ -1,0 +1,63 @@
+"""Compile the HIP library, the command-line harness and (optionally) the CPU oracle.
+
+Run as a script or call build().  Everything lands in-tree next to this file
+(libawq_infer.so, qwen3_awq_infer) so that a source snapshot carries the
+binaries along.
+"""
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "libawq_infer.so")
+CLI = os.path.join(HERE, "qwen3_awq_infer")
+
+HIP_SOURCES = ["gemv.hip", "ops.hip", "attention.hip", "engine.cpp", "synth.cpp"]
+
+# -ffp-contract=off: every fma in the sources is written out; a contracted
+#   a*b-c*d would break bit parity with the reference's __hmul/__hsub sequence.
+# packed-fp32 ops are switched off for the whole library.
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fopenmp",
+    "-ffp-contract=off", "-fno-fast-math", "-fhip-fp32-correctly-rounded-divide-sqrt",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-function", "-x", "hip",
+]
+
+
+def _run(cmd):
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        sys.stderr.write(" ".join(cmd) + "\n" + res.stdout + res.stderr)
+        raise RuntimeError("build step failed: " + cmd[0])
+    return res
+
+
+def build(verbose=False, oracle=True):
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    objdir = os.path.join(HERE, "build")
+    os.makedirs(objdir, exist_ok=True)
+
+    def compile_one(src):
+        obj = os.path.join(objdir, src + ".o")
+        _run([hipcc] + HIPCC_FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj])
+        return obj
+
+    with ThreadPoolExecutor(max_workers=min(8, len(HIP_SOURCES))) as pool:
+        objs = list(pool.map(compile_one, HIP_SOURCES))
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fopenmp", "-o", LIB] + objs)
+    # the drop-in C++ class and the reference's command line on top of the C ABI
+    _run([hipcc, "-O2", "-std=c++17", os.path.join(CSRC, "qwen3_awq_infer.cpp"), os.path.join(CSRC, "main.cpp"),
+          "-o", CLI, "-L" + HERE, "-lawq_infer", "-Wl,-rpath,$ORIGIN"])
+    if oracle:
+        _run(["make", "-C", os.path.join(ROOT, "oracle"), "-B"])
+    if verbose:
+        print("built", LIB)
+    return LIB
+
+
+if __name__ == "__main__":
+    build(verbose=True)

@@ -1,0 +1,89 @@
+// Shared declarations of the HIP side: FP16 vector types, error plumbing and
+// the launcher prototypes that the C ABI (api.cpp) and the engine call.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <string>
+
+#include "../../include/awq_canon_math.h"
+#include "../../include/awq_infer.h"
+
+typedef _Float16 half_t;
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+
+// error string of the calling thread (awq_last_error)
+void awq_set_error(const std::string& msg);
+
+#define AWQ_HIP_TRY(expr)                                                                                 \
+  do {                                                                                                    \
+    hipError_t err__ = (expr);                                                                            \
+    if (err__ != hipSuccess) {                                                                            \
+      awq_set_error(std::string("HIP error at ") + __FILE__ + ":" + std::to_string(__LINE__) + " code=" + \
+                    std::to_string((int)err__) + " \"" + hipGetErrorString(err__) + "\" in " #expr);       \
+      return AWQ_ERR_HIP;                                                                                 \
+    }                                                                                                     \
+  } while (0)
+
+#define AWQ_REQUIRE(cond, msg)                                       \
+  do {                                                               \
+    if (!(cond)) {                                                   \
+      awq_set_error(std::string(__func__) + ": " + (msg));           \
+      return AWQ_ERR_ARG;                                            \
+    }                                                                \
+  } while (0)
+
+// Values that change from step to step live in device memory so that a
+// captured graph can be replayed unchanged: kernels read them from here.
+struct StepState {
+  int32_t pos;        // position written to the KV cache this step
+  int32_t len_lo;     // attended length for layers <  split
+  int32_t len_hi;     // attended length for layers >= split
+  int32_t token;      // token to embed at the start of the step, -1 = keep the hidden state
+  int32_t out_index;  // where the sampled token goes in the output array
+  int32_t sample;     // 1 = run the sampler at the end of the step
+};
+
+// epilogues of the fused linear kernel
+enum LinearEpilogue {
+  EPI_STORE = 0,     // y = h(acc)
+  EPI_RESIDUAL = 1,  // y = h(res + h(acc))
+  EPI_GELU = 2,      // y = h(gelu(h(acc)))
+};
+
+struct LinearArgs {
+  const void* wq;      // repacked int4
+  const half_t* scale; // [m/128]
+  const half_t* zp;    // [m/128]
+  const half_t* x;     // [k]
+  half_t* y;           // [m]
+  const half_t* res;   // EPI_RESIDUAL: [m], may alias y
+  float* partials;     // split-k workspace
+  int32_t* counters;   // one per 64-row group, zero between launches
+  int64_t m, k;
+  int zp_integral;     // all zero-points are integers in [0,1024]: take the 2-op dequant
+  int epilogue;
+};
+
+int launch_dequant(const uint8_t* packed, const half_t* scale, const half_t* zp, half_t* out, int64_t rows,
+                   int64_t cols, int64_t n_groups, hipStream_t st);
+int launch_repack(const uint8_t* in, void* out, int64_t m, int64_t k, hipStream_t st);
+int64_t gemv_workspace_bytes(int64_t m, int64_t k);
+int launch_gemv(const LinearArgs& a, hipStream_t st);
+int launch_rmsnorm(const half_t* x, const half_t* gamma, half_t* out, int64_t n, float eps, hipStream_t st);
+int launch_rope_kv_append(const half_t* qkv, const half_t* cos_t, const half_t* sin_t, half_t* q_out, half_t* kc,
+                          half_t* vc, int n_heads, int64_t max_pos, int64_t pos, const StepState* dyn, hipStream_t st);
+int64_t attention_workspace_bytes(int n_heads, int64_t max_pos);
+int launch_attention(const half_t* q, const half_t* kc, const half_t* vc, half_t* ctx, int n_heads, int64_t max_pos,
+                     int64_t L, const StepState* dyn, int use_len_hi, void* ws, hipStream_t st);
+int launch_residual(const half_t* a, const half_t* b, half_t* out, int64_t n, hipStream_t st);
+int launch_gelu(half_t* x, int64_t n, hipStream_t st);
+int64_t argmax_workspace_bytes(int64_t n);
+int launch_argmax(const half_t* logits, int64_t n, int32_t* out_token, void* ws, const StepState* dyn,
+                  int32_t* out_array, hipStream_t st);
+int launch_embed(const uint8_t* packed, const half_t* scale, const half_t* zp, int64_t hidden, int64_t vocab,
+                 int32_t tok, const StepState* dyn, const int32_t* tok_dev, half_t* out, hipStream_t st);
+int launch_set_state(StepState* dst, StepState v, hipStream_t st);
+int launch_fill_zero(void* p, int64_t bytes, hipStream_t st);

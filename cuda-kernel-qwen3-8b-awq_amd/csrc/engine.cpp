@@ -1,0 +1,704 @@
+// Host side of the engine: the C ABI of include/awq_infer.h.
+//
+// Replaces class QWen3AWQInfer of the reference (Inference.cu:356-415):
+// constructor (:422-470), loader (:766-903), runOneLayer (:1029-1230),
+// sampleNextToken (:1235-1292) and generateResponse (:1297-1408), with all
+// layers, the embedding and the unembedding on the current device, weights kept
+// as packed int4, and no host round trip inside a step.
+#include "engine.hpp"
+
+#include <stdio.h>
+#include <string.h>
+#include <sys/stat.h>
+
+#include <memory>
+
+static thread_local std::string g_last_error;
+void awq_set_error(const std::string& msg) { g_last_error = msg; }
+extern "C" const char* awq_last_error(void) { return g_last_error.c_str(); }
+
+extern "C" void awq_default_config(awq_config* cfg) {
+  cfg->n_layers = 36;      // Inference.cu:37
+  cfg->hidden = 4096;      // :33
+  cfg->inter = 12288;      // :34
+  cfg->vocab = 151936;     // :38
+  cfg->max_pos = 40960;    // :39
+  cfg->split_idx = 18;     // :47
+  cfg->eps = 1e-6f;        // :41
+}
+
+int awq_check_config(const awq_config* c) {
+  AWQ_REQUIRE(c != nullptr, "config is NULL");
+  AWQ_REQUIRE(c->n_layers >= 1 && c->n_layers <= 4096, "n_layers out of range");
+  AWQ_REQUIRE(c->hidden >= 512 && c->hidden % 512 == 0, "hidden must be a positive multiple of 512");
+  AWQ_REQUIRE(c->inter >= 512 && c->inter % 512 == 0, "inter must be a positive multiple of 512");
+  AWQ_REQUIRE(c->vocab >= 128 && c->vocab % 128 == 0, "vocab must be a positive multiple of 128");
+  AWQ_REQUIRE(c->max_pos >= 1 && c->max_pos <= 65536, "max_pos must be in 1..65536");
+  AWQ_REQUIRE(c->split_idx >= 0 && c->split_idx <= c->n_layers, "split_idx out of range");
+  AWQ_REQUIRE(c->eps > 0.0f, "eps must be positive");
+  int C = awq_group_period(c->vocab, c->hidden);
+  AWQ_REQUIRE((c->hidden / AWQ_BLOCK_K) % C == 0, "hidden/32 must be a multiple of the unembedding's scale-group period");
+  return AWQ_OK;
+}
+
+void awq_tensor_dims(const awq_config& cfg, int kind, int64_t* out_dim, int64_t* in_dim) {
+  const int64_t H = cfg.hidden, I = cfg.inter, V = cfg.vocab;
+  switch (kind) {
+    case AWQ_T_WQKV: *out_dim = 3 * H; *in_dim = H; break;  // Inference.cu:616
+    case AWQ_T_WO: *out_dim = H; *in_dim = H; break;        // :630
+    case AWQ_T_W1: *out_dim = I; *in_dim = H; break;        // :644
+    case AWQ_T_W2: *out_dim = H; *in_dim = I; break;        // :658
+    case AWQ_T_EMBED: *out_dim = H; *in_dim = V; break;     // :693
+    case AWQ_T_UNEMBED: *out_dim = V; *in_dim = H; break;   // :708
+    default: *out_dim = 0; *in_dim = 0;
+  }
+}
+
+static int64_t part_bytes(const awq_config& cfg, int kind, int part) {
+  if (kind == AWQ_T_GAMMA) return (int64_t)cfg.hidden * 2;
+  int64_t o, i;
+  awq_tensor_dims(cfg, kind, &o, &i);
+  if (part == AWQ_P_PACKED) return o * ((i + 1) / 2);  // Inference.cu:775
+  return (o / AWQ_GROUP_SIZE) * 2;                      // :776: out_dim/128 entries
+}
+
+std::vector<WeightFile> awq_weight_files(const awq_config& cfg) {
+  std::vector<WeightFile> v;
+  static const struct {
+    int kind;
+    const char *w, *s, *z;
+  } per_layer[4] = {{AWQ_T_WQKV, "_wqkv.bin", "_bqkv_scale.bin", "_bqkv_zp.bin"},  // Inference.cu:780-790
+                    {AWQ_T_WO, "_wo.bin", "_wo_scale.bin", "_wo_zp.bin"},            // :802-810
+                    {AWQ_T_W1, "_w1.bin", "_w1_scale.bin", "_w1_zp.bin"},            // :822-830
+                    {AWQ_T_W2, "_w2.bin", "_w2_scale.bin", "_w2_zp.bin"}};           // :842-850
+  for (int l = 0; l < cfg.n_layers; ++l) {
+    std::string p = "layer_" + std::to_string(l);
+    for (const auto& t : per_layer) {
+      v.push_back({p + t.w, l, t.kind, AWQ_P_PACKED, part_bytes(cfg, t.kind, AWQ_P_PACKED)});
+      v.push_back({p + t.s, l, t.kind, AWQ_P_SCALE, part_bytes(cfg, t.kind, AWQ_P_SCALE)});
+      v.push_back({p + t.z, l, t.kind, AWQ_P_ZP, part_bytes(cfg, t.kind, AWQ_P_ZP)});
+    }
+    v.push_back({"rms_norm_gamma_" + std::to_string(l) + ".bin", l, AWQ_T_GAMMA, 0, part_bytes(cfg, AWQ_T_GAMMA, 0)});  // :856
+  }
+  v.push_back({"word_embedding.bin", 0, AWQ_T_EMBED, AWQ_P_PACKED, part_bytes(cfg, AWQ_T_EMBED, AWQ_P_PACKED)});  // :870
+  v.push_back({"word_embed_scale.bin", 0, AWQ_T_EMBED, AWQ_P_SCALE, part_bytes(cfg, AWQ_T_EMBED, AWQ_P_SCALE)});
+  v.push_back({"word_embed_zp.bin", 0, AWQ_T_EMBED, AWQ_P_ZP, part_bytes(cfg, AWQ_T_EMBED, AWQ_P_ZP)});
+  v.push_back({"unembed.bin", 0, AWQ_T_UNEMBED, AWQ_P_PACKED, part_bytes(cfg, AWQ_T_UNEMBED, AWQ_P_PACKED)});     // :891
+  v.push_back({"unembed_scale.bin", 0, AWQ_T_UNEMBED, AWQ_P_SCALE, part_bytes(cfg, AWQ_T_UNEMBED, AWQ_P_SCALE)});
+  v.push_back({"unembed_zp.bin", 0, AWQ_T_UNEMBED, AWQ_P_ZP, part_bytes(cfg, AWQ_T_UNEMBED, AWQ_P_ZP)});
+  return v;
+}
+
+extern "C" int awq_validate_weight_dir(const char* dir, const awq_config* cfg_in) {
+  AWQ_REQUIRE(dir != nullptr, "dir is NULL");
+  awq_config cfg;
+  if (cfg_in) cfg = *cfg_in;
+  else awq_default_config(&cfg);
+  if (int rc = awq_check_config(&cfg)) return rc;
+  for (const WeightFile& wf : awq_weight_files(cfg)) {
+    std::string path = std::string(dir) + "/" + wf.name;
+    struct stat st;
+    if (stat(path.c_str(), &st) != 0 || !S_ISREG(st.st_mode)) {
+      awq_set_error("could not open " + path);  // Inference.cu:299-302
+      return AWQ_ERR_IO;
+    }
+    if ((int64_t)st.st_size < wf.bytes) {
+      awq_set_error("read failed for " + path + ": " + std::to_string((long long)st.st_size) + " bytes, need " +
+                    std::to_string((long long)wf.bytes));  // :305-308
+      return AWQ_ERR_IO;
+    }
+  }
+  return AWQ_OK;
+}
+
+// ---------------------------------------------------------------------------
+
+namespace {
+
+struct DevLinear {
+  uint8_t* packed = nullptr;  // file order; freed after reordering except for the embedding
+  void* stream_order = nullptr;
+  half_t* scale = nullptr;
+  half_t* zp = nullptr;
+  int64_t m = 0, k = 0;
+  int zp_integral = 0;
+  bool have[3] = {false, false, false};
+};
+
+struct LayerDev {
+  DevLinear wqkv, wo, w1, w2;
+  half_t* gamma = nullptr;
+  bool have_gamma = false;
+  half_t* kcache = nullptr;
+  half_t* vcache = nullptr;
+};
+
+}  // namespace
+
+struct awq_engine {
+  awq_config cfg;
+  int n_heads = 0;
+  int device = 0;
+  hipStream_t stream = nullptr;
+  std::vector<LayerDev> layers;
+  DevLinear embed, unembed;
+  half_t *cos_t = nullptr, *sin_t = nullptr;
+  // activations (Inference.cu:334-348)
+  half_t *hidden = nullptr, *normed = nullptr, *qkv = nullptr, *q = nullptr, *ctx = nullptr, *mid = nullptr,
+         *logits = nullptr;
+  // workspaces
+  float* gemv_partials = nullptr;
+  int32_t* gemv_counters = nullptr;
+  void* attn_ws = nullptr;
+  void* argmax_ws = nullptr;
+  StepState* d_state = nullptr;
+  int32_t* d_token = nullptr;
+  int32_t* d_out = nullptr;
+  // sequence state
+  int current_seq_len = 0;  // current_seq_len_ of Inference.cu:408
+  int n_positions = 0;      // forward passes since reset
+  int n_generated = 0;
+  bool finalized = false;
+  bool graph_mode = true;
+  hipGraphExec_t graph_prompt = nullptr, graph_gen = nullptr;
+  std::vector<void*> allocations;
+};
+
+namespace {
+
+int dev_alloc(awq_engine* e, void** p, int64_t bytes) {
+  AWQ_HIP_TRY(hipMalloc(p, (size_t)(bytes > 0 ? bytes : 4)));
+  e->allocations.push_back(*p);
+  return AWQ_OK;
+}
+
+int dev_free(awq_engine* e, void* p) {
+  for (auto& a : e->allocations)
+    if (a == p) {
+      a = nullptr;
+      AWQ_HIP_TRY(hipFree(p));
+      return AWQ_OK;
+    }
+  return AWQ_OK;
+}
+
+DevLinear* find_linear(awq_engine* e, int layer, int kind) {
+  if (kind == AWQ_T_EMBED) return &e->embed;
+  if (kind == AWQ_T_UNEMBED) return &e->unembed;
+  if (layer < 0 || layer >= e->cfg.n_layers) return nullptr;
+  switch (kind) {
+    case AWQ_T_WQKV: return &e->layers[layer].wqkv;
+    case AWQ_T_WO: return &e->layers[layer].wo;
+    case AWQ_T_W1: return &e->layers[layer].w1;
+    case AWQ_T_W2: return &e->layers[layer].w2;
+  }
+  return nullptr;
+}
+
+int alloc_linear(awq_engine* e, DevLinear& t, int kind) {
+  awq_tensor_dims(e->cfg, kind, &t.m, &t.k);
+  if (int rc = dev_alloc(e, (void**)&t.packed, part_bytes(e->cfg, kind, AWQ_P_PACKED))) return rc;
+  if (int rc = dev_alloc(e, (void**)&t.scale, part_bytes(e->cfg, kind, AWQ_P_SCALE))) return rc;
+  if (int rc = dev_alloc(e, (void**)&t.zp, part_bytes(e->cfg, kind, AWQ_P_ZP))) return rc;
+  return AWQ_OK;
+}
+
+bool zp_all_integral(const uint16_t* zp, int64_t n) {
+  for (int64_t i = 0; i < n; ++i) {
+    half_t h;
+    memcpy(&h, &zp[i], 2);
+    float f = (float)h;
+    if (!(f >= 0.0f && f <= 1024.0f) || f != (float)(int)f) return false;
+  }
+  return true;
+}
+
+// one fused-linear launch on the engine's stream
+int linear(awq_engine* e, const DevLinear& t, const half_t* x, half_t* y, int epilogue, const half_t* res) {
+  LinearArgs a;
+  a.wq = t.stream_order;
+  a.scale = t.scale;
+  a.zp = t.zp;
+  a.x = x;
+  a.y = y;
+  a.res = res;
+  a.partials = e->gemv_partials;
+  a.counters = e->gemv_counters;
+  a.m = t.m;
+  a.k = t.k;
+  a.zp_integral = t.zp_integral;
+  a.epilogue = epilogue;
+  return launch_gemv(a, e->stream);
+}
+
+// runOneLayer, Inference.cu:1029-1230.  The attended length comes from the
+// device-side step state: len_lo or len_hi.
+int enqueue_layer(awq_engine* e, int l, int use_len_hi) {
+  LayerDev& L = e->layers[l];
+  const int H = e->cfg.hidden;
+  hipStream_t st = e->stream;
+  if (int rc = launch_rmsnorm(e->hidden, L.gamma, e->normed, H, e->cfg.eps, st)) return rc;  // :1040
+  if (int rc = linear(e, L.wqkv, e->normed, e->qkv, EPI_STORE, nullptr)) return rc;          // :1052
+  if (int rc = launch_rope_kv_append(e->qkv, e->cos_t, e->sin_t, e->q, L.kcache, L.vcache, e->n_heads, e->cfg.max_pos,
+                                     0, e->d_state, st))
+    return rc;  // :1070-1103
+  if (int rc = launch_attention(e->q, L.kcache, L.vcache, e->ctx, e->n_heads, e->cfg.max_pos, 0, e->d_state,
+                                use_len_hi, e->attn_ws, st))
+    return rc;  // :1110
+  // :1128-1155, Wo product and residual add in one launch; input and output
+  // are distinct buffers (they alias in the reference)
+  if (int rc = linear(e, L.wo, e->ctx, e->hidden, EPI_RESIDUAL, e->hidden)) return rc;
+  if (int rc = launch_rmsnorm(e->hidden, L.gamma, e->normed, H, e->cfg.eps, st)) return rc;  // :1163, same gamma
+  if (int rc = linear(e, L.w1, e->normed, e->mid, EPI_GELU, nullptr)) return rc;             // :1176, :1196
+  if (int rc = linear(e, L.w2, e->mid, e->hidden, EPI_RESIDUAL, e->hidden)) return rc;       // :1201, :1227
+  return AWQ_OK;
+}
+
+// sampleNextToken, Inference.cu:1235-1292
+int enqueue_sample(awq_engine* e) {
+  hipStream_t st = e->stream;
+  const int NL = e->cfg.n_layers;
+  if (int rc = launch_rmsnorm(e->hidden, e->layers[NL - 1].gamma, e->normed, e->cfg.hidden, e->cfg.eps, st)) return rc;
+  if (int rc = linear(e, e->unembed, e->normed, e->logits, EPI_STORE, nullptr)) return rc;
+  return launch_argmax(e->logits, e->cfg.vocab, e->d_token, e->argmax_ws, e->d_state, e->d_out, st);
+}
+
+// everything of one position after the step state has been written
+int enqueue_step_body(awq_engine* e, bool gen) {
+  // embedding gather (Inference.cu:1310-1324, 1384-1398), skipped on the device
+  // when the state says to keep the hidden state (:1357)
+  if (int rc = launch_embed(e->embed.packed, e->embed.scale, e->embed.zp, e->cfg.hidden, e->cfg.vocab, 0, e->d_state,
+                            e->d_token, e->hidden, e->stream))
+    return rc;
+  const int split = gen ? e->cfg.split_idx : 1;
+  for (int l = 0; l < e->cfg.n_layers; ++l)
+    if (int rc = enqueue_layer(e, l, l >= split)) return rc;
+  if (gen) return enqueue_sample(e);
+  return AWQ_OK;
+}
+
+int build_graph(awq_engine* e, bool gen, hipGraphExec_t* out) {
+  hipGraph_t graph = nullptr;
+  AWQ_HIP_TRY(hipStreamBeginCapture(e->stream, hipStreamCaptureModeThreadLocal));
+  int rc = enqueue_step_body(e, gen);
+  hipError_t err = hipStreamEndCapture(e->stream, &graph);
+  if (rc) {
+    if (graph) hipGraphDestroy(graph);
+    return rc;
+  }
+  AWQ_HIP_TRY(err);
+  AWQ_HIP_TRY(hipGraphInstantiate(out, graph, nullptr, nullptr, 0));
+  AWQ_HIP_TRY(hipGraphDestroy(graph));
+  return AWQ_OK;
+}
+
+int run_step(awq_engine* e, bool gen, const StepState& s) {
+  if (int rc = launch_set_state(e->d_state, s, e->stream)) return rc;
+  if (e->graph_mode) {
+    hipGraphExec_t* g = gen ? &e->graph_gen : &e->graph_prompt;
+    if (!*g)
+      if (int rc = build_graph(e, gen, g)) return rc;
+    AWQ_HIP_TRY(hipGraphLaunch(*g, e->stream));
+    return AWQ_OK;
+  }
+  return enqueue_step_body(e, gen);
+}
+
+int read_file(const std::string& path, int64_t bytes, std::vector<uint8_t>& staging) {
+  FILE* f = fopen(path.c_str(), "rb");
+  if (!f) {
+    awq_set_error("could not open " + path);  // Inference.cu:299-302
+    return AWQ_ERR_IO;
+  }
+  staging.resize((size_t)bytes);
+  size_t got = fread(staging.data(), 1, (size_t)bytes, f);
+  fclose(f);
+  if ((int64_t)got != bytes) {
+    awq_set_error("read failed for " + path);  // :305-308
+    return AWQ_ERR_IO;
+  }
+  return AWQ_OK;
+}
+
+}  // namespace
+
+extern "C" int awq_create_empty(const awq_config* cfg_in, awq_engine** out) {
+  AWQ_REQUIRE(out != nullptr, "out is NULL");
+  *out = nullptr;
+  awq_config cfg;
+  if (cfg_in) cfg = *cfg_in;
+  else awq_default_config(&cfg);
+  if (int rc = awq_check_config(&cfg)) return rc;
+  int ndev = 0;
+  AWQ_HIP_TRY(hipGetDeviceCount(&ndev));
+  if (ndev < 1) {
+    awq_set_error("no HIP device found");
+    return AWQ_ERR_HIP;
+  }
+  std::unique_ptr<awq_engine> e(new awq_engine());
+  e->cfg = cfg;
+  e->n_heads = cfg.hidden / AWQ_HEAD_DIM;
+  AWQ_HIP_TRY(hipGetDevice(&e->device));
+  AWQ_HIP_TRY(hipStreamCreateWithFlags(&e->stream, hipStreamNonBlocking));
+  e->layers.resize(cfg.n_layers);
+  awq_engine* ep = e.get();
+  auto fail = [&](int rc) {
+    awq_destroy(e.release());
+    return rc;
+  };
+  const int64_t H = cfg.hidden, I = cfg.inter, V = cfg.vocab;
+  const int64_t kv_bytes = (int64_t)e->n_heads * cfg.max_pos * AWQ_HEAD_DIM * 2;  // Inference.cu:676
+  for (int l = 0; l < cfg.n_layers; ++l) {
+    LayerDev& L = e->layers[l];
+    if (int rc = alloc_linear(ep, L.wqkv, AWQ_T_WQKV)) return fail(rc);
+    if (int rc = alloc_linear(ep, L.wo, AWQ_T_WO)) return fail(rc);
+    if (int rc = alloc_linear(ep, L.w1, AWQ_T_W1)) return fail(rc);
+    if (int rc = alloc_linear(ep, L.w2, AWQ_T_W2)) return fail(rc);
+    if (int rc = dev_alloc(ep, (void**)&L.gamma, H * 2)) return fail(rc);
+    if (int rc = dev_alloc(ep, (void**)&L.kcache, kv_bytes)) return fail(rc);
+    if (int rc = dev_alloc(ep, (void**)&L.vcache, kv_bytes)) return fail(rc);
+  }
+  if (int rc = alloc_linear(ep, e->embed, AWQ_T_EMBED)) return fail(rc);
+  if (int rc = alloc_linear(ep, e->unembed, AWQ_T_UNEMBED)) return fail(rc);
+  const int64_t table_bytes = (int64_t)cfg.max_pos * (AWQ_HEAD_DIM / 2) * 2;
+  if (int rc = dev_alloc(ep, (void**)&e->cos_t, table_bytes)) return fail(rc);
+  if (int rc = dev_alloc(ep, (void**)&e->sin_t, table_bytes)) return fail(rc);
+  struct {
+    half_t** p;
+    int64_t n;
+  } acts[] = {{&e->hidden, H}, {&e->normed, H}, {&e->qkv, 3 * H}, {&e->q, H},     {&e->ctx, H},
+              {&e->mid, I},    {&e->logits, V}};
+  for (auto& a : acts)
+    if (int rc = dev_alloc(ep, (void**)a.p, a.n * 2)) return fail(rc);
+  int64_t max_m = std::max<int64_t>(std::max<int64_t>(3 * H, I), V);
+  if (int rc = dev_alloc(ep, (void**)&e->gemv_partials, 16 * max_m * 4)) return fail(rc);
+  if (int rc = dev_alloc(ep, (void**)&e->gemv_counters, (max_m / 64 + 1) * 4)) return fail(rc);
+  if (int rc = dev_alloc(ep, &e->attn_ws, attention_workspace_bytes(e->n_heads, cfg.max_pos))) return fail(rc);
+  if (int rc = dev_alloc(ep, &e->argmax_ws, argmax_workspace_bytes(V))) return fail(rc);
+  if (int rc = dev_alloc(ep, (void**)&e->d_state, sizeof(StepState))) return fail(rc);
+  if (int rc = dev_alloc(ep, (void**)&e->d_token, 4)) return fail(rc);
+  if (int rc = dev_alloc(ep, (void**)&e->d_out, (int64_t)cfg.max_pos * 4)) return fail(rc);
+  *out = e.release();
+  return AWQ_OK;
+}
+
+extern "C" int awq_upload(awq_engine* e, int layer, int kind, int part, const void* host_src, int64_t bytes) {
+  AWQ_REQUIRE(e && host_src, "NULL argument");
+  if (e->finalized) {
+    awq_set_error("awq_upload after awq_finalize");
+    return AWQ_ERR_STATE;
+  }
+  AWQ_REQUIRE(kind >= AWQ_T_WQKV && kind <= AWQ_T_UNEMBED, "bad tensor kind");
+  int64_t need = part_bytes(e->cfg, kind, part);
+  AWQ_REQUIRE(bytes == need, "byte count " + std::to_string((long long)bytes) + " != expected " +
+                                 std::to_string((long long)need));
+  if (kind == AWQ_T_GAMMA) {
+    AWQ_REQUIRE(layer >= 0 && layer < e->cfg.n_layers, "layer out of range");
+    AWQ_HIP_TRY(hipMemcpy(e->layers[layer].gamma, host_src, (size_t)bytes, hipMemcpyHostToDevice));  // :309
+    e->layers[layer].have_gamma = true;
+    return AWQ_OK;
+  }
+  AWQ_REQUIRE(part >= AWQ_P_PACKED && part <= AWQ_P_ZP, "bad tensor part");
+  DevLinear* t = find_linear(e, layer, kind);
+  AWQ_REQUIRE(t != nullptr, "layer out of range");
+  void* dst = part == AWQ_P_PACKED ? (void*)t->packed : part == AWQ_P_SCALE ? (void*)t->scale : (void*)t->zp;
+  AWQ_HIP_TRY(hipMemcpy(dst, host_src, (size_t)bytes, hipMemcpyHostToDevice));
+  if (part == AWQ_P_ZP) t->zp_integral = zp_all_integral((const uint16_t*)host_src, bytes / 2);
+  t->have[part] = true;
+  return AWQ_OK;
+}
+
+extern "C" int awq_finalize(awq_engine* e) {
+  AWQ_REQUIRE(e != nullptr, "engine is NULL");
+  if (e->finalized) return AWQ_OK;
+  // everything uploaded?
+  for (int l = 0; l < e->cfg.n_layers; ++l) {
+    LayerDev& L = e->layers[l];
+    DevLinear* ts[4] = {&L.wqkv, &L.wo, &L.w1, &L.w2};
+    for (DevLinear* t : ts)
+      if (!(t->have[0] && t->have[1] && t->have[2])) {
+        awq_set_error("layer " + std::to_string(l) + " has tensors that were never uploaded");
+        return AWQ_ERR_STATE;
+      }
+    if (!L.have_gamma) {
+      awq_set_error("gamma of layer " + std::to_string(l) + " was never uploaded");
+      return AWQ_ERR_STATE;
+    }
+  }
+  for (DevLinear* t : {&e->embed, &e->unembed})
+    if (!(t->have[0] && t->have[1] && t->have[2])) {
+      awq_set_error("embedding or unembedding was never uploaded");
+      return AWQ_ERR_STATE;
+    }
+  hipStream_t st = e->stream;
+  // reorder every linear layer's stream; the file-order copy is then dropped.
+  // The embedding is only ever gathered from, so it stays in file order.
+  std::vector<DevLinear*> all;
+  for (auto& L : e->layers) {
+    all.push_back(&L.wqkv);
+    all.push_back(&L.wo);
+    all.push_back(&L.w1);
+    all.push_back(&L.w2);
+  }
+  all.push_back(&e->unembed);
+  for (DevLinear* t : all) {
+    if (int rc = dev_alloc(e, &t->stream_order, t->m * (t->k / 2))) return rc;
+    if (int rc = launch_repack(t->packed, t->stream_order, t->m, t->k, st)) return rc;
+    AWQ_HIP_TRY(hipStreamSynchronize(st));
+    if (int rc = dev_free(e, t->packed)) return rc;
+    t->packed = nullptr;
+  }
+  // rotary tables, Inference.cu:443-464
+  {
+    std::vector<uint16_t> c((size_t)e->cfg.max_pos * 64), s(c.size());
+    if (int rc = awq_rope_tables_host(c.data(), s.data(), e->cfg.max_pos)) return rc;
+    AWQ_HIP_TRY(hipMemcpy(e->cos_t, c.data(), c.size() * 2, hipMemcpyHostToDevice));
+    AWQ_HIP_TRY(hipMemcpy(e->sin_t, s.data(), s.size() * 2, hipMemcpyHostToDevice));
+  }
+  // zero the KV caches (Inference.cu:431-437) and the self-resetting workspaces
+  const int64_t kv_bytes = (int64_t)e->n_heads * e->cfg.max_pos * AWQ_HEAD_DIM * 2;
+  for (auto& L : e->layers) {
+    if (int rc = launch_fill_zero(L.kcache, kv_bytes, st)) return rc;
+    if (int rc = launch_fill_zero(L.vcache, kv_bytes, st)) return rc;
+  }
+  int64_t max_m = std::max<int64_t>(std::max<int64_t>(3 * (int64_t)e->cfg.hidden, e->cfg.inter), e->cfg.vocab);
+  if (int rc = launch_fill_zero(e->gemv_counters, (max_m / 64 + 1) * 4, st)) return rc;
+  if (int rc = launch_fill_zero(e->argmax_ws, 64, st)) return rc;
+  if (int rc = launch_fill_zero(e->d_token, 4, st)) return rc;
+  if (int rc = launch_fill_zero(e->hidden, (int64_t)e->cfg.hidden * 2, st)) return rc;
+  AWQ_HIP_TRY(hipStreamSynchronize(st));
+  e->finalized = true;
+  return awq_reset(e);
+}
+
+extern "C" int awq_create(const char* weight_dir, const awq_config* cfg_in, awq_engine** out) {
+  AWQ_REQUIRE(weight_dir != nullptr && out != nullptr, "NULL argument");
+  *out = nullptr;
+  // look at the directory before touching the GPU
+  if (int rc = awq_validate_weight_dir(weight_dir, cfg_in)) return rc;
+  awq_engine* e = nullptr;
+  if (int rc = awq_create_empty(cfg_in, &e)) return rc;
+  std::vector<uint8_t> staging;
+  for (const WeightFile& wf : awq_weight_files(e->cfg)) {
+    int rc = read_file(std::string(weight_dir) + "/" + wf.name, wf.bytes, staging);
+    if (!rc) rc = awq_upload(e, wf.layer, wf.kind, wf.part, staging.data(), wf.bytes);
+    if (rc) {
+      awq_destroy(e);
+      return rc;
+    }
+  }
+  if (int rc = awq_finalize(e)) {
+    awq_destroy(e);
+    return rc;
+  }
+  *out = e;
+  return AWQ_OK;
+}
+
+extern "C" void awq_destroy(awq_engine* e) {
+  if (!e) return;
+  if (e->stream) (void)hipStreamSynchronize(e->stream);
+  if (e->graph_prompt) (void)hipGraphExecDestroy(e->graph_prompt);
+  if (e->graph_gen) (void)hipGraphExecDestroy(e->graph_gen);
+  for (void* p : e->allocations)
+    if (p) (void)hipFree(p);
+  if (e->stream) (void)hipStreamDestroy(e->stream);
+  delete e;
+}
+
+extern "C" int awq_set_graph_mode(awq_engine* e, int enabled) {
+  AWQ_REQUIRE(e != nullptr, "engine is NULL");
+  e->graph_mode = enabled != 0;
+  return AWQ_OK;
+}
+
+extern "C" int awq_reset(awq_engine* e) {
+  AWQ_REQUIRE(e != nullptr, "engine is NULL");
+  if (!e->finalized) {
+    awq_set_error("awq_reset before awq_finalize");
+    return AWQ_ERR_STATE;
+  }
+  // The reference initialises current_seq_len_ in the constructor only
+  // (Inference.cu:430); a second generateResponse would attend stale positions.
+  // Each sequence starts clean here, with a zero hidden state.
+  e->current_seq_len = 0;
+  e->n_positions = 0;
+  e->n_generated = 0;
+  if (int rc = launch_fill_zero(e->hidden, (int64_t)e->cfg.hidden * 2, e->stream)) return rc;
+  AWQ_HIP_TRY(hipStreamSynchronize(e->stream));
+  return AWQ_OK;
+}
+
+// prompt loop, Inference.cu:1304-1343
+extern "C" int awq_prefill(awq_engine* e, const int32_t* prompt_ids, int32_t n_prompt) {
+  AWQ_REQUIRE(e != nullptr && n_prompt >= 0 && (n_prompt == 0 || prompt_ids), "bad arguments");
+  if (!e->finalized) {
+    awq_set_error("awq_prefill before awq_finalize");
+    return AWQ_ERR_STATE;
+  }
+  AWQ_REQUIRE(e->n_generated == 0, "prompt tokens cannot follow generated ones; call awq_reset");
+  AWQ_REQUIRE((int64_t)e->n_positions + n_prompt <= e->cfg.max_pos, "prompt does not fit max_pos");
+  for (int32_t i = 0; i < n_prompt; ++i) {
+    AWQ_REQUIRE(prompt_ids[i] >= 0 && prompt_ids[i] < e->cfg.vocab, "token id out of range");
+    const int t = e->n_positions;
+    StepState s;
+    s.pos = t;
+    s.len_lo = e->current_seq_len + 1;  // layer 0 still sees the previous value (:1118 before :1331)
+    s.len_hi = t + 1;                   // later layers see current_seq_len_ = t
+    s.token = prompt_ids[i];
+    s.out_index = 0;
+    s.sample = 0;
+    if (int rc = run_step(e, false, s)) return rc;
+    e->current_seq_len = t;
+    e->n_positions = t + 1;
+  }
+  AWQ_HIP_TRY(hipStreamSynchronize(e->stream));
+  return AWQ_OK;
+}
+
+// generation loop, Inference.cu:1352-1405
+extern "C" int awq_decode(awq_engine* e, int32_t n_steps, int32_t* out_ids) {
+  AWQ_REQUIRE(e != nullptr && n_steps >= 0 && (n_steps == 0 || out_ids), "bad arguments");
+  if (!e->finalized) {
+    awq_set_error("awq_decode before awq_finalize");
+    return AWQ_ERR_STATE;
+  }
+  AWQ_REQUIRE((int64_t)e->n_positions + n_steps <= e->cfg.max_pos, "sequence does not fit max_pos");
+  const int first = e->n_generated;
+  for (int32_t i = 0; i < n_steps; ++i) {
+    const int pos = e->n_positions;
+    StepState s;
+    s.pos = pos;
+    s.len_lo = e->current_seq_len + 1;  // layers below split_idx run before :1364
+    s.len_hi = pos + 1;                 // the others after it
+    // first step: the hidden state left by the last layer is the input (:1357);
+    // afterwards: the embedding of the token sampled by the previous step (:1392)
+    s.token = (e->n_generated == 0) ? -1 : -2;
+    s.out_index = e->n_generated;
+    s.sample = 1;
+    if (int rc = run_step(e, true, s)) return rc;
+    e->current_seq_len = pos;
+    e->n_positions = pos + 1;
+    e->n_generated += 1;
+  }
+  AWQ_HIP_TRY(hipStreamSynchronize(e->stream));
+  if (n_steps > 0)
+    AWQ_HIP_TRY(hipMemcpy(out_ids, e->d_out + first, (size_t)n_steps * 4, hipMemcpyDeviceToHost));
+  return AWQ_OK;
+}
+
+extern "C" int awq_generate(awq_engine* e, const int32_t* prompt_ids, int32_t n_prompt, int32_t max_new_tokens,
+                            int32_t* out_ids) {
+  AWQ_REQUIRE(e != nullptr, "engine is NULL");
+  AWQ_REQUIRE(n_prompt >= 0 && max_new_tokens >= 0, "negative count");
+  AWQ_REQUIRE((int64_t)n_prompt + max_new_tokens <= e->cfg.max_pos, "prompt + new tokens exceed max_pos");
+  if (int rc = awq_reset(e)) return rc;
+  if (int rc = awq_prefill(e, prompt_ids, n_prompt)) return rc;
+  return awq_decode(e, max_new_tokens, out_ids);
+}
+
+extern "C" int awq_read_hidden(awq_engine* e, uint16_t* host_dst) {
+  AWQ_REQUIRE(e && host_dst, "NULL argument");
+  AWQ_HIP_TRY(hipStreamSynchronize(e->stream));
+  AWQ_HIP_TRY(hipMemcpy(host_dst, e->hidden, (size_t)e->cfg.hidden * 2, hipMemcpyDeviceToHost));
+  return AWQ_OK;
+}
+
+extern "C" int awq_read_logits(awq_engine* e, uint16_t* host_dst) {
+  AWQ_REQUIRE(e && host_dst, "NULL argument");
+  AWQ_HIP_TRY(hipStreamSynchronize(e->stream));
+  AWQ_HIP_TRY(hipMemcpy(host_dst, e->logits, (size_t)e->cfg.vocab * 2, hipMemcpyDeviceToHost));
+  return AWQ_OK;
+}
+
+// ---------------------------------------------------------------------------
+// kernel-level entry points
+// ---------------------------------------------------------------------------
+extern "C" int awq_dequant(const void* packed, const void* scale, const void* zp, void* out, int64_t rows, int64_t cols,
+                           int64_t n_groups, void* stream) {
+  AWQ_REQUIRE(packed && scale && zp && out, "NULL pointer");
+  return launch_dequant((const uint8_t*)packed, (const half_t*)scale, (const half_t*)zp, (half_t*)out, rows, cols,
+                        n_groups, (hipStream_t)stream);
+}
+
+extern "C" int awq_linear_repack(const void* packed_in, void* repacked_out, int64_t m, int64_t k, void* stream) {
+  AWQ_REQUIRE(packed_in && repacked_out && packed_in != repacked_out, "NULL or aliased pointers");
+  return launch_repack((const uint8_t*)packed_in, repacked_out, m, k, (hipStream_t)stream);
+}
+
+extern "C" int64_t awq_gemv_workspace_bytes(int64_t m, int64_t k) { return gemv_workspace_bytes(m, k); }
+
+extern "C" int awq_gemv(const void* repacked, const void* scale, const void* zp, int64_t m, int64_t k, const void* x,
+                        void* y, int32_t zp_integral, void* workspace, void* stream) {
+  AWQ_REQUIRE(repacked && scale && zp && x && y && workspace, "NULL pointer");
+  AWQ_REQUIRE(m > 0 && m % 128 == 0, "m must be a positive multiple of 128");
+  if (zp_integral < 0) {
+    // look at the zero-points on the device (synchronises the stream)
+    std::vector<uint16_t> zph((size_t)(m / 128));
+    AWQ_HIP_TRY(hipMemcpyAsync(zph.data(), zp, zph.size() * 2, hipMemcpyDeviceToHost, (hipStream_t)stream));
+    AWQ_HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+    zp_integral = zp_all_integral(zph.data(), (int64_t)zph.size());
+  }
+  LinearArgs a;
+  a.wq = repacked;
+  a.scale = (const half_t*)scale;
+  a.zp = (const half_t*)zp;
+  a.x = (const half_t*)x;
+  a.y = (half_t*)y;
+  a.res = nullptr;
+  a.counters = (int32_t*)workspace;
+  a.partials = (float*)((char*)workspace + ((m / 64) * 4 + 255) / 256 * 256);
+  a.m = m;
+  a.k = k;
+  a.zp_integral = zp_integral != 0;
+  a.epilogue = EPI_STORE;
+  return launch_gemv(a, (hipStream_t)stream);
+}
+
+extern "C" int awq_rmsnorm(const void* x, const void* gamma, void* out, int64_t n, float eps, void* stream) {
+  AWQ_REQUIRE(x && gamma && out, "NULL pointer");
+  return launch_rmsnorm((const half_t*)x, (const half_t*)gamma, (half_t*)out, n, eps, (hipStream_t)stream);
+}
+
+extern "C" int awq_rope_kv_append(const void* qkv, const void* cos_t, const void* sin_t, void* q_out, void* k_cache,
+                                  void* v_cache, int32_t n_heads, int64_t max_pos, int64_t pos, void* stream) {
+  AWQ_REQUIRE(qkv && cos_t && sin_t && q_out && k_cache && v_cache, "NULL pointer");
+  return launch_rope_kv_append((const half_t*)qkv, (const half_t*)cos_t, (const half_t*)sin_t, (half_t*)q_out,
+                               (half_t*)k_cache, (half_t*)v_cache, n_heads, max_pos, pos, nullptr,
+                               (hipStream_t)stream);
+}
+
+extern "C" int64_t awq_attention_workspace_bytes(int32_t n_heads, int64_t max_pos) {
+  return attention_workspace_bytes(n_heads, max_pos);
+}
+
+extern "C" int awq_decode_attention(const void* q, const void* k_cache, const void* v_cache, void* ctx, int32_t n_heads,
+                                    int64_t max_pos, int64_t L, void* workspace, void* stream) {
+  AWQ_REQUIRE(q && k_cache && v_cache && ctx, "NULL pointer");
+  return launch_attention((const half_t*)q, (const half_t*)k_cache, (const half_t*)v_cache, (half_t*)ctx, n_heads,
+                          max_pos, L, nullptr, 0, workspace, (hipStream_t)stream);
+}
+
+extern "C" int awq_residual_add(const void* a, const void* b, void* out, int64_t n, void* stream) {
+  AWQ_REQUIRE(a && b && out, "NULL pointer");
+  return launch_residual((const half_t*)a, (const half_t*)b, (half_t*)out, n, (hipStream_t)stream);
+}
+
+extern "C" int awq_gelu(void* x, int64_t n, void* stream) {
+  AWQ_REQUIRE(x != nullptr, "NULL pointer");
+  return launch_gelu((half_t*)x, n, (hipStream_t)stream);
+}
+
+extern "C" int64_t awq_argmax_workspace_bytes(int64_t n) { return argmax_workspace_bytes(n); }
+
+extern "C" int awq_logits_argmax(const void* logits, int64_t n, void* out_token, void* workspace, void* stream) {
+  AWQ_REQUIRE(logits && out_token, "NULL pointer");
+  return launch_argmax((const half_t*)logits, n, (int32_t*)out_token, workspace, nullptr, nullptr, (hipStream_t)stream);
+}
+
+extern "C" int awq_embed_gather(const void* packed, const void* scale, const void* zp, int64_t hidden, int64_t vocab,
+                                int32_t tok, void* out, void* stream) {
+  AWQ_REQUIRE(packed && scale && zp && out, "NULL pointer");
+  return launch_embed((const uint8_t*)packed, (const half_t*)scale, (const half_t*)zp, hidden, vocab, tok, nullptr,
+                      nullptr, (half_t*)out, (hipStream_t)stream);
+}

@@ -1,0 +1,170 @@
+/*
+ * awq_infer.h -- C ABI of the MI355X AWQ int4 decode engine.
+ *
+ * Plain pointers and sizes only.  Every function that can fail returns 0 on
+ * success and a non-zero code otherwise; awq_last_error() then describes the
+ * failure for the calling thread.  (The reference prints to stderr and calls
+ * exit(1), Inference.cu:52-71; the C++ wrapper class QWen3AWQInfer restores
+ * that behaviour on top of these codes.)
+ *
+ * Device pointers are HIP device addresses; `stream` is a hipStream_t passed
+ * as void* (NULL = the default stream).  Kernel entry points only enqueue
+ * work; they do not synchronise.  FP16 data is IEEE binary16 stored as
+ * uint16_t.
+ */
+#ifndef AWQ_INFER_H
+#define AWQ_INFER_H
+
+#include <stdint.h>
+#include "awq_synth.h" /* enum awq_tensor_kind / awq_tensor_part */
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define AWQ_OK 0
+#define AWQ_ERR_ARG 1     /* bad argument or unsupported shape */
+#define AWQ_ERR_IO 2      /* missing or short weight file */
+#define AWQ_ERR_HIP 3     /* a HIP runtime call failed */
+#define AWQ_ERR_STATE 4   /* call order violated (e.g. generate before finalize) */
+
+/* Model shape.  awq_default_config gives the constants of Inference.cu:33-47. */
+typedef struct awq_config {
+  int32_t n_layers;   /* NUM_HIDDEN_LAYERS 36    Inference.cu:37 */
+  int32_t hidden;     /* HIDDEN_SIZE 4096        Inference.cu:33, multiple of 256 */
+  int32_t inter;      /* INTERMEDIATE_SIZE 12288 Inference.cu:34, multiple of 128 */
+  int32_t vocab;      /* VOCAB_SIZE 151936       Inference.cu:38, multiple of 128 */
+  int32_t max_pos;    /* MAX_POS_EMBEDDINGS 40960 Inference.cu:39, KV cache rows per head */
+  int32_t split_idx;  /* SPLIT_IDX 18            Inference.cu:47: layers below it attend one
+                         position fewer during generation (Inference.cu:1118 with 1364) */
+  float eps;          /* RMS_NORM_EPS 1e-6       Inference.cu:41 */
+} awq_config;
+
+typedef struct awq_engine awq_engine;
+
+const char* awq_last_error(void);
+void awq_default_config(awq_config* cfg);
+
+/* ----------------------------------------------------------------------------
+ * Engine: replaces class QWen3AWQInfer (Inference.cu:356-415).
+ * ------------------------------------------------------------------------- */
+
+/* Host-only check that `dir` holds every file of Inference.cu:780-899 with at
+ * least the expected byte count.  Touches no GPU. */
+int awq_validate_weight_dir(const char* dir, const awq_config* cfg);
+
+/* Constructor, Inference.cu:422-470: loads the weight directory onto the
+ * current device, repacks, builds rotary tables, zeroes the KV cache.
+ * cfg == NULL means the reference constants. */
+int awq_create(const char* weight_dir, const awq_config* cfg, awq_engine** out);
+
+/* Same engine without a directory: allocate, then awq_upload every array, then
+ * awq_finalize.  Used with in-memory synthetic weights. */
+int awq_create_empty(const awq_config* cfg, awq_engine** out);
+int awq_upload(awq_engine* e, int layer, int kind, int part, const void* host_src, int64_t bytes);
+int awq_finalize(awq_engine* e);
+
+/* generateResponse, Inference.cu:1297-1408.  Writes max_new_tokens ids to
+ * out_ids.  Restarts from an empty sequence on every call.  Fails (instead of
+ * the reference's assert / cache overrun) when n_prompt + max_new_tokens >
+ * max_pos. */
+int awq_generate(awq_engine* e, const int32_t* prompt_ids, int32_t n_prompt, int32_t max_new_tokens,
+                 int32_t* out_ids);
+
+/* The same loop in pieces, for timing: reset, the prompt loop
+ * (Inference.cu:1304-1343), then n_steps generation steps
+ * (Inference.cu:1352-1405).  awq_decode returns after the device finished. */
+int awq_reset(awq_engine* e);
+int awq_prefill(awq_engine* e, const int32_t* prompt_ids, int32_t n_prompt);
+int awq_decode(awq_engine* e, int32_t n_steps, int32_t* out_ids);
+
+/* Copies of internal state for tests: hidden state [hidden] and the logits of
+ * the last sampled position [vocab], both FP16, to host memory. */
+int awq_read_hidden(awq_engine* e, uint16_t* host_dst);
+int awq_read_logits(awq_engine* e, uint16_t* host_dst);
+/* 0: every op is its own launch; 1 (default): one captured graph per step */
+int awq_set_graph_mode(awq_engine* e, int enabled);
+
+/* Destructor, Inference.cu:475-558 */
+void awq_destroy(awq_engine* e);
+
+/* Writes a weight directory in the layout of Inference.cu:780-899 filled from
+ * awq_synth.h under `seed` (the reference ships no producer of its format). */
+int awq_write_weight_dir(const char* dir, const awq_config* cfg, uint64_t seed);
+
+/* Host-side synthetic data (awq_synth.h).  `count` is in elements of the
+ * array: bytes for AWQ_P_PACKED, halves otherwise. */
+int awq_synth_fill(uint64_t seed, int layer, int kind, int part, void* host_dst, int64_t count);
+int awq_synth_normal_f16(uint64_t seed, uint64_t stream, uint16_t* host_dst, int64_t count, float mean, float std);
+int awq_synth_tokens(uint64_t seed, uint64_t stream, int32_t* host_dst, int64_t count, int32_t vocab);
+
+/* Rotary tables, Inference.cu:443-454, computed on the host with libm as the
+ * reference does; cos_t / sin_t are host arrays of max_pos*64 halves. */
+int awq_rope_tables_host(uint16_t* cos_t, uint16_t* sin_t, int64_t max_pos);
+
+/* ----------------------------------------------------------------------------
+ * Kernels (device pointers).
+ * ------------------------------------------------------------------------- */
+
+/* dequantAwqKernel and its launches, Inference.cu:76-106, 908-1008.
+ * packed [rows][cols/2] bytes, scale/zp [n_groups] FP16, out [rows][cols] FP16.
+ * group = (col/128) % n_groups.  cols must be even. */
+int awq_dequant(const void* packed, const void* scale, const void* zp, void* out, int64_t rows, int64_t cols,
+                int64_t n_groups, void* stream);
+
+/* Load-time reordering of the packed int4 stream of an [m outputs x k inputs]
+ * matrix (file layout: nibble p = j*m + i, Inference.cu:1059 read of :105)
+ * into the order the product kernels stream it in.  Same byte count. */
+int awq_linear_repack(const void* packed_in, void* repacked_out, int64_t m, int64_t k, void* stream);
+
+/* cublasGemmEx with n = 1, Inference.cu:1052-1065, 1128-1141, 1176-1189,
+ * 1201-1214, 1260-1273, fused with the dequantisation:
+ *     y[i] = h( sum_j w(i,j) * x[j] ),  FP32 accumulation in the blocked order
+ *     of awq_canon_math.h.
+ * repacked from awq_linear_repack; scale/zp [m/128]; x [k], y [m] FP16.
+ * zp_integral: 1 when every zero-point is an integer in [0,1024] (true of AWQ
+ * checkpoints) -- a shorter instruction sequence with the same bits; 0 for
+ * arbitrary zero-points; -1 to have the call inspect them (synchronises).
+ * workspace: awq_gemv_workspace_bytes(m,k) bytes, zero-filled once before its
+ * first use (the kernel leaves it zeroed); must not be shared by launches that
+ * may overlap. */
+int64_t awq_gemv_workspace_bytes(int64_t m, int64_t k);
+int awq_gemv(const void* repacked, const void* scale, const void* zp, int64_t m, int64_t k, const void* x, void* y,
+             int32_t zp_integral, void* workspace, void* stream);
+
+/* rmsNormKernel, Inference.cu:111-145.  n multiple of 256. */
+int awq_rmsnorm(const void* x, const void* gamma, void* out, int64_t n, float eps, void* stream);
+
+/* QKV split (Inference.cu:1070-1077), applyRotaryKernel on Q and K
+ * (:1082-1091) and the KV-cache append (:1094-1103) in one launch.
+ * qkv [3*n_heads*128]; q_out [n_heads*128]; caches [n_heads][max_pos][128]. */
+int awq_rope_kv_append(const void* qkv, const void* cos_t, const void* sin_t, void* q_out, void* k_cache,
+                       void* v_cache, int32_t n_heads, int64_t max_pos, int64_t pos, void* stream);
+
+/* attentionKernel, Inference.cu:182-266, for one query over L cached
+ * positions.  workspace: awq_attention_workspace_bytes(n_heads, max_pos). */
+int64_t awq_attention_workspace_bytes(int32_t n_heads, int64_t max_pos);
+int awq_decode_attention(const void* q, const void* k_cache, const void* v_cache, void* ctx, int32_t n_heads,
+                         int64_t max_pos, int64_t L, void* workspace, void* stream);
+
+/* residual add lambda, Inference.cu:1149-1155: out = h(a + b); out may be a */
+int awq_residual_add(const void* a, const void* b, void* out, int64_t n, void* stream);
+
+/* geluKernel, Inference.cu:271-279, in place */
+int awq_gelu(void* x, int64_t n, void* stream);
+
+/* finalSoftmaxKernel + D2H + host argmax, Inference.cu:1278-1290, on device:
+ * *out_token (device int32) = lowest index of the largest FP16 logit.
+ * workspace: awq_argmax_workspace_bytes(n) bytes, zero-filled once. */
+int64_t awq_argmax_workspace_bytes(int64_t n);
+int awq_logits_argmax(const void* logits, int64_t n, void* out_token, void* workspace, void* stream);
+
+/* gather lambda, Inference.cu:1310-1324: out[idx] = dequantised
+ * word_embedding[idx][tok], read from the packed [hidden][vocab] file layout. */
+int awq_embed_gather(const void* packed, const void* scale, const void* zp, int64_t hidden, int64_t vocab,
+                     int32_t tok, void* out, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AWQ_INFER_H */

@@ -1,0 +1,135 @@
+"""numpy utilities shared by the tests: pointer plumbing, an independent numpy
+version of the seeded generator, reference packing helpers."""
+import ctypes
+
+import numpy as np
+
+MASK64 = (1 << 64) - 1
+
+
+def ptr(a):
+    """void* of a contiguous numpy array"""
+    assert a.flags["C_CONTIGUOUS"]
+    return a.ctypes.data_as(ctypes.c_void_p)
+
+
+def f16(bits):
+    return np.asarray(bits, dtype=np.uint16).view(np.float16)
+
+
+def bits16(x):
+    return np.asarray(x, dtype=np.float16).view(np.uint16)
+
+
+# ---- independent numpy statement of include/awq_synth.h ----------------------
+def synth_hash(seed, sid, idx):
+    idx = np.asarray(idx, dtype=np.uint64)
+    with np.errstate(over="ignore"):
+        z = (np.uint64((seed * 0x9E3779B97F4A7C15) & MASK64) + np.uint64(((sid + 1) * 0xD1B54A32D192ED03) & MASK64)
+             + idx * np.uint64(0xA0761D6478BD642F))
+        z ^= z >> np.uint64(30)
+        z *= np.uint64(0xBF58476D1CE4E5B9)
+        z ^= z >> np.uint64(27)
+        z *= np.uint64(0x94D049BB133111EB)
+        z ^= z >> np.uint64(31)
+    return z
+
+
+def synth_stream(layer, kind, part):
+    l = 0 if kind in (5, 6) else layer + 1
+    return l * 64 + kind * 4 + part
+
+
+def synth_packed(seed, layer, kind, nbytes):
+    words = synth_hash(seed, synth_stream(layer, kind, 0), np.arange((nbytes + 7) // 8, dtype=np.uint64))
+    return words.view(np.uint8)[:nbytes].copy()  # little endian host
+
+
+def synth_scale(seed, layer, kind, n):
+    h = synth_hash(seed, synth_stream(layer, kind, 1), np.arange(n, dtype=np.uint64))
+    u = (h >> np.uint64(40)).astype(np.float32) * np.float32(1.0 / 16777216.0)
+    return (np.float32(0.002) + np.float32(0.018) * u).astype(np.float16)
+
+
+def synth_zp(seed, layer, kind, n):
+    h = synth_hash(seed, synth_stream(layer, kind, 2), np.arange(n, dtype=np.uint64))
+    return (h & np.uint64(15)).astype(np.float32).astype(np.float16)
+
+
+def synth_normal(seed, sid, n):
+    idx = np.arange(n, dtype=np.uint64)
+    a = synth_hash(seed, sid, idx * np.uint64(2))
+    b = synth_hash(seed, sid, idx * np.uint64(2) + np.uint64(1))
+    u1 = ((a >> np.uint64(11)).astype(np.float64) + 1.0) * (1.0 / 9007199254740992.0)
+    u2 = (b >> np.uint64(11)).astype(np.float64) * (1.0 / 9007199254740992.0)
+    return np.sqrt(-2.0 * np.log(u1)) * np.cos(6.283185307179586 * u2)
+
+
+# ---- AWQ helpers --------------------------------------------------------------
+def nibbles_flat(packed):
+    """flat nibble stream: low nibble first (Inference.cu:95-99)"""
+    p = np.asarray(packed, dtype=np.uint8)
+    out = np.empty(p.size * 2, dtype=np.uint8)
+    out[0::2] = p & 15
+    out[1::2] = p >> 4
+    return out
+
+
+def dequant_numpy(packed, scale, zp, rows, cols, n_groups):
+    """(q - z) * s with binary16 rounding after each op, via numpy float16 arithmetic"""
+    q = nibbles_flat(packed).reshape(rows, cols).astype(np.float16)
+    g = (np.arange(cols) // 128) % n_groups
+    sub = (q - zp[g][None, :]).astype(np.float16)
+    return (sub * scale[g][None, :]).astype(np.float16)
+
+
+def effective_weights_f64(packed, scale, zp, m, k):
+    """W_eff[i, j] = dequantised flat element j*m + i (column-major read, Inference.cu:1059)"""
+    flat = dequant_numpy(packed, scale, zp, m, k, m // 128).reshape(-1)
+    return flat.astype(np.float64).reshape(k, m).T
+
+
+def block_elem(k, C, blk, t):
+    U = k // (32 * C)
+    c, u = divmod(blk, U)
+    return c + C * (32 * u + t)
+
+
+def repack_numpy(packed, m, k, C):
+    """numpy statement of the streaming order of the GPU kernels (see csrc/gemv.hip)"""
+    nib = nibbles_flat(packed).astype(np.uint32)
+    nblk = k // 32
+    out = np.zeros((m // 64, nblk, 64, 4), dtype=np.uint32)
+    rows = np.arange(m).reshape(m // 64, 64)
+    for blk in range(nblk):
+        for t in range(32):
+            j = block_elem(k, C, blk, t)
+            q = nib[j * m + rows]
+            tt = t & 7
+            pos = (tt >> 1) * 4 + (tt & 1) * 16
+            out[:, blk, :, t >> 3] |= q << np.uint32(pos)
+    return out.reshape(-1)
+
+
+# ---- engine / oracle pairs ----------------------------------------------------
+def make_oracle_model(oracle, cfg):
+    import oracle_lib
+    ocfg = oracle_lib.OracleConfig(cfg.n_layers, cfg.hidden, cfg.inter, cfg.vocab, cfg.max_pos, cfg.split_idx, cfg.eps)
+    return oracle.awqo_model_create(ctypes.byref(ocfg))
+
+
+def fill_pair(awq, oracle, cfg, seed, engine=None, model=None):
+    """Fill the oracle model's host arrays from the seeded generator and upload the very same
+    bytes to the engine."""
+    lib = awq.load_library()
+    for layer, kind, part in awq.tensor_list(cfg):
+        count = cfg.part_count(kind, part)
+        nbytes = count if (part == awq.P_PACKED and kind != awq.T_GAMMA) else 2 * count
+        got = ctypes.c_int64(0)
+        p = oracle.awqo_model_tensor(model, layer, kind, part, ctypes.byref(got))
+        assert got.value == nbytes, (layer, kind, part, got.value, nbytes)
+        awq.check(lib.awq_synth_fill(seed, layer, kind, part, p, count))
+        if engine is not None:
+            engine.upload(layer, kind, part, p, nbytes)
+    if engine is not None:
+        engine.finalize()

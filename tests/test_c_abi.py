@@ -1,0 +1,141 @@
+"""CPU-side checks of the drop-in boundary: the shared library loads without a GPU, exports every
+symbol that include/awq_infer.h declares, validates weight directories before touching HIP, and the
+seeded generator agrees with an independent numpy statement and with the committed fixture."""
+import ctypes
+import json
+import os
+import re
+import subprocess
+
+import numpy as np
+import pytest
+
+import helpers
+from helpers import ptr
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "awq_infer.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(awq_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol(awq, lib):
+    names = declared_functions()
+    assert len(names) >= 30
+    for n in names:
+        assert hasattr(lib, n), n
+        assert n in awq.SIGNATURES, "binding missing for " + n
+    assert set(awq.SIGNATURES) == set(names)
+
+
+def test_default_config_is_the_reference(awq):
+    c = awq.default_config()
+    assert (c.n_layers, c.hidden, c.inter, c.vocab, c.max_pos, c.split_idx) == (36, 4096, 12288, 151936, 40960, 18)
+    assert abs(c.eps - 1e-6) < 1e-12
+
+
+def test_weight_file_table_matches_reference_sizes(awq, lib, tmp_path):
+    """write the directory for a small shape and check names and sizes follow Inference.cu:780-899;
+    the full-size byte counts are checked arithmetically"""
+    cfg = awq.make_config(n_layers=2, hidden=512, inter=1024, vocab=1280, max_pos=16)
+    d = str(tmp_path)
+    awq.check(lib.awq_write_weight_dir(d.encode(), ctypes.byref(cfg), 5))
+    files = sorted(os.listdir(d))
+    assert len(files) == 2 * 13 + 6
+    assert os.path.getsize(os.path.join(d, "layer_1_w1.bin")) == 1024 * 512 // 2
+    assert os.path.getsize(os.path.join(d, "layer_1_w2_scale.bin")) == (512 // 128) * 2
+    assert os.path.getsize(os.path.join(d, "word_embedding.bin")) == 512 * 1280 // 2
+    assert os.path.getsize(os.path.join(d, "word_embed_zp.bin")) == (512 // 128) * 2
+    assert os.path.getsize(os.path.join(d, "unembed_scale.bin")) == (1280 // 128) * 2
+    assert lib.awq_validate_weight_dir(d.encode(), ctypes.byref(cfg)) == 0
+    # contents are the seeded stream
+    got = np.fromfile(os.path.join(d, "layer_1_wo.bin"), dtype=np.uint8)
+    assert np.array_equal(got, helpers.synth_packed(5, 1, awq.T_WO, got.size))
+    # missing file
+    os.remove(os.path.join(d, "rms_norm_gamma_0.bin"))
+    assert lib.awq_validate_weight_dir(d.encode(), ctypes.byref(cfg)) == 2
+    assert b"could not open" in lib.awq_last_error() and b"rms_norm_gamma_0.bin" in lib.awq_last_error()
+    # short file
+    open(os.path.join(d, "rms_norm_gamma_0.bin"), "wb").write(b"\0" * 10)
+    assert lib.awq_validate_weight_dir(d.encode(), ctypes.byref(cfg)) == 2
+    assert b"read failed" in lib.awq_last_error()
+    # awq_create refuses the directory before any GPU call
+    h = ctypes.c_void_p()
+    assert lib.awq_create(d.encode(), ctypes.byref(cfg), ctypes.byref(h)) == 2 and not h.value
+    # full-size totals of the reference layout
+    full = awq.default_config()
+    total = sum((n if (p == awq.P_PACKED and k != awq.T_GAMMA) else 2 * n)
+                for (l, k, p) in awq.tensor_list(full) for n in [full.part_count(k, p)])
+    assert total == 3642565388
+    assert len(awq.tensor_list(full)) == 474
+
+
+def test_bad_configs_are_rejected(awq, lib, tmp_path):
+    for kw in [dict(hidden=500), dict(inter=100), dict(vocab=100), dict(max_pos=0), dict(n_layers=0),
+               dict(max_pos=70000)]:
+        base = dict(n_layers=2, hidden=512, inter=1024, vocab=1280, max_pos=16)
+        base.update(kw)
+        cfg = awq.make_config(**base)
+        assert lib.awq_validate_weight_dir(str(tmp_path).encode(), ctypes.byref(cfg)) == 1, kw
+
+
+def test_cli_usage_error():
+    exe = os.path.join(ROOT, "cuda-kernel-qwen3-8b-awq_amd", "qwen3_awq_infer")
+    res = subprocess.run([exe], capture_output=True, text=True)
+    assert res.returncode == 1 and "Usage:" in res.stderr          # Inference.cu:1414-1417
+    res = subprocess.run([exe, "/nonexistent-dir"], capture_output=True, text=True)
+    assert res.returncode == 1 and "could not open" in res.stderr  # Inference.cu:299-302
+
+
+def test_synth_matches_numpy_and_fixture(awq, lib):
+    seed = 42
+    fx = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "synth_seed42.json")))
+    # packed bytes
+    buf = np.zeros(1000, dtype=np.uint8)
+    awq.check(lib.awq_synth_fill(seed, 3, awq.T_W1, awq.P_PACKED, ptr(buf), buf.size))
+    assert np.array_equal(buf, helpers.synth_packed(seed, 3, awq.T_W1, 1000))
+    assert buf[:16].tolist() == fx["w1_layer3_packed_first16"]
+    # scale and zero-point
+    sc = np.zeros(96, dtype=np.float16)
+    awq.check(lib.awq_synth_fill(seed, 3, awq.T_W1, awq.P_SCALE, ptr(sc), sc.size))
+    assert np.array_equal(sc.view(np.uint16), helpers.synth_scale(seed, 3, awq.T_W1, 96).view(np.uint16))
+    assert sc[:8].view(np.uint16).tolist() == fx["w1_layer3_scale_first8_bits"]
+    assert sc.min() >= 0.002 - 1e-5 and sc.max() <= 0.02
+    zp = np.zeros(96, dtype=np.float16)
+    awq.check(lib.awq_synth_fill(seed, 3, awq.T_W1, awq.P_ZP, ptr(zp), zp.size))
+    assert np.array_equal(zp.view(np.uint16), helpers.synth_zp(seed, 3, awq.T_W1, 96).view(np.uint16))
+    assert zp[:8].astype(int).tolist() == fx["w1_layer3_zp_first8"]
+    assert set(np.unique(zp).tolist()) <= set(float(i) for i in range(16))
+    # the two global tensors ignore the layer argument
+    a = np.zeros(64, dtype=np.uint8); b = np.zeros(64, dtype=np.uint8)
+    awq.check(lib.awq_synth_fill(seed, 0, awq.T_UNEMBED, awq.P_PACKED, ptr(a), 64))
+    awq.check(lib.awq_synth_fill(seed, 7, awq.T_UNEMBED, awq.P_PACKED, ptr(b), 64))
+    assert np.array_equal(a, b)
+    # normals: numpy statement of the same Box-Muller, then distribution checks
+    x = np.zeros(200000, dtype=np.float16)
+    awq.check(lib.awq_synth_normal_f16(seed, awq.SYNTH_STREAM_INPUT, ptr(x), x.size, 0.0, 1.0))
+    ref = helpers.synth_normal(seed, awq.SYNTH_STREAM_INPUT, x.size).astype(np.float16)
+    assert np.mean(x.view(np.uint16) == ref.view(np.uint16)) > 0.9999
+    assert abs(float(x.astype(np.float64).mean())) < 0.01 and abs(float(x.astype(np.float64).std()) - 1.0) < 0.01
+    assert x[:8].view(np.uint16).tolist() == fx["normal_first8_bits"]
+    g = np.zeros(4096, dtype=np.float16)
+    awq.check(lib.awq_synth_fill(seed, 0, awq.T_GAMMA, 0, ptr(g), g.size))
+    assert abs(float(g.astype(np.float64).mean()) - 1.0) < 2e-3 and abs(float(g.astype(np.float64).std()) - 0.02) < 2e-3
+    # token ids
+    t = np.zeros(128, dtype=np.int32)
+    awq.check(lib.awq_synth_tokens(seed, awq.SYNTH_STREAM_INPUT + 1, ptr(t), t.size, 151936))
+    h = helpers.synth_hash(seed, awq.SYNTH_STREAM_INPUT + 1, np.arange(128, dtype=np.uint64))
+    assert np.array_equal(t, (h % np.uint64(151936)).astype(np.int32))
+    assert t[:8].tolist() == fx["tokens_first8"]
+
+
+def test_rope_tables_host_match_oracle(awq, lib, oracle):
+    mp = 4096
+    a, b = np.zeros((mp, 64), np.float16), np.zeros((mp, 64), np.float16)
+    c, d = np.zeros((mp, 64), np.float16), np.zeros((mp, 64), np.float16)
+    awq.check(lib.awq_rope_tables_host(ptr(a), ptr(b), mp))
+    oracle.awqo_rope_tables(ptr(c), ptr(d), mp)
+    assert np.array_equal(a.view(np.uint16), c.view(np.uint16)) and np.array_equal(b.view(np.uint16), d.view(np.uint16))

@@ -1,0 +1,438 @@
+"""Pins the CPU oracle (oracle/awq_oracle.cpp) without running the reference:
+closed forms, invariants, brute force in FP64 and second implementations.
+The reference (Inference.cu) has no tests or golden vectors of its own."""
+import ctypes
+import math
+
+import numpy as np
+import pytest
+
+from helpers import (bits16, block_elem, dequant_numpy, effective_weights_f64, f16, nibbles_flat, ptr)
+
+RNG = np.random.default_rng(20240607)
+
+
+def rand_awq(m, k, n_groups=None, zp_int=True, rng=RNG):
+    n_groups = n_groups or m // 128
+    packed = rng.integers(0, 256, size=m * k // 2, dtype=np.uint8)
+    scale = rng.uniform(0.002, 0.02, size=n_groups).astype(np.float16)
+    if zp_int:
+        zp = rng.integers(0, 16, size=n_groups).astype(np.float16)
+    else:
+        zp = rng.uniform(0, 15, size=n_groups).astype(np.float16)
+    return packed, scale, zp
+
+
+# ----------------------------------------------------------------------------- half conversions
+def test_half_to_float_exhaustive(oracle):
+    allh = np.arange(65536, dtype=np.uint16)
+    ref = allh.view(np.float16).astype(np.float32)
+    for h in range(0, 65536, 1):
+        a = oracle.awqo_soft_h2f(h)
+        b = oracle.awqo_h2f(h)
+        r = float(ref[h])
+        if math.isnan(r):
+            assert math.isnan(a) and math.isnan(b)
+        else:
+            assert a == r and b == r, h
+
+
+def test_float_to_half_three_ways(oracle):
+    # random bit patterns, every half-way point between adjacent halves, and the edges of the range
+    bits = RNG.integers(0, 2**32, size=40000, dtype=np.uint64).astype(np.uint32)
+    finite16 = np.arange(0x7c00, dtype=np.uint16).view(np.float16).astype(np.float64)
+    mids = ((finite16[:-1] + finite16[1:]) / 2).astype(np.float32)
+    edge = np.array([65504.0, 65519.99, 65520.0, 65536.0, 1e10, 5.96e-8, 2.98e-8, 2.9802322e-8, 2.99e-8, 0.0, -0.0,
+                     6.1035156e-5, 6.1e-5], dtype=np.float32)
+    vals = np.concatenate([bits.view(np.float32), mids, -mids, np.nextafter(mids, np.float32(np.inf)),
+                           np.nextafter(mids, np.float32(-np.inf)), edge, -edge])
+    with np.errstate(over="ignore"):
+        ref = vals.astype(np.float16).view(np.uint16)
+    for v, r in zip(vals, ref):
+        a = oracle.awqo_soft_f2h(float(v))
+        b = oracle.awqo_f2h(float(v))
+        if np.isnan(v):
+            assert (a & 0x7c00) == 0x7c00 and (a & 0x3ff) and (b & 0x7c00) == 0x7c00 and (b & 0x3ff)
+        else:
+            assert a == int(r) and b == int(r), (float(v), a, b, int(r))
+
+
+# ----------------------------------------------------------------------------- dequant (Inference.cu:76-106)
+def test_dequant_known_answer_byte_a3(oracle):
+    # byte 0xA3: low nibble 3 is the even column, high nibble 10 the odd one (Inference.cu:95-99)
+    packed = np.full(64, 0xA3, dtype=np.uint8)
+    scale = np.array([1.0], dtype=np.float16)
+    zp = np.array([0.0], dtype=np.float16)
+    out = np.zeros(128, dtype=np.float16)
+    oracle.awqo_dequant(ptr(packed), ptr(scale), ptr(zp), ptr(out), 1, 128, 1)
+    assert np.all(out[0::2] == 3.0) and np.all(out[1::2] == 10.0)
+    scale[0], zp[0] = 0.5, 8.0
+    oracle.awqo_dequant(ptr(packed), ptr(scale), ptr(zp), ptr(out), 1, 128, 1)
+    assert np.all(out[0::2] == -2.5) and np.all(out[1::2] == 1.0)
+
+
+def test_dequant_exhaustive_nibble_scale_zp_grid(oracle):
+    # every nibble against a grid of (scale, zp) bit patterns, including non-integral zero-points,
+    # subnormal scales and values whose product needs rounding; second implementation: numpy float16
+    scales = np.concatenate([f16(np.arange(0x1800, 0x2600, 7, dtype=np.uint16)),  # 0.002 .. 0.02 region
+                             f16(np.array([0x0001, 0x03ff, 0x0400, 0x3c00, 0x3555, 0x7bff], dtype=np.uint16))])
+    zps = np.concatenate([np.arange(16).astype(np.float16), f16(np.arange(0x3c00, 0x4b80, 97, dtype=np.uint16)),
+                          np.array([0.5, 7.25, 1e-4, 1023.0, -3.0], dtype=np.float16)])
+    S, Z = np.meshgrid(scales, zps, indexing="ij")
+    S, Z = S.reshape(-1), Z.reshape(-1)
+    n = S.size
+    # one group per row-of-128: make cols = 128*n, one row; nibbles cycle 0..15
+    cols = 128 * n
+    nib = (np.arange(cols) % 16).astype(np.uint8)
+    packed = (nib[0::2] | (nib[1::2] << 4)).astype(np.uint8)
+    out = np.zeros(cols, dtype=np.float16)
+    oracle.awqo_dequant(ptr(packed), ptr(S), ptr(Z), ptr(out), 1, cols, n)
+    with np.errstate(over="ignore", invalid="ignore"):
+        ref = dequant_numpy(packed, S, Z, 1, cols, n).reshape(-1)
+    assert np.array_equal(out.view(np.uint16), ref.view(np.uint16))
+
+
+def test_dequant_group_wrap_and_row_layout(oracle):
+    # more column groups than stored entries: the index wraps (the reference reads out of bounds there)
+    rows, cols, ng = 3, 512, 2
+    packed, scale, zp = rand_awq(rows * 2, cols // 2 * 1, n_groups=ng)  # sizes only
+    packed = RNG.integers(0, 256, size=rows * cols // 2, dtype=np.uint8)
+    out = np.zeros(rows * cols, dtype=np.float16)
+    oracle.awqo_dequant(ptr(packed), ptr(scale), ptr(zp), ptr(out), rows, cols, ng)
+    ref = np.empty((rows, cols), dtype=np.float16)
+    for r in range(rows):
+        for c in range(cols):
+            b = int(packed[r * (cols // 2) + c // 2])
+            q = (b >> 4) if c & 1 else (b & 15)
+            g = (c // 128) % ng
+            ref[r, c] = np.float16(np.float16(np.float16(q) - zp[g]) * scale[g])
+    assert np.array_equal(out.reshape(rows, cols).view(np.uint16), ref.view(np.uint16))
+
+
+def test_dequant_odd_cols_follow_reference_stride(oracle):
+    rows, cols = 2, 7  # packed row stride (cols+1)/2 = 4 (Inference.cu:93)
+    packed = RNG.integers(0, 256, size=rows * 4, dtype=np.uint8)
+    scale = np.array([0.25], dtype=np.float16)
+    zp = np.array([2.0], dtype=np.float16)
+    out = np.zeros(rows * cols, dtype=np.float16)
+    oracle.awqo_dequant(ptr(packed), ptr(scale), ptr(zp), ptr(out), rows, cols, 1)
+    for r in range(rows):
+        for c in range(cols):
+            b = int(packed[r * 4 + c // 2])
+            q = (b >> 4) if c & 1 else (b & 15)
+            assert out[r * cols + c] == np.float16((q - 2.0) * 0.25)
+
+
+# ----------------------------------------------------------------------------- group index
+@pytest.mark.parametrize("m,k", [(12288, 4096), (4096, 4096), (4096, 12288), (151936, 4096), (384, 256), (640, 512)])
+def test_group_index_and_period(oracle, m, k):
+    rng = np.random.default_rng(m + k)
+    C = oracle.awqo_group_period(m, k)
+    expect = {(12288, 4096): 1, (4096, 4096): 1, (4096, 12288): 1, (151936, 4096): 32}.get((m, k))
+    if expect:
+        assert C == expect
+    for _ in range(300):
+        i, j = int(rng.integers(0, m)), int(rng.integers(0, k))
+        g = oracle.awqo_group_index(m, k, i, j)
+        p = j * m + i
+        assert g == ((p % k) // 128) % (m // 128)  # Inference.cu:88-90 on flat element p, wrapped
+        if j + C < k:
+            assert g == oracle.awqo_group_index(m, k, i, j + C)
+    # C is the smallest period: some i, j must differ for every smaller step
+    for c in range(1, C):
+        assert any(oracle.awqo_group_index(m, k, i, 0) != oracle.awqo_group_index(m, k, i, c)
+                   for i in range(0, m, 128))
+    # the closed forms used in the build notes
+    if (m, k) == (151936, 4096):
+        for i, j in [(0, 0), (130, 1), (151935, 4095), (77777, 1234)]:
+            assert oracle.awqo_group_index(m, k, i, j) == (3 * j + i // 128) % 32
+    if (m, k) == (4096, 12288):
+        for i, j in [(0, 0), (130, 1), (4095, 12287)]:
+            assert oracle.awqo_group_index(m, k, i, j) == i // 128
+
+
+# ----------------------------------------------------------------------------- linear (Inference.cu:1052-1065)
+LIN_SHAPES = [(128, 512), (256, 1024), (384, 512), (128, 1536), (640, 512)]
+
+
+def run_linear(oracle, fn, packed, scale, zp, m, k, x, M, out_dtype):
+    y = np.zeros((M, m), dtype=out_dtype)
+    getattr(oracle, fn)(ptr(packed), ptr(scale), ptr(zp), m, k, ptr(x), ptr(y), M)
+    return y
+
+
+@pytest.mark.parametrize("m,k", LIN_SHAPES)
+def test_linear_f64_brute_force(oracle, m, k):
+    packed, scale, zp = rand_awq(m, k, zp_int=False)
+    x = RNG.standard_normal((2, k)).astype(np.float16)
+    W = effective_weights_f64(packed, scale, zp, m, k)  # W[i,j] = flat[j*m+i]
+    ref = x.astype(np.float64) @ W.T
+    y = run_linear(oracle, "awqo_linear_f64", packed, scale, zp, m, k, x, 2, np.float64)
+    assert np.allclose(y, ref, rtol=1e-12, atol=1e-12)
+
+
+def test_linear_one_hot_pins_column_major_reading(oracle):
+    # scale 1, zp 0, all nibbles 0 except one at flat position p: only y[p % m] moves, by q * x[p // m]
+    m, k = 256, 512
+    scale = np.ones(m // 128, dtype=np.float16)
+    zp = np.zeros(m // 128, dtype=np.float16)
+    x = (np.arange(k) % 13 + 1).astype(np.float16)
+    for p, q in [(0, 5), (1, 9), (m - 1, 3), (m, 7), (3 * m + 17, 15), (k * m - 1, 1), (200 * m + 255, 12)]:
+        packed = np.zeros(m * k // 2, dtype=np.uint8)
+        packed[p >> 1] = q << (4 * (p & 1))
+        for fn, dt in [("awqo_linear_f64", np.float64), ("awqo_linear_seq", np.float16), ("awqo_linear", np.float16),
+                       ("awqo_linear_scalar", np.float16)]:
+            y = run_linear(oracle, fn, packed, scale, zp, m, k, x[None, :], 1, dt)[0].astype(np.float64)
+            expect = np.zeros(m)
+            expect[p % m] = q * float(x[p // m])
+            assert np.array_equal(y, expect), (fn, p)
+
+
+@pytest.mark.parametrize("m,k", LIN_SHAPES)
+def test_linear_orders_agree(oracle, m, k):
+    packed, scale, zp = rand_awq(m, k)
+    x = RNG.standard_normal((3, k)).astype(np.float16)
+    y64 = run_linear(oracle, "awqo_linear_f64", packed, scale, zp, m, k, x, 3, np.float64)
+    seq = run_linear(oracle, "awqo_linear_seq", packed, scale, zp, m, k, x, 3, np.float16)
+    blk = run_linear(oracle, "awqo_linear", packed, scale, zp, m, k, x, 3, np.float16)
+    sca = run_linear(oracle, "awqo_linear_scalar", packed, scale, zp, m, k, x, 3, np.float16)
+    # the vector and the scalar statement of the blocked order are the same arithmetic
+    assert np.array_equal(blk.view(np.uint16), sca.view(np.uint16))
+    # both binary32 orders sit within FP16 rounding of the exact sum
+    tol = 2.0 ** -10 * np.maximum(np.abs(y64), 1e-3) + 1e-3
+    assert np.all(np.abs(seq.astype(np.float64) - y64) <= tol)
+    assert np.all(np.abs(blk.astype(np.float64) - y64) <= tol)
+    # M > 1 is M independent products
+    for t in range(3):
+        one = run_linear(oracle, "awqo_linear", packed, scale, zp, m, k, x[t:t + 1].copy(), 1, np.float16)
+        assert np.array_equal(one[0].view(np.uint16), blk[t].view(np.uint16))
+
+
+def test_linear_blocked_order_definition(oracle):
+    # independent numpy statement of the blocked order: fma chains of 32, adjacent-pair tree
+    m, k = 384, 512  # period 4
+    C = oracle.awqo_group_period(m, k)
+    assert C == 4
+    packed, scale, zp = rand_awq(m, k)
+    x = RNG.standard_normal(k).astype(np.float16)
+    W = effective_weights_f64(packed, scale, zp, m, k)
+    y = run_linear(oracle, "awqo_linear", packed, scale, zp, m, k, x[None, :].copy(), 1, np.float16)[0]
+    nblk = k // 32
+    for i in [0, 1, 127, 128, 383]:
+        parts = []
+        for blk in range(nblk):
+            acc = np.float32(0)
+            for t in range(32):
+                j = block_elem(k, C, blk, t)
+                # fma in binary32: the product of two halves is exact in float64, one rounding of the sum
+                acc = np.float32(np.float64(W[i, j]) * np.float64(x[j]) + np.float64(acc))
+            parts.append(acc)
+        n = nblk
+        while n > 1 and n % 2 == 0:
+            parts = [np.float32(parts[2 * a] + parts[2 * a + 1]) for a in range(n // 2)]
+            n //= 2
+        tot = parts[0]
+        for a in range(1, n):
+            tot = np.float32(tot + parts[a])
+        assert np.float16(tot) == y[i], i
+
+
+# ----------------------------------------------------------------------------- RMSNorm (Inference.cu:111-145)
+def test_rmsnorm_constant_vector_closed_form(oracle):
+    n = 4096
+    for c in [1.0, -0.5, 3.25, 0.001]:
+        x = np.full(n, c, dtype=np.float16)
+        gamma = (1 + 0.02 * RNG.standard_normal(n)).astype(np.float16)
+        out = np.zeros(n, dtype=np.float16)
+        oracle.awqo_rmsnorm(ptr(x), ptr(gamma), ptr(out), n, 1e-6)
+        cf = np.float32(x[0])
+        # 4096 equal squares summed in binary32 by the tree are exact multiples; mean = c^2 exactly
+        ms = np.float32(cf * cf)
+        sc = np.float16(np.float32(1.0) / np.sqrt(np.float32(ms + np.float32(1e-6))))
+        ref = (np.float16(x[0] * sc) * gamma).astype(np.float16)
+        assert np.array_equal(out.view(np.uint16), ref.view(np.uint16))
+
+
+def test_rmsnorm_matches_fp64(oracle):
+    n = 4096
+    x = (RNG.standard_normal(n) * 3).astype(np.float16)
+    gamma = (1 + 0.02 * RNG.standard_normal(n)).astype(np.float16)
+    out = np.zeros(n, dtype=np.float16)
+    oracle.awqo_rmsnorm(ptr(x), ptr(gamma), ptr(out), n, 1e-6)
+    xd = x.astype(np.float64)
+    ref = xd / np.sqrt(np.mean(xd * xd) + 1e-6) * gamma.astype(np.float64)
+    assert np.all(np.abs(out.astype(np.float64) - ref) <= 3 * 2.0 ** -11 * np.abs(ref) + 1e-6)
+
+
+# ----------------------------------------------------------------------------- rotary (Inference.cu:150-177, 443-454)
+def test_rope_tables(oracle):
+    max_pos = 2048
+    c = np.zeros((max_pos, 64), dtype=np.float16)
+    s = np.zeros((max_pos, 64), dtype=np.float16)
+    oracle.awqo_rope_tables(ptr(c), ptr(s), max_pos)
+    assert np.all(c[0] == 1.0) and np.all(s[0] == 0.0)
+    i = np.arange(64, dtype=np.float32)
+    inv = (np.float32(1.0) / np.power(np.float32(10000.0), (2 * i) / np.float32(128.0))).astype(np.float32)
+    ang = (np.arange(max_pos, dtype=np.float32)[:, None] * inv[None, :]).astype(np.float32)
+    # the angle is a binary32 number in the reference; its cosine in FP64 must round to the same half,
+    # up to one ulp where cosf's own error straddles a rounding boundary
+    cref, sref = np.cos(ang.astype(np.float64)), np.sin(ang.astype(np.float64))
+    ulp = 2.0 ** -11
+    assert np.all(np.abs(c.astype(np.float64) - cref) <= ulp * 1.01)
+    assert np.all(np.abs(s.astype(np.float64) - sref) <= ulp * 1.01)
+    assert np.mean(c.view(np.uint16) == cref.astype(np.float16).view(np.uint16)) > 0.99  # numpy power vs powf: last-bit angle differences
+
+
+def test_rotary_identity_pairs_and_norm(oracle):
+    max_pos, nh = 64, 4
+    c = np.zeros((max_pos, 64), dtype=np.float16)
+    s = np.zeros((max_pos, 64), dtype=np.float16)
+    oracle.awqo_rope_tables(ptr(c), ptr(s), max_pos)
+    x = RNG.standard_normal(nh * 128).astype(np.float16)
+    y = x.copy()
+    oracle.awqo_rotary(ptr(y), ptr(c), ptr(s), nh, 0)
+    assert np.array_equal(x.view(np.uint16), y.view(np.uint16))  # cos=1, sin=0 exactly
+    y = x.copy()
+    oracle.awqo_rotary(ptr(y), ptr(c), ptr(s), nh, 37)
+    # closed form per pair with binary16 rounding after every op (Inference.cu:172-173)
+    xr = x.reshape(nh, 64, 2)
+    cc, ss = c[37][None, :], s[37][None, :]
+    r0 = ((xr[:, :, 0] * cc).astype(np.float16) - (xr[:, :, 1] * ss).astype(np.float16)).astype(np.float16)
+    r1 = ((xr[:, :, 0] * ss).astype(np.float16) + (xr[:, :, 1] * cc).astype(np.float16)).astype(np.float16)
+    ref = np.stack([r0, r1], axis=-1).reshape(-1)
+    assert np.array_equal(y.view(np.uint16), ref.view(np.uint16))
+    # a rotation keeps pair norms (up to FP16 rounding)
+    n0 = np.linalg.norm(xr.astype(np.float64), axis=-1)
+    n1 = np.linalg.norm(y.reshape(nh, 64, 2).astype(np.float64), axis=-1)
+    assert np.all(np.abs(n0 - n1) <= 4e-3 * np.maximum(n0, 1))
+    # touching element 2i changes outputs 2i and 2i+1 only
+    x2 = x.copy()
+    x2[130] = np.float16(5.0)
+    y2 = x2.copy()
+    oracle.awqo_rotary(ptr(y2), ptr(c), ptr(s), nh, 37)
+    diff = np.nonzero(y2.view(np.uint16) != y.view(np.uint16))[0]
+    assert set(diff.tolist()) <= {130, 131} and len(diff) > 0
+
+
+# ----------------------------------------------------------------------------- attention (Inference.cu:182-266)
+def attention_inputs(nh, max_pos, L, rng=RNG):
+    q = rng.standard_normal(nh * 128).astype(np.float16)
+    kc = np.zeros((nh, max_pos, 128), dtype=np.float16)
+    vc = np.zeros((nh, max_pos, 128), dtype=np.float16)
+    kc[:, :L] = rng.standard_normal((nh, L, 128)).astype(np.float16)
+    vc[:, :L] = rng.standard_normal((nh, L, 128)).astype(np.float16)
+    return q, kc, vc
+
+
+def test_attention_length_one_returns_v0(oracle):
+    # the only case in which the reference kernel itself is well defined
+    nh, mp = 4, 16
+    q, kc, vc = attention_inputs(nh, mp, 1)
+    ctx = np.zeros(nh * 128, dtype=np.float16)
+    oracle.awqo_attention(ptr(q), ptr(kc), ptr(vc), ptr(ctx), nh, mp, 1, None)
+    assert np.array_equal(ctx.reshape(nh, 128).view(np.uint16), vc[:, 0].view(np.uint16))
+
+
+def test_attention_equal_keys_give_mean_of_values(oracle):
+    nh, mp, L = 2, 256, 200
+    q, kc, vc = attention_inputs(nh, mp, L)
+    kc[:, :L] = kc[:, :1]
+    ctx = np.zeros(nh * 128, dtype=np.float16)
+    oracle.awqo_attention(ptr(q), ptr(kc), ptr(vc), ptr(ctx), nh, mp, L, None)
+    ref = vc[:, :L].astype(np.float64).mean(axis=1).reshape(-1)
+    assert np.all(np.abs(ctx.astype(np.float64) - ref) <= 2.0 ** -10 * np.abs(ref) + 1e-4)
+
+
+@pytest.mark.parametrize("L", [1, 2, 63, 64, 65, 129, 513])
+def test_attention_matches_fp64_softmax(oracle, L):
+    nh, mp = 3, 640
+    q, kc, vc = attention_inputs(nh, mp, L)
+    ctx = np.zeros(nh * 128, dtype=np.float16)
+    scores = np.zeros((nh, L), dtype=np.float32)
+    oracle.awqo_attention(ptr(q), ptr(kc), ptr(vc), ptr(ctx), nh, mp, L, ptr(scores))
+    qd = q.astype(np.float64).reshape(nh, 128)
+    s = np.einsum("hd,htd->ht", qd, kc[:, :L].astype(np.float64)) / math.sqrt(128.0)
+    assert np.allclose(scores, s, rtol=2e-6, atol=2e-6)
+    p = np.exp(s - s.max(axis=1, keepdims=True))
+    p /= p.sum(axis=1, keepdims=True)
+    ref = np.einsum("ht,htd->hd", p, vc[:, :L].astype(np.float64)).reshape(-1)
+    assert np.all(np.abs(ctx.astype(np.float64) - ref) <= 2.0 ** -10 * np.abs(ref) + 2e-4)
+
+
+# ----------------------------------------------------------------------------- GeLU, residual, argmax, embedding
+def test_gelu_points_and_fp64(oracle):
+    x = np.array([0.0, -0.0, 10.0, -10.0, 60000.0, -60000.0, 1.0, -1.0], dtype=np.float16)
+    y = x.copy()
+    oracle.awqo_gelu(ptr(y), y.size)
+    assert y[0] == 0 and y[1] == 0 and y[2] == 10.0 and y[3] == 0 and y[4] == 60000.0 and y[5] == 0
+    assert abs(float(y[6]) - 0.8413447) < 1e-3 and abs(float(y[7]) + 0.1586553) < 2e-4
+    allh = np.arange(65536, dtype=np.uint16).view(np.float16)
+    allh = allh[np.isfinite(allh)].copy()
+    y = allh.copy()
+    oracle.awqo_gelu(ptr(y), y.size)
+    v = allh.astype(np.float64)
+    erf = np.vectorize(math.erf)
+    ref = 0.5 * v * (1.0 + erf(v * 0.70710678))
+    err = np.abs(y.astype(np.float64) - ref)
+    # one FP16 ulp of the result, plus the binary32 cancellation in 1+erf that the reference has too
+    tol = 2.0 ** -10 * np.abs(ref) + np.abs(v) * 2.0 ** -24 + 6e-8
+    assert np.all(err <= tol)
+
+
+def test_residual_is_fp16_add(oracle):
+    a = (RNG.standard_normal(4096) * 4).astype(np.float16)
+    b = (RNG.standard_normal(4096) * 4).astype(np.float16)
+    out = np.zeros_like(a)
+    oracle.awqo_residual(ptr(a), ptr(b), ptr(out), a.size)
+    assert np.array_equal(out.view(np.uint16), (a + b).astype(np.float16).view(np.uint16))
+
+
+def test_argmax_ties_and_nan(oracle):
+    x = np.zeros(1000, dtype=np.float16)
+    assert oracle.awqo_argmax(ptr(x), x.size) == 0
+    x[[10, 500, 999]] = 3.5
+    assert oracle.awqo_argmax(ptr(x), x.size) == 10  # strict '>' keeps the first (Inference.cu:1285)
+    x[700] = np.float16("nan")
+    assert oracle.awqo_argmax(ptr(x), x.size) == 10  # NaN never beats anything
+    x[0] = np.float16("nan")
+    assert oracle.awqo_argmax(ptr(x), x.size) == 0   # and nothing beats a NaN at index 0
+    x[:] = -np.inf
+    x[3] = -65504.0
+    assert oracle.awqo_argmax(ptr(x), x.size) == 3
+    x[:] = 0.0
+    x[5] = -0.0
+    assert oracle.awqo_argmax(ptr(x), x.size) == 0   # -0 == +0
+
+
+def test_embed_is_column_of_dequantised_matrix(oracle):
+    H, V = 256, 1024
+    packed, scale, zp = rand_awq(H, V)
+    full = np.zeros(H * V, dtype=np.float16)
+    oracle.awqo_dequant(ptr(packed), ptr(scale), ptr(zp), ptr(full), H, V, H // 128)
+    full = full.reshape(H, V)
+    out = np.zeros(H, dtype=np.float16)
+    for tok in [0, 1, 127, 128, 255, 256, 511, 1023]:
+        oracle.awqo_embed(ptr(packed), ptr(scale), ptr(zp), H, V, tok, ptr(out))
+        assert np.array_equal(out.view(np.uint16), full[:, tok].view(np.uint16)), tok
+
+
+# ----------------------------------------------------------------------------- canonical math
+def test_canonical_exp_erf_accuracy(oracle):
+    xs = np.concatenate([np.linspace(-104, 88.7, 20001), -np.logspace(-8, 2, 2000)]).astype(np.float32)
+    for x in xs[::7]:
+        t = math.exp(float(x))
+        y = oracle.awqo_expf(float(x))
+        if t > 1.2e-38:
+            assert abs(y - t) <= 1.01 * np.spacing(np.float32(t))
+        else:
+            assert abs(y - t) <= 1.5e-45
+    assert oracle.awqo_expf(0.0) == 1.0
+    assert oracle.awqo_expf(-200.0) == 0.0
+    for x in np.linspace(-5, 5, 4001).astype(np.float32):
+        t = math.erf(float(x))
+        y = oracle.awqo_erff(float(x))
+        if abs(x) < 1:
+            assert abs(y - t) <= 2.6 * np.spacing(np.float32(abs(t))) + 1e-45
+        else:
+            assert abs(y - t) <= 1.2 * 2.0 ** -24
+    assert oracle.awqo_erff(0.0) == 0.0 and oracle.awqo_erff(9.0) == 1.0 and oracle.awqo_erff(-9.0) == -1.0
