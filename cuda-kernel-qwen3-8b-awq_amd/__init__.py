@@ -66,6 +66,7 @@ SIGNATURES = {
     "awq_read_hidden": (ctypes.c_int, [_vp, _vp]),
     "awq_read_logits": (ctypes.c_int, [_vp, _vp]),
     "awq_set_graph_mode": (ctypes.c_int, [_vp, ctypes.c_int]),
+    "awq_time_linear": (ctypes.c_int, [_vp, ctypes.c_int, _i32, ctypes.POINTER(_f32), ctypes.POINTER(_i64)]),
     "awq_destroy": (None, [_vp]),
     "awq_write_weight_dir": (ctypes.c_int, [ctypes.c_char_p, _cfgp, _u64]),
     "awq_synth_fill": (ctypes.c_int, [_u64, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp, _i64]),
@@ -99,6 +100,13 @@ def load_library():
         raise RuntimeError(
             "libawq_infer.so is not built: run `python %s` (needs hipcc); there is no CPU fallback"
             % os.path.join(_HERE, "build.py"))
+    # PyTorch (used by callers for device memory and streams) bundles its own HIP runtime.  Two
+    # HIP runtimes in one process cannot both own the GPU, so torch is imported first: the loader
+    # then resolves this library's libamdhip64.so.7 to the copy that is already mapped.
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     lib = ctypes.CDLL(LIB_PATH)
     for name, (res, args) in SIGNATURES.items():
         fn = getattr(lib, name)
@@ -223,6 +231,12 @@ class QWen3AWQInfer:
         buf = (ctypes.c_uint16 * self.config.vocab)()
         check(self._lib.awq_read_logits(self._h, buf))
         return buf
+
+    def time_linear(self, kind, n_rounds=20):
+        """(mean microseconds per launch, algorithmic bytes per launch) of the fused linear kernel"""
+        us, nbytes = _f32(0), _i64(0)
+        check(self._lib.awq_time_linear(self._h, kind, n_rounds, ctypes.byref(us), ctypes.byref(nbytes)))
+        return us.value, nbytes.value
 
     def close(self):
         if self._h:

@@ -14,6 +14,16 @@ typedef _Float16 half_t;
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 
+// binary32 -> binary16, round to nearest even, as its own instruction.  Without
+// the barrier the compiler folds a preceding multiply into v_fma_mixlo_f16 with
+// a +0 addend, which turns a product of -0 into +0.
+__device__ __forceinline__ half_t to_half_rn(float v) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("" : "+v"(v));
+#endif
+  return (half_t)v;
+}
+
 // error string of the calling thread (awq_last_error)
 void awq_set_error(const std::string& msg);
 

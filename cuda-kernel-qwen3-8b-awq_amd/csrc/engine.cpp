@@ -611,6 +611,56 @@ extern "C" int awq_read_logits(awq_engine* e, uint16_t* host_dst) {
   return AWQ_OK;
 }
 
+// Times the engine's own fused-linear launches of one tensor kind over all
+// layers' resident weights (a different matrix every launch, so the working
+// set is n_layers matrices), with HIP events on the engine's stream.
+extern "C" int awq_time_linear(awq_engine* e, int kind, int32_t n_rounds, float* avg_us_per_launch,
+                               int64_t* bytes_per_launch) {
+  AWQ_REQUIRE(e && avg_us_per_launch && n_rounds > 0, "bad arguments");
+  if (!e->finalized) {
+    awq_set_error("awq_time_linear before awq_finalize");
+    return AWQ_ERR_STATE;
+  }
+  AWQ_REQUIRE(kind == AWQ_T_WQKV || kind == AWQ_T_WO || kind == AWQ_T_W1 || kind == AWQ_T_W2 || kind == AWQ_T_UNEMBED,
+              "kind must be a linear layer");
+  hipEvent_t ev0, ev1;
+  AWQ_HIP_TRY(hipEventCreate(&ev0));
+  AWQ_HIP_TRY(hipEventCreate(&ev1));
+  const int n_mats = kind == AWQ_T_UNEMBED ? 1 : e->cfg.n_layers;
+  auto one_round = [&]() -> int {
+    for (int l = 0; l < n_mats; ++l) {
+      const DevLinear& t = *find_linear(e, l, kind);
+      int rc = AWQ_OK;
+      switch (kind) {
+        case AWQ_T_WQKV: rc = linear(e, t, e->normed, e->qkv, EPI_STORE, nullptr); break;
+        case AWQ_T_WO: rc = linear(e, t, e->ctx, e->hidden, EPI_RESIDUAL, e->hidden); break;
+        case AWQ_T_W1: rc = linear(e, t, e->normed, e->mid, EPI_GELU, nullptr); break;
+        case AWQ_T_W2: rc = linear(e, t, e->mid, e->hidden, EPI_RESIDUAL, e->hidden); break;
+        default: rc = linear(e, t, e->normed, e->logits, EPI_STORE, nullptr); break;
+      }
+      if (rc) return rc;
+    }
+    return AWQ_OK;
+  };
+  if (int rc = one_round()) return rc;  // warm-up
+  AWQ_HIP_TRY(hipEventRecord(ev0, e->stream));
+  for (int r = 0; r < n_rounds; ++r)
+    if (int rc = one_round()) return rc;
+  AWQ_HIP_TRY(hipEventRecord(ev1, e->stream));
+  AWQ_HIP_TRY(hipEventSynchronize(ev1));
+  float ms = 0.0f;
+  AWQ_HIP_TRY(hipEventElapsedTime(&ms, ev0, ev1));
+  *avg_us_per_launch = ms * 1000.0f / (float)((int64_t)n_rounds * n_mats);
+  if (bytes_per_launch) {
+    const DevLinear& t = *find_linear(e, 0, kind);
+    // packed weights + scales + zero-points + input vector + output vector
+    *bytes_per_launch = t.m * (t.k / 2) + 2 * (t.m / 128) * 2 + t.k * 2 + t.m * 2;
+  }
+  (void)hipEventDestroy(ev0);
+  (void)hipEventDestroy(ev1);
+  return awq_reset(e);
+}
+
 // ---------------------------------------------------------------------------
 // kernel-level entry points
 // ---------------------------------------------------------------------------

@@ -174,7 +174,7 @@ __device__ __forceinline__ void epilogue(const GemvParams& p, int row, float acc
   if (EPI == EPI_RESIDUAL) {
     v = p.res[row] + v;
   } else if (EPI == EPI_GELU) {
-    v = (half_t)awq_gelu_f32((float)v);
+    v = to_half_rn(awq_gelu_f32((float)v));
   }
   p.y[row] = v;
 }

@@ -67,7 +67,7 @@ __global__ __launch_bounds__(256) void residual_kernel(const half_t* a, const ha
 // geluKernel (Inference.cu:271-279)
 __global__ __launch_bounds__(256) void gelu_kernel(half_t* x, int64_t n) {
   int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i < n) x[i] = (half_t)awq_gelu_f32((float)x[i]);
+  if (i < n) x[i] = to_half_rn(awq_gelu_f32((float)x[i]));
 }
 
 // gather lambda (Inference.cu:1310-1324) straight from the packed [hidden][vocab]

@@ -85,6 +85,14 @@ int awq_read_logits(awq_engine* e, uint16_t* host_dst);
 /* 0: every op is its own launch; 1 (default): one captured graph per step */
 int awq_set_graph_mode(awq_engine* e, int enabled);
 
+/* Measurement aid with no counterpart in the reference: runs the engine's own
+ * fused-linear launch of `kind` (AWQ_T_WQKV/WO/W1/W2/UNEMBED) over every
+ * layer's resident matrix, n_rounds times, between two HIP events on the
+ * engine's stream.  Returns the mean launch duration and the algorithmic bytes
+ * of one launch (packed weights + scales + zero-points + input + output).
+ * Resets the sequence. */
+int awq_time_linear(awq_engine* e, int kind, int32_t n_rounds, float* avg_us_per_launch, int64_t* bytes_per_launch);
+
 /* Destructor, Inference.cu:475-558 */
 void awq_destroy(awq_engine* e);
 

@@ -515,6 +515,7 @@ struct awqo_model {
   std::vector<std::vector<half_t>> kcache, vcache;
   std::vector<half_t> cos_t, sin_t;
   std::vector<half_t> hidden, normed, qkv, ctx, attn_out, mid, mlp_out, logits;
+  std::vector<half_t> last_layer_out;  // hidden state after the last layer of the latest position
   int current_seq_len = 0;
   bool luts_ready = false;
   // statistics of the last generate call
@@ -728,6 +729,7 @@ AWQO_API int awqo_model_generate(awqo_model* m, const int* prompt, int n_prompt,
       awqo_model_layer(m, l, t, m->current_seq_len + 1);
       m->current_seq_len = t;  // I:1331, 1341: updated after every layer
     }
+    m->last_layer_out = m->hidden;
   }
   for (int step = 0; step < max_new; ++step) {  // I:1352
     int pos = n_prompt + step;
@@ -740,6 +742,7 @@ AWQO_API int awqo_model_generate(awqo_model* m, const int* prompt, int n_prompt,
     m->current_seq_len = pos;                                                           // I:1374
     int tok = awqo_model_sample(m);                                                     // I:1377
     out[step] = tok;
+    m->last_layer_out = m->hidden;
     model_embed(m, tok);  // I:1392
   }
   return max_new;
@@ -747,6 +750,10 @@ AWQO_API int awqo_model_generate(awqo_model* m, const int* prompt, int n_prompt,
 
 AWQO_API const uint16_t* awqo_model_hidden(awqo_model* m) { return m->hidden.data(); }
 AWQO_API const uint16_t* awqo_model_logits(awqo_model* m) { return m->logits.data(); }
+AWQO_API const uint16_t* awqo_model_last_layer_out(awqo_model* m) {
+  if (m->last_layer_out.empty()) m->last_layer_out = m->hidden;
+  return m->last_layer_out.data();
+}
 AWQO_API uint16_t* awqo_model_hidden_mut(awqo_model* m) { return m->hidden.data(); }
 AWQO_API uint16_t* awqo_model_kcache(awqo_model* m, int l) { return m->kcache[l].data(); }
 AWQO_API uint16_t* awqo_model_vcache(awqo_model* m, int l) { return m->vcache[l].data(); }

@@ -49,6 +49,7 @@ SIG = {
     "awqo_model_generate": (ctypes.c_int, [vp, vp, ctypes.c_int, ctypes.c_int, vp]),
     "awqo_model_hidden": (vp, [vp]),
     "awqo_model_logits": (vp, [vp]),
+    "awqo_model_last_layer_out": (vp, [vp]),
     "awqo_model_hidden_mut": (vp, [vp]),
     "awqo_model_kcache": (vp, [vp, ctypes.c_int]),
     "awqo_model_vcache": (vp, [vp, ctypes.c_int]),

@@ -23,7 +23,7 @@ def oracle_generate(oracle, model, prompt, n_new):
 
 def compare_state(awq, oracle, eng, model, cfg):
     hid = np.ctypeslib.as_array(eng.read_hidden())
-    oh = np.ctypeslib.as_array(ctypes.cast(oracle.awqo_model_hidden(model), ctypes.POINTER(ctypes.c_uint16)), (cfg.hidden,))
+    oh = np.ctypeslib.as_array(ctypes.cast(oracle.awqo_model_last_layer_out(model), ctypes.POINTER(ctypes.c_uint16)), (cfg.hidden,))
     assert np.array_equal(hid, oh)
     lg = np.ctypeslib.as_array(eng.read_logits())
     ol = np.ctypeslib.as_array(ctypes.cast(oracle.awqo_model_logits(model), ctypes.POINTER(ctypes.c_uint16)), (cfg.vocab,))
