@@ -88,6 +88,22 @@ SIGNATURES = {
     "awq_embed_gather": (ctypes.c_int, [_vp, _vp, _vp, _i64, _i64, _i32, _vp, _vp]),
 }
 
+
+
+class AwqLinearArgs(ctypes.Structure):
+    """struct awq_linear_args"""
+    _fields_ = [
+        ("repacked", _vp), ("scale", _vp), ("zp", _vp), ("m", _i64), ("k", _i64), ("x", _vp), ("y", _vp),
+        ("zp_integral", _i32), ("prologue", _i32), ("epilogue", _i32), ("eps", _f32), ("gamma", _vp),
+        ("residual", _vp), ("cos_t", _vp), ("sin_t", _vp), ("k_cache", _vp), ("v_cache", _vp), ("hidden", _i32),
+        ("reserved", _i32), ("max_pos", _i64), ("pos", _i64), ("out_token", _vp), ("workspace", _vp),
+    ]
+
+
+PRO_NONE, PRO_RMSNORM = 0, 1
+EPI_STORE, EPI_RESIDUAL, EPI_GELU, EPI_QKV_ROPE, EPI_ARGMAX = range(5)
+SIGNATURES["awq_gemv_fused"] = (ctypes.c_int, [ctypes.POINTER(AwqLinearArgs), _vp])
+
 _lib = None
 
 

@@ -56,26 +56,59 @@ struct StepState {
   int32_t sample;     // 1 = run the sampler at the end of the step
 };
 
-// epilogues of the fused linear kernel
+// what the fused linear kernel does to its input and its output
+enum LinearPrologue {
+  PRO_NONE = 0,     // x is used as is
+  PRO_RMSNORM = 1,  // x is the un-normalised hidden state: rmsNormKernel (Inference.cu:111-145) first
+};
 enum LinearEpilogue {
   EPI_STORE = 0,     // y = h(acc)
-  EPI_RESIDUAL = 1,  // y = h(res + h(acc))
-  EPI_GELU = 2,      // y = h(gelu(h(acc)))
+  EPI_RESIDUAL = 1,  // y = h(res + h(acc))                              Inference.cu:1149-1155
+  EPI_GELU = 2,      // y = h(gelu(h(acc)))                              Inference.cu:271-279
+  EPI_QKV_ROPE = 3,  // split, rotary on Q and K, K/V appended to the cache  Inference.cu:1070-1103
+  EPI_ARGMAX = 4,    // y = h(acc) and the greedy token                  Inference.cu:1278-1290
 };
 
 struct LinearArgs {
-  const void* wq;      // repacked int4
-  const half_t* scale; // [m/128]
-  const half_t* zp;    // [m/128]
-  const half_t* x;     // [k]
-  half_t* y;           // [m]
-  const half_t* res;   // EPI_RESIDUAL: [m], may alias y
-  float* partials;     // split-k workspace
-  int32_t* counters;   // one per 64-row group, zero between launches
-  int64_t m, k;
-  int zp_integral;     // all zero-points are integers in [0,1024]: take the 2-op dequant
-  int epilogue;
+  const void* wq = nullptr;       // repacked int4
+  const half_t* scale = nullptr;  // [m/128]
+  const half_t* zp = nullptr;     // [m/128]
+  const half_t* x = nullptr;      // [k]
+  half_t* y = nullptr;            // [m] ([hidden] rotated Q for EPI_QKV_ROPE)
+  const half_t* res = nullptr;    // EPI_RESIDUAL: [m], may alias y
+  float* partials = nullptr;      // split-k workspace
+  int32_t* counters = nullptr;    // one per 64-row group, zero between launches
+  int64_t m = 0, k = 0;
+  int zp_integral = 0;            // all zero-points are integers in [0,1024]: take the 2-op dequant
+  int prologue = PRO_NONE;
+  int epilogue = EPI_STORE;
+  const half_t* gamma = nullptr;  // PRO_RMSNORM: [k]
+  float eps = 0.0f;
+  const half_t* cos_t = nullptr;  // EPI_QKV_ROPE
+  const half_t* sin_t = nullptr;
+  half_t* k_cache = nullptr;
+  half_t* v_cache = nullptr;
+  int32_t hidden = 0;
+  int32_t pos = 0;
+  int64_t max_pos = 0;
+  const StepState* dyn = nullptr;     // pos / out_index come from here when set
+  unsigned long long* best = nullptr;  // EPI_ARGMAX: zero between launches
+  int32_t* done = nullptr;             // EPI_ARGMAX: zero between launches
+  int32_t* out_token = nullptr;
+  int32_t* out_array = nullptr;
 };
+
+// Greedy sampling key: an order-preserving integer image of a binary16 logit
+// with NaN lowest, so that the reference's scan "strict > from index 0"
+// (Inference.cu:1282-1289) becomes a maximum over (key, -index).
+__host__ __device__ inline int32_t awq_logit_key(uint16_t bits) {
+  if ((bits & 0x7fffu) > 0x7c00u) return INT32_MIN;  // NaN never wins
+  if ((bits & 0x7fffu) == 0) return 0;               // -0 == +0 in a float compare
+  return (bits & 0x8000u) ? -(int32_t)(bits & 0x7fffu) : (int32_t)bits;
+}
+__host__ __device__ inline unsigned long long awq_pack_candidate(int32_t key, uint32_t idx) {
+  return ((unsigned long long)((uint32_t)key ^ 0x80000000u) << 32) | (uint32_t)(0xffffffffu - idx);
+}
 
 int launch_dequant(const uint8_t* packed, const half_t* scale, const half_t* zp, half_t* out, int64_t rows,
                    int64_t cols, int64_t n_groups, hipStream_t st);

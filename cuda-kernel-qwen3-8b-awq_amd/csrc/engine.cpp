@@ -144,13 +144,12 @@ struct awq_engine {
   DevLinear embed, unembed;
   half_t *cos_t = nullptr, *sin_t = nullptr;
   // activations (Inference.cu:334-348)
-  half_t *hidden = nullptr, *normed = nullptr, *qkv = nullptr, *q = nullptr, *ctx = nullptr, *mid = nullptr,
-         *logits = nullptr;
+  half_t *hidden = nullptr, *q = nullptr, *ctx = nullptr, *mid = nullptr, *logits = nullptr;
   // workspaces
   float* gemv_partials = nullptr;
   int32_t* gemv_counters = nullptr;
   void* attn_ws = nullptr;
-  void* argmax_ws = nullptr;
+  void* sample_ws = nullptr;  // 64-bit best candidate + finished-row-group counter
   StepState* d_state = nullptr;
   int32_t* d_token = nullptr;
   int32_t* d_out = nullptr;
@@ -214,53 +213,80 @@ bool zp_all_integral(const uint16_t* zp, int64_t n) {
 }
 
 // one fused-linear launch on the engine's stream
-int linear(awq_engine* e, const DevLinear& t, const half_t* x, half_t* y, int epilogue, const half_t* res) {
+LinearArgs linear_args(awq_engine* e, const DevLinear& t, const half_t* x, half_t* y) {
   LinearArgs a;
   a.wq = t.stream_order;
   a.scale = t.scale;
   a.zp = t.zp;
   a.x = x;
   a.y = y;
-  a.res = res;
   a.partials = e->gemv_partials;
   a.counters = e->gemv_counters;
   a.m = t.m;
   a.k = t.k;
   a.zp_integral = t.zp_integral;
-  a.epilogue = epilogue;
-  return launch_gemv(a, e->stream);
+  a.eps = e->cfg.eps;
+  a.dyn = e->d_state;
+  return a;
 }
 
-// runOneLayer, Inference.cu:1029-1230.  The attended length comes from the
-// device-side step state: len_lo or len_hi.
+// runOneLayer, Inference.cu:1029-1230, as five launches.  The position and the
+// attended length come from the device-side step state.
 int enqueue_layer(awq_engine* e, int l, int use_len_hi) {
   LayerDev& L = e->layers[l];
-  const int H = e->cfg.hidden;
   hipStream_t st = e->stream;
-  if (int rc = launch_rmsnorm(e->hidden, L.gamma, e->normed, H, e->cfg.eps, st)) return rc;  // :1040
-  if (int rc = linear(e, L.wqkv, e->normed, e->qkv, EPI_STORE, nullptr)) return rc;          // :1052
-  if (int rc = launch_rope_kv_append(e->qkv, e->cos_t, e->sin_t, e->q, L.kcache, L.vcache, e->n_heads, e->cfg.max_pos,
-                                     0, e->d_state, st))
-    return rc;  // :1070-1103
+  {  // :1040 RMSNorm, :1052 Wqkv, :1070-1103 split + rotary + KV append
+    LinearArgs a = linear_args(e, L.wqkv, e->hidden, e->q);
+    a.prologue = PRO_RMSNORM;
+    a.gamma = L.gamma;
+    a.epilogue = EPI_QKV_ROPE;
+    a.cos_t = e->cos_t;
+    a.sin_t = e->sin_t;
+    a.k_cache = L.kcache;
+    a.v_cache = L.vcache;
+    a.hidden = e->cfg.hidden;
+    a.max_pos = e->cfg.max_pos;
+    if (int rc = launch_gemv(a, st)) return rc;
+  }
   if (int rc = launch_attention(e->q, L.kcache, L.vcache, e->ctx, e->n_heads, e->cfg.max_pos, 0, e->d_state,
                                 use_len_hi, e->attn_ws, st))
     return rc;  // :1110
-  // :1128-1155, Wo product and residual add in one launch; input and output
-  // are distinct buffers (they alias in the reference)
-  if (int rc = linear(e, L.wo, e->ctx, e->hidden, EPI_RESIDUAL, e->hidden)) return rc;
-  if (int rc = launch_rmsnorm(e->hidden, L.gamma, e->normed, H, e->cfg.eps, st)) return rc;  // :1163, same gamma
-  if (int rc = linear(e, L.w1, e->normed, e->mid, EPI_GELU, nullptr)) return rc;             // :1176, :1196
-  if (int rc = linear(e, L.w2, e->mid, e->hidden, EPI_RESIDUAL, e->hidden)) return rc;       // :1201, :1227
+  {  // :1128-1155 Wo product and residual add; input and output are distinct
+     // buffers (they alias in the reference)
+    LinearArgs a = linear_args(e, L.wo, e->ctx, e->hidden);
+    a.epilogue = EPI_RESIDUAL;
+    a.res = e->hidden;
+    if (int rc = launch_gemv(a, st)) return rc;
+  }
+  {  // :1163 RMSNorm with the same gamma, :1176 W1, :1196 GeLU
+    LinearArgs a = linear_args(e, L.w1, e->hidden, e->mid);
+    a.prologue = PRO_RMSNORM;
+    a.gamma = L.gamma;
+    a.epilogue = EPI_GELU;
+    if (int rc = launch_gemv(a, st)) return rc;
+  }
+  {  // :1201 W2, :1227 residual add
+    LinearArgs a = linear_args(e, L.w2, e->mid, e->hidden);
+    a.epilogue = EPI_RESIDUAL;
+    a.res = e->hidden;
+    if (int rc = launch_gemv(a, st)) return rc;
+  }
   return AWQ_OK;
 }
 
-// sampleNextToken, Inference.cu:1235-1292
+// sampleNextToken, Inference.cu:1235-1292: final RMSNorm (gamma of the last
+// layer), unembedding and greedy argmax in one launch
 int enqueue_sample(awq_engine* e) {
-  hipStream_t st = e->stream;
   const int NL = e->cfg.n_layers;
-  if (int rc = launch_rmsnorm(e->hidden, e->layers[NL - 1].gamma, e->normed, e->cfg.hidden, e->cfg.eps, st)) return rc;
-  if (int rc = linear(e, e->unembed, e->normed, e->logits, EPI_STORE, nullptr)) return rc;
-  return launch_argmax(e->logits, e->cfg.vocab, e->d_token, e->argmax_ws, e->d_state, e->d_out, st);
+  LinearArgs a = linear_args(e, e->unembed, e->hidden, e->logits);
+  a.prologue = PRO_RMSNORM;
+  a.gamma = e->layers[NL - 1].gamma;
+  a.epilogue = EPI_ARGMAX;
+  a.best = (unsigned long long*)e->sample_ws;
+  a.done = (int32_t*)((char*)e->sample_ws + 8);
+  a.out_token = e->d_token;
+  a.out_array = e->d_out;
+  return launch_gemv(a, e->stream);
 }
 
 // everything of one position after the step state has been written
@@ -366,15 +392,14 @@ extern "C" int awq_create_empty(const awq_config* cfg_in, awq_engine** out) {
   struct {
     half_t** p;
     int64_t n;
-  } acts[] = {{&e->hidden, H}, {&e->normed, H}, {&e->qkv, 3 * H}, {&e->q, H},     {&e->ctx, H},
-              {&e->mid, I},    {&e->logits, V}};
+  } acts[] = {{&e->hidden, H}, {&e->q, H}, {&e->ctx, H}, {&e->mid, I}, {&e->logits, V}};
   for (auto& a : acts)
     if (int rc = dev_alloc(ep, (void**)a.p, a.n * 2)) return fail(rc);
   int64_t max_m = std::max<int64_t>(std::max<int64_t>(3 * H, I), V);
   if (int rc = dev_alloc(ep, (void**)&e->gemv_partials, 16 * max_m * 4)) return fail(rc);
   if (int rc = dev_alloc(ep, (void**)&e->gemv_counters, (max_m / 64 + 1) * 4)) return fail(rc);
   if (int rc = dev_alloc(ep, &e->attn_ws, attention_workspace_bytes(e->n_heads, cfg.max_pos))) return fail(rc);
-  if (int rc = dev_alloc(ep, &e->argmax_ws, argmax_workspace_bytes(V))) return fail(rc);
+  if (int rc = dev_alloc(ep, &e->sample_ws, 64)) return fail(rc);
   if (int rc = dev_alloc(ep, (void**)&e->d_state, sizeof(StepState))) return fail(rc);
   if (int rc = dev_alloc(ep, (void**)&e->d_token, 4)) return fail(rc);
   if (int rc = dev_alloc(ep, (void**)&e->d_out, (int64_t)cfg.max_pos * 4)) return fail(rc);
@@ -463,7 +488,7 @@ extern "C" int awq_finalize(awq_engine* e) {
   }
   int64_t max_m = std::max<int64_t>(std::max<int64_t>(3 * (int64_t)e->cfg.hidden, e->cfg.inter), e->cfg.vocab);
   if (int rc = launch_fill_zero(e->gemv_counters, (max_m / 64 + 1) * 4, st)) return rc;
-  if (int rc = launch_fill_zero(e->argmax_ws, 64, st)) return rc;
+  if (int rc = launch_fill_zero(e->sample_ws, 64, st)) return rc;
   if (int rc = launch_fill_zero(e->d_token, 4, st)) return rc;
   if (int rc = launch_fill_zero(e->hidden, (int64_t)e->cfg.hidden * 2, st)) return rc;
   AWQ_HIP_TRY(hipStreamSynchronize(st));
@@ -631,17 +656,49 @@ extern "C" int awq_time_linear(awq_engine* e, int kind, int32_t n_rounds, float*
     for (int l = 0; l < n_mats; ++l) {
       const DevLinear& t = *find_linear(e, l, kind);
       int rc = AWQ_OK;
+      LinearArgs a;
       switch (kind) {
-        case AWQ_T_WQKV: rc = linear(e, t, e->normed, e->qkv, EPI_STORE, nullptr); break;
-        case AWQ_T_WO: rc = linear(e, t, e->ctx, e->hidden, EPI_RESIDUAL, e->hidden); break;
-        case AWQ_T_W1: rc = linear(e, t, e->normed, e->mid, EPI_GELU, nullptr); break;
-        case AWQ_T_W2: rc = linear(e, t, e->mid, e->hidden, EPI_RESIDUAL, e->hidden); break;
-        default: rc = linear(e, t, e->normed, e->logits, EPI_STORE, nullptr); break;
+        case AWQ_T_WQKV:
+          a = linear_args(e, t, e->hidden, e->q);
+          a.prologue = PRO_RMSNORM;
+          a.gamma = e->layers[l].gamma;
+          a.epilogue = EPI_QKV_ROPE;
+          a.cos_t = e->cos_t;
+          a.sin_t = e->sin_t;
+          a.k_cache = e->layers[l].kcache;
+          a.v_cache = e->layers[l].vcache;
+          a.hidden = e->cfg.hidden;
+          a.max_pos = e->cfg.max_pos;
+          break;
+        case AWQ_T_WO:
+          a = linear_args(e, t, e->ctx, e->hidden);
+          a.epilogue = EPI_RESIDUAL;
+          a.res = e->hidden;
+          break;
+        case AWQ_T_W1:
+          a = linear_args(e, t, e->hidden, e->mid);
+          a.prologue = PRO_RMSNORM;
+          a.gamma = e->layers[l].gamma;
+          a.epilogue = EPI_GELU;
+          break;
+        case AWQ_T_W2:
+          a = linear_args(e, t, e->mid, e->hidden);
+          a.epilogue = EPI_RESIDUAL;
+          a.res = e->hidden;
+          break;
+        default:
+          a = linear_args(e, t, e->hidden, e->logits);
+          a.prologue = PRO_RMSNORM;
+          a.gamma = e->layers[e->cfg.n_layers - 1].gamma;
+          break;
       }
+      rc = launch_gemv(a, e->stream);
       if (rc) return rc;
     }
     return AWQ_OK;
   };
+  StepState s0{0, 1, 1, -1, 0, 0};
+  if (int rc = launch_set_state(e->d_state, s0, e->stream)) return rc;
   if (int rc = one_round()) return rc;  // warm-up
   AWQ_HIP_TRY(hipEventRecord(ev0, e->stream));
   for (int r = 0; r < n_rounds; ++r)
@@ -678,31 +735,66 @@ extern "C" int awq_linear_repack(const void* packed_in, void* repacked_out, int6
 
 extern "C" int64_t awq_gemv_workspace_bytes(int64_t m, int64_t k) { return gemv_workspace_bytes(m, k); }
 
-extern "C" int awq_gemv(const void* repacked, const void* scale, const void* zp, int64_t m, int64_t k, const void* x,
-                        void* y, int32_t zp_integral, void* workspace, void* stream) {
-  AWQ_REQUIRE(repacked && scale && zp && x && y && workspace, "NULL pointer");
-  AWQ_REQUIRE(m > 0 && m % 128 == 0, "m must be a positive multiple of 128");
+extern "C" int awq_gemv_fused(const awq_linear_args* u, void* stream) {
+  AWQ_REQUIRE(u != nullptr, "args is NULL");
+  AWQ_REQUIRE(u->repacked && u->scale && u->zp && u->x && u->y && u->workspace, "NULL pointer");
+  AWQ_REQUIRE(u->m > 0 && u->m % 128 == 0, "m must be a positive multiple of 128");
+  AWQ_REQUIRE(u->prologue == AWQ_PRO_NONE || u->prologue == AWQ_PRO_RMSNORM, "bad prologue");
+  AWQ_REQUIRE(u->epilogue >= AWQ_EPI_STORE && u->epilogue <= AWQ_EPI_ARGMAX, "bad epilogue");
+  int zp_integral = u->zp_integral;
   if (zp_integral < 0) {
     // look at the zero-points on the device (synchronises the stream)
-    std::vector<uint16_t> zph((size_t)(m / 128));
-    AWQ_HIP_TRY(hipMemcpyAsync(zph.data(), zp, zph.size() * 2, hipMemcpyDeviceToHost, (hipStream_t)stream));
+    std::vector<uint16_t> zph((size_t)(u->m / 128));
+    AWQ_HIP_TRY(hipMemcpyAsync(zph.data(), u->zp, zph.size() * 2, hipMemcpyDeviceToHost, (hipStream_t)stream));
     AWQ_HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
     zp_integral = zp_all_integral(zph.data(), (int64_t)zph.size());
   }
   LinearArgs a;
-  a.wq = repacked;
-  a.scale = (const half_t*)scale;
-  a.zp = (const half_t*)zp;
-  a.x = (const half_t*)x;
-  a.y = (half_t*)y;
-  a.res = nullptr;
-  a.counters = (int32_t*)workspace;
-  a.partials = (float*)((char*)workspace + ((m / 64) * 4 + 255) / 256 * 256);
-  a.m = m;
-  a.k = k;
+  a.wq = u->repacked;
+  a.scale = (const half_t*)u->scale;
+  a.zp = (const half_t*)u->zp;
+  a.x = (const half_t*)u->x;
+  a.y = (half_t*)u->y;
+  a.res = (const half_t*)u->residual;
+  // workspace: [0,8) best candidate, [8,12) finished counter, [64,..) one counter
+  // per 64-row group, then the split-k partial sums
+  char* ws = (char*)u->workspace;
+  a.best = (unsigned long long*)ws;
+  a.done = (int32_t*)(ws + 8);
+  a.counters = (int32_t*)(ws + 64);
+  a.partials = (float*)(ws + 64 + ((u->m / 64) * 4 + 255) / 256 * 256);
+  a.m = u->m;
+  a.k = u->k;
   a.zp_integral = zp_integral != 0;
-  a.epilogue = EPI_STORE;
+  a.prologue = u->prologue;
+  a.epilogue = u->epilogue;
+  a.gamma = (const half_t*)u->gamma;
+  a.eps = u->eps;
+  a.cos_t = (const half_t*)u->cos_t;
+  a.sin_t = (const half_t*)u->sin_t;
+  a.k_cache = (half_t*)u->k_cache;
+  a.v_cache = (half_t*)u->v_cache;
+  a.hidden = u->hidden;
+  a.pos = (int32_t)u->pos;
+  a.max_pos = u->max_pos;
+  a.out_token = (int32_t*)u->out_token;
   return launch_gemv(a, (hipStream_t)stream);
+}
+
+extern "C" int awq_gemv(const void* repacked, const void* scale, const void* zp, int64_t m, int64_t k, const void* x,
+                        void* y, int32_t zp_integral, void* workspace, void* stream) {
+  awq_linear_args u;
+  memset(&u, 0, sizeof(u));
+  u.repacked = repacked;
+  u.scale = scale;
+  u.zp = zp;
+  u.m = m;
+  u.k = k;
+  u.x = x;
+  u.y = y;
+  u.zp_integral = zp_integral;
+  u.workspace = workspace;
+  return awq_gemv_fused(&u, stream);
 }
 
 extern "C" int awq_rmsnorm(const void* x, const void* gamma, void* out, int64_t n, float eps, void* stream) {

@@ -13,6 +13,7 @@
 // (and the same after one shift by 8) yields two weights as the low mantissa
 // bits of a packed pair of binary16 numbers 1024+q or 1024+16q.
 #include "common.hpp"
+#include <stdlib.h>
 
 namespace {
 
@@ -166,27 +167,109 @@ struct GemvParams {
   int32_t C;         // group period
   int32_t n_slabs;   // workgroups along k
   int32_t mg, kg;    // m/128, k/128
+  int32_t prologue, epilogue;
+  // PRO_RMSNORM
+  const half_t* gamma;
+  float eps;
+  // EPI_QKV_ROPE
+  const half_t* cos_t;
+  const half_t* sin_t;
+  half_t* k_cache;
+  half_t* v_cache;
+  int32_t hidden;
+  int32_t pos;
+  int64_t max_pos;
+  const StepState* dyn;
+  // EPI_ARGMAX
+  unsigned long long* best;
+  int32_t* done;
+  int32_t* out_token;
+  int32_t* out_array;
 };
 
-template <int EPI>
-__device__ __forceinline__ void epilogue(const GemvParams& p, int row, float acc) {
+__device__ __forceinline__ void epilogue(const GemvParams& p, int row, int lane, float acc) {
   half_t v = (half_t)acc;
-  if (EPI == EPI_RESIDUAL) {
-    v = p.res[row] + v;
-  } else if (EPI == EPI_GELU) {
-    v = to_half_rn(awq_gelu_f32((float)v));
+  switch (p.epilogue) {
+    case EPI_RESIDUAL:  // Inference.cu:1149-1155
+      p.y[row] = p.res[row] + v;
+      return;
+    case EPI_GELU:  // Inference.cu:271-279
+      p.y[row] = to_half_rn(awq_gelu_f32((float)v));
+      return;
+    case EPI_QKV_ROPE: {
+      // Inference.cu:1070-1103: rows [0,H) are Q, [H,2H) K, [2H,3H) V.  Q and K
+      // are rotated pairwise (Inference.cu:158-176); K and V go to the cache
+      // row of this position, Q to y.
+      const int pos = p.dyn ? p.dyn->pos : p.pos;
+      const int H = p.hidden;
+      const int sec = row / H;  // same for the whole wavefront
+      const int r = row - sec * H;
+      const int d = r & (AWQ_HEAD_DIM - 1);
+      half_t other = __builtin_bit_cast(half_t, (unsigned short)__shfl_xor((int)__builtin_bit_cast(unsigned short, v), 1, 64));
+      half_t out = v;
+      if (sec < 2) {
+        const half_t c = p.cos_t[(int64_t)pos * 64 + (d >> 1)], s = p.sin_t[(int64_t)pos * 64 + (d >> 1)];
+        const half_t a = (lane & 1) ? other : v, b = (lane & 1) ? v : other;
+        if (lane & 1) {
+          half_t as = a * s, bc = b * c;
+          out = as + bc;
+        } else {
+          half_t ac = a * c, bs = b * s;
+          out = ac - bs;
+        }
+      }
+      if (sec == 0) {
+        p.y[r] = out;
+      } else {
+        half_t* cache = sec == 1 ? p.k_cache : p.v_cache;
+        cache[((int64_t)(r >> 7) * p.max_pos + pos) * AWQ_HEAD_DIM + d] = out;
+      }
+      return;
+    }
+    case EPI_ARGMAX: {
+      // Inference.cu:1278-1290 on the device: the best (value, lowest index)
+      // pair of the vocabulary is kept with a 64-bit atomic max, which does
+      // not depend on arrival order.
+      p.y[row] = v;
+      const unsigned short bits = __builtin_bit_cast(unsigned short, v);
+      int32_t key = awq_logit_key(bits);
+      if (row == 0 && (bits & 0x7fffu) > 0x7c00u) key = INT32_MAX;  // a NaN at index 0 is never displaced
+      unsigned long long cand = awq_pack_candidate(key, (uint32_t)row);
+#pragma unroll
+      for (int mask = 1; mask < 64; mask <<= 1) {
+        unsigned long long o = __shfl_xor(cand, mask, 64);
+        cand = o > cand ? o : cand;
+      }
+      if (lane == 0) {
+        __hip_atomic_fetch_max(p.best, cand, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __builtin_amdgcn_s_waitcnt(0);
+        int old = __hip_atomic_fetch_add(p.done, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (old == p.m / 64 - 1) {
+          unsigned long long b = __hip_atomic_load(p.best, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          int32_t tok = (int32_t)(0xffffffffu - (uint32_t)(b & 0xffffffffull));
+          *p.out_token = tok;
+          if (p.out_array && p.dyn) p.out_array[p.dyn->out_index] = tok;
+          __hip_atomic_store(p.best, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(p.done, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+      }
+      return;
+    }
+    default:
+      p.y[row] = v;
   }
-  p.y[row] = v;
 }
 
 // NI groups of four blocks per wavefront; 4 wavefronts per workgroup cover
 // 16*NI consecutive blocks of one 64-row group.
-template <int NI, bool ZINT, bool PERIODIC, int EPI>
+template <int NI, bool ZINT, bool PERIODIC>
 __global__ __launch_bounds__(256) void gemv_kernel(GemvParams p) {
   constexpr int NB = 4 * NI;
   __shared__ __attribute__((aligned(16))) half_t xs[4 * NB * AWQ_BLOCK_K];
   __shared__ float red[4][64];
   __shared__ float fin[16][64];  // slab partials of the finishing wavefront
+  __shared__ GroupConst gtab[PERIODIC ? 64 : 1];
+  __shared__ float nbuf[256];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -201,11 +284,38 @@ __global__ __launch_bounds__(256) void gemv_kernel(GemvParams p) {
 #pragma unroll
   for (int n = 0; n < 4; ++n) wreg[0][n] = __builtin_nontemporal_load(wp + n * 64);
 
-  // stage this workgroup's slice of x in block order
-  if (PERIODIC) {
+  // stage this workgroup's slice of x in block order, normalising it on the
+  // way when the RMSNorm is fused in (Inference.cu:111-145: 256 strided fma
+  // partial sums, stride-halving tree, then two binary16 multiplies)
+  half_t sc = (half_t)1.0f;
+  if (p.prologue == PRO_RMSNORM) {
+    float acc = 0.0f;
+    for (int i = tid; i < p.k; i += 256) {
+      float v = (float)p.x[i];
+      acc = __builtin_fmaf(v, v, acc);
+    }
+    nbuf[tid] = acc;
+    __syncthreads();
+    if (tid < 128) nbuf[tid] += nbuf[tid + 128];
+    __syncthreads();
+    if (tid < 64) {
+      float v = nbuf[tid] + nbuf[tid + 64];
+#pragma unroll
+      for (int stride = 32; stride > 0; stride >>= 1) v += __shfl_down(v, stride, 64);
+      if (tid == 0) nbuf[0] = v;
+    }
+    __syncthreads();
+    sc = (half_t)awq_rsqrtf(nbuf[0] / (float)p.k + p.eps);
+  }
+  if (PERIODIC || p.prologue == PRO_RMSNORM) {
     for (int e = tid; e < 4 * NB * AWQ_BLOCK_K; e += 256) {
-      int64_t j = awq_block_elem(p.k, p.C, blk_wg + (e >> 5), e & 31);
-      xs[e] = p.x[j];
+      int64_t j = PERIODIC ? awq_block_elem(p.k, p.C, blk_wg + (e >> 5), e & 31) : (int64_t)blk_wg * AWQ_BLOCK_K + e;
+      half_t v = p.x[j];
+      if (p.prologue == PRO_RMSNORM) {
+        half_t t = v * sc;
+        v = t * p.gamma[j];
+      }
+      xs[e] = v;
     }
   } else {
     const uint2* src = reinterpret_cast<const uint2*>(p.x + (int64_t)blk_wg * AWQ_BLOCK_K);
@@ -213,14 +323,24 @@ __global__ __launch_bounds__(256) void gemv_kernel(GemvParams p) {
   }
 
   // scale group of this wavefront's 64 rows: row/128, then Inference.cu:90 with
-  // the index wrapped to the m/128 stored entries
+  // the index wrapped to the m/128 stored entries.  When the group depends on
+  // the input index it is constant within a class of blocks; the (at most 64)
+  // classes go through a table in LDS.
   const int a = rg >> 1;
   GroupConst g;
   if (!PERIODIC) {
     int gi = (a % p.kg) % p.mg;
     g = make_group<ZINT>(p.scale[gi], p.zp[gi]);
+  } else if (tid < p.C) {
+    int gi = (int)((((int64_t)tid * p.mg + a) % p.kg) % p.mg);
+    gtab[tid] = make_group<ZINT>(p.scale[gi], p.zp[gi]);
   }
   const int U = p.nblk / p.C;  // blocks per class (PERIODIC)
+  int cls = 0, cls_left = 0;   // class of the next block and blocks left in it
+  if (PERIODIC) {
+    cls = blk_wave / U;
+    cls_left = U - (blk_wave - cls * U);
+  }
   __syncthreads();
 
   float g4[NI];
@@ -235,9 +355,11 @@ __global__ __launch_bounds__(256) void gemv_kernel(GemvParams p) {
     for (int n = 0; n < 4; ++n) {
       const int bl = it * 4 + n;
       if (PERIODIC) {
-        int c = (blk_wave + bl) / U;
-        int gi = (int)((((int64_t)c * p.mg + a) % p.kg) % p.mg);
-        g = make_group<ZINT>(p.scale[gi], p.zp[gi]);
+        g = gtab[cls];
+        if (--cls_left == 0) {
+          ++cls;
+          cls_left = U;
+        }
       }
       bs[n] = block_dot<ZINT>(wreg[it & 1][n], xs + (wave * NB + bl) * AWQ_BLOCK_K, g);
     }
@@ -255,18 +377,20 @@ __global__ __launch_bounds__(256) void gemv_kernel(GemvParams p) {
   float v = (red[0][lane] + red[1][lane]) + (red[2][lane] + red[3][lane]);
   const int row = rg * 64 + lane;
   if (p.n_slabs == 1) {
-    epilogue<EPI>(p, row, v);
+    epilogue(p, row, lane, v);
     return;
   }
-  // split along k: publish, and let the last workgroup of this row group
-  // finish the tree in slab order
-  p.partials[(int64_t)slab * p.m + row] = v;
-  __threadfence();
+  // Split along k: publish, and let the last workgroup of this row group
+  // finish the tree in slab order.  The partial sums travel as device-scope
+  // atomic stores and loads (they go to the level of the memory system that
+  // all compute dies share), so no cache write-back or invalidate is needed:
+  // wait until this wavefront's stores have been acknowledged, then count.
+  __hip_atomic_store(&p.partials[(int64_t)slab * p.m + row], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __builtin_amdgcn_s_waitcnt(0);
   int old = 0;
-  if (lane == 0) old = __hip_atomic_fetch_add(&p.counters[rg], 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+  if (lane == 0) old = __hip_atomic_fetch_add(&p.counters[rg], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   old = __builtin_amdgcn_readfirstlane(old);
   if (old != p.n_slabs - 1) return;
-  __threadfence();
   int n = p.n_slabs;
   for (int s = 0; s < n; ++s)
     fin[s][lane] = __hip_atomic_load(&p.partials[(int64_t)s * p.m + row], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -276,8 +400,8 @@ __global__ __launch_bounds__(256) void gemv_kernel(GemvParams p) {
   }
   float tot = fin[0][lane];
   for (int q = 1; q < n; ++q) tot += fin[q][lane];
-  epilogue<EPI>(p, row, tot);
   if (lane == 0) __hip_atomic_store(&p.counters[rg], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  epilogue(p, row, lane, tot);
 }
 
 struct GemvPlan {
@@ -291,6 +415,10 @@ GemvPlan plan_gemv(int64_t m, int64_t k) {
   int64_t units = k / AWQ_BLOCK_K / 16;  // NI * n_slabs
   int64_t rgs = m / 64;
   GemvPlan best{1, (int)units};
+  if (const char* f = getenv("AWQ_DEV_NI")) {
+    int ni = atoi(f);
+    if (ni >= 1 && units % ni == 0 && units / ni <= 16) return GemvPlan{ni, (int)(units / ni)};
+  }
   for (int ni = 8; ni >= 1; ni >>= 1) {
     if (units % ni) continue;
     int64_t slabs = units / ni;
@@ -301,23 +429,14 @@ GemvPlan plan_gemv(int64_t m, int64_t k) {
   return best;
 }
 
-template <int NI, bool ZINT, bool PERIODIC>
-void launch_epi(const GemvParams& p, int epi, dim3 grid, hipStream_t st) {
-  switch (epi) {
-    case EPI_RESIDUAL: hipLaunchKernelGGL((gemv_kernel<NI, ZINT, PERIODIC, EPI_RESIDUAL>), grid, dim3(256), 0, st, p); break;
-    case EPI_GELU: hipLaunchKernelGGL((gemv_kernel<NI, ZINT, PERIODIC, EPI_GELU>), grid, dim3(256), 0, st, p); break;
-    default: hipLaunchKernelGGL((gemv_kernel<NI, ZINT, PERIODIC, EPI_STORE>), grid, dim3(256), 0, st, p); break;
-  }
-}
-
 template <int NI>
-void launch_ni(const GemvParams& p, bool zint, bool periodic, int epi, dim3 grid, hipStream_t st) {
+void launch_ni(const GemvParams& p, bool zint, bool periodic, dim3 grid, hipStream_t st) {
   if (zint) {
-    if (periodic) launch_epi<NI, true, true>(p, epi, grid, st);
-    else launch_epi<NI, true, false>(p, epi, grid, st);
+    if (periodic) hipLaunchKernelGGL((gemv_kernel<NI, true, true>), grid, dim3(256), 0, st, p);
+    else hipLaunchKernelGGL((gemv_kernel<NI, true, false>), grid, dim3(256), 0, st, p);
   } else {
-    if (periodic) launch_epi<NI, false, true>(p, epi, grid, st);
-    else launch_epi<NI, false, false>(p, epi, grid, st);
+    if (periodic) hipLaunchKernelGGL((gemv_kernel<NI, false, true>), grid, dim3(256), 0, st, p);
+    else hipLaunchKernelGGL((gemv_kernel<NI, false, false>), grid, dim3(256), 0, st, p);
   }
 }
 
@@ -342,6 +461,7 @@ static int check_linear_shape(int64_t m, int64_t k) {
   AWQ_REQUIRE(m < (1ll << 31) && k < (1ll << 31) && m / 64 < 2147483647ll, "shape too large");
   int C = awq_group_period(m, k);
   AWQ_REQUIRE((k / AWQ_BLOCK_K) % C == 0, "k/32 must be a multiple of the scale-group period");
+  AWQ_REQUIRE(C <= 64, "scale-group period above 64 is not supported");
   return AWQ_OK;
 }
 
@@ -355,9 +475,9 @@ int launch_repack(const uint8_t* in, void* out, int64_t m, int64_t k, hipStream_
 }
 
 int64_t gemv_workspace_bytes(int64_t m, int64_t k) {
-  // up to 16 slabs of FP32 partials plus one counter per 64-row group
+  // 64 bytes for the sampler, one counter per 64-row group, up to 16 slabs of FP32 partials
   (void)k;
-  return 16 * m * 4 + ((m / 64) * 4 + 255) / 256 * 256;
+  return 64 + 16 * m * 4 + ((m / 64) * 4 + 255) / 256 * 256;
 }
 
 int launch_gemv(const LinearArgs& a, hipStream_t st) {
@@ -365,6 +485,15 @@ int launch_gemv(const LinearArgs& a, hipStream_t st) {
   GemvPlan plan = plan_gemv(a.m, a.k);
   AWQ_REQUIRE(plan.n_slabs <= 16, "k too large for the split workspace");
   AWQ_REQUIRE(plan.n_slabs == 1 || (a.partials && a.counters), "split-k launch needs a workspace");
+  AWQ_REQUIRE(a.prologue != PRO_RMSNORM || (a.gamma && a.k % 256 == 0), "fused RMSNorm needs gamma and k % 256 == 0");
+  AWQ_REQUIRE(a.epilogue != EPI_RESIDUAL || a.res, "residual epilogue needs res");
+  if (a.epilogue == EPI_QKV_ROPE) {
+    AWQ_REQUIRE(a.cos_t && a.sin_t && a.k_cache && a.v_cache && a.hidden > 0 && a.m == 3 * (int64_t)a.hidden &&
+                    a.hidden % AWQ_HEAD_DIM == 0 && a.max_pos > 0,
+                "QKV epilogue needs rotary tables, caches and m == 3*hidden");
+    AWQ_REQUIRE(a.dyn || (a.pos >= 0 && a.pos < a.max_pos), "pos out of range");
+  }
+  if (a.epilogue == EPI_ARGMAX) AWQ_REQUIRE(a.best && a.done && a.out_token, "argmax epilogue needs its workspace");
   GemvParams p;
   p.wq = (const u32x4*)a.wq;
   p.scale = a.scale;
@@ -381,13 +510,29 @@ int launch_gemv(const LinearArgs& a, hipStream_t st) {
   p.n_slabs = plan.n_slabs;
   p.mg = (int32_t)(a.m / 128);
   p.kg = (int32_t)(a.k / 128);
+  p.prologue = a.prologue;
+  p.epilogue = a.epilogue;
+  p.gamma = a.gamma;
+  p.eps = a.eps;
+  p.cos_t = a.cos_t;
+  p.sin_t = a.sin_t;
+  p.k_cache = a.k_cache;
+  p.v_cache = a.v_cache;
+  p.hidden = a.hidden;
+  p.pos = a.pos;
+  p.max_pos = a.max_pos;
+  p.dyn = a.dyn;
+  p.best = a.best;
+  p.done = a.done;
+  p.out_token = a.out_token;
+  p.out_array = a.out_array;
   bool periodic = p.C > 1;
   dim3 grid((unsigned)(a.m / 64), (unsigned)plan.n_slabs);
   switch (plan.ni) {
-    case 1: launch_ni<1>(p, a.zp_integral, periodic, a.epilogue, grid, st); break;
-    case 2: launch_ni<2>(p, a.zp_integral, periodic, a.epilogue, grid, st); break;
-    case 4: launch_ni<4>(p, a.zp_integral, periodic, a.epilogue, grid, st); break;
-    default: launch_ni<8>(p, a.zp_integral, periodic, a.epilogue, grid, st); break;
+    case 1: launch_ni<1>(p, a.zp_integral, periodic, grid, st); break;
+    case 2: launch_ni<2>(p, a.zp_integral, periodic, grid, st); break;
+    case 4: launch_ni<4>(p, a.zp_integral, periodic, grid, st); break;
+    default: launch_ni<8>(p, a.zp_integral, periodic, grid, st); break;
   }
   AWQ_HIP_TRY(hipGetLastError());
   return AWQ_OK;

@@ -92,18 +92,6 @@ __global__ __launch_bounds__(256) void embed_kernel(const uint8_t* __restrict__ 
 }
 
 // Greedy sampling (Inference.cu:1278-1290) without leaving the device.
-// key = order-preserving integer image of the binary16 logit, NaN lowest, so
-// the scan "strict > from index 0" becomes max over (key, -index).
-__device__ __forceinline__ int32_t logit_key(uint16_t bits) {
-  if ((bits & 0x7fffu) > 0x7c00u) return INT32_MIN;       // NaN never wins
-  if ((bits & 0x7fffu) == 0) return 0;                    // -0 == +0 in a float compare
-  return (bits & 0x8000u) ? -(int32_t)(bits & 0x7fffu) : (int32_t)bits;
-}
-__device__ __forceinline__ unsigned long long pack_cand(int32_t key, uint32_t idx) {
-  // larger key first, then smaller index
-  return ((unsigned long long)((uint32_t)key ^ 0x80000000u) << 32) | (uint32_t)(0xffffffffu - idx);
-}
-
 __global__ __launch_bounds__(256) void argmax_kernel(const uint16_t* __restrict__ logits, int64_t n,
                                                      unsigned long long* cand, int32_t* counter, int32_t* out_token,
                                                      const StepState* dyn, int32_t* out_array) {
@@ -111,7 +99,7 @@ __global__ __launch_bounds__(256) void argmax_kernel(const uint16_t* __restrict_
   const int tid = threadIdx.x;
   unsigned long long best = 0;
   for (int64_t i = (int64_t)blockIdx.x * 256 + tid; i < n; i += (int64_t)gridDim.x * 256) {
-    unsigned long long c = pack_cand(logit_key(logits[i]), (uint32_t)i);
+    unsigned long long c = awq_pack_candidate(awq_logit_key(logits[i]), (uint32_t)i);
     best = c > best ? c : best;
   }
   sh[tid] = best;

@@ -140,6 +140,50 @@ int64_t awq_gemv_workspace_bytes(int64_t m, int64_t k);
 int awq_gemv(const void* repacked, const void* scale, const void* zp, int64_t m, int64_t k, const void* x, void* y,
              int32_t zp_integral, void* workspace, void* stream);
 
+/* The same kernel with the neighbouring operators of runOneLayer /
+ * sampleNextToken fused in, as the engine launches it:
+ *   prologue AWQ_PRO_RMSNORM   x is the un-normalised hidden state; rmsNormKernel
+ *                              (Inference.cu:111-145) with gamma/eps runs first (k % 256 == 0)
+ *   epilogue AWQ_EPI_RESIDUAL  y = h(residual + h(acc))          Inference.cu:1149-1155
+ *            AWQ_EPI_GELU      y = h(gelu(h(acc)))               Inference.cu:271-279
+ *            AWQ_EPI_QKV_ROPE  m == 3*hidden: rows [0,hidden) rotated to y (Q), rows
+ *                              [hidden,2*hidden) rotated into k_cache at pos, the rest
+ *                              into v_cache at pos                Inference.cu:1070-1103
+ *            AWQ_EPI_ARGMAX    y = h(acc) and *out_token = greedy token  Inference.cu:1278-1290
+ * Unused pointers may be NULL. */
+#define AWQ_PRO_NONE 0
+#define AWQ_PRO_RMSNORM 1
+#define AWQ_EPI_STORE 0
+#define AWQ_EPI_RESIDUAL 1
+#define AWQ_EPI_GELU 2
+#define AWQ_EPI_QKV_ROPE 3
+#define AWQ_EPI_ARGMAX 4
+typedef struct awq_linear_args {
+  const void* repacked;
+  const void* scale;
+  const void* zp;
+  int64_t m, k;
+  const void* x;
+  void* y;
+  int32_t zp_integral;
+  int32_t prologue;
+  int32_t epilogue;
+  float eps;
+  const void* gamma;     /* [k] FP16 */
+  const void* residual;  /* [m] FP16, may alias y */
+  const void* cos_t;     /* [max_pos][64] FP16 */
+  const void* sin_t;
+  void* k_cache;         /* [hidden/128][max_pos][128] FP16 */
+  void* v_cache;
+  int32_t hidden;
+  int32_t reserved;
+  int64_t max_pos;
+  int64_t pos;
+  void* out_token;       /* device int32 */
+  void* workspace;       /* awq_gemv_workspace_bytes(m,k), zero-filled once */
+} awq_linear_args;
+int awq_gemv_fused(const awq_linear_args* args, void* stream);
+
 /* rmsNormKernel, Inference.cu:111-145.  n multiple of 256. */
 int awq_rmsnorm(const void* x, const void* gamma, void* out, int64_t n, float eps, void* stream);
 

@@ -320,3 +320,119 @@ def test_embed_gather_bit_exact(awq, lib, oracle, torch_gpu):
         torch.cuda.synchronize()
         assert np.array_equal(d_o.cpu().numpy().view(np.uint16), ref.view(np.uint16)), tok
     assert lib.awq_embed_gather(d_p.data_ptr(), d_s.data_ptr(), d_z.data_ptr(), H, V, V, d_o.data_ptr(), None) != 0
+
+
+# ----------------------------------------------------------------------------- fused linear launches
+def fused_setup(awq, lib, torch, rng, m, k, zp_int=True):
+    packed, scale, zp = rand_awq(rng, m, k, zp_int=zp_int)
+    d_in = dev(torch, packed)
+    d_w = torch.zeros(m * k // 2, dtype=torch.uint8, device="cuda")
+    awq.check(lib.awq_linear_repack(d_in.data_ptr(), d_w.data_ptr(), m, k, stream(torch)))
+    keep = dict(d_w=d_w, d_s=dev(torch, scale), d_z=dev(torch, zp),
+                ws=torch.zeros(lib.awq_gemv_workspace_bytes(m, k), dtype=torch.uint8, device="cuda"))
+    a = awq.AwqLinearArgs()
+    a.repacked, a.scale, a.zp = keep["d_w"].data_ptr(), keep["d_s"].data_ptr(), keep["d_z"].data_ptr()
+    a.m, a.k, a.zp_integral, a.workspace = m, k, 1 if zp_int else 0, keep["ws"].data_ptr()
+    return packed, scale, zp, a, keep
+
+
+@pytest.mark.parametrize("m,k", [(256, 512), (12288, 4096), (4096, 12288)])
+def test_gemv_fused_norm_gelu_residual(awq, lib, oracle, torch_gpu, m, k):
+    torch = torch_gpu
+    rng = np.random.default_rng(m + 3 * k)
+    packed, scale, zp, a, keep = fused_setup(awq, lib, torch, rng, m, k)
+    hidden = (rng.standard_normal(k) * 2).astype(np.float16)
+    gamma = (1 + 0.02 * rng.standard_normal(k)).astype(np.float16)
+    res = rng.standard_normal(m).astype(np.float16)
+    normed = np.zeros(k, dtype=np.float16)
+    oracle.awqo_rmsnorm(ptr(hidden), ptr(gamma), ptr(normed), k, 1e-6)
+    lin = np.zeros(m, dtype=np.float16)
+    oracle.awqo_linear(ptr(packed), ptr(scale), ptr(zp), m, k, ptr(normed), ptr(lin), 1)
+    d_h, d_g, d_r = dev(torch, hidden), dev(torch, gamma), dev(torch, res)
+    d_y = torch.zeros(m, dtype=torch.float16, device="cuda")
+    a.x, a.y, a.gamma, a.eps = d_h.data_ptr(), d_y.data_ptr(), d_g.data_ptr(), 1e-6
+    # RMSNorm prologue, plain store
+    a.prologue, a.epilogue = awq.PRO_RMSNORM, awq.EPI_STORE
+    awq.check(lib.awq_gemv_fused(ctypes.byref(a), stream(torch)))
+    torch.cuda.synchronize()
+    assert np.array_equal(d_y.cpu().numpy().view(np.uint16), lin.view(np.uint16))
+    # RMSNorm prologue + GeLU epilogue (the W1 launch)
+    a.epilogue = awq.EPI_GELU
+    awq.check(lib.awq_gemv_fused(ctypes.byref(a), stream(torch)))
+    torch.cuda.synchronize()
+    g = lin.copy()
+    oracle.awqo_gelu(ptr(g), m)
+    assert np.array_equal(d_y.cpu().numpy().view(np.uint16), g.view(np.uint16))
+    # residual epilogue in place (the Wo / W2 launches)
+    a.prologue, a.epilogue = awq.PRO_NONE, awq.EPI_RESIDUAL
+    d_n = dev(torch, normed)
+    a.x, a.y, a.residual = d_n.data_ptr(), d_r.data_ptr(), d_r.data_ptr()
+    awq.check(lib.awq_gemv_fused(ctypes.byref(a), stream(torch)))
+    torch.cuda.synchronize()
+    rr = np.zeros(m, dtype=np.float16)
+    oracle.awqo_residual(ptr(res), ptr(lin), ptr(rr), m)
+    assert np.array_equal(d_r.cpu().numpy().view(np.uint16), rr.view(np.uint16))
+
+
+@pytest.mark.parametrize("H,pos", [(512, 0), (512, 5), (4096, 512)])
+def test_gemv_fused_qkv_rope_kv_append(awq, lib, oracle, torch_gpu, H, pos):
+    """config 2's first launch: RMSNorm + Wqkv + split + rotary + KV append"""
+    torch = torch_gpu
+    m, k, nh, mp = 3 * H, H, H // 128, 640
+    rng = np.random.default_rng(H + pos)
+    packed, scale, zp, a, keep = fused_setup(awq, lib, torch, rng, m, k)
+    hidden = rng.standard_normal(k).astype(np.float16)
+    gamma = (1 + 0.02 * rng.standard_normal(k)).astype(np.float16)
+    cos_t, sin_t = np.zeros((mp, 64), np.float16), np.zeros((mp, 64), np.float16)
+    oracle.awqo_rope_tables(ptr(cos_t), ptr(sin_t), mp)
+    normed = np.zeros(k, dtype=np.float16)
+    oracle.awqo_rmsnorm(ptr(hidden), ptr(gamma), ptr(normed), k, 1e-6)
+    qkv = np.zeros(m, dtype=np.float16)
+    oracle.awqo_linear(ptr(packed), ptr(scale), ptr(zp), m, k, ptr(normed), ptr(qkv), 1)
+    q_ref, k_ref, v_ref = qkv[:H].copy(), qkv[H:2 * H].copy(), qkv[2 * H:].copy()
+    oracle.awqo_rotary(ptr(q_ref), ptr(cos_t), ptr(sin_t), nh, pos)
+    oracle.awqo_rotary(ptr(k_ref), ptr(cos_t), ptr(sin_t), nh, pos)
+    kc_ref = rng.standard_normal(nh * mp * 128).astype(np.float16)
+    vc_ref = rng.standard_normal(nh * mp * 128).astype(np.float16)
+    d_kc, d_vc = dev(torch, kc_ref), dev(torch, vc_ref)
+    oracle.awqo_kv_append(ptr(kc_ref), ptr(k_ref), nh, mp, pos)
+    oracle.awqo_kv_append(ptr(vc_ref), ptr(v_ref), nh, mp, pos)
+    d_h, d_g, d_c, d_s = dev(torch, hidden), dev(torch, gamma), dev(torch, cos_t), dev(torch, sin_t)
+    d_q = torch.zeros(H, dtype=torch.float16, device="cuda")
+    a.x, a.y, a.gamma, a.eps = d_h.data_ptr(), d_q.data_ptr(), d_g.data_ptr(), 1e-6
+    a.prologue, a.epilogue = awq.PRO_RMSNORM, awq.EPI_QKV_ROPE
+    a.cos_t, a.sin_t, a.k_cache, a.v_cache = d_c.data_ptr(), d_s.data_ptr(), d_kc.data_ptr(), d_vc.data_ptr()
+    a.hidden, a.max_pos, a.pos = H, mp, pos
+    awq.check(lib.awq_gemv_fused(ctypes.byref(a), stream(torch)))
+    torch.cuda.synchronize()
+    assert np.array_equal(d_q.cpu().numpy().view(np.uint16), q_ref.view(np.uint16))
+    assert np.array_equal(d_kc.cpu().numpy().view(np.uint16), kc_ref.view(np.uint16))
+    assert np.array_equal(d_vc.cpu().numpy().view(np.uint16), vc_ref.view(np.uint16))
+    a.pos = mp
+    assert lib.awq_gemv_fused(ctypes.byref(a), stream(torch)) != 0
+
+
+@pytest.mark.parametrize("m,k", [(128 * 37, 512), (151936, 4096)])
+def test_gemv_fused_norm_unembed_argmax(awq, lib, oracle, torch_gpu, m, k):
+    """config 3: final RMSNorm + unembedding + greedy argmax in one launch"""
+    torch = torch_gpu
+    rng = np.random.default_rng(m)
+    packed, scale, zp, a, keep = fused_setup(awq, lib, torch, rng, m, k)
+    gamma = (1 + 0.02 * rng.standard_normal(k)).astype(np.float16)
+    d_g = dev(torch, gamma)
+    tok = torch.full((1,), -1, dtype=torch.int32, device="cuda")
+    d_y = torch.zeros(m, dtype=torch.float16, device="cuda")
+    for trial in range(3):
+        hidden = rng.standard_normal(k).astype(np.float16)
+        normed = np.zeros(k, dtype=np.float16)
+        oracle.awqo_rmsnorm(ptr(hidden), ptr(gamma), ptr(normed), k, 1e-6)
+        logits = np.zeros(m, dtype=np.float16)
+        oracle.awqo_linear(ptr(packed), ptr(scale), ptr(zp), m, k, ptr(normed), ptr(logits), 1)
+        d_h = dev(torch, hidden)
+        a.x, a.y, a.gamma, a.eps, a.out_token = d_h.data_ptr(), d_y.data_ptr(), d_g.data_ptr(), 1e-6, tok.data_ptr()
+        a.prologue, a.epilogue = awq.PRO_RMSNORM, awq.EPI_ARGMAX
+        awq.check(lib.awq_gemv_fused(ctypes.byref(a), stream(torch)))
+        torch.cuda.synchronize()
+        assert np.array_equal(d_y.cpu().numpy().view(np.uint16), logits.view(np.uint16))
+        assert int(tok.item()) == oracle.awqo_argmax(ptr(logits), m)
+    assert int(keep["ws"][:64].to(torch.int32).abs().sum().item()) == 0  # sampler workspace left zeroed
