@@ -8,29 +8,72 @@
 //                 combined (0+1)+(2+3); chunk vectors added in order
 // Cache layout [head][max_pos][128] FP16 (Inference.cu:1097): a position is one
 // 256-byte row, so a wavefront load of 16 bytes per lane covers 4 positions.
+//
+// One workgroup of 16 wavefronts per head.  Scores: wavefront w takes the w-th
+// group of 4 positions of every 64-position chunk, so all wavefronts stream
+// keys even for short sequences.  Context: one wavefront per chunk.
 #include "common.hpp"
 
 namespace {
 
-constexpr int kMaxChunks = 1024;  // 65536 positions
+constexpr int kMaxChunks = 1024;    // 65536 positions
+constexpr int kLdsPositions = 8192; // scores kept in LDS up to this length
+constexpr int kLdsChunks = 32;      // chunk vectors kept in LDS up to this many chunks
+constexpr int kThreads = 1024;
+constexpr int kWaves = kThreads / 64;
 
+// v + (value of lane ^ mask) inside a row of 16 lanes.  After the xor-1 and
+// xor-2 steps all four lanes of a quad hold the same sum, so mirroring inside
+// 8 (resp. 16) lanes fetches exactly what an xor with 4 (resp. 8) would.
+__device__ __forceinline__ float dpp_add_xor1(float v) {
+  return v + __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float dpp_add_xor2(float v) {
+  return v + __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float dpp_add_half_mirror(float v) {
+  return v + __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x141, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float dpp_add_mirror(float v) {
+  return v + __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x140, 0xf, 0xf, true));
+}
 __device__ __forceinline__ float xor_add(float v, int mask) { return v + __shfl_xor(v, mask, 64); }
 
-__global__ __launch_bounds__(256) void attention_kernel(const half_t* __restrict__ q, const half_t* __restrict__ kc,
-                                                        const half_t* __restrict__ vc, half_t* __restrict__ ctx,
-                                                        int64_t max_pos, int L_arg, const StepState* dyn,
-                                                        int use_len_hi, float* __restrict__ ws_scores,
-                                                        float* __restrict__ ws_cv, int max_chunks) {
+// sum over the 16 lanes of a row, adjacent pairs first
+__device__ __forceinline__ float row16_tree_sum(float v) {
+  v = dpp_add_xor1(v);
+  v = dpp_add_xor2(v);
+  v = dpp_add_half_mirror(v);
+  v = dpp_add_mirror(v);
+  return v;
+}
+// sum over the 64 lanes of a wavefront, adjacent pairs first
+__device__ __forceinline__ float wave_tree_sum(float v) {
+  v = row16_tree_sum(v);
+  v = xor_add(v, 16);
+  v = xor_add(v, 32);
+  return v;
+}
+
+template <bool LDS_SCORES, bool LDS_CV>
+__global__ __launch_bounds__(kThreads) void attention_kernel(const half_t* __restrict__ q,
+                                                             const half_t* __restrict__ kc,
+                                                             const half_t* __restrict__ vc, half_t* __restrict__ ctx,
+                                                             int64_t max_pos, int L_arg, const StepState* dyn,
+                                                             int use_len_hi, float* __restrict__ ws_scores,
+                                                             float* __restrict__ ws_cv, int max_chunks) {
   __shared__ float cs[kMaxChunks];
-  __shared__ float wmax[4];
+  __shared__ float wmax[kWaves];
+  __shared__ float s_lds[LDS_SCORES ? kLdsPositions : 1];
+  __shared__ float cv_lds[LDS_CV ? kLdsChunks * AWQ_HEAD_DIM : 1];
   const int L = dyn ? (use_len_hi ? dyn->len_hi : dyn->len_lo) : L_arg;
   const int head = blockIdx.x;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int tq = lane >> 4, dl = lane & 15;
   const half_t* kh = kc + (int64_t)head * max_pos * AWQ_HEAD_DIM;
   const half_t* vh = vc + (int64_t)head * max_pos * AWQ_HEAD_DIM;
-  float* s = ws_scores + (int64_t)head * max_pos;
-  float* cv = ws_cv + (int64_t)head * max_chunks * AWQ_HEAD_DIM;
+  float* s = LDS_SCORES ? s_lds : ws_scores + (int64_t)head * max_pos;
+  float* cv = LDS_CV ? cv_lds : ws_cv + (int64_t)head * max_chunks * AWQ_HEAD_DIM;
   const int nchunks = (L + 63) >> 6;
   const float scale = 1.0f / sqrtf((float)AWQ_HEAD_DIM);  // Inference.cu:218
 
@@ -41,23 +84,25 @@ __global__ __launch_bounds__(256) void attention_kernel(const half_t* __restrict
     for (int i = 0; i < 8; ++i) qf[i] = (float)qv[i];
   }
 
-  // scores (Inference.cu:202-226) and their maximum (:229-233)
+  // scores (Inference.cu:202-226) and their maximum (:229-233): this
+  // wavefront's four positions of each chunk, eight chunks' loads in flight
   float lmax = -1e9f;
-  for (int chunk = wave; chunk < nchunks; chunk += 4) {
-    const int base = chunk << 6;
-#pragma unroll 4
-    for (int nl = 0; nl < 16; ++nl) {
-      const int t = base + 4 * nl + tq;
+  for (int c0 = 0; c0 < nchunks; c0 += 8) {
+    half8_t kv[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int t = ((c0 + u) << 6) + 4 * wave + tq;
+      if (t < L) kv[u] = *reinterpret_cast<const half8_t*>(kh + (int64_t)t * AWQ_HEAD_DIM + 8 * dl);
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int t = ((c0 + u) << 6) + 4 * wave + tq;
       float part = 0.0f;
       if (t < L) {
-        half8_t kv = *reinterpret_cast<const half8_t*>(kh + (int64_t)t * AWQ_HEAD_DIM + 8 * dl);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) part = __builtin_fmaf(qf[i], (float)kv[i], part);
+        for (int i = 0; i < 8; ++i) part = __builtin_fmaf(qf[i], (float)kv[u][i], part);
       }
-      part = xor_add(part, 1);
-      part = xor_add(part, 2);
-      part = xor_add(part, 4);
-      part = xor_add(part, 8);
+      part = row16_tree_sum(part);
       const float sc = part * scale;
       if (t < L) {
         if (dl == 0) s[t] = sc;
@@ -69,38 +114,45 @@ __global__ __launch_bounds__(256) void attention_kernel(const half_t* __restrict
   for (int mask = 1; mask < 64; mask <<= 1) lmax = fmaxf(lmax, __shfl_xor(lmax, mask, 64));
   if (lane == 0) wmax[wave] = lmax;
   __syncthreads();
-  const float mx = fmaxf(fmaxf(wmax[0], wmax[1]), fmaxf(wmax[2], wmax[3]));
+  float mx = wmax[0];
+#pragma unroll
+  for (int w = 1; w < kWaves; ++w) mx = fmaxf(mx, wmax[w]);
 
-  // exponentials and their sum (Inference.cu:239-249)
-  for (int chunk = wave; chunk < nchunks; chunk += 4) {
+  // exponentials and their sum (Inference.cu:239-249), one wavefront per chunk
+  for (int chunk = wave; chunk < nchunks; chunk += kWaves) {
     const int t = (chunk << 6) + lane;
     float e = 0.0f;
     if (t < L) {
       e = awq_expf(s[t] - mx);
       s[t] = e;
     }
-#pragma unroll
-    for (int mask = 1; mask < 64; mask <<= 1) e = xor_add(e, mask);
+    e = wave_tree_sum(e);
     if (lane == 0) cs[chunk] = e;
   }
   __syncthreads();
   float Z = cs[0];
   for (int c = 1; c < nchunks; ++c) Z += cs[c];
 
-  // weighted sum of V (Inference.cu:251-265)
-  for (int chunk = wave; chunk < nchunks; chunk += 4) {
+  // weighted sum of V (Inference.cu:251-265), one wavefront per chunk; the 16
+  // loads of a chunk are issued together
+  for (int chunk = wave; chunk < nchunks; chunk += kWaves) {
     const int base = chunk << 6;
+    half8_t vv[16];
+#pragma unroll
+    for (int nl = 0; nl < 16; ++nl) {
+      const int t = base + 4 * nl + tq;
+      if (t < L) vv[nl] = *reinterpret_cast<const half8_t*>(vh + (int64_t)t * AWQ_HEAD_DIM + 8 * dl);
+    }
     float acc[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
-#pragma unroll 4
+#pragma unroll
     for (int nl = 0; nl < 16; ++nl) {
       const int t = base + 4 * nl + tq;
       if (t < L) {
         const float p = s[t] / Z;
-        half8_t vv = *reinterpret_cast<const half8_t*>(vh + (int64_t)t * AWQ_HEAD_DIM + 8 * dl);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) acc[i] = __builtin_fmaf(p, (float)vv[i], acc[i]);
+        for (int i = 0; i < 8; ++i) acc[i] = __builtin_fmaf(p, (float)vv[nl][i], acc[i]);
       }
     }
 #pragma unroll
@@ -130,14 +182,26 @@ int64_t attention_workspace_bytes(int n_heads, int64_t max_pos) {
 }
 
 int launch_attention(const half_t* q, const half_t* kc, const half_t* vc, half_t* ctx, int n_heads, int64_t max_pos,
-                     int64_t L, const StepState* dyn, int use_len_hi, void* ws, hipStream_t st) {
+                     int64_t L, const StepState* dyn, int use_len_hi, int64_t len_bound, void* ws, hipStream_t st) {
   AWQ_REQUIRE(n_heads > 0 && max_pos > 0 && max_pos <= (int64_t)kMaxChunks * 64, "max_pos must be in 1..65536");
   AWQ_REQUIRE(dyn || (L >= 1 && L <= max_pos), "attended length out of range");
   AWQ_REQUIRE(ws != nullptr, "workspace required");
   float* scores = (float*)ws;
   float* cv = scores + (int64_t)n_heads * max_pos;
-  hipLaunchKernelGGL(attention_kernel, dim3(n_heads), dim3(256), 0, st, q, kc, vc, ctx, max_pos, (int)L, dyn,
-                     use_len_hi, scores, cv, (int)chunks_for(max_pos));
+  // With a device-side length the caller states an upper bound for it (it
+  // decides where the scores live); with a length known here, the length itself.
+  const int64_t bound = dyn ? (len_bound > 0 ? len_bound : max_pos) : L;
+  const int mc = (int)chunks_for(max_pos);
+  if (bound <= kLdsChunks * 64) {
+    hipLaunchKernelGGL((attention_kernel<true, true>), dim3(n_heads), dim3(kThreads), 0, st, q, kc, vc, ctx, max_pos,
+                       (int)L, dyn, use_len_hi, scores, cv, mc);
+  } else if (bound <= kLdsPositions) {
+    hipLaunchKernelGGL((attention_kernel<true, false>), dim3(n_heads), dim3(kThreads), 0, st, q, kc, vc, ctx, max_pos,
+                       (int)L, dyn, use_len_hi, scores, cv, mc);
+  } else {
+    hipLaunchKernelGGL((attention_kernel<false, false>), dim3(n_heads), dim3(kThreads), 0, st, q, kc, vc, ctx,
+                       max_pos, (int)L, dyn, use_len_hi, scores, cv, mc);
+  }
   AWQ_HIP_TRY(hipGetLastError());
   return AWQ_OK;
 }

@@ -159,7 +159,7 @@ struct awq_engine {
   int n_generated = 0;
   bool finalized = false;
   bool graph_mode = true;
-  hipGraphExec_t graph_prompt = nullptr, graph_gen = nullptr;
+  hipGraphExec_t graphs[2][3] = {{nullptr, nullptr, nullptr}, {nullptr, nullptr, nullptr}};  // [prompt|gen][length bound]
   std::vector<void*> allocations;
 };
 
@@ -232,7 +232,7 @@ LinearArgs linear_args(awq_engine* e, const DevLinear& t, const half_t* x, half_
 
 // runOneLayer, Inference.cu:1029-1230, as five launches.  The position and the
 // attended length come from the device-side step state.
-int enqueue_layer(awq_engine* e, int l, int use_len_hi) {
+int enqueue_layer(awq_engine* e, int l, int use_len_hi, int64_t len_bound) {
   LayerDev& L = e->layers[l];
   hipStream_t st = e->stream;
   {  // :1040 RMSNorm, :1052 Wqkv, :1070-1103 split + rotary + KV append
@@ -249,7 +249,7 @@ int enqueue_layer(awq_engine* e, int l, int use_len_hi) {
     if (int rc = launch_gemv(a, st)) return rc;
   }
   if (int rc = launch_attention(e->q, L.kcache, L.vcache, e->ctx, e->n_heads, e->cfg.max_pos, 0, e->d_state,
-                                use_len_hi, e->attn_ws, st))
+                                use_len_hi, len_bound, e->attn_ws, st))
     return rc;  // :1110
   {  // :1128-1155 Wo product and residual add; input and output are distinct
      // buffers (they alias in the reference)
@@ -290,7 +290,7 @@ int enqueue_sample(awq_engine* e) {
 }
 
 // everything of one position after the step state has been written
-int enqueue_step_body(awq_engine* e, bool gen) {
+int enqueue_step_body(awq_engine* e, bool gen, int64_t len_bound) {
   // embedding gather (Inference.cu:1310-1324, 1384-1398), skipped on the device
   // when the state says to keep the hidden state (:1357)
   if (int rc = launch_embed(e->embed.packed, e->embed.scale, e->embed.zp, e->cfg.hidden, e->cfg.vocab, 0, e->d_state,
@@ -298,15 +298,15 @@ int enqueue_step_body(awq_engine* e, bool gen) {
     return rc;
   const int split = gen ? e->cfg.split_idx : 1;
   for (int l = 0; l < e->cfg.n_layers; ++l)
-    if (int rc = enqueue_layer(e, l, l >= split)) return rc;
+    if (int rc = enqueue_layer(e, l, l >= split, len_bound)) return rc;
   if (gen) return enqueue_sample(e);
   return AWQ_OK;
 }
 
-int build_graph(awq_engine* e, bool gen, hipGraphExec_t* out) {
+int build_graph(awq_engine* e, bool gen, int64_t len_bound, hipGraphExec_t* out) {
   hipGraph_t graph = nullptr;
   AWQ_HIP_TRY(hipStreamBeginCapture(e->stream, hipStreamCaptureModeThreadLocal));
-  int rc = enqueue_step_body(e, gen);
+  int rc = enqueue_step_body(e, gen, len_bound);
   hipError_t err = hipStreamEndCapture(e->stream, &graph);
   if (rc) {
     if (graph) hipGraphDestroy(graph);
@@ -320,14 +320,20 @@ int build_graph(awq_engine* e, bool gen, hipGraphExec_t* out) {
 
 int run_step(awq_engine* e, bool gen, const StepState& s) {
   if (int rc = launch_set_state(e->d_state, s, e->stream)) return rc;
+  // the attention launch is specialised by an upper bound of the attended
+  // length (where its scores live); one captured graph per bound
+  static const int64_t kBounds[3] = {2048, 8192, 1 << 30};
+  int bucket = 0;
+  while (s.len_hi > kBounds[bucket]) ++bucket;
+  const int64_t len_bound = kBounds[bucket] < e->cfg.max_pos ? kBounds[bucket] : e->cfg.max_pos;
   if (e->graph_mode) {
-    hipGraphExec_t* g = gen ? &e->graph_gen : &e->graph_prompt;
+    hipGraphExec_t* g = &e->graphs[gen ? 1 : 0][bucket];
     if (!*g)
-      if (int rc = build_graph(e, gen, g)) return rc;
+      if (int rc = build_graph(e, gen, len_bound, g)) return rc;
     AWQ_HIP_TRY(hipGraphLaunch(*g, e->stream));
     return AWQ_OK;
   }
-  return enqueue_step_body(e, gen);
+  return enqueue_step_body(e, gen, len_bound);
 }
 
 int read_file(const std::string& path, int64_t bytes, std::vector<uint8_t>& staging) {
@@ -523,8 +529,9 @@ extern "C" int awq_create(const char* weight_dir, const awq_config* cfg_in, awq_
 extern "C" void awq_destroy(awq_engine* e) {
   if (!e) return;
   if (e->stream) (void)hipStreamSynchronize(e->stream);
-  if (e->graph_prompt) (void)hipGraphExecDestroy(e->graph_prompt);
-  if (e->graph_gen) (void)hipGraphExecDestroy(e->graph_gen);
+  for (auto& row : e->graphs)
+    for (hipGraphExec_t g : row)
+      if (g) (void)hipGraphExecDestroy(g);
   for (void* p : e->allocations)
     if (p) (void)hipFree(p);
   if (e->stream) (void)hipStreamDestroy(e->stream);
@@ -818,7 +825,7 @@ extern "C" int awq_decode_attention(const void* q, const void* k_cache, const vo
                                     int64_t max_pos, int64_t L, void* workspace, void* stream) {
   AWQ_REQUIRE(q && k_cache && v_cache && ctx, "NULL pointer");
   return launch_attention((const half_t*)q, (const half_t*)k_cache, (const half_t*)v_cache, (half_t*)ctx, n_heads,
-                          max_pos, L, nullptr, 0, workspace, (hipStream_t)stream);
+                          max_pos, L, nullptr, 0, 0, workspace, (hipStream_t)stream);
 }
 
 extern "C" int awq_residual_add(const void* a, const void* b, void* out, int64_t n, void* stream) {
