@@ -76,8 +76,6 @@ struct LinearArgs {
   const half_t* x = nullptr;      // [k]
   half_t* y = nullptr;            // [m] ([hidden] rotated Q for EPI_QKV_ROPE)
   const half_t* res = nullptr;    // EPI_RESIDUAL: [m], may alias y
-  float* partials = nullptr;      // split-k workspace
-  int32_t* counters = nullptr;    // one per 64-row group, zero between launches
   int64_t m = 0, k = 0;
   int zp_integral = 0;            // all zero-points are integers in [0,1024]: take the 2-op dequant
   int prologue = PRO_NONE;
@@ -93,7 +91,6 @@ struct LinearArgs {
   int64_t max_pos = 0;
   const StepState* dyn = nullptr;     // pos / out_index come from here when set
   unsigned long long* best = nullptr;  // EPI_ARGMAX: zero between launches
-  int32_t* done = nullptr;             // EPI_ARGMAX: zero between launches
   int32_t* out_token = nullptr;
   int32_t* out_array = nullptr;
 };

@@ -146,10 +146,8 @@ struct awq_engine {
   // activations (Inference.cu:334-348)
   half_t *hidden = nullptr, *q = nullptr, *ctx = nullptr, *mid = nullptr, *logits = nullptr;
   // workspaces
-  float* gemv_partials = nullptr;
-  int32_t* gemv_counters = nullptr;
   void* attn_ws = nullptr;
-  void* sample_ws = nullptr;  // 64-bit best candidate + finished-row-group counter
+  void* sample_ws = nullptr;  // 64-bit best candidate of the sampler
   StepState* d_state = nullptr;
   int32_t* d_token = nullptr;
   int32_t* d_out = nullptr;
@@ -220,8 +218,6 @@ LinearArgs linear_args(awq_engine* e, const DevLinear& t, const half_t* x, half_
   a.zp = t.zp;
   a.x = x;
   a.y = y;
-  a.partials = e->gemv_partials;
-  a.counters = e->gemv_counters;
   a.m = t.m;
   a.k = t.k;
   a.zp_integral = t.zp_integral;
@@ -283,7 +279,6 @@ int enqueue_sample(awq_engine* e) {
   a.gamma = e->layers[NL - 1].gamma;
   a.epilogue = EPI_ARGMAX;
   a.best = (unsigned long long*)e->sample_ws;
-  a.done = (int32_t*)((char*)e->sample_ws + 8);
   a.out_token = e->d_token;
   a.out_array = e->d_out;
   return launch_gemv(a, e->stream);
@@ -401,9 +396,6 @@ extern "C" int awq_create_empty(const awq_config* cfg_in, awq_engine** out) {
   } acts[] = {{&e->hidden, H}, {&e->q, H}, {&e->ctx, H}, {&e->mid, I}, {&e->logits, V}};
   for (auto& a : acts)
     if (int rc = dev_alloc(ep, (void**)a.p, a.n * 2)) return fail(rc);
-  int64_t max_m = std::max<int64_t>(std::max<int64_t>(3 * H, I), V);
-  if (int rc = dev_alloc(ep, (void**)&e->gemv_partials, 16 * max_m * 4)) return fail(rc);
-  if (int rc = dev_alloc(ep, (void**)&e->gemv_counters, (max_m / 64 + 1) * 4)) return fail(rc);
   if (int rc = dev_alloc(ep, &e->attn_ws, attention_workspace_bytes(e->n_heads, cfg.max_pos))) return fail(rc);
   if (int rc = dev_alloc(ep, &e->sample_ws, 64)) return fail(rc);
   if (int rc = dev_alloc(ep, (void**)&e->d_state, sizeof(StepState))) return fail(rc);
@@ -492,8 +484,6 @@ extern "C" int awq_finalize(awq_engine* e) {
     if (int rc = launch_fill_zero(L.kcache, kv_bytes, st)) return rc;
     if (int rc = launch_fill_zero(L.vcache, kv_bytes, st)) return rc;
   }
-  int64_t max_m = std::max<int64_t>(std::max<int64_t>(3 * (int64_t)e->cfg.hidden, e->cfg.inter), e->cfg.vocab);
-  if (int rc = launch_fill_zero(e->gemv_counters, (max_m / 64 + 1) * 4, st)) return rc;
   if (int rc = launch_fill_zero(e->sample_ws, 64, st)) return rc;
   if (int rc = launch_fill_zero(e->d_token, 4, st)) return rc;
   if (int rc = launch_fill_zero(e->hidden, (int64_t)e->cfg.hidden * 2, st)) return rc;
@@ -763,13 +753,7 @@ extern "C" int awq_gemv_fused(const awq_linear_args* u, void* stream) {
   a.x = (const half_t*)u->x;
   a.y = (half_t*)u->y;
   a.res = (const half_t*)u->residual;
-  // workspace: [0,8) best candidate, [8,12) finished counter, [64,..) one counter
-  // per 64-row group, then the split-k partial sums
-  char* ws = (char*)u->workspace;
-  a.best = (unsigned long long*)ws;
-  a.done = (int32_t*)(ws + 8);
-  a.counters = (int32_t*)(ws + 64);
-  a.partials = (float*)(ws + 64 + ((u->m / 64) * 4 + 255) / 256 * 256);
+  a.best = (unsigned long long*)u->workspace;  // the sampler's best candidate
   a.m = u->m;
   a.k = u->k;
   a.zp_integral = zp_integral != 0;

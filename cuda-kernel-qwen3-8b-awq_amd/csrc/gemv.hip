@@ -3,15 +3,19 @@
 // vector product used for decode.
 //
 // Weight stream after reordering.  The [m outputs x k inputs] matrix is cut
-// into groups of 64 output rows; the k inputs of a row into blocks of 32 in
-// the order of awq_block_elem (awq_canon_math.h).  Lane l of a wavefront owns
-// row 64*rg + l, and one 16-byte load hands it one whole block:
-//     byte offset = ((rg * (k/32) + blk) * 64 + l) * 16
-// so a wavefront load is 1 KiB contiguous and successive blocks follow each
-// other.  Inside the 16 bytes, dword c holds elements 8c..8c+7 with nibble
-// positions {0,16,4,20,8,24,12,28}[t & 7]: masking with 0x000f000f / 0x00f000f0
-// (and the same after one shift by 8) yields two weights as the low mantissa
-// bits of a packed pair of binary16 numbers 1024+q or 1024+16q.
+// into groups of 16 output rows; the k inputs of a row into blocks of 32 in
+// the order of awq_block_elem (awq_canon_math.h).  One 16-byte load hands a
+// lane one whole block of its row:
+//     byte offset = ((rg * (k/32) + blk) * 16 + r) * 16,   rg = row/16, r = row%16
+// A workgroup owns one row group and all of k, so no partial sums ever leave
+// the workgroup: lane (wavefront w, quarter q = lane/16, r = lane%16) takes the
+// G consecutive blocks starting at (4w+q)*G of row 16*rg + r; a wavefront load
+// is four contiguous 256-byte pieces, and the G loads of a lane walk 256*G
+// contiguous bytes per quarter.  Inside the 16 bytes, dword c holds elements
+// 8c..8c+7 with nibble positions {0,16,4,20,8,24,12,28}[t & 7]: masking with
+// 0x000f000f / 0x00f000f0 (and the same after one shift by 8) yields two
+// weights as the low mantissa bits of a packed pair of binary16 numbers 1024+q
+// or 1024+16q.
 #include "common.hpp"
 #include <stdlib.h>
 
@@ -53,13 +57,13 @@ __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict_
 __global__ __launch_bounds__(256) void repack_kernel(const uint8_t* __restrict__ in, uint4* __restrict__ out,
                                                      int64_t m, int64_t k, int C) {
   const int64_t nblk = k / AWQ_BLOCK_K;
-  const int64_t total = (m / 64) * nblk * 64;
+  const int64_t total = (m / 16) * nblk * 16;
   int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (id >= total) return;
-  int lane = (int)(id & 63);
-  int64_t blk = (id >> 6) % nblk;
-  int64_t rg = (id >> 6) / nblk;
-  int64_t row = rg * 64 + lane;
+  int r = (int)(id & 15);
+  int64_t blk = (id >> 4) % nblk;
+  int64_t rg = (id >> 4) / nblk;
+  int64_t row = rg * 16 + r;
   uint32_t d[4] = {0, 0, 0, 0};
   for (int t = 0; t < AWQ_BLOCK_K; ++t) {
     int64_t j = awq_block_elem(k, C, blk, t);
@@ -160,12 +164,10 @@ struct GemvParams {
   const half_t* x;
   half_t* y;
   const half_t* res;
-  float* partials;
-  int32_t* counters;
   int32_t m, k;
   int32_t nblk;      // k/32
   int32_t C;         // group period
-  int32_t n_slabs;   // workgroups along k
+  int32_t n_waves;   // wavefronts per workgroup = k/32/G/4
   int32_t mg, kg;    // m/128, k/128
   int32_t prologue, epilogue;
   // PRO_RMSNORM
@@ -182,12 +184,10 @@ struct GemvParams {
   const StepState* dyn;
   // EPI_ARGMAX
   unsigned long long* best;
-  int32_t* done;
-  int32_t* out_token;
-  int32_t* out_array;
 };
 
-__device__ __forceinline__ void epilogue(const GemvParams& p, int row, int lane, float acc) {
+// the 16 finished rows of a workgroup; r = lane = row % 16, lanes 0..15 of wavefront 0
+__device__ __forceinline__ void epilogue(const GemvParams& p, int row, int r, float acc) {
   half_t v = (half_t)acc;
   switch (p.epilogue) {
     case EPI_RESIDUAL:  // Inference.cu:1149-1155
@@ -202,15 +202,15 @@ __device__ __forceinline__ void epilogue(const GemvParams& p, int row, int lane,
       // row of this position, Q to y.
       const int pos = p.dyn ? p.dyn->pos : p.pos;
       const int H = p.hidden;
-      const int sec = row / H;  // same for the whole wavefront
-      const int r = row - sec * H;
-      const int d = r & (AWQ_HEAD_DIM - 1);
+      const int sec = row / H;  // same for the whole workgroup
+      const int rr = row - sec * H;
+      const int d = rr & (AWQ_HEAD_DIM - 1);
       half_t other = __builtin_bit_cast(half_t, (unsigned short)__shfl_xor((int)__builtin_bit_cast(unsigned short, v), 1, 64));
       half_t out = v;
       if (sec < 2) {
         const half_t c = p.cos_t[(int64_t)pos * 64 + (d >> 1)], s = p.sin_t[(int64_t)pos * 64 + (d >> 1)];
-        const half_t a = (lane & 1) ? other : v, b = (lane & 1) ? v : other;
-        if (lane & 1) {
+        const half_t a = (r & 1) ? other : v, b = (r & 1) ? v : other;
+        if (r & 1) {
           half_t as = a * s, bc = b * c;
           out = as + bc;
         } else {
@@ -219,40 +219,30 @@ __device__ __forceinline__ void epilogue(const GemvParams& p, int row, int lane,
         }
       }
       if (sec == 0) {
-        p.y[r] = out;
+        p.y[rr] = out;
       } else {
         half_t* cache = sec == 1 ? p.k_cache : p.v_cache;
-        cache[((int64_t)(r >> 7) * p.max_pos + pos) * AWQ_HEAD_DIM + d] = out;
+        cache[((int64_t)(rr >> 7) * p.max_pos + pos) * AWQ_HEAD_DIM + d] = out;
       }
       return;
     }
     case EPI_ARGMAX: {
       // Inference.cu:1278-1290 on the device: the best (value, lowest index)
       // pair of the vocabulary is kept with a 64-bit atomic max, which does
-      // not depend on arrival order.
+      // not depend on arrival order.  Most workgroups find a better candidate
+      // already there and skip the atomic.
       p.y[row] = v;
       const unsigned short bits = __builtin_bit_cast(unsigned short, v);
       int32_t key = awq_logit_key(bits);
       if (row == 0 && (bits & 0x7fffu) > 0x7c00u) key = INT32_MAX;  // a NaN at index 0 is never displaced
       unsigned long long cand = awq_pack_candidate(key, (uint32_t)row);
 #pragma unroll
-      for (int mask = 1; mask < 64; mask <<= 1) {
+      for (int mask = 1; mask < 16; mask <<= 1) {
         unsigned long long o = __shfl_xor(cand, mask, 64);
         cand = o > cand ? o : cand;
       }
-      if (lane == 0) {
+      if (r == 0 && cand > __hip_atomic_load(p.best, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
         __hip_atomic_fetch_max(p.best, cand, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __builtin_amdgcn_s_waitcnt(0);
-        int old = __hip_atomic_fetch_add(p.done, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (old == p.m / 64 - 1) {
-          unsigned long long b = __hip_atomic_load(p.best, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          int32_t tok = (int32_t)(0xffffffffu - (uint32_t)(b & 0xffffffffull));
-          *p.out_token = tok;
-          if (p.out_array && p.dyn) p.out_array[p.dyn->out_index] = tok;
-          __hip_atomic_store(p.best, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          __hip_atomic_store(p.done, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-      }
       return;
     }
     default:
@@ -260,41 +250,89 @@ __device__ __forceinline__ void epilogue(const GemvParams& p, int row, int lane,
   }
 }
 
-// NI groups of four blocks per wavefront; 4 wavefronts per workgroup cover
-// 16*NI consecutive blocks of one 64-row group.
-template <int NI, bool ZINT, bool PERIODIC>
-__global__ __launch_bounds__(256) void gemv_kernel(GemvParams p) {
-  constexpr int NB = 4 * NI;
-  __shared__ __attribute__((aligned(16))) half_t xs[4 * NB * AWQ_BLOCK_K];
-  __shared__ float red[4][64];
-  __shared__ float fin[16][64];  // slab partials of the finishing wavefront
-  __shared__ GroupConst gtab[PERIODIC ? 64 : 1];
+// A workgroup takes row groups blockIdx.x, blockIdx.x + gridDim.x, ... (16
+// output rows x all of k each).  n_waves wavefronts; lane (w, q, r) owns blocks
+// (4w+q)*G .. +G-1 of row 16*rg + r.  x is staged (and normalised) once per
+// workgroup; the weights of the next row group are in flight while the current
+// one is multiplied.
+template <int G, bool ZINT, bool PERIODIC>
+__global__ __launch_bounds__(1024) void gemv_kernel(GemvParams p) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  half_t* xs = reinterpret_cast<half_t*>(smem);  // x in block order, k halves
+  __shared__ float red[16][16];
   __shared__ float nbuf[256];
+  __shared__ GroupConst gtab[PERIODIC ? 64 : 1];
+  constexpr int MAXU = 8;  // 8-byte units of x a thread may hold in registers
 
   const int tid = threadIdx.x;
+  const int nthreads = p.n_waves * 64;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int rg = blockIdx.x;
-  const int slab = blockIdx.y;
-  const int blk_wg = slab * 4 * NB;
-  const int blk_wave = blk_wg + wave * NB;
+  const int q = lane >> 4, r = lane & 15;
+  const int n_rg = p.m >> 4;
+  const int blk0 = (4 * wave + q) * G;
+  const int U = p.nblk / p.C;  // blocks per class (PERIODIC)
 
-  const u32x4* wp = p.wq + ((int64_t)rg * p.nblk + blk_wave) * 64 + lane;
-  u32x4 wreg[2][4];
+  int rg = blockIdx.x;
+  const u32x4* wp = p.wq + ((int64_t)rg * p.nblk + blk0) * 16 + r;
+  u32x4 w[G], wn[G];
 #pragma unroll
-  for (int n = 0; n < 4; ++n) wreg[0][n] = __builtin_nontemporal_load(wp + n * 64);
+  for (int b = 0; b < G; ++b) w[b] = __builtin_nontemporal_load(wp + b * 16);
 
-  // stage this workgroup's slice of x in block order, normalising it on the
-  // way when the RMSNorm is fused in (Inference.cu:111-145: 256 strided fma
-  // partial sums, stride-halving tree, then two binary16 multiplies)
-  half_t sc = (half_t)1.0f;
-  if (p.prologue == PRO_RMSNORM) {
-    float acc = 0.0f;
-    for (int i = tid; i < p.k; i += 256) {
-      float v = (float)p.x[i];
-      acc = __builtin_fmaf(v, v, acc);
+  // ---- x into LDS in block order ------------------------------------------
+  // Unit u of a thread is the 4 consecutive block-order elements 4*(tid + u*nthreads)..+3;
+  // in natural order they are 4 consecutive indices too unless the matrix is
+  // periodic (then they are C apart and are gathered one by one).
+  const int total_units = p.k >> 2;  // at most MAXU * nthreads (checked by the launcher)
+  const bool norm = p.prologue == PRO_RMSNORM;
+  uint2 xu[MAXU], gu[MAXU];
+#pragma unroll
+  for (int u = 0; u < MAXU; ++u) {
+    if (tid + u * nthreads < total_units) {
+      const int e = 4 * (tid + u * nthreads);
+      if (PERIODIC) {
+        half_t hx[4], hg[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int j = (int)awq_block_elem(p.k, p.C, (e + i) >> 5, (e + i) & 31);
+          hx[i] = p.x[j];
+          hg[i] = norm ? p.gamma[j] : (half_t)0.0f;
+        }
+        xu[u] = __builtin_bit_cast(uint2, *reinterpret_cast<uint64_t*>(hx));
+        gu[u] = __builtin_bit_cast(uint2, *reinterpret_cast<uint64_t*>(hg));
+      } else {
+        xu[u] = reinterpret_cast<const uint2*>(p.x)[tid + u * nthreads];
+        if (norm) gu[u] = reinterpret_cast<const uint2*>(p.gamma)[tid + u * nthreads];
+      }
     }
-    nbuf[tid] = acc;
+  }
+  if (norm) {
+    // rmsNormKernel, Inference.cu:111-145: 256 strided fma partial sums over the
+    // natural order, the stride-halving tree, then two binary16 multiplies.
+    // The raw values go through LDS in natural order for the partial sums.
+#pragma unroll
+    for (int u = 0; u < MAXU; ++u) {
+      if (tid + u * nthreads < total_units) {
+        const int e = 4 * (tid + u * nthreads);
+        if (PERIODIC) {
+          half_t hx[4];
+          *reinterpret_cast<uint64_t*>(hx) = __builtin_bit_cast(uint64_t, xu[u]);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) xs[awq_block_elem(p.k, p.C, (e + i) >> 5, (e + i) & 31)] = hx[i];
+        } else {
+          reinterpret_cast<uint2*>(xs)[tid + u * nthreads] = xu[u];
+        }
+      }
+    }
+    __syncthreads();
+    if (tid < 256) {
+      float acc = 0.0f;
+      for (int i = tid; i < p.k; i += 256) {
+        float v = (float)xs[i];
+        acc = __builtin_fmaf(v, v, acc);
+      }
+      nbuf[tid] = acc;
+    }
     __syncthreads();
     if (tid < 128) nbuf[tid] += nbuf[tid + 128];
     __syncthreads();
@@ -305,55 +343,53 @@ __global__ __launch_bounds__(256) void gemv_kernel(GemvParams p) {
       if (tid == 0) nbuf[0] = v;
     }
     __syncthreads();
-    sc = (half_t)awq_rsqrtf(nbuf[0] / (float)p.k + p.eps);
-  }
-  if (PERIODIC || p.prologue == PRO_RMSNORM) {
-    for (int e = tid; e < 4 * NB * AWQ_BLOCK_K; e += 256) {
-      int64_t j = PERIODIC ? awq_block_elem(p.k, p.C, blk_wg + (e >> 5), e & 31) : (int64_t)blk_wg * AWQ_BLOCK_K + e;
-      half_t v = p.x[j];
-      if (p.prologue == PRO_RMSNORM) {
-        half_t t = v * sc;
-        v = t * p.gamma[j];
+    const half_t sc = (half_t)awq_rsqrtf(nbuf[0] / (float)p.k + p.eps);
+    const half2_t sc2 = half2_t{sc, sc};
+#pragma unroll
+    for (int u = 0; u < MAXU; ++u) {
+      if (tid + u * nthreads < total_units) {
+        half2_t t0 = as_half2(xu[u].x) * sc2, t1 = as_half2(xu[u].y) * sc2;
+        t0 = t0 * as_half2(gu[u].x);
+        t1 = t1 * as_half2(gu[u].y);
+        xu[u].x = __builtin_bit_cast(uint32_t, t0);
+        xu[u].y = __builtin_bit_cast(uint32_t, t1);
       }
-      xs[e] = v;
     }
-  } else {
-    const uint2* src = reinterpret_cast<const uint2*>(p.x + (int64_t)blk_wg * AWQ_BLOCK_K);
-    for (int e = tid; e < NB * AWQ_BLOCK_K; e += 256) reinterpret_cast<uint2*>(xs)[e] = src[e];
   }
-
-  // scale group of this wavefront's 64 rows: row/128, then Inference.cu:90 with
-  // the index wrapped to the m/128 stored entries.  When the group depends on
-  // the input index it is constant within a class of blocks; the (at most 64)
-  // classes go through a table in LDS.
-  const int a = rg >> 1;
-  GroupConst g;
-  if (!PERIODIC) {
-    int gi = (a % p.kg) % p.mg;
-    g = make_group<ZINT>(p.scale[gi], p.zp[gi]);
-  } else if (tid < p.C) {
-    int gi = (int)((((int64_t)tid * p.mg + a) % p.kg) % p.mg);
-    gtab[tid] = make_group<ZINT>(p.scale[gi], p.zp[gi]);
-  }
-  const int U = p.nblk / p.C;  // blocks per class (PERIODIC)
-  int cls = 0, cls_left = 0;   // class of the next block and blocks left in it
-  if (PERIODIC) {
-    cls = blk_wave / U;
-    cls_left = U - (blk_wave - cls * U);
-  }
-  __syncthreads();
-
-  float g4[NI];
 #pragma unroll
-  for (int it = 0; it < NI; ++it) {
-    if (it + 1 < NI) {
+  for (int u = 0; u < MAXU; ++u)
+    if (tid + u * nthreads < total_units) reinterpret_cast<uint2*>(xs)[tid + u * nthreads] = xu[u];
+
+  for (; rg < n_rg; rg += gridDim.x) {
+    const int rg_next = rg + gridDim.x;
+    if (rg_next < n_rg) {
+      const u32x4* wpn = p.wq + ((int64_t)rg_next * p.nblk + blk0) * 16 + r;
 #pragma unroll
-      for (int n = 0; n < 4; ++n) wreg[(it + 1) & 1][n] = __builtin_nontemporal_load(wp + ((it + 1) * 4 + n) * 64);
+      for (int b = 0; b < G; ++b) wn[b] = __builtin_nontemporal_load(wpn + b * 16);
     }
-    float bs[4];
+    // scale group of these 16 rows: row/128, then Inference.cu:90 with the index
+    // wrapped to the m/128 stored entries.  When the group depends on the input
+    // index it is constant within a class of blocks; the (at most 64) classes go
+    // through a table in LDS.
+    const int a = rg >> 3;
+    GroupConst g;
+    if (!PERIODIC) {
+      int gi = (a % p.kg) % p.mg;
+      g = make_group<ZINT>(p.scale[gi], p.zp[gi]);
+    } else if (tid < p.C) {
+      int gi = (int)((((int64_t)tid * p.mg + a) % p.kg) % p.mg);
+      gtab[tid] = make_group<ZINT>(p.scale[gi], p.zp[gi]);
+    }
+    int cls = 0, cls_left = 0;  // class of the next block and blocks left in it
+    if (PERIODIC) {
+      cls = blk0 / U;
+      cls_left = U - (blk0 - cls * U);
+    }
+    __syncthreads();  // xs (first pass), gtab, and the previous pass's use of red
+
+    float bs[G];
 #pragma unroll
-    for (int n = 0; n < 4; ++n) {
-      const int bl = it * 4 + n;
+    for (int b = 0; b < G; ++b) {
       if (PERIODIC) {
         g = gtab[cls];
         if (--cls_left == 0) {
@@ -361,82 +397,80 @@ __global__ __launch_bounds__(256) void gemv_kernel(GemvParams p) {
           cls_left = U;
         }
       }
-      bs[n] = block_dot<ZINT>(wreg[it & 1][n], xs + (wave * NB + bl) * AWQ_BLOCK_K, g);
+      bs[b] = block_dot<ZINT>(w[b], xs + (blk0 + b) * AWQ_BLOCK_K, g);
     }
-    g4[it] = (bs[0] + bs[1]) + (bs[2] + bs[3]);
-  }
-  // adjacent-pair tree over this lane's groups
+    // adjacent-pair tree: this lane's G blocks, then the four quarters of the
+    // wavefront (consecutive block ranges), then the wavefronts
 #pragma unroll
-  for (int n = NI; n > 1; n >>= 1) {
+    for (int n = G; n > 1; n >>= 1) {
 #pragma unroll
-    for (int q = 0; q < n / 2; ++q) g4[q] = g4[2 * q] + g4[2 * q + 1];
+      for (int i = 0; i < n / 2; ++i) bs[i] = bs[2 * i] + bs[2 * i + 1];
+    }
+    float v = bs[0];
+    v += __shfl_xor(v, 16, 64);
+    v += __shfl_xor(v, 32, 64);
+    if (q == 0) red[wave][r] = v;
+    __syncthreads();
+    if (tid < 16) {
+      int n = p.n_waves;
+      while (n > 1 && (n & 1) == 0) {
+        n >>= 1;
+        for (int i = 0; i < n; ++i) red[i][r] = red[2 * i][r] + red[2 * i + 1][r];
+      }
+      float tot = red[0][r];
+      for (int i = 1; i < n; ++i) tot += red[i][r];
+      epilogue(p, rg * 16 + r, r, tot);
+    }
+#pragma unroll
+    for (int b = 0; b < G; ++b) w[b] = wn[b];
   }
-  red[wave][lane] = g4[0];
-  __syncthreads();
-  if (wave != 0) return;
-  float v = (red[0][lane] + red[1][lane]) + (red[2][lane] + red[3][lane]);
-  const int row = rg * 64 + lane;
-  if (p.n_slabs == 1) {
-    epilogue(p, row, lane, v);
-    return;
-  }
-  // Split along k: publish, and let the last workgroup of this row group
-  // finish the tree in slab order.  The partial sums travel as device-scope
-  // atomic stores and loads (they go to the level of the memory system that
-  // all compute dies share), so no cache write-back or invalidate is needed:
-  // wait until this wavefront's stores have been acknowledged, then count.
-  __hip_atomic_store(&p.partials[(int64_t)slab * p.m + row], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  __builtin_amdgcn_s_waitcnt(0);
-  int old = 0;
-  if (lane == 0) old = __hip_atomic_fetch_add(&p.counters[rg], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  old = __builtin_amdgcn_readfirstlane(old);
-  if (old != p.n_slabs - 1) return;
-  int n = p.n_slabs;
-  for (int s = 0; s < n; ++s)
-    fin[s][lane] = __hip_atomic_load(&p.partials[(int64_t)s * p.m + row], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  while (n > 1 && (n & 1) == 0) {
-    n >>= 1;
-    for (int q = 0; q < n; ++q) fin[q][lane] = fin[2 * q][lane] + fin[2 * q + 1][lane];
-  }
-  float tot = fin[0][lane];
-  for (int q = 1; q < n; ++q) tot += fin[q][lane];
-  if (lane == 0) __hip_atomic_store(&p.counters[rg], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  epilogue(p, row, lane, tot);
+}
+
+// Inference.cu:1282-1290, last step: turn the best candidate into the token id
+__global__ void sample_finish_kernel(unsigned long long* best, int32_t* out_token, const StepState* dyn,
+                                     int32_t* out_array) {
+  if (threadIdx.x != 0) return;
+  unsigned long long b = *best;
+  int32_t tok = (int32_t)(0xffffffffu - (uint32_t)(b & 0xffffffffull));
+  *out_token = tok;
+  if (out_array && dyn) out_array[dyn->out_index] = tok;
+  *best = 0;
 }
 
 struct GemvPlan {
-  int ni;       // 1, 2, 4 or 8
-  int n_slabs;  // workgroups along k
+  int g;        // blocks per lane: 1, 2, 4 or 8
+  int n_waves;  // wavefronts per workgroup
 };
 
-// 16*NI blocks per workgroup; pick the split so that the launch has at least
-// ~2 workgroups per compute unit when the shape allows it
-GemvPlan plan_gemv(int64_t m, int64_t k) {
-  int64_t units = k / AWQ_BLOCK_K / 16;  // NI * n_slabs
-  int64_t rgs = m / 64;
-  GemvPlan best{1, (int)units};
-  if (const char* f = getenv("AWQ_DEV_NI")) {
-    int ni = atoi(f);
-    if (ni >= 1 && units % ni == 0 && units / ni <= 16) return GemvPlan{ni, (int)(units / ni)};
+// Lane groups per workgroup = (k/32)/G must be a multiple of 4 and at most 64.
+// Prefer long per-lane runs (G = 8) unless that leaves the device with few
+// wavefronts.
+bool plan_gemv(int64_t m, int64_t k, GemvPlan* out) {
+  const int64_t nblk = k / AWQ_BLOCK_K;
+  bool found = false;
+  for (int g = 8; g >= 1; g >>= 1) {
+    if (nblk % g) continue;
+    int64_t groups = nblk / g;
+    if (groups % 4 || groups > 64) continue;
+    *out = GemvPlan{g, (int)(groups / 4)};
+    found = true;
+    if ((m / 16) * (groups / 4) >= 2048) break;
   }
-  for (int ni = 8; ni >= 1; ni >>= 1) {
-    if (units % ni) continue;
-    int64_t slabs = units / ni;
-    if (slabs > 16) continue;
-    best = GemvPlan{ni, (int)slabs};
-    if (rgs * slabs >= 512) break;
+  if (const char* f = getenv("AWQ_DEV_G")) {
+    int g = atoi(f);
+    if (g >= 1 && nblk % g == 0 && (nblk / g) % 4 == 0 && nblk / g <= 64) *out = GemvPlan{g, (int)(nblk / g / 4)};
   }
-  return best;
+  return found;
 }
 
-template <int NI>
-void launch_ni(const GemvParams& p, bool zint, bool periodic, dim3 grid, hipStream_t st) {
+template <int G>
+void launch_g(const GemvParams& p, bool zint, bool periodic, dim3 grid, dim3 block, size_t lds, hipStream_t st) {
   if (zint) {
-    if (periodic) hipLaunchKernelGGL((gemv_kernel<NI, true, true>), grid, dim3(256), 0, st, p);
-    else hipLaunchKernelGGL((gemv_kernel<NI, true, false>), grid, dim3(256), 0, st, p);
+    if (periodic) hipLaunchKernelGGL((gemv_kernel<G, true, true>), grid, block, lds, st, p);
+    else hipLaunchKernelGGL((gemv_kernel<G, true, false>), grid, block, lds, st, p);
   } else {
-    if (periodic) hipLaunchKernelGGL((gemv_kernel<NI, false, true>), grid, dim3(256), 0, st, p);
-    else hipLaunchKernelGGL((gemv_kernel<NI, false, false>), grid, dim3(256), 0, st, p);
+    if (periodic) hipLaunchKernelGGL((gemv_kernel<G, false, true>), grid, block, lds, st, p);
+    else hipLaunchKernelGGL((gemv_kernel<G, false, false>), grid, block, lds, st, p);
   }
 }
 
@@ -458,10 +492,12 @@ int launch_dequant(const uint8_t* packed, const half_t* scale, const half_t* zp,
 static int check_linear_shape(int64_t m, int64_t k) {
   AWQ_REQUIRE(m > 0 && k > 0 && m % 128 == 0, "m must be a positive multiple of 128");
   AWQ_REQUIRE(k % 512 == 0, "k must be a positive multiple of 512");
-  AWQ_REQUIRE(m < (1ll << 31) && k < (1ll << 31) && m / 64 < 2147483647ll, "shape too large");
+  AWQ_REQUIRE(m < (1ll << 31) && k <= 24576, "shape too large (k is limited to 24576 by the LDS copy of x)");
   int C = awq_group_period(m, k);
   AWQ_REQUIRE((k / AWQ_BLOCK_K) % C == 0, "k/32 must be a multiple of the scale-group period");
   AWQ_REQUIRE(C <= 64, "scale-group period above 64 is not supported");
+  GemvPlan plan;
+  AWQ_REQUIRE(plan_gemv(m, k, &plan), "k/32 has no supported split into lane groups");
   return AWQ_OK;
 }
 
@@ -475,16 +511,16 @@ int launch_repack(const uint8_t* in, void* out, int64_t m, int64_t k, hipStream_
 }
 
 int64_t gemv_workspace_bytes(int64_t m, int64_t k) {
-  // 64 bytes for the sampler, one counter per 64-row group, up to 16 slabs of FP32 partials
+  // the sampler's 64-bit best candidate; the product itself needs no scratch
+  (void)m;
   (void)k;
-  return 64 + 16 * m * 4 + ((m / 64) * 4 + 255) / 256 * 256;
+  return 256;
 }
 
 int launch_gemv(const LinearArgs& a, hipStream_t st) {
   if (int rc = check_linear_shape(a.m, a.k)) return rc;
-  GemvPlan plan = plan_gemv(a.m, a.k);
-  AWQ_REQUIRE(plan.n_slabs <= 16, "k too large for the split workspace");
-  AWQ_REQUIRE(plan.n_slabs == 1 || (a.partials && a.counters), "split-k launch needs a workspace");
+  GemvPlan plan;
+  plan_gemv(a.m, a.k, &plan);
   AWQ_REQUIRE(a.prologue != PRO_RMSNORM || (a.gamma && a.k % 256 == 0), "fused RMSNorm needs gamma and k % 256 == 0");
   AWQ_REQUIRE(a.epilogue != EPI_RESIDUAL || a.res, "residual epilogue needs res");
   if (a.epilogue == EPI_QKV_ROPE) {
@@ -493,7 +529,7 @@ int launch_gemv(const LinearArgs& a, hipStream_t st) {
                 "QKV epilogue needs rotary tables, caches and m == 3*hidden");
     AWQ_REQUIRE(a.dyn || (a.pos >= 0 && a.pos < a.max_pos), "pos out of range");
   }
-  if (a.epilogue == EPI_ARGMAX) AWQ_REQUIRE(a.best && a.done && a.out_token, "argmax epilogue needs its workspace");
+  if (a.epilogue == EPI_ARGMAX) AWQ_REQUIRE(a.best && a.out_token, "argmax epilogue needs its workspace");
   GemvParams p;
   p.wq = (const u32x4*)a.wq;
   p.scale = a.scale;
@@ -501,13 +537,11 @@ int launch_gemv(const LinearArgs& a, hipStream_t st) {
   p.x = a.x;
   p.y = a.y;
   p.res = a.res;
-  p.partials = a.partials;
-  p.counters = a.counters;
   p.m = (int32_t)a.m;
   p.k = (int32_t)a.k;
   p.nblk = (int32_t)(a.k / AWQ_BLOCK_K);
   p.C = awq_group_period(a.m, a.k);
-  p.n_slabs = plan.n_slabs;
+  p.n_waves = plan.n_waves;
   p.mg = (int32_t)(a.m / 128);
   p.kg = (int32_t)(a.k / 128);
   p.prologue = a.prologue;
@@ -523,17 +557,28 @@ int launch_gemv(const LinearArgs& a, hipStream_t st) {
   p.max_pos = a.max_pos;
   p.dyn = a.dyn;
   p.best = a.best;
-  p.done = a.done;
-  p.out_token = a.out_token;
-  p.out_array = a.out_array;
-  bool periodic = p.C > 1;
-  dim3 grid((unsigned)(a.m / 64), (unsigned)plan.n_slabs);
-  switch (plan.ni) {
-    case 1: launch_ni<1>(p, a.zp_integral, periodic, grid, st); break;
-    case 2: launch_ni<2>(p, a.zp_integral, periodic, grid, st); break;
-    case 4: launch_ni<4>(p, a.zp_integral, periodic, grid, st); break;
-    default: launch_ni<8>(p, a.zp_integral, periodic, grid, st); break;
+  const bool periodic = p.C > 1;
+  AWQ_REQUIRE(a.k / 4 <= 8 * plan.n_waves * 64, "k too large for this workgroup size");
+  // one workgroup per row group while that fits the device a few times over;
+  // beyond that a workgroup walks several row groups and stages x once
+  int64_t n_rg = a.m / 16, n_wg = n_rg;
+  if (n_rg > 1024) n_wg = 1024;
+  if (const char* f = getenv("AWQ_DEV_WGS")) {
+    int64_t v = atoll(f);
+    if (v >= 1 && v < n_rg) n_wg = v;
+  }
+  dim3 grid((unsigned)n_wg), block((unsigned)(plan.n_waves * 64));
+  size_t lds = (size_t)a.k * 2;
+  switch (plan.g) {
+    case 1: launch_g<1>(p, a.zp_integral, periodic, grid, block, lds, st); break;
+    case 2: launch_g<2>(p, a.zp_integral, periodic, grid, block, lds, st); break;
+    case 4: launch_g<4>(p, a.zp_integral, periodic, grid, block, lds, st); break;
+    default: launch_g<8>(p, a.zp_integral, periodic, grid, block, lds, st); break;
   }
   AWQ_HIP_TRY(hipGetLastError());
+  if (a.epilogue == EPI_ARGMAX) {
+    hipLaunchKernelGGL(sample_finish_kernel, dim3(1), dim3(64), 0, st, a.best, a.out_token, a.dyn, a.out_array);
+    AWQ_HIP_TRY(hipGetLastError());
+  }
   return AWQ_OK;
 }

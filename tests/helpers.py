@@ -96,11 +96,12 @@ def block_elem(k, C, blk, t):
 
 
 def repack_numpy(packed, m, k, C):
-    """numpy statement of the streaming order of the GPU kernels (see csrc/gemv.hip)"""
+    """numpy statement of the streaming order of the GPU kernels (see csrc/gemv.hip):
+    [row group of 16][block][row % 16][4 dwords]"""
     nib = nibbles_flat(packed).astype(np.uint32)
     nblk = k // 32
-    out = np.zeros((m // 64, nblk, 64, 4), dtype=np.uint32)
-    rows = np.arange(m).reshape(m // 64, 64)
+    out = np.zeros((m // 16, nblk, 16, 4), dtype=np.uint32)
+    rows = np.arange(m).reshape(m // 16, 16)
     for blk in range(nblk):
         for t in range(32):
             j = block_elem(k, C, blk, t)
