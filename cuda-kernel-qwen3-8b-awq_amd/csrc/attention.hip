@@ -85,17 +85,27 @@ __global__ __launch_bounds__(kThreads) void attention_kernel(const half_t* __res
   }
 
   // scores (Inference.cu:202-226) and their maximum (:229-233): this
-  // wavefront's four positions of each chunk, eight chunks' loads in flight
+  // wavefront's four positions of each chunk, six chunks' loads in flight.
+  // The values of this wavefront's first chunk are requested right behind the
+  // first keys, so that both arrive in one memory round trip.
+  half8_t vv[16];
   float lmax = -1e9f;
-  for (int c0 = 0; c0 < nchunks; c0 += 8) {
-    half8_t kv[8];
+  for (int c0 = 0; c0 < nchunks; c0 += 6) {
+    half8_t kv[6];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
+    for (int u = 0; u < 6; ++u) {
       const int t = ((c0 + u) << 6) + 4 * wave + tq;
       if (t < L) kv[u] = *reinterpret_cast<const half8_t*>(kh + (int64_t)t * AWQ_HEAD_DIM + 8 * dl);
     }
+    if (c0 == 0 && wave < nchunks) {
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
+      for (int nl = 0; nl < 16; ++nl) {
+        const int t = (wave << 6) + 4 * nl + tq;
+        if (t < L) vv[nl] = *reinterpret_cast<const half8_t*>(vh + (int64_t)t * AWQ_HEAD_DIM + 8 * dl);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 6; ++u) {
       const int t = ((c0 + u) << 6) + 4 * wave + tq;
       float part = 0.0f;
       if (t < L) {
@@ -137,11 +147,12 @@ __global__ __launch_bounds__(kThreads) void attention_kernel(const half_t* __res
   // loads of a chunk are issued together
   for (int chunk = wave; chunk < nchunks; chunk += kWaves) {
     const int base = chunk << 6;
-    half8_t vv[16];
+    if (chunk != wave) {  // the first chunk's values were requested at the start
 #pragma unroll
-    for (int nl = 0; nl < 16; ++nl) {
-      const int t = base + 4 * nl + tq;
-      if (t < L) vv[nl] = *reinterpret_cast<const half8_t*>(vh + (int64_t)t * AWQ_HEAD_DIM + 8 * dl);
+      for (int nl = 0; nl < 16; ++nl) {
+        const int t = base + 4 * nl + tq;
+        if (t < L) vv[nl] = *reinterpret_cast<const half8_t*>(vh + (int64_t)t * AWQ_HEAD_DIM + 8 * dl);
+      }
     }
     float acc[8];
 #pragma unroll

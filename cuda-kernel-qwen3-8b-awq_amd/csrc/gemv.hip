@@ -250,6 +250,14 @@ __device__ __forceinline__ void epilogue(const GemvParams& p, int row, int r, fl
   }
 }
 
+// LDS position (in halves) of block-order element e of x.  The four quarters of
+// a wavefront read four different lane groups at the same time; 16 bytes of
+// skew per lane group keep those reads in different banks.
+template <int G>
+__device__ __forceinline__ int xs_index(int e) {
+  return e + (e / (G * AWQ_BLOCK_K)) * 8;
+}
+
 // A workgroup takes row groups blockIdx.x, blockIdx.x + gridDim.x, ... (16
 // output rows x all of k each).  n_waves wavefronts; lane (w, q, r) owns blocks
 // (4w+q)*G .. +G-1 of row 16*rg + r.  x is staged (and normalised) once per
@@ -276,8 +284,6 @@ __global__ __launch_bounds__(1024) void gemv_kernel(GemvParams p) {
   int rg = blockIdx.x;
   const u32x4* wp = p.wq + ((int64_t)rg * p.nblk + blk0) * 16 + r;
   u32x4 w[G], wn[G];
-#pragma unroll
-  for (int b = 0; b < G; ++b) w[b] = __builtin_nontemporal_load(wp + b * 16);
 
   // ---- x into LDS in block order ------------------------------------------
   // Unit u of a thread is the 4 consecutive block-order elements 4*(tid + u*nthreads)..+3;
@@ -306,10 +312,18 @@ __global__ __launch_bounds__(1024) void gemv_kernel(GemvParams p) {
       }
     }
   }
+  // x first, and alone: once every wavefront of the device has its 8 KiB of
+  // weight loads in flight, a small load of x (an L2 hit) waits microseconds in
+  // the same queues.  So the weight stream starts only when x has arrived.
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+  for (int b = 0; b < G; ++b) w[b] = __builtin_nontemporal_load(wp + b * 16);
   if (norm) {
     // rmsNormKernel, Inference.cu:111-145: 256 strided fma partial sums over the
     // natural order, the stride-halving tree, then two binary16 multiplies.
-    // The raw values go through LDS in natural order for the partial sums.
+    // The raw values go through LDS in natural order (unskewed, in the same
+    // buffer; it is overwritten afterwards) for the partial sums.
+    half_t* xn = xs;
 #pragma unroll
     for (int u = 0; u < MAXU; ++u) {
       if (tid + u * nthreads < total_units) {
@@ -318,9 +332,9 @@ __global__ __launch_bounds__(1024) void gemv_kernel(GemvParams p) {
           half_t hx[4];
           *reinterpret_cast<uint64_t*>(hx) = __builtin_bit_cast(uint64_t, xu[u]);
 #pragma unroll
-          for (int i = 0; i < 4; ++i) xs[awq_block_elem(p.k, p.C, (e + i) >> 5, (e + i) & 31)] = hx[i];
+          for (int i = 0; i < 4; ++i) xn[awq_block_elem(p.k, p.C, (e + i) >> 5, (e + i) & 31)] = hx[i];
         } else {
-          reinterpret_cast<uint2*>(xs)[tid + u * nthreads] = xu[u];
+          reinterpret_cast<uint2*>(xn)[tid + u * nthreads] = xu[u];
         }
       }
     }
@@ -328,7 +342,7 @@ __global__ __launch_bounds__(1024) void gemv_kernel(GemvParams p) {
     if (tid < 256) {
       float acc = 0.0f;
       for (int i = tid; i < p.k; i += 256) {
-        float v = (float)xs[i];
+        float v = (float)xn[i];
         acc = __builtin_fmaf(v, v, acc);
       }
       nbuf[tid] = acc;
@@ -356,9 +370,11 @@ __global__ __launch_bounds__(1024) void gemv_kernel(GemvParams p) {
       }
     }
   }
+  if (norm) __syncthreads();  // everyone is done with the natural-order copy
 #pragma unroll
   for (int u = 0; u < MAXU; ++u)
-    if (tid + u * nthreads < total_units) reinterpret_cast<uint2*>(xs)[tid + u * nthreads] = xu[u];
+    if (tid + u * nthreads < total_units)
+      *reinterpret_cast<uint2*>(xs + xs_index<G>(4 * (tid + u * nthreads))) = xu[u];
 
   for (; rg < n_rg; rg += gridDim.x) {
     const int rg_next = rg + gridDim.x;
@@ -397,7 +413,7 @@ __global__ __launch_bounds__(1024) void gemv_kernel(GemvParams p) {
           cls_left = U;
         }
       }
-      bs[b] = block_dot<ZINT>(w[b], xs + (blk0 + b) * AWQ_BLOCK_K, g);
+      bs[b] = block_dot<ZINT>(w[b], xs + xs_index<G>((blk0 + b) * AWQ_BLOCK_K), g);
     }
     // adjacent-pair tree: this lane's G blocks, then the four quarters of the
     // wavefront (consecutive block ranges), then the wavefronts
@@ -568,7 +584,7 @@ int launch_gemv(const LinearArgs& a, hipStream_t st) {
     if (v >= 1 && v < n_rg) n_wg = v;
   }
   dim3 grid((unsigned)n_wg), block((unsigned)(plan.n_waves * 64));
-  size_t lds = (size_t)a.k * 2;
+  size_t lds = (size_t)a.k * 2 + (size_t)(a.k / AWQ_BLOCK_K / plan.g) * 16;  // x plus 16 bytes of skew per lane group
   switch (plan.g) {
     case 1: launch_g<1>(p, a.zp_integral, periodic, grid, block, lds, st); break;
     case 2: launch_g<2>(p, a.zp_integral, periodic, grid, block, lds, st); break;
