@@ -788,6 +788,20 @@ extern "C" int awq_gemv(const void* repacked, const void* scale, const void* zp,
   return awq_gemv_fused(&u, stream);
 }
 
+extern "C" int awq_gemm(const void* repacked, const void* scale, const void* zp, int64_t m, int64_t k, const void* x,
+                        void* y, int64_t M, int32_t zp_integral, void* stream) {
+  AWQ_REQUIRE(repacked && scale && zp && x && y, "NULL pointer");
+  AWQ_REQUIRE(m > 0 && m % 128 == 0, "m must be a positive multiple of 128");
+  if (zp_integral < 0) {
+    std::vector<uint16_t> zph((size_t)(m / 128));
+    AWQ_HIP_TRY(hipMemcpyAsync(zph.data(), zp, zph.size() * 2, hipMemcpyDeviceToHost, (hipStream_t)stream));
+    AWQ_HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+    zp_integral = zp_all_integral(zph.data(), (int64_t)zph.size());
+  }
+  return launch_gemm(repacked, (const half_t*)scale, (const half_t*)zp, m, k, (const half_t*)x, (half_t*)y, M,
+                     zp_integral != 0, (hipStream_t)stream);
+}
+
 extern "C" int awq_rmsnorm(const void* x, const void* gamma, void* out, int64_t n, float eps, void* stream) {
   AWQ_REQUIRE(x && gamma && out, "NULL pointer");
   return launch_rmsnorm((const half_t*)x, (const half_t*)gamma, (half_t*)out, n, eps, (hipStream_t)stream);

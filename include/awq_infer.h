@@ -185,6 +185,16 @@ typedef struct awq_linear_args {
 } awq_linear_args;
 int awq_gemv_fused(const awq_linear_args* args, void* stream);
 
+/* The same product for M tokens at once (prefill, batched decode): the
+ * reference's cublasGemmEx with n = M, ldb = k, ldc = m (it only ever calls it
+ * with n = 1, Inference.cu:1056).  x [M][k], y [M][m] row-major FP16.  Weights
+ * are dequantised on load and contracted on the matrix cores with FP32
+ * accumulation: within rounding noise of awq_gemv applied to each token, not
+ * bit-identical to it.  Matrices whose scale group depends on the input index
+ * (the 151936 x 4096 unembedding) are not supported. */
+int awq_gemm(const void* repacked, const void* scale, const void* zp, int64_t m, int64_t k, const void* x, void* y,
+             int64_t M, int32_t zp_integral, void* stream);
+
 /* rmsNormKernel, Inference.cu:111-145.  n multiple of 256. */
 int awq_rmsnorm(const void* x, const void* gamma, void* out, int64_t n, float eps, void* stream);
 

@@ -436,3 +436,62 @@ def test_gemv_fused_norm_unembed_argmax(awq, lib, oracle, torch_gpu, m, k):
         assert np.array_equal(d_y.cpu().numpy().view(np.uint16), logits.view(np.uint16))
         assert int(tok.item()) == oracle.awqo_argmax(ptr(logits), m)
     assert int(keep["ws"][:64].to(torch.int32).abs().sum().item()) == 0  # sampler workspace left zeroed
+
+
+# ----------------------------------------------------------------------------- W4A16 GEMM on the matrix cores
+@pytest.mark.parametrize("m,k,M,zp_int", [(256, 512, 3, True), (256, 512, 17, False), (384, 1536, 130, True),
+                                          (12288, 4096, 16, True), (12288, 4096, 200, True), (4096, 12288, 64, False)])
+def test_gemm_matches_fp32_accumulate_reference(awq, lib, oracle, torch_gpu, m, k, M, zp_int):
+    """config 5: dequant-on-load MFMA product; 1e-2 relative against the sequential FP32-accumulate
+    reference, and the weights it multiplies are the bit-exact dequantised ones (one-hot check below)"""
+    torch = torch_gpu
+    rng = np.random.default_rng(m + k + M)
+    packed, scale, zp = rand_awq(rng, m, k, zp_int=zp_int)
+    x = rng.standard_normal((M, k)).astype(np.float16)
+    Mo = min(M, 24)  # the oracle is slow on the large shapes: check a subset of tokens there
+    sel = np.sort(rng.choice(M, size=Mo, replace=False))
+    ref = np.zeros((Mo, m), dtype=np.float16)
+    xs = np.ascontiguousarray(x[sel])
+    oracle.awqo_linear(ptr(packed), ptr(scale), ptr(zp), m, k, ptr(xs), ptr(ref), Mo)
+    d_in = dev(torch, packed)
+    d_w = torch.zeros(m * k // 2, dtype=torch.uint8, device="cuda")
+    awq.check(lib.awq_linear_repack(d_in.data_ptr(), d_w.data_ptr(), m, k, stream(torch)))
+    d_s, d_z, d_x = dev(torch, scale), dev(torch, zp), dev(torch, x)
+    d_y = torch.full((M, m), float("nan"), dtype=torch.float16, device="cuda")
+    print("gemm", m, k, M, flush=True)
+    awq.check(lib.awq_gemm(d_w.data_ptr(), d_s.data_ptr(), d_z.data_ptr(), m, k, d_x.data_ptr(), d_y.data_ptr(), M,
+                           1 if zp_int else 0, stream(torch)))
+    torch.cuda.synchronize()
+    got = d_y.cpu().numpy()[sel].astype(np.float64)
+    want = ref.astype(np.float64)
+    denom = np.maximum(np.abs(want), 1e-2 * np.abs(want).max())
+    assert np.all(np.isfinite(got))
+    assert np.all(np.abs(got - want) <= 1e-2 * denom)
+    # much tighter in practice: FP32 accumulation either way
+    assert np.mean(d_y.cpu().numpy()[sel].view(np.uint16) == ref.view(np.uint16)) > 0.9
+
+
+def test_gemm_one_hot_and_token_independence(awq, lib, torch_gpu):
+    torch = torch_gpu
+    m, k, M = 256, 512, 20
+    scale = np.ones(m // 128, dtype=np.float16)
+    zp = np.zeros(m // 128, dtype=np.float16)
+    x = ((np.arange(M * k).reshape(M, k) % 13) + 1).astype(np.float16)
+    for p, q in [(0, 5), (m + 1, 9), (3 * m + 17, 15), (k * m - 1, 1)]:
+        packed = np.zeros(m * k // 2, dtype=np.uint8)
+        packed[p >> 1] = q << (4 * (p & 1))
+        d_in = dev(torch, packed)
+        d_w = torch.zeros(m * k // 2, dtype=torch.uint8, device="cuda")
+        awq.check(lib.awq_linear_repack(d_in.data_ptr(), d_w.data_ptr(), m, k, stream(torch)))
+        d_s, d_z, d_x = dev(torch, scale), dev(torch, zp), dev(torch, x)
+        d_y = torch.zeros((M, m), dtype=torch.float16, device="cuda")
+        awq.check(lib.awq_gemm(d_w.data_ptr(), d_s.data_ptr(), d_z.data_ptr(), m, k, d_x.data_ptr(), d_y.data_ptr(), M,
+                               1, stream(torch)))
+        torch.cuda.synchronize()
+        y = d_y.cpu().numpy().astype(np.float64)
+        expect = np.zeros((M, m))
+        expect[:, p % m] = q * x[:, p // m].astype(np.float64)
+        assert np.array_equal(y, expect), p
+    buf = torch.zeros(1 << 20, dtype=torch.uint8, device="cuda")
+    b = buf.data_ptr()
+    assert lib.awq_gemm(b, b, b, 128 * 37, 512, b, b, 4, 1, None) != 0   # input-dependent scale groups: refused
