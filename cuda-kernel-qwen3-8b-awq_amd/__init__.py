@@ -21,6 +21,7 @@ INCLUDE_DIR = os.path.join(os.path.dirname(_HERE), "include")
 T_WQKV, T_WO, T_W1, T_W2, T_GAMMA, T_EMBED, T_UNEMBED = range(7)
 P_PACKED, P_SCALE, P_ZP = range(3)
 SYNTH_STREAM_INPUT = 0x100000
+SYNTH_SPEC, SYNTH_BALANCED = 0, 1
 
 
 class AwqConfig(ctypes.Structure):
@@ -70,6 +71,7 @@ SIGNATURES = {
     "awq_destroy": (None, [_vp]),
     "awq_write_weight_dir": (ctypes.c_int, [ctypes.c_char_p, _cfgp, _u64]),
     "awq_synth_fill": (ctypes.c_int, [_u64, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp, _i64]),
+    "awq_synth_fill_profile": (ctypes.c_int, [ctypes.c_int, _u64, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp, _i64]),
     "awq_synth_normal_f16": (ctypes.c_int, [_u64, _u64, _vp, _i64, _f32, _f32]),
     "awq_synth_tokens": (ctypes.c_int, [_u64, _u64, _vp, _i64, _i32]),
     "awq_rope_tables_host": (ctypes.c_int, [_vp, _vp, _i64]),

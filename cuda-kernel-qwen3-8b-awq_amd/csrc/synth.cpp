@@ -16,7 +16,13 @@ static uint16_t to_half_bits(float f) {
 }
 
 extern "C" int awq_synth_fill(uint64_t seed, int layer, int kind, int part, void* host_dst, int64_t count) {
+  return awq_synth_fill_profile(AWQ_SYNTH_SPEC, seed, layer, kind, part, host_dst, count);
+}
+
+extern "C" int awq_synth_fill_profile(int profile, uint64_t seed, int layer, int kind, int part, void* host_dst,
+                                      int64_t count) {
   AWQ_REQUIRE(host_dst && count >= 0, "bad destination");
+  AWQ_REQUIRE(profile == AWQ_SYNTH_SPEC || profile == AWQ_SYNTH_BALANCED, "bad profile");
   AWQ_REQUIRE(kind >= AWQ_T_WQKV && kind <= AWQ_T_UNEMBED, "bad tensor kind");
   const uint64_t sid = awq_synth_stream(layer, kind, part);
   if (kind == AWQ_T_GAMMA) {
@@ -44,10 +50,10 @@ extern "C" int awq_synth_fill(uint64_t seed, int layer, int kind, int part, void
     uint64_t h = awq_synth_hash(seed, sid, (uint64_t)i);
     if (part == AWQ_P_SCALE) {
       float u = awq_synth_uniform(h);
-      float v = 0.018f * u;
-      d[i] = to_half_bits(0.002f + v);
+      float v = (profile == AWQ_SYNTH_BALANCED ? 0.0015f : 0.018f) * u;
+      d[i] = to_half_bits((profile == AWQ_SYNTH_BALANCED ? 0.0025f : 0.002f) + v);
     } else {
-      d[i] = to_half_bits((float)(h & 15u));
+      d[i] = to_half_bits(profile == AWQ_SYNTH_BALANCED ? (float)(7u + (unsigned)(h & 1u)) : (float)(h & 15u));
     }
   }
   return AWQ_OK;

@@ -103,6 +103,8 @@ int awq_write_weight_dir(const char* dir, const awq_config* cfg, uint64_t seed);
 /* Host-side synthetic data (awq_synth.h).  `count` is in elements of the
  * array: bytes for AWQ_P_PACKED, halves otherwise. */
 int awq_synth_fill(uint64_t seed, int layer, int kind, int part, void* host_dst, int64_t count);
+/* profile: AWQ_SYNTH_SPEC (what awq_synth_fill draws) or AWQ_SYNTH_BALANCED (awq_synth.h) */
+int awq_synth_fill_profile(int profile, uint64_t seed, int layer, int kind, int part, void* host_dst, int64_t count);
 int awq_synth_normal_f16(uint64_t seed, uint64_t stream, uint16_t* host_dst, int64_t count, float mean, float std);
 int awq_synth_tokens(uint64_t seed, uint64_t stream, int32_t* host_dst, int64_t count, int32_t vocab);
 

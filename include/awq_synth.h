@@ -15,6 +15,15 @@
  *   token ids           r mod vocab
  *
  * Normals use Box-Muller in double precision and are rounded to binary16 once.
+ *
+ * Those are the distributions of the benchmark definition.  A 36-layer model
+ * drawn from them overflows binary16 within four layers (the zero-points give
+ * every weight row a large mean), after which every logit is NaN and greedy
+ * decoding returns token 0 whatever the arithmetic does.  AWQ_SYNTH_BALANCED
+ * keeps the same format and generator but draws
+ *   scale               h(0.0025 + 0.0015*u)
+ *   zero-point          h(7 + (r mod 2)), i.e. 7 or 8
+ * so that activations stay finite and token identity is a real test.
  */
 #ifndef AWQ_SYNTH_H
 #define AWQ_SYNTH_H
@@ -33,6 +42,7 @@ enum awq_tensor_kind {
   AWQ_T_UNEMBED = 6  /* unembed.bin, [V x H]                  Inference.cu:891 */
 };
 enum awq_tensor_part { AWQ_P_PACKED = 0, AWQ_P_SCALE = 1, AWQ_P_ZP = 2 };
+enum awq_synth_profile { AWQ_SYNTH_SPEC = 0, AWQ_SYNTH_BALANCED = 1 };
 
 static inline uint64_t awq_synth_hash(uint64_t seed, uint64_t sid, uint64_t idx) {
   uint64_t z = seed * 0x9E3779B97F4A7C15ull + (sid + 1) * 0xD1B54A32D192ED03ull + idx * 0xA0761D6478BD642Full;

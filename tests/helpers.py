@@ -119,7 +119,7 @@ def make_oracle_model(oracle, cfg):
     return oracle.awqo_model_create(ctypes.byref(ocfg))
 
 
-def fill_pair(awq, oracle, cfg, seed, engine=None, model=None):
+def fill_pair(awq, oracle, cfg, seed, engine=None, model=None, profile=0):
     """Fill the oracle model's host arrays from the seeded generator and upload the very same
     bytes to the engine."""
     lib = awq.load_library()
@@ -129,7 +129,7 @@ def fill_pair(awq, oracle, cfg, seed, engine=None, model=None):
         got = ctypes.c_int64(0)
         p = oracle.awqo_model_tensor(model, layer, kind, part, ctypes.byref(got))
         assert got.value == nbytes, (layer, kind, part, got.value, nbytes)
-        awq.check(lib.awq_synth_fill(seed, layer, kind, part, p, count))
+        awq.check(lib.awq_synth_fill_profile(profile, seed, layer, kind, part, p, count))
         if engine is not None:
             engine.upload(layer, kind, part, p, nbytes)
     if engine is not None:

@@ -121,3 +121,126 @@ def test_full_width_model_token_identity(awq, oracle, torch_gpu, n_layers, promp
     compare_state(awq, oracle, eng, model, cfg)
     eng.close()
     oracle.awqo_model_destroy(model)
+
+
+def test_config2_one_decoder_layer_at_position_512(awq, lib, oracle, torch_gpu):
+    """config 2: one full decoder layer at decode batch 1, reference widths, 512 prior cached positions of
+    N(0,1) values, attention over L = 513 -- composed from the C ABI's kernel entry points exactly as
+    runOneLayer (Inference.cu:1029-1230) orders them, against the oracle's layer"""
+    import ctypes as C
+    torch = torch_gpu
+    H, I, nh, mp, pos, L = 4096, 12288, 32, 640, 512, 513
+    cfg = awq.make_config(n_layers=1, max_pos=mp, vocab=128)
+    model = make_oracle_model(oracle, cfg)
+    fill_pair(awq, oracle, cfg, 4242, engine=None, model=model)
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def host(kind, part):
+        n = C.c_int64(0)
+        p = oracle.awqo_model_tensor(model, 0, kind, part, C.byref(n))
+        return np.ctypeslib.as_array(C.cast(p, C.POINTER(C.c_uint8)), (n.value,))
+
+    def upload(a):
+        return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+    # seeded inputs: hidden state and the first 512 cache rows of every head
+    hidden = np.zeros(H, dtype=np.float16)
+    awq.check(lib.awq_synth_normal_f16(4242, awq.SYNTH_STREAM_INPUT + 2, ptr(hidden), H, 0.0, 1.0))
+    kv = np.zeros((2, nh, mp, 128), dtype=np.float16)
+    for which in range(2):
+        rows = np.zeros((nh, pos, 128), dtype=np.float16)
+        awq.check(lib.awq_synth_normal_f16(4242, awq.SYNTH_STREAM_INPUT + 3 + which, ptr(rows), rows.size, 0.0, 1.0))
+        kv[which, :, :pos] = rows
+    for which, getter in ((0, oracle.awqo_model_kcache), (1, oracle.awqo_model_vcache)):
+        dst = np.ctypeslib.as_array(C.cast(getter(model, 0), C.POINTER(C.c_uint16)), (nh * mp * 128,))
+        dst[:] = kv[which].reshape(-1).view(np.uint16)
+    oh = np.ctypeslib.as_array(C.cast(oracle.awqo_model_hidden_mut(model), C.POINTER(C.c_uint16)), (H,))
+    oh[:] = hidden.view(np.uint16)
+    oracle.awqo_model_layer(model, 0, pos, L)
+    ref_hidden = oh.copy()
+    ref_k = np.ctypeslib.as_array(C.cast(oracle.awqo_model_kcache(model, 0), C.POINTER(C.c_uint16)), (nh * mp * 128,)).copy()
+
+    # device side
+    dims = {awq.T_WQKV: (3 * H, H), awq.T_WO: (H, H), awq.T_W1: (I, H), awq.T_W2: (H, I)}
+    dev_w = {}
+    for kind, (m, k) in dims.items():
+        d_in = upload(host(kind, awq.P_PACKED))
+        d_w = torch.empty_like(d_in)
+        awq.check(lib.awq_linear_repack(d_in.data_ptr(), d_w.data_ptr(), m, k, st))
+        dev_w[kind] = (d_w, upload(host(kind, awq.P_SCALE)), upload(host(kind, awq.P_ZP)))
+    d_gamma = upload(host(awq.T_GAMMA, 0))
+    cos_t, sin_t = np.zeros((mp, 64), np.float16), np.zeros((mp, 64), np.float16)
+    awq.check(lib.awq_rope_tables_host(ptr(cos_t), ptr(sin_t), mp))
+    d_cos, d_sin = upload(cos_t), upload(sin_t)
+    d_k, d_v = upload(kv[0]), upload(kv[1])
+    d_hidden = upload(hidden)
+    d_q = torch.zeros(H, dtype=torch.float16, device="cuda")
+    d_ctx = torch.zeros(H, dtype=torch.float16, device="cuda")
+    d_mid = torch.zeros(I, dtype=torch.float16, device="cuda")
+    ws = torch.zeros(4096, dtype=torch.uint8, device="cuda")
+    att_ws = torch.zeros(lib.awq_attention_workspace_bytes(nh, mp), dtype=torch.uint8, device="cuda")
+
+    def linear(kind, x, y, **kw):
+        a = awq.AwqLinearArgs()
+        w, s, z = dev_w[kind]
+        a.repacked, a.scale, a.zp = w.data_ptr(), s.data_ptr(), z.data_ptr()
+        a.m, a.k = dims[kind]
+        a.x, a.y, a.zp_integral, a.workspace, a.eps = x.data_ptr(), y.data_ptr(), 1, ws.data_ptr(), 1e-6
+        for key, val in kw.items():
+            setattr(a, key, val)
+        awq.check(lib.awq_gemv_fused(C.byref(a), st))
+
+    linear(awq.T_WQKV, d_hidden, d_q, prologue=awq.PRO_RMSNORM, gamma=d_gamma.data_ptr(), epilogue=awq.EPI_QKV_ROPE,
+           cos_t=d_cos.data_ptr(), sin_t=d_sin.data_ptr(), k_cache=d_k.data_ptr(), v_cache=d_v.data_ptr(),
+           hidden=H, max_pos=mp, pos=pos)
+    awq.check(lib.awq_decode_attention(d_q.data_ptr(), d_k.data_ptr(), d_v.data_ptr(), d_ctx.data_ptr(), nh, mp, L,
+                                       att_ws.data_ptr(), st))
+    linear(awq.T_WO, d_ctx, d_hidden, epilogue=awq.EPI_RESIDUAL, residual=d_hidden.data_ptr())
+    linear(awq.T_W1, d_hidden, d_mid, prologue=awq.PRO_RMSNORM, gamma=d_gamma.data_ptr(), epilogue=awq.EPI_GELU)
+    linear(awq.T_W2, d_mid, d_hidden, epilogue=awq.EPI_RESIDUAL, residual=d_hidden.data_ptr())
+    torch.cuda.synchronize()
+    assert np.array_equal(d_hidden.cpu().numpy().view(np.uint16), ref_hidden)
+    assert np.array_equal(d_k.cpu().numpy().reshape(-1).view(np.uint16), ref_k)
+    oracle.awqo_model_destroy(model)
+
+
+def test_full_model_32_greedy_tokens_identical(awq, oracle, torch_gpu):
+    """config 4 at reduced length: all 36 layers at the reference widths, random-init seeded weights, greedy
+    decode of 32 tokens; ids, final hidden state and last logits must equal the CPU path bit for bit.
+    Weights come from the balanced profile (include/awq_synth.h): with the benchmark's own distributions the
+    activations overflow binary16 by layer 3 and every token is 0, which would test nothing (that regime is
+    covered by the next test).  Here the logits are finite and the top-1/top-2 margin is a few FP16 ulps, so
+    any rounding difference between the two paths changes the ids."""
+    cfg = awq.make_config(max_pos=64)
+    assert (cfg.n_layers, cfg.hidden, cfg.inter, cfg.vocab, cfg.split_idx) == (36, 4096, 12288, 151936, 18)
+    model = make_oracle_model(oracle, cfg)
+    eng = awq.QWen3AWQInfer.empty(cfg)
+    fill_pair(awq, oracle, cfg, 2025, engine=eng, model=model, profile=awq.SYNTH_BALANCED)
+    prompt = np.zeros(4, dtype=np.int32)
+    awq.check(awq.load_library().awq_synth_tokens(2025, awq.SYNTH_STREAM_INPUT, ptr(prompt), prompt.size, cfg.vocab))
+    print("36-layer model: 32 greedy tokens", flush=True)
+    got = eng.generateResponse(prompt.tolist(), 32)
+    ref = oracle_generate(oracle, model, prompt.tolist(), 32)
+    margins = np.zeros(64, dtype=np.float32)
+    n = oracle.awqo_model_margins(model, ptr(margins), 64)
+    print("top-1/top-2 logit margins: min %.4f median %.4f" % (margins[:n].min(), np.median(margins[:n])), flush=True)
+    assert got == ref
+    assert len(set(got)) > 1 and np.isfinite(margins[:n]).all() and margins[:n].min() < 0.5
+    compare_state(awq, oracle, eng, model, cfg)
+    eng.close()
+    oracle.awqo_model_destroy(model)
+
+
+def test_full_model_benchmark_distributions_overflow_identically(awq, oracle, torch_gpu):
+    """the benchmark's own value distributions on the 36-layer model: activations reach inf/NaN within four
+    layers on both paths; the hidden state, the logits (NaN patterns included) and the ids still agree"""
+    cfg = awq.make_config(max_pos=32)
+    model = make_oracle_model(oracle, cfg)
+    eng = awq.QWen3AWQInfer.empty(cfg)
+    fill_pair(awq, oracle, cfg, 2026, engine=eng, model=model, profile=awq.SYNTH_SPEC)
+    prompt = [151643, 17]
+    got = eng.generateResponse(prompt, 6)
+    assert got == oracle_generate(oracle, model, prompt, 6)
+    compare_state(awq, oracle, eng, model, cfg)
+    eng.close()
+    oracle.awqo_model_destroy(model)
