@@ -24,6 +24,8 @@ HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fopenmp",
     "-ffp-contract=off", "-fno-fast-math", "-fhip-fp32-correctly-rounded-divide-sqrt",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # first 16 dwords of a kernel's arguments arrive in scalar registers at wavefront launch
+    "-mllvm", "-amdgpu-kernarg-preload-count=16",
     "-Wall", "-Wno-unused-function", "-x", "hip",
 ]
 

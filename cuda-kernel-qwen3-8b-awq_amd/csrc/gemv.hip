@@ -263,8 +263,16 @@ __device__ __forceinline__ int xs_index(int e) {
 // (4w+q)*G .. +G-1 of row 16*rg + r.  x is staged (and normalised) once per
 // workgroup; the weights of the next row group are in flight while the current
 // one is multiplied.
+// The arguments every wavefront needs before its first load come first and
+// one by one: the first 16 dwords of the argument block are preloaded into
+// scalar registers at wavefront launch (see the build flags), which takes one
+// memory round trip off the start of the kernel.
 template <int G, bool ZINT, bool PERIODIC>
-__global__ __launch_bounds__(1024) void gemv_kernel(GemvParams p) {
+__global__ __launch_bounds__(1024) void gemv_kernel(const u32x4* __restrict__ wq, const half_t* __restrict__ x,
+                                                    const half_t* __restrict__ gamma, const half_t* __restrict__ scale,
+                                                    const half_t* __restrict__ zp, int32_t k, int32_t nblk,
+                                                    int32_t n_waves, int32_t m, int32_t prologue, int32_t C,
+                                                    GemvParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   half_t* xs = reinterpret_cast<half_t*>(smem);  // x in block order, k halves
   __shared__ float red[16][16];
@@ -273,24 +281,24 @@ __global__ __launch_bounds__(1024) void gemv_kernel(GemvParams p) {
   constexpr int MAXU = 8;  // 8-byte units of x a thread may hold in registers
 
   const int tid = threadIdx.x;
-  const int nthreads = p.n_waves * 64;
+  const int nthreads = n_waves * 64;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int q = lane >> 4, r = lane & 15;
-  const int n_rg = p.m >> 4;
+  const int n_rg = m >> 4;
   const int blk0 = (4 * wave + q) * G;
-  const int U = p.nblk / p.C;  // blocks per class (PERIODIC)
+  const int U = nblk / C;  // blocks per class (PERIODIC)
 
   int rg = blockIdx.x;
-  const u32x4* wp = p.wq + ((int64_t)rg * p.nblk + blk0) * 16 + r;
+  const u32x4* wp = wq + ((int64_t)rg * nblk + blk0) * 16 + r;
   u32x4 w[G], wn[G];
 
   // ---- x into LDS in block order ------------------------------------------
   // Unit u of a thread is the 4 consecutive block-order elements 4*(tid + u*nthreads)..+3;
   // in natural order they are 4 consecutive indices too unless the matrix is
   // periodic (then they are C apart and are gathered one by one).
-  const int total_units = p.k >> 2;  // at most MAXU * nthreads (checked by the launcher)
-  const bool norm = p.prologue == PRO_RMSNORM;
+  const int total_units = k >> 2;  // at most MAXU * nthreads (checked by the launcher)
+  const bool norm = prologue == PRO_RMSNORM;
   uint2 xu[MAXU], gu[MAXU];
 #pragma unroll
   for (int u = 0; u < MAXU; ++u) {
@@ -300,15 +308,15 @@ __global__ __launch_bounds__(1024) void gemv_kernel(GemvParams p) {
         half_t hx[4], hg[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const int j = (int)awq_block_elem(p.k, p.C, (e + i) >> 5, (e + i) & 31);
-          hx[i] = p.x[j];
-          hg[i] = norm ? p.gamma[j] : (half_t)0.0f;
+          const int j = (int)awq_block_elem(k, C, (e + i) >> 5, (e + i) & 31);
+          hx[i] = x[j];
+          hg[i] = norm ? gamma[j] : (half_t)0.0f;
         }
         xu[u] = __builtin_bit_cast(uint2, *reinterpret_cast<uint64_t*>(hx));
         gu[u] = __builtin_bit_cast(uint2, *reinterpret_cast<uint64_t*>(hg));
       } else {
-        xu[u] = reinterpret_cast<const uint2*>(p.x)[tid + u * nthreads];
-        if (norm) gu[u] = reinterpret_cast<const uint2*>(p.gamma)[tid + u * nthreads];
+        xu[u] = reinterpret_cast<const uint2*>(x)[tid + u * nthreads];
+        if (norm) gu[u] = reinterpret_cast<const uint2*>(gamma)[tid + u * nthreads];
       }
     }
   }
@@ -332,7 +340,7 @@ __global__ __launch_bounds__(1024) void gemv_kernel(GemvParams p) {
           half_t hx[4];
           *reinterpret_cast<uint64_t*>(hx) = __builtin_bit_cast(uint64_t, xu[u]);
 #pragma unroll
-          for (int i = 0; i < 4; ++i) xn[awq_block_elem(p.k, p.C, (e + i) >> 5, (e + i) & 31)] = hx[i];
+          for (int i = 0; i < 4; ++i) xn[awq_block_elem(k, C, (e + i) >> 5, (e + i) & 31)] = hx[i];
         } else {
           reinterpret_cast<uint2*>(xn)[tid + u * nthreads] = xu[u];
         }
@@ -341,7 +349,7 @@ __global__ __launch_bounds__(1024) void gemv_kernel(GemvParams p) {
     __syncthreads();
     if (tid < 256) {
       float acc = 0.0f;
-      for (int i = tid; i < p.k; i += 256) {
+      for (int i = tid; i < k; i += 256) {
         float v = (float)xn[i];
         acc = __builtin_fmaf(v, v, acc);
       }
@@ -357,7 +365,7 @@ __global__ __launch_bounds__(1024) void gemv_kernel(GemvParams p) {
       if (tid == 0) nbuf[0] = v;
     }
     __syncthreads();
-    const half_t sc = (half_t)awq_rsqrtf(nbuf[0] / (float)p.k + p.eps);
+    const half_t sc = (half_t)awq_rsqrtf(nbuf[0] / (float)k + p.eps);
     const half2_t sc2 = half2_t{sc, sc};
 #pragma unroll
     for (int u = 0; u < MAXU; ++u) {
@@ -379,7 +387,7 @@ __global__ __launch_bounds__(1024) void gemv_kernel(GemvParams p) {
   for (; rg < n_rg; rg += gridDim.x) {
     const int rg_next = rg + gridDim.x;
     if (rg_next < n_rg) {
-      const u32x4* wpn = p.wq + ((int64_t)rg_next * p.nblk + blk0) * 16 + r;
+      const u32x4* wpn = wq + ((int64_t)rg_next * nblk + blk0) * 16 + r;
 #pragma unroll
       for (int b = 0; b < G; ++b) wn[b] = __builtin_nontemporal_load(wpn + b * 16);
     }
@@ -391,10 +399,10 @@ __global__ __launch_bounds__(1024) void gemv_kernel(GemvParams p) {
     GroupConst g;
     if (!PERIODIC) {
       int gi = (a % p.kg) % p.mg;
-      g = make_group<ZINT>(p.scale[gi], p.zp[gi]);
-    } else if (tid < p.C) {
+      g = make_group<ZINT>(scale[gi], zp[gi]);
+    } else if (tid < C) {
       int gi = (int)((((int64_t)tid * p.mg + a) % p.kg) % p.mg);
-      gtab[tid] = make_group<ZINT>(p.scale[gi], p.zp[gi]);
+      gtab[tid] = make_group<ZINT>(scale[gi], zp[gi]);
     }
     int cls = 0, cls_left = 0;  // class of the next block and blocks left in it
     if (PERIODIC) {
@@ -428,7 +436,7 @@ __global__ __launch_bounds__(1024) void gemv_kernel(GemvParams p) {
     if (q == 0) red[wave][r] = v;
     __syncthreads();
     if (tid < 16) {
-      int n = p.n_waves;
+      int n = n_waves;
       while (n > 1 && (n & 1) == 0) {
         n >>= 1;
         for (int i = 0; i < n; ++i) red[i][r] = red[2 * i][r] + red[2 * i + 1][r];
@@ -470,7 +478,8 @@ bool plan_gemv(int64_t m, int64_t k, GemvPlan* out) {
     if (groups % 4 || groups > 64) continue;
     *out = GemvPlan{g, (int)(groups / 4)};
     found = true;
-    if ((m / 16) * (groups / 4) >= 2048) break;
+    // at least 4 wavefronts: the fused norm sums with 256 threads
+    if (groups / 4 >= 4 && (m / 16) * (groups / 4) >= 2048) break;
   }
   if (const char* f = getenv("AWQ_DEV_G")) {
     int g = atoi(f);
@@ -479,14 +488,15 @@ bool plan_gemv(int64_t m, int64_t k, GemvPlan* out) {
   return found;
 }
 
+#define GEMV_HOT_ARGS p.wq, p.x, p.gamma, p.scale, p.zp, p.k, p.nblk, p.n_waves, p.m, p.prologue, p.C
 template <int G>
 void launch_g(const GemvParams& p, bool zint, bool periodic, dim3 grid, dim3 block, size_t lds, hipStream_t st) {
   if (zint) {
-    if (periodic) hipLaunchKernelGGL((gemv_kernel<G, true, true>), grid, block, lds, st, p);
-    else hipLaunchKernelGGL((gemv_kernel<G, true, false>), grid, block, lds, st, p);
+    if (periodic) hipLaunchKernelGGL((gemv_kernel<G, true, true>), grid, block, lds, st, GEMV_HOT_ARGS, p);
+    else hipLaunchKernelGGL((gemv_kernel<G, true, false>), grid, block, lds, st, GEMV_HOT_ARGS, p);
   } else {
-    if (periodic) hipLaunchKernelGGL((gemv_kernel<G, false, true>), grid, block, lds, st, p);
-    else hipLaunchKernelGGL((gemv_kernel<G, false, false>), grid, block, lds, st, p);
+    if (periodic) hipLaunchKernelGGL((gemv_kernel<G, false, true>), grid, block, lds, st, GEMV_HOT_ARGS, p);
+    else hipLaunchKernelGGL((gemv_kernel<G, false, false>), grid, block, lds, st, GEMV_HOT_ARGS, p);
   }
 }
 
