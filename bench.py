@@ -85,6 +85,19 @@ def main():
     prompt = np.zeros(args.prompt_len, dtype=np.int32)
     awq.check(lib.awq_synth_tokens(args.seed, awq.SYNTH_STREAM_INPUT, ptr(prompt), prompt.size, cfg.vocab))
 
+    # ---- the prompt pass, both ways (not part of `value`): token by token as the reference does,
+    #      and all positions through each layer together on the matrix cores ---------------------
+    prefill_ms = {}
+    for name, batched in (("batched", True), ("sequential", False)):
+        for rep in range(2):                       # the first pass builds graphs / allocates buffers
+            eng.reset()
+            torch.cuda.synchronize()
+            tp = time.perf_counter()
+            eng.prefill(prompt.tolist(), batched=batched)   # returns after the device finished
+            prefill_ms[name] = round(1000.0 * (time.perf_counter() - tp), 3)
+    log("prompt of %d tokens: %.2f ms token by token, %.2f ms batched" %
+        (args.prompt_len, prefill_ms["sequential"], prefill_ms["batched"]))
+
     # ---- timed decode: K steps after the prompt and W warm-up steps ------------------------------
     eng.reset()
     eng.prefill(prompt.tolist())
@@ -158,6 +171,7 @@ def main():
         "step_algorithmic_bytes": int(step_bytes),
         "step_hbm_frac": round(step_bytes * tok_s / (HBM_PEAK_GBS * 1e9), 4),
         "greedy_tokens_identical_to_cpu": tokens_match,
+        "prompt_pass_ms": prefill_ms,
         "roofline": roofline,
         "cpu_baseline": cpu,
     }

@@ -64,6 +64,8 @@ SIGNATURES = {
     "awq_reset": (ctypes.c_int, [_vp]),
     "awq_prefill": (ctypes.c_int, [_vp, _vp, _i32]),
     "awq_decode": (ctypes.c_int, [_vp, _i32, _vp]),
+    "awq_prefill_batched": (ctypes.c_int, [_vp, _vp, _i32]),
+    "awq_set_prefill_mode": (ctypes.c_int, [_vp, ctypes.c_int]),
     "awq_read_hidden": (ctypes.c_int, [_vp, _vp]),
     "awq_read_logits": (ctypes.c_int, [_vp, _vp]),
     "awq_set_graph_mode": (ctypes.c_int, [_vp, ctypes.c_int]),
@@ -230,8 +232,14 @@ class QWen3AWQInfer:
     def reset(self):
         check(self._lib.awq_reset(self._h))
 
-    def prefill(self, prompt_ids):
-        check(self._lib.awq_prefill(self._h, _int32_array(prompt_ids), len(prompt_ids)))
+    def prefill(self, prompt_ids, batched=False):
+        """The prompt loop; batched=True sends all positions through each layer together."""
+        fn = self._lib.awq_prefill_batched if batched else self._lib.awq_prefill
+        check(fn(self._h, _int32_array(prompt_ids), len(prompt_ids)))
+
+    def set_prefill_mode(self, batched):
+        """Which prompt loop generateResponse uses (default: token by token)."""
+        check(self._lib.awq_set_prefill_mode(self._h, 1 if batched else 0))
 
     def decode(self, n_steps):
         out = (ctypes.c_int32 * max(1, n_steps))()

@@ -4,8 +4,10 @@
 
   * M = 2048 tokens through the dequant-on-load MFMA kernel: TFLOP/s and the fraction of the
     MI355X dense FP16 matrix peak (2.5 PFLOP/s);
-  * M = 1 through the decode kernel, M = 4, 16, 64 through the MFMA kernel: microseconds, algorithmic
-    GB/s and the fraction of the 8 TB/s HBM peak.
+  * M = 1 through the decode kernel, M = 4, 16, 64, 128, 512 through the MFMA kernels: microseconds,
+    algorithmic GB/s and the fraction of the 8 TB/s HBM peak.
+
+An optional argument lists the token counts to run, e.g. 128,2048.
 
 Weights rotate over several distinct matrices so that they come from HBM, not from cache.
 Prints one JSON object.  Run on the GPU box: python cuda-kernel-qwen3-8b-awq_amd/bench_w4a16.py
@@ -21,6 +23,9 @@ sys.path.insert(0, ROOT)
 
 
 def main():
+    tokens = (1, 4, 16, 64, 128, 512, 2048)
+    if len(sys.argv) > 1:
+        tokens = tuple(int(v) for v in sys.argv[1].split(","))
     import numpy as np
     import torch
     awq = importlib.import_module("cuda-kernel-qwen3-8b-awq_amd")
@@ -46,7 +51,7 @@ def main():
         d_s, d_z = torch.from_numpy(sc).cuda(), torch.from_numpy(zp).cuda()
         ws = torch.zeros(lib.awq_gemv_workspace_bytes(m, k), dtype=torch.uint8, device="cuda")
         res = {}
-        for M in (1, 4, 16, 64, 2048):
+        for M in tokens:
             x = torch.randn(M, k, dtype=torch.float16, device="cuda")
             y = torch.empty(M, m, dtype=torch.float16, device="cuda")
 
@@ -58,7 +63,7 @@ def main():
                 else:
                     awq.check(lib.awq_gemm(w.data_ptr(), d_s.data_ptr(), d_z.data_ptr(), m, k, x.data_ptr(),
                                            y.data_ptr(), M, 1, st))
-            iters = 24 if M == 2048 else 120
+            iters = 24 if M >= 512 else 120
             for i in range(n_mat):
                 launch(i)
             torch.cuda.synchronize()

@@ -55,7 +55,11 @@ __device__ __forceinline__ float wave_tree_sum(float v) {
   return v;
 }
 
-template <bool LDS_SCORES, bool LDS_CV>
+// BATCH: blockIdx.y is a prompt token at position L_arg + blockIdx.y with its
+// own query and output rows ([token][head][128]); it attends the positions the
+// prompt loop gives it (Inference.cu:1118 read before or after :1331):
+// max(pos, 1) when use_len_hi is 0, pos + 1 otherwise.
+template <bool LDS_SCORES, bool LDS_CV, bool BATCH>
 __global__ __launch_bounds__(kThreads) void attention_kernel(const half_t* __restrict__ q,
                                                              const half_t* __restrict__ kc,
                                                              const half_t* __restrict__ vc, half_t* __restrict__ ctx,
@@ -66,7 +70,15 @@ __global__ __launch_bounds__(kThreads) void attention_kernel(const half_t* __res
   __shared__ float wmax[kWaves];
   __shared__ float s_lds[LDS_SCORES ? kLdsPositions : 1];
   __shared__ float cv_lds[LDS_CV ? kLdsChunks * AWQ_HEAD_DIM : 1];
-  const int L = dyn ? (use_len_hi ? dyn->len_hi : dyn->len_lo) : L_arg;
+  int L;
+  if (BATCH) {
+    const int pos = L_arg + blockIdx.y;
+    L = use_len_hi ? pos + 1 : (pos > 1 ? pos : 1);
+    q += (int64_t)blockIdx.y * gridDim.x * AWQ_HEAD_DIM;
+    ctx += (int64_t)blockIdx.y * gridDim.x * AWQ_HEAD_DIM;
+  } else {
+    L = dyn ? (use_len_hi ? dyn->len_hi : dyn->len_lo) : L_arg;
+  }
   const int head = blockIdx.x;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int tq = lane >> 4, dl = lane & 15;
@@ -204,15 +216,39 @@ int launch_attention(const half_t* q, const half_t* kc, const half_t* vc, half_t
   const int64_t bound = dyn ? (len_bound > 0 ? len_bound : max_pos) : L;
   const int mc = (int)chunks_for(max_pos);
   if (bound <= kLdsChunks * 64) {
-    hipLaunchKernelGGL((attention_kernel<true, true>), dim3(n_heads), dim3(kThreads), 0, st, q, kc, vc, ctx, max_pos,
+    hipLaunchKernelGGL((attention_kernel<true, true, false>), dim3(n_heads), dim3(kThreads), 0, st, q, kc, vc, ctx, max_pos,
                        (int)L, dyn, use_len_hi, scores, cv, mc);
   } else if (bound <= kLdsPositions) {
-    hipLaunchKernelGGL((attention_kernel<true, false>), dim3(n_heads), dim3(kThreads), 0, st, q, kc, vc, ctx, max_pos,
+    hipLaunchKernelGGL((attention_kernel<true, false, false>), dim3(n_heads), dim3(kThreads), 0, st, q, kc, vc, ctx, max_pos,
                        (int)L, dyn, use_len_hi, scores, cv, mc);
   } else {
-    hipLaunchKernelGGL((attention_kernel<false, false>), dim3(n_heads), dim3(kThreads), 0, st, q, kc, vc, ctx,
+    hipLaunchKernelGGL((attention_kernel<false, false, false>), dim3(n_heads), dim3(kThreads), 0, st, q, kc, vc, ctx,
                        max_pos, (int)L, dyn, use_len_hi, scores, cv, mc);
   }
   AWQ_HIP_TRY(hipGetLastError());
+  return AWQ_OK;
+}
+
+// Attention of M consecutive prompt positions pos0 .. pos0+M-1, whose keys and
+// values are already in the cache.  While the longest attended length fits the
+// LDS variant all tokens go in one launch; beyond that, one launch per token.
+int launch_attention_batch(const half_t* q, const half_t* kc, const half_t* vc, half_t* ctx, int n_heads,
+                           int64_t max_pos, int64_t pos0, int64_t M, int use_len_hi, void* ws, hipStream_t st) {
+  AWQ_REQUIRE(n_heads > 0 && max_pos > 0 && max_pos <= (int64_t)kMaxChunks * 64, "max_pos must be in 1..65536");
+  AWQ_REQUIRE(M >= 1 && M <= 65535 && pos0 >= 0 && pos0 + M <= max_pos, "positions out of range");
+  AWQ_REQUIRE(ws != nullptr, "workspace required");
+  if (pos0 + M <= kLdsChunks * 64) {
+    hipLaunchKernelGGL((attention_kernel<true, true, true>), dim3(n_heads, (unsigned)M), dim3(kThreads), 0, st, q, kc,
+                       vc, ctx, max_pos, (int)pos0, nullptr, use_len_hi, nullptr, nullptr, 0);
+    AWQ_HIP_TRY(hipGetLastError());
+    return AWQ_OK;
+  }
+  const int64_t H = (int64_t)n_heads * AWQ_HEAD_DIM;
+  for (int64_t t = 0; t < M; ++t) {
+    const int64_t pos = pos0 + t;
+    const int64_t L = use_len_hi ? pos + 1 : (pos > 1 ? pos : 1);
+    if (int rc = launch_attention(q + t * H, kc, vc, ctx + t * H, n_heads, max_pos, L, nullptr, 0, 0, ws, st))
+      return rc;
+  }
   return AWQ_OK;
 }

@@ -11,6 +11,7 @@
 #include <string.h>
 #include <sys/stat.h>
 
+#include <algorithm>
 #include <memory>
 
 static thread_local std::string g_last_error;
@@ -158,6 +159,14 @@ struct awq_engine {
   bool finalized = false;
   bool graph_mode = true;
   hipGraphExec_t graphs[2][3] = {{nullptr, nullptr, nullptr}, {nullptr, nullptr, nullptr}};  // [prompt|gen][length bound]
+  // activations of the batched prompt pass, [chunk][n] each; allocated at first use
+  struct {
+    half_t *hidden = nullptr, *norm = nullptr, *qkv = nullptr, *q = nullptr, *ctx = nullptr, *mid = nullptr,
+           *tmp = nullptr;
+    int32_t* tokens = nullptr;
+    int64_t chunk = 0;
+  } pb;
+  bool batched_prefill = false;
   std::vector<void*> allocations;
 };
 
@@ -578,6 +587,98 @@ extern "C" int awq_prefill(awq_engine* e, const int32_t* prompt_ids, int32_t n_p
   return AWQ_OK;
 }
 
+namespace {
+
+constexpr int64_t kPrefillChunk = 1024;  // prompt positions per batched pass
+
+int ensure_prefill_buffers(awq_engine* e) {
+  if (e->pb.chunk) return AWQ_OK;
+  const int64_t C = std::min<int64_t>(kPrefillChunk, e->cfg.max_pos), H = e->cfg.hidden, I = e->cfg.inter;
+  if (int rc = dev_alloc(e, (void**)&e->pb.hidden, C * H * 2)) return rc;
+  if (int rc = dev_alloc(e, (void**)&e->pb.norm, C * H * 2)) return rc;
+  if (int rc = dev_alloc(e, (void**)&e->pb.qkv, C * 3 * H * 2)) return rc;
+  if (int rc = dev_alloc(e, (void**)&e->pb.q, C * H * 2)) return rc;
+  if (int rc = dev_alloc(e, (void**)&e->pb.ctx, C * H * 2)) return rc;
+  if (int rc = dev_alloc(e, (void**)&e->pb.mid, C * I * 2)) return rc;
+  if (int rc = dev_alloc(e, (void**)&e->pb.tmp, C * H * 2)) return rc;
+  if (int rc = dev_alloc(e, (void**)&e->pb.tokens, C * 4)) return rc;
+  e->pb.chunk = C;
+  return AWQ_OK;
+}
+
+int gemm_of(awq_engine* e, const DevLinear& t, const half_t* x, half_t* y, int64_t M) {
+  return launch_gemm(t.stream_order, t.scale, t.zp, t.m, t.k, x, y, M, t.zp_integral, e->stream);
+}
+
+// runOneLayer, Inference.cu:1029-1230, for M prompt positions pos0.. at once.
+// Layer 0 reads current_seq_len_ before the prompt loop updates it (:1118, :1331).
+int enqueue_layer_batch(awq_engine* e, int l, int64_t pos0, int64_t M) {
+  LayerDev& L = e->layers[l];
+  hipStream_t st = e->stream;
+  const int64_t H = e->cfg.hidden, I = e->cfg.inter;
+  auto& b = e->pb;
+  if (int rc = launch_rmsnorm_batch(b.hidden, L.gamma, b.norm, H, M, e->cfg.eps, st)) return rc;  // :1040
+  if (int rc = gemm_of(e, L.wqkv, b.norm, b.qkv, M)) return rc;                                    // :1052
+  if (int rc = launch_rope_kv_append_batch(b.qkv, e->cos_t, e->sin_t, b.q, L.kcache, L.vcache, e->n_heads,
+                                           e->cfg.max_pos, pos0, M, st))
+    return rc;  // :1070-1103
+  if (int rc = launch_attention_batch(b.q, L.kcache, L.vcache, b.ctx, e->n_heads, e->cfg.max_pos, pos0, M, l >= 1,
+                                      e->attn_ws, st))
+    return rc;                                                         // :1110
+  if (int rc = gemm_of(e, L.wo, b.ctx, b.tmp, M)) return rc;           // :1128
+  if (int rc = launch_residual(b.hidden, b.tmp, b.hidden, M * H, st)) return rc;  // :1149
+  if (int rc = launch_rmsnorm_batch(b.hidden, L.gamma, b.norm, H, M, e->cfg.eps, st)) return rc;  // :1163
+  if (int rc = gemm_of(e, L.w1, b.norm, b.mid, M)) return rc;          // :1176
+  if (int rc = launch_gelu(b.mid, M * I, st)) return rc;               // :1196
+  if (int rc = gemm_of(e, L.w2, b.mid, b.tmp, M)) return rc;           // :1201
+  return launch_residual(b.hidden, b.tmp, b.hidden, M * H, st);        // :1221
+}
+
+}  // namespace
+
+// The prompt loop (Inference.cu:1304-1343) with all prompt positions of a chunk
+// going through each layer together: the weights are read once per chunk and
+// the products run on the matrix cores.  Every token still sees exactly the
+// positions the sequential loop shows it.  The products are summed in another
+// order than the one-token kernel's, so the cache it leaves agrees with
+// awq_prefill's to binary16 rounding noise, not bit for bit.
+extern "C" int awq_prefill_batched(awq_engine* e, const int32_t* prompt_ids, int32_t n_prompt) {
+  AWQ_REQUIRE(e != nullptr && n_prompt >= 0 && (n_prompt == 0 || prompt_ids), "bad arguments");
+  if (!e->finalized) {
+    awq_set_error("awq_prefill_batched before awq_finalize");
+    return AWQ_ERR_STATE;
+  }
+  AWQ_REQUIRE(e->n_generated == 0, "prompt tokens cannot follow generated ones; call awq_reset");
+  AWQ_REQUIRE((int64_t)e->n_positions + n_prompt <= e->cfg.max_pos, "prompt does not fit max_pos");
+  for (int32_t i = 0; i < n_prompt; ++i)
+    AWQ_REQUIRE(prompt_ids[i] >= 0 && prompt_ids[i] < e->cfg.vocab, "token id out of range");
+  if (n_prompt == 0) return AWQ_OK;
+  if (int rc = ensure_prefill_buffers(e)) return rc;
+  const int64_t H = e->cfg.hidden;
+  for (int64_t off = 0; off < n_prompt; off += e->pb.chunk) {
+    const int64_t M = std::min<int64_t>(e->pb.chunk, n_prompt - off), pos0 = e->n_positions;
+    AWQ_HIP_TRY(hipMemcpyAsync(e->pb.tokens, prompt_ids + off, (size_t)M * 4, hipMemcpyHostToDevice, e->stream));
+    if (int rc = launch_embed_batch(e->embed.packed, e->embed.scale, e->embed.zp, H, e->cfg.vocab, e->pb.tokens, M,
+                                    e->pb.hidden, e->stream))
+      return rc;
+    for (int l = 0; l < e->cfg.n_layers; ++l)
+      if (int rc = enqueue_layer_batch(e, l, pos0, M)) return rc;
+    // the state the generation loop starts from (:1357): the last position's output
+    AWQ_HIP_TRY(hipMemcpyAsync(e->hidden, e->pb.hidden + (M - 1) * H, (size_t)H * 2, hipMemcpyDeviceToDevice,
+                               e->stream));
+    AWQ_HIP_TRY(hipStreamSynchronize(e->stream));  // the token ids were read from the caller's buffer
+    e->current_seq_len = (int)(pos0 + M - 1);
+    e->n_positions = (int)(pos0 + M);
+  }
+  return AWQ_OK;
+}
+
+extern "C" int awq_set_prefill_mode(awq_engine* e, int batched) {
+  AWQ_REQUIRE(e != nullptr, "engine is NULL");
+  e->batched_prefill = batched != 0;
+  return AWQ_OK;
+}
+
 // generation loop, Inference.cu:1352-1405
 extern "C" int awq_decode(awq_engine* e, int32_t n_steps, int32_t* out_ids) {
   AWQ_REQUIRE(e != nullptr && n_steps >= 0 && (n_steps == 0 || out_ids), "bad arguments");
@@ -615,7 +716,8 @@ extern "C" int awq_generate(awq_engine* e, const int32_t* prompt_ids, int32_t n_
   AWQ_REQUIRE(n_prompt >= 0 && max_new_tokens >= 0, "negative count");
   AWQ_REQUIRE((int64_t)n_prompt + max_new_tokens <= e->cfg.max_pos, "prompt + new tokens exceed max_pos");
   if (int rc = awq_reset(e)) return rc;
-  if (int rc = awq_prefill(e, prompt_ids, n_prompt)) return rc;
+  if (int rc = e->batched_prefill ? awq_prefill_batched(e, prompt_ids, n_prompt) : awq_prefill(e, prompt_ids, n_prompt))
+    return rc;
   return awq_decode(e, max_new_tokens, out_ids);
 }
 

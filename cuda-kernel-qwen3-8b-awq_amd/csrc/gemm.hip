@@ -4,19 +4,17 @@
 // Inference.cu:1052-1065) applied to the same column-major reading of the
 // dequantised weights.  The weights stay packed int4 in memory and are turned
 // into binary16 in registers, bit-exactly as Inference.cu:102-104 rounds them;
-// the contraction runs on the matrix cores (v_mfma_f32_16x16x32_f16) with FP32
-// accumulation, so results agree with a sequential FP32 sum to rounding noise,
-// not bit for bit.
+// the contraction runs on the matrix cores with FP32 accumulation, so results
+// agree with a sequential FP32 sum to rounding noise, not bit for bit.
 //
-// Same weight stream as the decode kernel: [16-row group][32-wide block][row][16 B].
-// Lane l of a wavefront takes dword l/16 of row l%16 of a block: its 8 nibbles are
-// elements 8*(l/16)..+7 of that row, which is exactly the per-lane operand shape
-// of the 16x16x32 instruction (index l%16, 8 consecutive k at 8*(l/16)).  The
-// tokens ride in the other operand, read from an LDS tile [token][32 k].
-//
-// Workgroup tile: 128 weight rows x TN tokens, 4 wavefronts x 2 row groups each;
-// a wavefront reuses every token operand for its two row groups.
+// Same weight stream as the decode kernel: [16-row group][32-wide block][row][16 B],
+// dword c of a row holding elements 8c..8c+7 of the block.  Two kernels:
+//   few tokens   the decode kernel's decomposition, products on v_mfma_f32_16x16x32_f16
+//   many tokens  64 rows x 128 tokens per wavefront on v_mfma_f32_32x32x16_f16,
+//                tokens staged through LDS
 #include "common.hpp"
+
+#include <type_traits>
 
 namespace {
 
@@ -61,105 +59,6 @@ __device__ __forceinline__ half8_t dequant8(uint32_t v, half_t s, half_t z) {
   }
   const half2_t w0 = u0 * s2, w1 = u1 * s2, w2 = u2 * s2, w3 = u3 * s2;
   return half8_t{w0.x, w0.y, w1.x, w1.y, w2.x, w2.y, w3.x, w3.y};
-}
-
-constexpr int kXStride = 40;  // halves per token row of the LDS tile: 32 + 8 of padding
-
-template <int TT, bool ZINT>  // TT 16-token tiles per workgroup
-__global__ __launch_bounds__(256) void gemm_kernel(GemmParams p) {
-  constexpr int TN = 16 * TT;
-  __shared__ __attribute__((aligned(16))) half_t xs[2][TN * kXStride];
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int r = lane & 15, kq = lane >> 4;
-  const int rg0 = blockIdx.x * 8 + wave * 2;  // this wavefront's two 16-row groups
-  const int t0 = blockIdx.y * TN;
-
-  // scale group of a row group: (row/128) folded as in Inference.cu:90 (see the decode kernel)
-  half_t sc[2], zz[2];
-#pragma unroll
-  for (int a = 0; a < 2; ++a) {
-    const int gi = (((rg0 + a) >> 3) % p.kg) % p.mg;
-    sc[a] = p.scale[gi];
-    zz[a] = p.zp[gi];
-  }
-
-  // staging of the token tile: thread -> (token, 16-byte piece) pairs
-  constexpr int PIECES = TN * 4;  // 16-byte pieces per k-block
-  constexpr int PPT = (PIECES + 255) / 256;
-  uint4 xr[PPT];
-  auto load_x = [&](int kb) {
-#pragma unroll
-    for (int i = 0; i < PPT; ++i) {
-      const int pc = tid + i * 256;
-      const int tok = pc >> 2, part = pc & 3;
-      xr[i] = make_uint4(0, 0, 0, 0);
-      if (pc < PIECES && t0 + tok < p.M)
-        xr[i] = *reinterpret_cast<const uint4*>(p.x + (int64_t)(t0 + tok) * p.k + kb * 32 + part * 8);
-    }
-  };
-  auto store_x = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < PPT; ++i) {
-      const int pc = tid + i * 256;
-      if (pc < PIECES) *reinterpret_cast<uint4*>(&xs[buf][(pc >> 2) * kXStride + (pc & 3) * 8]) = xr[i];
-    }
-  };
-
-  const uint32_t* wp[2];
-#pragma unroll
-  for (int a = 0; a < 2; ++a) wp[a] = p.wq + ((int64_t)(rg0 + a) * p.nblk * 16 + r) * 4 + kq;
-  constexpr int PF = 4;  // weight dwords in flight per row group
-  uint32_t wd[2][PF];
-#pragma unroll
-  for (int f = 0; f < PF; ++f)
-#pragma unroll
-    for (int a = 0; a < 2; ++a) wd[a][f] = f < p.nblk ? wp[a][(int64_t)f * 64] : 0u;
-
-  float4_t acc[2][TT];
-#pragma unroll
-  for (int a = 0; a < 2; ++a)
-#pragma unroll
-    for (int t = 0; t < TT; ++t) acc[a][t] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
-
-  load_x(0);
-  store_x(0);
-  for (int kb0 = 0; kb0 < p.nblk; kb0 += PF) {
-#pragma unroll
-    for (int f = 0; f < PF; ++f) {
-      const int kb = kb0 + f;
-      if (kb >= p.nblk) break;
-      if (kb + 1 < p.nblk) load_x(kb + 1);
-      __syncthreads();  // tile kb is in xs[kb & 1]; tile kb-1's readers are done
-      half8_t wop[2];
-#pragma unroll
-      for (int a = 0; a < 2; ++a) {
-        wop[a] = dequant8<ZINT>(wd[a][f], sc[a], zz[a]);
-        wd[a][f] = kb + PF < p.nblk ? wp[a][(int64_t)(kb + PF) * 64] : 0u;
-      }
-      const half_t* xb = &xs[kb & 1][0];
-#pragma unroll
-      for (int t = 0; t < TT; ++t) {
-        const half8_t xop = *reinterpret_cast<const half8_t*>(xb + (t * 16 + r) * kXStride + kq * 8);
-#pragma unroll
-        for (int a = 0; a < 2; ++a) acc[a][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xop, wop[a], acc[a][t], 0, 0, 0);
-      }
-      if (kb + 1 < p.nblk) store_x((kb + 1) & 1);
-    }
-  }
-  // D[token 4*(lane/16)+i][row lane%16]
-#pragma unroll
-  for (int a = 0; a < 2; ++a) {
-    const int row = (rg0 + a) * 16 + r;
-#pragma unroll
-    for (int t = 0; t < TT; ++t) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int tok = t0 + t * 16 + kq * 4 + i;
-        if (tok < p.M) p.y[(int64_t)tok * p.m + row] = (half_t)acc[a][t][i];
-      }
-    }
-  }
 }
 
 // Few tokens (batched decode): the work is streaming the weights once, so the
@@ -221,16 +120,217 @@ __global__ __launch_bounds__(1024) void gemm_small_kernel(GemmParams p, int n_wa
   }
 }
 
+// Many tokens: a wavefront owns 64 weight rows x 128 tokens as 2 x 4 accumulator
+// tiles of v_mfma_f32_32x32x16_f16 (twice the rate of the 16x16x32 shape on this
+// device).  Every token operand read from LDS feeds two products and every
+// dequantised weight operand four.  Operand shapes: lane (n, kh) = (lane % 32,
+// lane / 32) supplies 8 consecutive k of token / weight row n; a 32-wide block
+// of k goes through two instructions, slice j taking dwords j (kh = 0) and
+// j + 2 (kh = 1) of each row's 16 bytes, so that a lane's two weight dwords
+// (2kh, 2kh + 1) are adjacent in the weight stream.
+// Two workgroup shapes:
+//   rows split (KSPLIT = false): 4 wavefronts x 64 rows = 256 rows, one shared
+//     token tile per step; for products with many tiles.
+//   k split (KSPLIT = true): the 4 wavefronts share 64 rows and take a quarter
+//     of k each (a token tile of their own per step), partial sums meet in LDS;
+//     four times as many workgroups for products with few tiles.
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t xvec_t __attribute__((ext_vector_type(4)));  // 16 bytes of tokens in flight
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+constexpr int kWideRP = 2;                              // 32-row pairs of row groups per wavefront
+constexpr int kWideTT = 4;                              // 32-token tiles per wavefront
+constexpr int kWideTokens = 32 * kWideTT;               // 128
+constexpr int kWideNH = 2;                              // 32-wide blocks of k per step
+constexpr int kWideStride = 32 * kWideNH + 8;           // halves per token row of a tile in LDS (16 bytes of padding)
+constexpr int kWideSlot = kWideTokens * kWideStride;    // halves per token tile in LDS
+constexpr int kWideLdsRows = 2 * kWideSlot * 2;                          // bytes, rows split
+constexpr int kWideLdsK = 4 * kWideRP * kWideTT * 64 * 16 * 4;           // bytes, k split: the partial sums
+
+template <bool ZINT, bool KSPLIT>
+__global__ __launch_bounds__(256, 1) void gemm_wide_kernel(GemmParams p) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  half_t* xs = reinterpret_cast<half_t*>(smem_raw);  // [2][NKB][128 tokens][kWideStride]
+  constexpr int NKB = KSPLIT ? 4 : 1;
+  constexpr int NH = kWideNH;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 31, kh = lane >> 5;
+  const int rg0 = KSPLIT ? blockIdx.x * 4 : (blockIdx.x * 4 + wave) * 4;  // first of this wavefront's 4 row groups
+  const bool rows_ok = rg0 * 16 < p.m;  // rows split: the last workgroup may hang over the edge
+  const int t0 = blockIdx.y * kWideTokens;
+  // a step is NH blocks of k; the step count is even (checked by the launcher)
+  const int steps = (KSPLIT ? p.nblk / 4 : p.nblk) / NH;
+  const int kb_base = KSPLIT ? wave * steps * NH : 0;
+  const int slot = KSPLIT ? wave : 0;
+
+  // the 64 rows share one scale group (rg0 is a multiple of 4, a group is 8 row groups)
+  const int gi = rows_ok ? ((rg0 >> 3) % p.kg) % p.mg : 0;
+  const half_t sc = p.scale[gi], zz = p.zp[gi];
+
+  // Token tile staging: piece = (slot, token, 16 bytes).  Two tiles are on their
+  // way in registers while a third is multiplied: a tile is requested two steps
+  // before its use and written to LDS one step before.  The main loop has no
+  // conditionals: loads past the end repeat the last tile (never used), tokens
+  // past M repeat token M-1 (never stored).
+  constexpr int PCS = kWideTokens * 4 * NH;  // pieces per slot
+  constexpr int PPT = NKB * PCS / 256;
+  const half_t* xsrc[PPT];
+  int xdst[PPT];
+#pragma unroll
+  for (int i = 0; i < PPT; ++i) {
+    const int pc = tid + i * 256;
+    const int j = pc / PCS, tok = (pc % PCS) / (4 * NH), part = pc % (4 * NH);
+    const int tg = t0 + tok < p.M ? t0 + tok : p.M - 1;
+    xsrc[i] = p.x + (int64_t)tg * p.k + (KSPLIT ? j * steps * NH : 0) * 32 + part * 8;
+    xdst[i] = j * kWideSlot + tok * kWideStride + part * 8;
+  }
+  xvec_t xr0[PPT], xr1[PPT];  // two named register sets (an indexed array would live in scratch memory)
+  auto load_x = [&](int s, xvec_t (&dst)[PPT]) __attribute__((always_inline)) {
+    const int sc_ = s < steps ? s : steps - 1;
+#pragma unroll
+    for (int i = 0; i < PPT; ++i) dst[i] = *reinterpret_cast<const xvec_t*>(xsrc[i] + sc_ * (32 * NH));
+  };
+  auto store_x = [&](int buf, const xvec_t (&src)[PPT]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < PPT; ++i) *reinterpret_cast<xvec_t*>(xs + buf * NKB * kWideSlot + xdst[i]) = src[i];
+  };
+
+  // weights: row n of pair rp is row n % 16 of row group rg0 + 2 rp + n / 16; dwords 2kh, 2kh + 1 of its block
+  const u32x2_t* wp[kWideRP];
+#pragma unroll
+  for (int a = 0; a < kWideRP; ++a) {
+    const int rg = rows_ok ? rg0 + 2 * a + (n >> 4) : 0;
+    wp[a] = reinterpret_cast<const u32x2_t*>(p.wq + (((int64_t)rg * p.nblk + kb_base) * 16 + (n & 15)) * 4 + 2 * kh);
+  }
+  constexpr int PF = 2;  // steps of weight dwords in flight
+  u32x2_t wd[kWideRP][PF][NH];
+#pragma unroll
+  for (int f = 0; f < PF; ++f)
+#pragma unroll
+    for (int h = 0; h < NH; ++h)
+#pragma unroll
+      for (int a = 0; a < kWideRP; ++a) wd[a][f][h] = __builtin_nontemporal_load(wp[a] + (int64_t)(f * NH + h) * 32);
+
+  f32x16_t acc[kWideRP][kWideTT];
+#pragma unroll
+  for (int a = 0; a < kWideRP; ++a)
+#pragma unroll
+    for (int t = 0; t < kWideTT; ++t)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[a][t][i] = 0.0f;
+
+  load_x(0, xr0);
+  store_x(0, xr0);
+  load_x(1, xr1);
+  // one step; F is its index inside the unrolled pair (a compile-time constant)
+  auto step = [&](int s0, auto F) __attribute__((always_inline)) {
+    constexpr int f = decltype(F)::value;
+    const int s = s0 + f;
+    // tile s left these registers one step ago
+    if constexpr (f & 1) load_x(s + 2, xr1);
+    else load_x(s + 2, xr0);
+    __syncthreads();  // tile s is in buffer s & 1; the readers of tile s-1 are done
+    const half_t* xb = xs + ((s & 1) * NKB + slot) * kWideSlot + n * kWideStride + 16 * kh;
+    const int sn = s + PF < steps ? s + PF : steps - 1;
+#pragma unroll
+    for (int h = 0; h < NH; ++h) {
+      half8_t wop[kWideRP][2];
+#pragma unroll
+      for (int a = 0; a < kWideRP; ++a) {
+        wop[a][0] = dequant8<ZINT>(wd[a][f][h].x, sc, zz);
+        wop[a][1] = dequant8<ZINT>(wd[a][f][h].y, sc, zz);
+        wd[a][f][h] = __builtin_nontemporal_load(wp[a] + (int64_t)(sn * NH + h) * 32);
+      }
+#pragma unroll
+      for (int t = 0; t < kWideTT; ++t) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          // slice j: k = 8 (j + 2 kh) .. + 7 of block h
+          const half8_t xop = *reinterpret_cast<const half8_t*>(xb + t * 32 * kWideStride + h * 32 + 8 * j);
+#pragma unroll
+          for (int a = 0; a < kWideRP; ++a)
+            acc[a][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xop, wop[a][j], acc[a][t], 0, 0, 0);
+        }
+      }
+    }
+    if constexpr (f & 1) store_x((s + 1) & 1, xr0);
+    else store_x((s + 1) & 1, xr1);
+  };
+  for (int s0 = 0; s0 < steps; s0 += 2) {
+    step(s0, std::integral_constant<int, 0>{});
+    step(s0, std::integral_constant<int, 1>{});
+  }
+
+  // acc[a][t][i] is D[token 32 t + 8 (i / 4) + 4 kh + i % 4][row 32 a + n]
+  if (!KSPLIT) {
+    if (!rows_ok) return;
+#pragma unroll
+    for (int a = 0; a < kWideRP; ++a) {
+      const int row = rg0 * 16 + a * 32 + n;
+#pragma unroll
+      for (int t = 0; t < kWideTT; ++t) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int tok = t0 + t * 32 + (i >> 2) * 8 + kh * 4 + (i & 3);
+          if (tok < p.M) p.y[(int64_t)tok * p.m + row] = (half_t)acc[a][t][i];
+        }
+      }
+    }
+    return;
+  }
+  // k split: the four partial sums of every output meet in LDS (the token tiles
+  // are dead by now); wavefront w finishes token tile w
+  float4_t* red = reinterpret_cast<float4_t*>(smem_raw);  // [wave][pair][tile][quarter][lane]
+  __syncthreads();
+#pragma unroll
+  for (int a = 0; a < kWideRP; ++a)
+#pragma unroll
+    for (int t = 0; t < kWideTT; ++t)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4)
+        red[(((wave * kWideRP + a) * kWideTT + t) * 4 + i4) * 64 + lane] =
+            float4_t{acc[a][t][4 * i4], acc[a][t][4 * i4 + 1], acc[a][t][4 * i4 + 2], acc[a][t][4 * i4 + 3]};
+  __syncthreads();
+#pragma unroll
+  for (int a = 0; a < kWideRP; ++a) {
+    const int row = rg0 * 16 + a * 32 + n;
+    const int t = wave;
+#pragma unroll
+    for (int i4 = 0; i4 < 4; ++i4) {
+      float4_t v = red[(((0 * kWideRP + a) * kWideTT + t) * 4 + i4) * 64 + lane];
+#pragma unroll
+      for (int w = 1; w < 4; ++w) v += red[(((w * kWideRP + a) * kWideTT + t) * 4 + i4) * 64 + lane];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int tok = t0 + t * 32 + i4 * 8 + kh * 4 + i;
+        if (tok < p.M) p.y[(int64_t)tok * p.m + row] = (half_t)v[i];
+      }
+    }
+  }
+}
+
+template <bool KSPLIT>
+int launch_wide(const GemmParams& p, bool zint, hipStream_t st) {
+  // the main loop takes two steps of two 32-wide blocks per trip (per quarter of k when k is split)
+  AWQ_REQUIRE(p.nblk % (KSPLIT ? 16 : 4) == 0, "k must be a multiple of 512");
+  const int lds = KSPLIT ? (kWideLdsK > 4 * kWideLdsRows ? kWideLdsK : 4 * kWideLdsRows) : kWideLdsRows;
+  static_assert(4 * kWideLdsRows <= 160 * 1024 && kWideLdsK <= 160 * 1024, "LDS of one compute unit");
+  const unsigned gx = KSPLIT ? (unsigned)(p.m / 64) : (unsigned)((p.m + 255) / 256);
+  dim3 grid(gx, (unsigned)((p.M + kWideTokens - 1) / kWideTokens));
+  auto kern = zint ? gemm_wide_kernel<true, KSPLIT> : gemm_wide_kernel<false, KSPLIT>;
+  if (lds > 65536) {
+    // more LDS than a launch gets by default: raise this kernel's limit (per device; cheap, so every time)
+    AWQ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+  }
+  hipLaunchKernelGGL(kern, grid, dim3(256), lds, st, p);
+  return AWQ_OK;
+}
+
 template <int G, int TT>
 void launch_small(const GemmParams& p, bool zint, int n_waves, dim3 grid, hipStream_t st) {
   if (zint) hipLaunchKernelGGL((gemm_small_kernel<G, TT, true>), grid, dim3(n_waves * 64), 0, st, p, n_waves);
   else hipLaunchKernelGGL((gemm_small_kernel<G, TT, false>), grid, dim3(n_waves * 64), 0, st, p, n_waves);
-}
-
-template <int TT>
-void launch_tt(const GemmParams& p, bool zint, dim3 grid, hipStream_t st) {
-  if (zint) hipLaunchKernelGGL((gemm_kernel<TT, true>), grid, dim3(256), 0, st, p);
-  else hipLaunchKernelGGL((gemm_kernel<TT, false>), grid, dim3(256), 0, st, p);
 }
 
 }  // namespace
@@ -253,32 +353,35 @@ int launch_gemm(const void* wq, const half_t* scale, const half_t* zp, int64_t m
   p.nblk = (int32_t)(k / AWQ_BLOCK_K);
   p.mg = (int32_t)(m / 128);
   p.kg = (int32_t)(k / 128);
-  if (M <= 64) {
+  // up to 16 tokens, and up to 32 on a matrix with few rows: the decode kernel's decomposition
+  int g = 0;
+  if (M <= 16 || (M <= 32 && m < 8192)) {
     // lane groups of G blocks: (k/32)/G of them, a multiple of 4 and at most 64
     const int64_t nblk = k / AWQ_BLOCK_K;
-    int g = 0;
     for (int c : {8, 4, 2, 1})
       if (nblk % c == 0 && (nblk / c) % 4 == 0 && nblk / c <= 64) {
         g = c;
         break;
       }
-    // 17..64 tokens on a matrix with many rows: the tiled kernel reads X less often
-    if (M > 16 && m >= 8192) g = 0;
-    if (g) {
-      const int n_waves = (int)(nblk / g / 4);
-      const bool one = M <= 16;
-      dim3 grid((unsigned)(m / 16), (unsigned)((M + (one ? 15 : 63)) / (one ? 16 : 64)));
-      switch (g) {
-        case 8: one ? launch_small<8, 1>(p, zp_integral, n_waves, grid, st) : launch_small<8, 4>(p, zp_integral, n_waves, grid, st); break;
-        case 4: one ? launch_small<4, 1>(p, zp_integral, n_waves, grid, st) : launch_small<4, 4>(p, zp_integral, n_waves, grid, st); break;
-        case 2: one ? launch_small<2, 1>(p, zp_integral, n_waves, grid, st) : launch_small<2, 4>(p, zp_integral, n_waves, grid, st); break;
-        default: one ? launch_small<1, 1>(p, zp_integral, n_waves, grid, st) : launch_small<1, 4>(p, zp_integral, n_waves, grid, st); break;
-      }
-    } else {
-      launch_tt<4>(p, zp_integral, dim3((unsigned)(m / 128), (unsigned)((M + 63) / 64)), st);
+  }
+  if (g) {
+    const int n_waves = (int)(k / AWQ_BLOCK_K / g / 4);
+    const bool one = M <= 16;
+    dim3 grid((unsigned)(m / 16), (unsigned)((M + (one ? 15 : 63)) / (one ? 16 : 64)));
+    switch (g) {
+      case 8: one ? launch_small<8, 1>(p, zp_integral, n_waves, grid, st) : launch_small<8, 4>(p, zp_integral, n_waves, grid, st); break;
+      case 4: one ? launch_small<4, 1>(p, zp_integral, n_waves, grid, st) : launch_small<4, 4>(p, zp_integral, n_waves, grid, st); break;
+      case 2: one ? launch_small<2, 1>(p, zp_integral, n_waves, grid, st) : launch_small<2, 4>(p, zp_integral, n_waves, grid, st); break;
+      default: one ? launch_small<1, 1>(p, zp_integral, n_waves, grid, st) : launch_small<1, 4>(p, zp_integral, n_waves, grid, st); break;
     }
   } else {
-    launch_tt<8>(p, zp_integral, dim3((unsigned)(m / 128), (unsigned)((M + 127) / 128)), st);
+    // enough 256-row x 128-token tiles to fill half the device: rows split; otherwise k split
+    const int64_t tiles = ((m + 255) / 256) * ((M + kWideTokens - 1) / kWideTokens);
+    if (tiles >= 128) {
+      if (int rc = launch_wide<false>(p, zp_integral, st)) return rc;
+    } else {
+      if (int rc = launch_wide<true>(p, zp_integral, st)) return rc;
+    }
   }
   AWQ_HIP_TRY(hipGetLastError());
   return AWQ_OK;

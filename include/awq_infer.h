@@ -78,6 +78,18 @@ int awq_reset(awq_engine* e);
 int awq_prefill(awq_engine* e, const int32_t* prompt_ids, int32_t n_prompt);
 int awq_decode(awq_engine* e, int32_t n_steps, int32_t* out_ids);
 
+/* The prompt loop (Inference.cu:1304-1343) for all prompt positions together:
+ * per layer one W4A16 matrix product over the prompt instead of one
+ * matrix-vector product per token (the reference streams every weight once per
+ * prompt token, Inference.cu:1326-1332).  Each token attends exactly the
+ * positions the sequential loop gives it.  Leaves the same state as awq_prefill
+ * up to rounding: the products are summed in a different order, so K/V and the
+ * hidden state agree to binary16 rounding noise, not bit for bit.
+ * awq_set_prefill_mode(e, 1) makes awq_generate use it; the default (0) is the
+ * token-by-token loop. */
+int awq_prefill_batched(awq_engine* e, const int32_t* prompt_ids, int32_t n_prompt);
+int awq_set_prefill_mode(awq_engine* e, int batched);
+
 /* Copies of internal state for tests: hidden state [hidden] and the logits of
  * the last sampled position [vocab], both FP16, to host memory. */
 int awq_read_hidden(awq_engine* e, uint16_t* host_dst);

@@ -440,7 +440,8 @@ def test_gemv_fused_norm_unembed_argmax(awq, lib, oracle, torch_gpu, m, k):
 
 # ----------------------------------------------------------------------------- W4A16 GEMM on the matrix cores
 @pytest.mark.parametrize("m,k,M,zp_int", [(256, 512, 3, True), (256, 512, 17, False), (384, 1536, 130, True),
-                                          (12288, 4096, 16, True), (12288, 4096, 200, True), (4096, 12288, 64, False)])
+                                          (12288, 4096, 16, True), (12288, 4096, 200, True), (4096, 12288, 64, False),
+                                          (4096, 12288, 128, True), (12288, 4096, 1030, True)])
 def test_gemm_matches_fp32_accumulate_reference(awq, lib, oracle, torch_gpu, m, k, M, zp_int):
     """config 5: dequant-on-load MFMA product; 1e-2 relative against the sequential FP32-accumulate
     reference, and the weights it multiplies are the bit-exact dequantised ones (one-hot check below)"""

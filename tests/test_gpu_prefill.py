@@ -1,0 +1,154 @@
+"""Batched prompt pass (all prompt positions through each layer together, products on the matrix
+cores) against the token-by-token prompt loop and the CPU oracle.
+
+The two prompt loops sum the products in different orders, so their states agree to binary16
+rounding noise (tolerance below), not bit for bit; greedy tokens must be identical except where the
+oracle's own top-1/top-2 logit margin is within that noise."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from helpers import fill_pair, make_oracle_model, ptr
+
+pytestmark = pytest.mark.gpu
+
+SMALL = dict(n_layers=4, hidden=512, inter=1536, vocab=1024, max_pos=160)
+REL_TOL = 1e-2      # of the largest magnitude of the vector compared
+MARGIN_TOL = 0.05   # logit units: a flip is only acceptable below this top-1/top-2 margin
+
+
+def as_f32(u16):
+    return np.ctypeslib.as_array(u16).view(np.float16).astype(np.float32)
+
+
+def close(a, b):
+    return np.abs(a - b).max() <= REL_TOL * max(np.abs(a).max(), 1e-6)
+
+
+def check_tokens(got, ref, margins, what):
+    for i, (g, r) in enumerate(zip(got, ref)):
+        if g != r:
+            assert margins[i] < MARGIN_TOL, "%s: token %d differs (%d vs %d) at margin %.4f" % (what, i, g, r, margins[i])
+            return i       # sequences diverge legitimately after a tie-like step
+    return len(ref)
+
+
+def oracle_run(oracle, model, prompt, n_new):
+    p = np.asarray(prompt, dtype=np.int32)
+    out = np.zeros(max(1, n_new), dtype=np.int32)
+    assert oracle.awqo_model_generate(model, ptr(p), p.size, n_new, ptr(out)) == n_new
+    margins = np.zeros(max(1, n_new), dtype=np.float32)
+    oracle.awqo_model_margins(model, ptr(margins), n_new)
+    return out[:n_new].tolist(), margins
+
+
+@pytest.mark.parametrize("n_prompt", [1, 2, 5, 37, 100])
+def test_small_model_batched_prompt_matches_sequential(awq, oracle, torch_gpu, n_prompt):
+    cfg = awq.make_config(**SMALL)
+    model = make_oracle_model(oracle, cfg)
+    eng = awq.QWen3AWQInfer.empty(cfg)
+    fill_pair(awq, oracle, cfg, 77, engine=eng, model=model, profile=awq.SYNTH_BALANCED)
+    rng = np.random.default_rng(n_prompt)
+    prompt = rng.integers(0, cfg.vocab, n_prompt).tolist()
+    n_new = 16
+    print("batched prompt pass, small model, P =", n_prompt, flush=True)
+
+    eng.reset()
+    eng.prefill(prompt)
+    hid_seq = as_f32(eng.read_hidden()).copy()
+    tok_seq = eng.decode(n_new)
+
+    eng.reset()
+    eng.prefill(prompt, batched=True)
+    hid_bat = as_f32(eng.read_hidden()).copy()
+    tok_bat = eng.decode(n_new)
+
+    assert np.isfinite(hid_seq).all() and np.abs(hid_seq).max() > 0
+    assert close(hid_seq, hid_bat)
+    ref, margins = oracle_run(oracle, model, prompt, n_new)
+    assert tok_seq == ref                      # the sequential loop is bit-exact with the oracle
+    same = check_tokens(tok_bat, ref, margins, "batched")
+    print("identical tokens: %d of %d; min margin %.4f" % (same, n_new, margins.min()), flush=True)
+
+    # generateResponse honours the mode switch
+    eng.set_prefill_mode(True)
+    assert eng.generateResponse(prompt, n_new) == tok_bat
+    eng.set_prefill_mode(False)
+    assert eng.generateResponse(prompt, n_new) == ref
+    eng.close()
+    oracle.awqo_model_destroy(model)
+
+
+def test_batched_prompt_in_pieces_equals_one_call(awq, oracle, torch_gpu):
+    """Positions, attended lengths and cache rows must not depend on how the prompt is cut into
+    calls.  The pieces are long enough (more than 32 tokens) for the same product kernel to serve
+    them and the whole prompt, and that kernel's result for a token does not depend on the other
+    tokens, so the state is bit-identical."""
+    cfg = awq.make_config(**SMALL)
+    model = make_oracle_model(oracle, cfg)   # only as the host buffer of the weights here
+    eng = awq.QWen3AWQInfer.empty(cfg)
+    fill_pair(awq, oracle, cfg, 78, engine=eng, model=model, profile=awq.SYNTH_BALANCED)
+    oracle.awqo_model_destroy(model)
+    rng = np.random.default_rng(5)
+    prompt = rng.integers(0, cfg.vocab, 90).tolist()
+    print("batched prompt pass in pieces", flush=True)
+    eng.reset()
+    eng.prefill(prompt, batched=True)
+    whole = np.ctypeslib.as_array(eng.read_hidden()).copy()
+    tok_whole = eng.decode(8)
+    eng.reset()
+    eng.prefill(prompt[:41], batched=True)
+    eng.prefill(prompt[41:], batched=True)
+    pieces = np.ctypeslib.as_array(eng.read_hidden()).copy()
+    assert np.array_equal(whole, pieces)
+    assert eng.decode(8) == tok_whole
+    # a sequential start followed by a batched rest stays within rounding noise of it
+    eng.reset()
+    eng.prefill(prompt[:7])
+    eng.prefill(prompt[7:], batched=True)
+    mixed = np.ctypeslib.as_array(eng.read_hidden()).copy()
+    assert close(whole.view(np.float16).astype(np.float32), mixed.view(np.float16).astype(np.float32))
+    # error paths: prompt tokens after generated ones, an id outside the vocabulary, overflow of max_pos
+    eng.decode(1)
+    with pytest.raises(awq.AwqError):
+        eng.prefill([1], batched=True)
+    eng.reset()
+    with pytest.raises(awq.AwqError):
+        eng.prefill([cfg.vocab], batched=True)
+    with pytest.raises(awq.AwqError):
+        eng.prefill([1] * (cfg.max_pos + 1), batched=True)
+    eng.prefill([], batched=True)
+    eng.close()
+
+
+def test_full_model_batched_prompt_tokens(awq, oracle, torch_gpu):
+    """36 layers at full width, 128-token prompt: the tokens after a batched prompt pass are the
+    oracle's."""
+    cfg = awq.make_config(max_pos=192)
+    model = make_oracle_model(oracle, cfg)
+    eng = awq.QWen3AWQInfer.empty(cfg)
+    fill_pair(awq, oracle, cfg, 2024, engine=eng, model=model, profile=awq.SYNTH_BALANCED)
+    lib = awq.load_library()
+    prompt = np.zeros(128, dtype=np.int32)
+    awq.check(lib.awq_synth_tokens(2024, awq.SYNTH_STREAM_INPUT, ptr(prompt), prompt.size, cfg.vocab))
+    n_new = 32
+    print("batched prompt pass, full model, P = 128", flush=True)
+    eng.reset()
+    eng.prefill(prompt.tolist(), batched=True)
+    hid_bat = as_f32(eng.read_hidden()).copy()
+    tok_bat = eng.decode(n_new)
+    eng.reset()
+    eng.prefill(prompt.tolist())
+    hid_seq = as_f32(eng.read_hidden()).copy()
+    tok_seq = eng.decode(n_new)
+    print("hidden: max |seq - batched| = %.5f at scale %.3f" % (np.abs(hid_seq - hid_bat).max(), np.abs(hid_seq).max()),
+          flush=True)
+    assert close(hid_seq, hid_bat)
+    ref, margins = oracle_run(oracle, model, prompt.tolist(), n_new)
+    assert tok_seq == ref
+    same = check_tokens(tok_bat, ref, margins, "batched")
+    print("identical tokens: %d of %d; min margin %.4f" % (same, n_new, margins.min()), flush=True)
+    assert same >= n_new // 2
+    eng.close()
+    oracle.awqo_model_destroy(model)
