@@ -54,6 +54,7 @@ def main():
         for M in tokens:
             x = torch.randn(M, k, dtype=torch.float16, device="cuda")
             y = torch.empty(M, m, dtype=torch.float16, device="cuda")
+            gws = torch.zeros(max(16, lib.awq_gemm_workspace_bytes(m, k, M)), dtype=torch.uint8, device="cuda")
 
             def launch(i):
                 w = mats[i % n_mat]
@@ -62,7 +63,7 @@ def main():
                                            y.data_ptr(), 1, ws.data_ptr(), st))
                 else:
                     awq.check(lib.awq_gemm(w.data_ptr(), d_s.data_ptr(), d_z.data_ptr(), m, k, x.data_ptr(),
-                                           y.data_ptr(), M, 1, st))
+                                           y.data_ptr(), M, 1, gws.data_ptr(), st))
             iters = 24 if M >= 512 else 120
             for i in range(n_mat):
                 launch(i)

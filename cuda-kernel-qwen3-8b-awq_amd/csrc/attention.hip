@@ -9,8 +9,8 @@
 // Cache layout [head][max_pos][128] FP16 (Inference.cu:1097): a position is one
 // 256-byte row, so a wavefront load of 16 bytes per lane covers 4 positions.
 //
-// One workgroup of 16 wavefronts per head.  Scores: wavefront w takes the w-th
-// group of 4 positions of every 64-position chunk, so all wavefronts stream
+// One workgroup of NW wavefronts per head (16 for decode).  Scores: the
+// positions go round the wavefronts in groups of 4, so all wavefronts stream
 // keys even for short sequences.  Context: one wavefront per chunk.
 #include "common.hpp"
 
@@ -19,8 +19,8 @@ namespace {
 constexpr int kMaxChunks = 1024;    // 65536 positions
 constexpr int kLdsPositions = 8192; // scores kept in LDS up to this length
 constexpr int kLdsChunks = 32;      // chunk vectors kept in LDS up to this many chunks
-constexpr int kThreads = 1024;
-constexpr int kWaves = kThreads / 64;
+constexpr int kWaves = 16;   // wavefronts per workgroup of the decode variants
+constexpr int kThreads = kWaves * 64;
 
 // v + (value of lane ^ mask) inside a row of 16 lanes.  After the xor-1 and
 // xor-2 steps all four lanes of a quad hold the same sum, so mirroring inside
@@ -59,17 +59,19 @@ __device__ __forceinline__ float wave_tree_sum(float v) {
 // own query and output rows ([token][head][128]); it attends the positions the
 // prompt loop gives it (Inference.cu:1118 read before or after :1331):
 // max(pos, 1) when use_len_hi is 0, pos + 1 otherwise.
-template <bool LDS_SCORES, bool LDS_CV, bool BATCH>
-__global__ __launch_bounds__(kThreads) void attention_kernel(const half_t* __restrict__ q,
+// NW wavefronts; SCAP positions of scores and CCAP chunks (sums, and vectors
+// when LDS_CV) fit the LDS arrays.
+template <bool LDS_SCORES, bool LDS_CV, bool BATCH, int NW, int SCAP, int CCAP>
+__global__ __launch_bounds__(NW * 64) void attention_kernel(const half_t* __restrict__ q,
                                                              const half_t* __restrict__ kc,
                                                              const half_t* __restrict__ vc, half_t* __restrict__ ctx,
                                                              int64_t max_pos, int L_arg, const StepState* dyn,
                                                              int use_len_hi, float* __restrict__ ws_scores,
                                                              float* __restrict__ ws_cv, int max_chunks) {
-  __shared__ float cs[kMaxChunks];
-  __shared__ float wmax[kWaves];
-  __shared__ float s_lds[LDS_SCORES ? kLdsPositions : 1];
-  __shared__ float cv_lds[LDS_CV ? kLdsChunks * AWQ_HEAD_DIM : 1];
+  __shared__ float cs[CCAP];
+  __shared__ float wmax[NW];
+  __shared__ float s_lds[LDS_SCORES ? SCAP : 1];
+  __shared__ float cv_lds[LDS_CV ? CCAP * AWQ_HEAD_DIM : 1];
   int L;
   if (BATCH) {
     const int pos = L_arg + blockIdx.y;
@@ -96,20 +98,21 @@ __global__ __launch_bounds__(kThreads) void attention_kernel(const half_t* __res
     for (int i = 0; i < 8; ++i) qf[i] = (float)qv[i];
   }
 
-  // scores (Inference.cu:202-226) and their maximum (:229-233): this
-  // wavefront's four positions of each chunk, six chunks' loads in flight.
-  // The values of this wavefront's first chunk are requested right behind the
-  // first keys, so that both arrive in one memory round trip.
+  // scores (Inference.cu:202-226) and their maximum (:229-233): groups of four
+  // positions go round the wavefronts, six groups' loads in flight.  The values
+  // of this wavefront's first chunk are requested right behind the first keys,
+  // so that both arrive in one memory round trip.
   half8_t vv[16];
   float lmax = -1e9f;
-  for (int c0 = 0; c0 < nchunks; c0 += 6) {
+  const int nquads = (L + 3) >> 2;
+  for (int q0 = wave; q0 < nquads; q0 += 6 * NW) {
     half8_t kv[6];
 #pragma unroll
     for (int u = 0; u < 6; ++u) {
-      const int t = ((c0 + u) << 6) + 4 * wave + tq;
+      const int t = 4 * (q0 + u * NW) + tq;
       if (t < L) kv[u] = *reinterpret_cast<const half8_t*>(kh + (int64_t)t * AWQ_HEAD_DIM + 8 * dl);
     }
-    if (c0 == 0 && wave < nchunks) {
+    if (q0 == wave && wave < nchunks) {
 #pragma unroll
       for (int nl = 0; nl < 16; ++nl) {
         const int t = (wave << 6) + 4 * nl + tq;
@@ -118,7 +121,7 @@ __global__ __launch_bounds__(kThreads) void attention_kernel(const half_t* __res
     }
 #pragma unroll
     for (int u = 0; u < 6; ++u) {
-      const int t = ((c0 + u) << 6) + 4 * wave + tq;
+      const int t = 4 * (q0 + u * NW) + tq;
       float part = 0.0f;
       if (t < L) {
 #pragma unroll
@@ -138,10 +141,10 @@ __global__ __launch_bounds__(kThreads) void attention_kernel(const half_t* __res
   __syncthreads();
   float mx = wmax[0];
 #pragma unroll
-  for (int w = 1; w < kWaves; ++w) mx = fmaxf(mx, wmax[w]);
+  for (int w = 1; w < NW; ++w) mx = fmaxf(mx, wmax[w]);
 
   // exponentials and their sum (Inference.cu:239-249), one wavefront per chunk
-  for (int chunk = wave; chunk < nchunks; chunk += kWaves) {
+  for (int chunk = wave; chunk < nchunks; chunk += NW) {
     const int t = (chunk << 6) + lane;
     float e = 0.0f;
     if (t < L) {
@@ -157,7 +160,7 @@ __global__ __launch_bounds__(kThreads) void attention_kernel(const half_t* __res
 
   // weighted sum of V (Inference.cu:251-265), one wavefront per chunk; the 16
   // loads of a chunk are issued together
-  for (int chunk = wave; chunk < nchunks; chunk += kWaves) {
+  for (int chunk = wave; chunk < nchunks; chunk += NW) {
     const int base = chunk << 6;
     if (chunk != wave) {  // the first chunk's values were requested at the start
 #pragma unroll
@@ -216,13 +219,16 @@ int launch_attention(const half_t* q, const half_t* kc, const half_t* vc, half_t
   const int64_t bound = dyn ? (len_bound > 0 ? len_bound : max_pos) : L;
   const int mc = (int)chunks_for(max_pos);
   if (bound <= kLdsChunks * 64) {
-    hipLaunchKernelGGL((attention_kernel<true, true, false>), dim3(n_heads), dim3(kThreads), 0, st, q, kc, vc, ctx, max_pos,
+    hipLaunchKernelGGL((attention_kernel<true, true, false, kWaves, kLdsChunks * 64, kLdsChunks>), dim3(n_heads),
+                       dim3(kThreads), 0, st, q, kc, vc, ctx, max_pos,
                        (int)L, dyn, use_len_hi, scores, cv, mc);
   } else if (bound <= kLdsPositions) {
-    hipLaunchKernelGGL((attention_kernel<true, false, false>), dim3(n_heads), dim3(kThreads), 0, st, q, kc, vc, ctx, max_pos,
+    hipLaunchKernelGGL((attention_kernel<true, false, false, kWaves, kLdsPositions, kMaxChunks>), dim3(n_heads),
+                       dim3(kThreads), 0, st, q, kc, vc, ctx, max_pos,
                        (int)L, dyn, use_len_hi, scores, cv, mc);
   } else {
-    hipLaunchKernelGGL((attention_kernel<false, false, false>), dim3(n_heads), dim3(kThreads), 0, st, q, kc, vc, ctx,
+    hipLaunchKernelGGL((attention_kernel<false, false, false, kWaves, 1, kMaxChunks>), dim3(n_heads),
+                       dim3(kThreads), 0, st, q, kc, vc, ctx,
                        max_pos, (int)L, dyn, use_len_hi, scores, cv, mc);
   }
   AWQ_HIP_TRY(hipGetLastError());
@@ -237,9 +243,17 @@ int launch_attention_batch(const half_t* q, const half_t* kc, const half_t* vc, 
   AWQ_REQUIRE(n_heads > 0 && max_pos > 0 && max_pos <= (int64_t)kMaxChunks * 64, "max_pos must be in 1..65536");
   AWQ_REQUIRE(M >= 1 && M <= 65535 && pos0 >= 0 && pos0 + M <= max_pos, "positions out of range");
   AWQ_REQUIRE(ws != nullptr, "workspace required");
+  // short prompts: small workgroups (4 wavefronts, 3 KiB of LDS), many of them per compute unit
+  if (pos0 + M <= 256) {
+    hipLaunchKernelGGL((attention_kernel<true, true, true, 4, 256, 4>), dim3(n_heads, (unsigned)M), dim3(256), 0, st,
+                       q, kc, vc, ctx, max_pos, (int)pos0, nullptr, use_len_hi, nullptr, nullptr, 0);
+    AWQ_HIP_TRY(hipGetLastError());
+    return AWQ_OK;
+  }
   if (pos0 + M <= kLdsChunks * 64) {
-    hipLaunchKernelGGL((attention_kernel<true, true, true>), dim3(n_heads, (unsigned)M), dim3(kThreads), 0, st, q, kc,
-                       vc, ctx, max_pos, (int)pos0, nullptr, use_len_hi, nullptr, nullptr, 0);
+    hipLaunchKernelGGL((attention_kernel<true, true, true, kWaves, kLdsChunks * 64, kLdsChunks>),
+                       dim3(n_heads, (unsigned)M), dim3(kThreads), 0, st, q, kc, vc, ctx, max_pos, (int)pos0, nullptr,
+                       use_len_hi, nullptr, nullptr, 0);
     AWQ_HIP_TRY(hipGetLastError());
     return AWQ_OK;
   }

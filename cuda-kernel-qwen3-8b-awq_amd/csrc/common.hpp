@@ -112,8 +112,10 @@ int launch_dequant(const uint8_t* packed, const half_t* scale, const half_t* zp,
 int launch_repack(const uint8_t* in, void* out, int64_t m, int64_t k, hipStream_t st);
 int64_t gemv_workspace_bytes(int64_t m, int64_t k);
 int launch_gemv(const LinearArgs& a, hipStream_t st);
+int64_t gemm_workspace_bytes(int64_t m, int64_t k, int64_t M);
 int launch_gemm(const void* wq, const half_t* scale, const half_t* zp, int64_t m, int64_t k, const half_t* x,
-                half_t* y, int64_t M, int zp_integral, hipStream_t st);
+                half_t* y, int64_t M, int zp_integral, int epilogue, const half_t* res, void* workspace,
+                int64_t workspace_bytes, hipStream_t st);
 int launch_rmsnorm(const half_t* x, const half_t* gamma, half_t* out, int64_t n, float eps, hipStream_t st);
 int launch_rope_kv_append(const half_t* qkv, const half_t* cos_t, const half_t* sin_t, half_t* q_out, half_t* kc,
                           half_t* vc, int n_heads, int64_t max_pos, int64_t pos, const StepState* dyn, hipStream_t st);

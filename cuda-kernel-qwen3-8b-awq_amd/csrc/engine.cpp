@@ -161,9 +161,9 @@ struct awq_engine {
   hipGraphExec_t graphs[2][3] = {{nullptr, nullptr, nullptr}, {nullptr, nullptr, nullptr}};  // [prompt|gen][length bound]
   // activations of the batched prompt pass, [chunk][n] each; allocated at first use
   struct {
-    half_t *hidden = nullptr, *norm = nullptr, *qkv = nullptr, *q = nullptr, *ctx = nullptr, *mid = nullptr,
-           *tmp = nullptr;
+    half_t *hidden = nullptr, *norm = nullptr, *qkv = nullptr, *q = nullptr, *ctx = nullptr, *mid = nullptr;
     int32_t* tokens = nullptr;
+    void* gemm_ws = nullptr;  // partial sums of products whose k is cut over workgroups
     int64_t chunk = 0;
   } pb;
   bool batched_prefill = false;
@@ -590,6 +590,7 @@ extern "C" int awq_prefill(awq_engine* e, const int32_t* prompt_ids, int32_t n_p
 namespace {
 
 constexpr int64_t kPrefillChunk = 1024;  // prompt positions per batched pass
+constexpr int64_t kGemmWsBytes = 64ll << 20;
 
 int ensure_prefill_buffers(awq_engine* e) {
   if (e->pb.chunk) return AWQ_OK;
@@ -600,14 +601,16 @@ int ensure_prefill_buffers(awq_engine* e) {
   if (int rc = dev_alloc(e, (void**)&e->pb.q, C * H * 2)) return rc;
   if (int rc = dev_alloc(e, (void**)&e->pb.ctx, C * H * 2)) return rc;
   if (int rc = dev_alloc(e, (void**)&e->pb.mid, C * I * 2)) return rc;
-  if (int rc = dev_alloc(e, (void**)&e->pb.tmp, C * H * 2)) return rc;
   if (int rc = dev_alloc(e, (void**)&e->pb.tokens, C * 4)) return rc;
+  if (int rc = dev_alloc(e, &e->pb.gemm_ws, kGemmWsBytes)) return rc;
   e->pb.chunk = C;
   return AWQ_OK;
 }
 
-int gemm_of(awq_engine* e, const DevLinear& t, const half_t* x, half_t* y, int64_t M) {
-  return launch_gemm(t.stream_order, t.scale, t.zp, t.m, t.k, x, y, M, t.zp_integral, e->stream);
+int gemm_of(awq_engine* e, const DevLinear& t, const half_t* x, half_t* y, int64_t M, int epilogue = EPI_STORE,
+            const half_t* res = nullptr) {
+  return launch_gemm(t.stream_order, t.scale, t.zp, t.m, t.k, x, y, M, t.zp_integral, epilogue, res, e->pb.gemm_ws,
+                     kGemmWsBytes, e->stream);
 }
 
 // runOneLayer, Inference.cu:1029-1230, for M prompt positions pos0.. at once.
@@ -615,7 +618,7 @@ int gemm_of(awq_engine* e, const DevLinear& t, const half_t* x, half_t* y, int64
 int enqueue_layer_batch(awq_engine* e, int l, int64_t pos0, int64_t M) {
   LayerDev& L = e->layers[l];
   hipStream_t st = e->stream;
-  const int64_t H = e->cfg.hidden, I = e->cfg.inter;
+  const int64_t H = e->cfg.hidden;
   auto& b = e->pb;
   if (int rc = launch_rmsnorm_batch(b.hidden, L.gamma, b.norm, H, M, e->cfg.eps, st)) return rc;  // :1040
   if (int rc = gemm_of(e, L.wqkv, b.norm, b.qkv, M)) return rc;                                    // :1052
@@ -625,13 +628,11 @@ int enqueue_layer_batch(awq_engine* e, int l, int64_t pos0, int64_t M) {
   if (int rc = launch_attention_batch(b.q, L.kcache, L.vcache, b.ctx, e->n_heads, e->cfg.max_pos, pos0, M, l >= 1,
                                       e->attn_ws, st))
     return rc;                                                         // :1110
-  if (int rc = gemm_of(e, L.wo, b.ctx, b.tmp, M)) return rc;           // :1128
-  if (int rc = launch_residual(b.hidden, b.tmp, b.hidden, M * H, st)) return rc;  // :1149
+  // :1128 Wo product, :1149 residual add in its epilogue
+  if (int rc = gemm_of(e, L.wo, b.ctx, b.hidden, M, EPI_RESIDUAL, b.hidden)) return rc;
   if (int rc = launch_rmsnorm_batch(b.hidden, L.gamma, b.norm, H, M, e->cfg.eps, st)) return rc;  // :1163
-  if (int rc = gemm_of(e, L.w1, b.norm, b.mid, M)) return rc;          // :1176
-  if (int rc = launch_gelu(b.mid, M * I, st)) return rc;               // :1196
-  if (int rc = gemm_of(e, L.w2, b.mid, b.tmp, M)) return rc;           // :1201
-  return launch_residual(b.hidden, b.tmp, b.hidden, M * H, st);        // :1221
+  if (int rc = gemm_of(e, L.w1, b.norm, b.mid, M, EPI_GELU)) return rc;  // :1176, :1196
+  return gemm_of(e, L.w2, b.mid, b.hidden, M, EPI_RESIDUAL, b.hidden);   // :1201, :1221
 }
 
 }  // namespace
@@ -890,8 +891,10 @@ extern "C" int awq_gemv(const void* repacked, const void* scale, const void* zp,
   return awq_gemv_fused(&u, stream);
 }
 
+extern "C" int64_t awq_gemm_workspace_bytes(int64_t m, int64_t k, int64_t M) { return gemm_workspace_bytes(m, k, M); }
+
 extern "C" int awq_gemm(const void* repacked, const void* scale, const void* zp, int64_t m, int64_t k, const void* x,
-                        void* y, int64_t M, int32_t zp_integral, void* stream) {
+                        void* y, int64_t M, int32_t zp_integral, void* workspace, void* stream) {
   AWQ_REQUIRE(repacked && scale && zp && x && y, "NULL pointer");
   AWQ_REQUIRE(m > 0 && m % 128 == 0, "m must be a positive multiple of 128");
   if (zp_integral < 0) {
@@ -901,7 +904,8 @@ extern "C" int awq_gemm(const void* repacked, const void* scale, const void* zp,
     zp_integral = zp_all_integral(zph.data(), (int64_t)zph.size());
   }
   return launch_gemm(repacked, (const half_t*)scale, (const half_t*)zp, m, k, (const half_t*)x, (half_t*)y, M,
-                     zp_integral != 0, (hipStream_t)stream);
+                     zp_integral != 0, EPI_STORE, nullptr, workspace, workspace ? gemm_workspace_bytes(m, k, M) : 0,
+                     (hipStream_t)stream);
 }
 
 extern "C" int awq_rmsnorm(const void* x, const void* gamma, void* out, int64_t n, float eps, void* stream) {

@@ -31,7 +31,31 @@ struct GemmParams {
   int32_t m, k, M;
   int32_t nblk;
   int32_t mg, kg;
+  int32_t epilogue;     // EPI_STORE, EPI_RESIDUAL or EPI_GELU
+  const half_t* res;    // EPI_RESIDUAL: [M][m], may be y itself
+  int32_t kz;           // k is cut into kz chunks over blockIdx.z (k-split workgroups only)
+  float* part;          // kz > 1: FP32 partial sums [kz][M][m], finished by reduce_parts_kernel
 };
+
+// one finished output: the same epilogues as the decode kernel's.  The kind is
+// a template argument so that the fully unrolled output loops stay free of
+// branches (a branch inside them makes the accumulators an indexed array in
+// scratch memory).
+template <int EPI>
+__device__ __forceinline__ void store_out(const GemmParams& p, int tok, int row, float acc) {
+  const int64_t at = (int64_t)tok * p.m + row;
+  const half_t v = (half_t)acc;
+  if (EPI == EPI_RESIDUAL) p.y[at] = p.res[at] + v;                          // Inference.cu:1149-1155
+  else if (EPI == EPI_GELU) p.y[at] = to_half_rn(awq_gelu_f32((float)v));    // Inference.cu:271-279
+  else p.y[at] = v;
+}
+// f(integral_constant<int, kind>) for the kind in p.epilogue
+template <class F>
+__device__ __forceinline__ void with_epilogue(const GemmParams& p, F&& f) {
+  if (p.epilogue == EPI_RESIDUAL) f(std::integral_constant<int, EPI_RESIDUAL>{});
+  else if (p.epilogue == EPI_GELU) f(std::integral_constant<int, EPI_GELU>{});
+  else f(std::integral_constant<int, EPI_STORE>{});
+}
 
 // 8 nibbles of one dword -> 8 binary16 weights in element order, h(h(q-z)*s)
 template <bool ZINT>
@@ -108,16 +132,18 @@ __global__ __launch_bounds__(1024) void gemm_small_kernel(GemmParams p, int n_wa
     for (int i = 0; i < 4; ++i) red[wave][t][lane][i] = acc[t][i];
   __syncthreads();
   if (wave != 0) return;
+  with_epilogue(p, [&](auto E) {
 #pragma unroll
-  for (int t = 0; t < TT; ++t) {
+    for (int t = 0; t < TT; ++t) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      float v = red[0][t][lane][i];
-      for (int wv = 1; wv < n_waves; ++wv) v += red[wv][t][lane][i];
-      const int tok = t0 + t * 16 + q * 4 + i;  // D[token 4*(lane/16)+i][row lane%16]
-      if (tok < p.M) p.y[(int64_t)tok * p.m + rg * 16 + r] = (half_t)v;
+      for (int i = 0; i < 4; ++i) {
+        float v = red[0][t][lane][i];
+        for (int wv = 1; wv < n_waves; ++wv) v += red[wv][t][lane][i];
+        const int tok = t0 + t * 16 + q * 4 + i;  // D[token 4*(lane/16)+i][row lane%16]
+        if (tok < p.M) store_out<decltype(E)::value>(p, tok, rg * 16 + r, v);
+      }
     }
-  }
+  });
 }
 
 // Many tokens: a wavefront owns 64 weight rows x 128 tokens as 2 x 4 accumulator
@@ -147,8 +173,8 @@ constexpr int kWideSlot = kWideTokens * kWideStride;    // halves per token tile
 constexpr int kWideLdsRows = 2 * kWideSlot * 2;                          // bytes, rows split
 constexpr int kWideLdsK = 4 * kWideRP * kWideTT * 64 * 16 * 4;           // bytes, k split: the partial sums
 
-template <bool ZINT, bool KSPLIT>
-__global__ __launch_bounds__(256, 1) void gemm_wide_kernel(GemmParams p) {
+template <bool ZINT, bool KSPLIT, int EPI>
+__global__ __launch_bounds__(256, KSPLIT ? 1 : 2) void gemm_wide_kernel(GemmParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   half_t* xs = reinterpret_cast<half_t*>(smem_raw);  // [2][NKB][128 tokens][kWideStride]
   constexpr int NKB = KSPLIT ? 4 : 1;
@@ -160,8 +186,10 @@ __global__ __launch_bounds__(256, 1) void gemm_wide_kernel(GemmParams p) {
   const bool rows_ok = rg0 * 16 < p.m;  // rows split: the last workgroup may hang over the edge
   const int t0 = blockIdx.y * kWideTokens;
   // a step is NH blocks of k; the step count is even (checked by the launcher)
-  const int steps = (KSPLIT ? p.nblk / 4 : p.nblk) / NH;
-  const int kb_base = KSPLIT ? wave * steps * NH : 0;
+  const int steps = (KSPLIT ? p.nblk / (4 * p.kz) : p.nblk) / NH;
+  // first block of this workgroup's chunk of k (k split only), then of this wavefront's quarter of it
+  const int kb_wg = KSPLIT ? (int)blockIdx.z * 4 * steps * NH : 0;
+  const int kb_base = kb_wg + (KSPLIT ? wave * steps * NH : 0);
   const int slot = KSPLIT ? wave : 0;
 
   // the 64 rows share one scale group (rg0 is a multiple of 4, a group is 8 row groups)
@@ -182,7 +210,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wide_kernel(GemmParams p) {
     const int pc = tid + i * 256;
     const int j = pc / PCS, tok = (pc % PCS) / (4 * NH), part = pc % (4 * NH);
     const int tg = t0 + tok < p.M ? t0 + tok : p.M - 1;
-    xsrc[i] = p.x + (int64_t)tg * p.k + (KSPLIT ? j * steps * NH : 0) * 32 + part * 8;
+    xsrc[i] = p.x + (int64_t)tg * p.k + (kb_wg + (KSPLIT ? j * steps * NH : 0)) * 32 + part * 8;
     xdst[i] = j * kWideSlot + tok * kWideStride + part * 8;
   }
   xvec_t xr0[PPT], xr1[PPT];  // two named register sets (an indexed array would live in scratch memory)
@@ -273,7 +301,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wide_kernel(GemmParams p) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
           const int tok = t0 + t * 32 + (i >> 2) * 8 + kh * 4 + (i & 3);
-          if (tok < p.M) p.y[(int64_t)tok * p.m + row] = (half_t)acc[a][t][i];
+          if (tok < p.M) store_out<EPI>(p, tok, row, acc[a][t][i]);
         }
       }
     }
@@ -292,38 +320,67 @@ __global__ __launch_bounds__(256, 1) void gemm_wide_kernel(GemmParams p) {
         red[(((wave * kWideRP + a) * kWideTT + t) * 4 + i4) * 64 + lane] =
             float4_t{acc[a][t][4 * i4], acc[a][t][4 * i4 + 1], acc[a][t][4 * i4 + 2], acc[a][t][4 * i4 + 3]};
   __syncthreads();
+  auto finish = [&](auto E) {
+    constexpr int epi = decltype(E)::value;  // -1: this workgroup's chunk of k only, as FP32 partial sums
 #pragma unroll
-  for (int a = 0; a < kWideRP; ++a) {
-    const int row = rg0 * 16 + a * 32 + n;
-    const int t = wave;
+    for (int a = 0; a < kWideRP; ++a) {
+      const int row = rg0 * 16 + a * 32 + n;
+      const int t = wave;
 #pragma unroll
-    for (int i4 = 0; i4 < 4; ++i4) {
-      float4_t v = red[(((0 * kWideRP + a) * kWideTT + t) * 4 + i4) * 64 + lane];
+      for (int i4 = 0; i4 < 4; ++i4) {
+        float4_t v = red[(((0 * kWideRP + a) * kWideTT + t) * 4 + i4) * 64 + lane];
 #pragma unroll
-      for (int w = 1; w < 4; ++w) v += red[(((w * kWideRP + a) * kWideTT + t) * 4 + i4) * 64 + lane];
+        for (int w = 1; w < 4; ++w) v += red[(((w * kWideRP + a) * kWideTT + t) * 4 + i4) * 64 + lane];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int tok = t0 + t * 32 + i4 * 8 + kh * 4 + i;
-        if (tok < p.M) p.y[(int64_t)tok * p.m + row] = (half_t)v[i];
+        for (int i = 0; i < 4; ++i) {
+          const int tok = t0 + t * 32 + i4 * 8 + kh * 4 + i;
+          if (tok < p.M) {
+            if (epi < 0) p.part[((int64_t)blockIdx.z * p.M + tok) * p.m + row] = v[i];
+            else store_out<(epi < 0 ? 0 : epi)>(p, tok, row, v[i]);
+          }
+        }
       }
     }
-  }
+  };
+  if (p.kz > 1) finish(std::integral_constant<int, -1>{});
+  else finish(std::integral_constant<int, EPI>{});
+}
+
+// k cut over several workgroups: the chunks' FP32 partial sums are added in
+// chunk order (whatever order the workgroups ran in), then the epilogue
+__global__ __launch_bounds__(256) void reduce_parts_kernel(GemmParams p) {
+  const int64_t total = (int64_t)p.M * p.m;
+  const int64_t at = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (at >= total) return;
+  float v = p.part[at];
+  for (int z = 1; z < p.kz; ++z) v += p.part[(int64_t)z * total + at];
+  with_epilogue(p, [&](auto E) { store_out<decltype(E)::value>(p, (int)(at / p.m), (int)(at % p.m), v); });
 }
 
 template <bool KSPLIT>
 int launch_wide(const GemmParams& p, bool zint, hipStream_t st) {
   // the main loop takes two steps of two 32-wide blocks per trip (per quarter of k when k is split)
-  AWQ_REQUIRE(p.nblk % (KSPLIT ? 16 : 4) == 0, "k must be a multiple of 512");
+  AWQ_REQUIRE(p.nblk % (KSPLIT ? 16 * p.kz : 4) == 0, "k must be a multiple of 512");
   const int lds = KSPLIT ? (kWideLdsK > 4 * kWideLdsRows ? kWideLdsK : 4 * kWideLdsRows) : kWideLdsRows;
   static_assert(4 * kWideLdsRows <= 160 * 1024 && kWideLdsK <= 160 * 1024, "LDS of one compute unit");
   const unsigned gx = KSPLIT ? (unsigned)(p.m / 64) : (unsigned)((p.m + 255) / 256);
-  dim3 grid(gx, (unsigned)((p.M + kWideTokens - 1) / kWideTokens));
-  auto kern = zint ? gemm_wide_kernel<true, KSPLIT> : gemm_wide_kernel<false, KSPLIT>;
+  dim3 grid(gx, (unsigned)((p.M + kWideTokens - 1) / kWideTokens), KSPLIT ? (unsigned)p.kz : 1u);
+  void (*kern)(GemmParams);
+  if (p.epilogue == EPI_RESIDUAL)
+    kern = zint ? gemm_wide_kernel<true, KSPLIT, EPI_RESIDUAL> : gemm_wide_kernel<false, KSPLIT, EPI_RESIDUAL>;
+  else if (p.epilogue == EPI_GELU)
+    kern = zint ? gemm_wide_kernel<true, KSPLIT, EPI_GELU> : gemm_wide_kernel<false, KSPLIT, EPI_GELU>;
+  else
+    kern = zint ? gemm_wide_kernel<true, KSPLIT, EPI_STORE> : gemm_wide_kernel<false, KSPLIT, EPI_STORE>;
   if (lds > 65536) {
     // more LDS than a launch gets by default: raise this kernel's limit (per device; cheap, so every time)
     AWQ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds));
   }
   hipLaunchKernelGGL(kern, grid, dim3(256), lds, st, p);
+  if (KSPLIT && p.kz > 1) {
+    const int64_t total = (int64_t)p.M * p.m;
+    hipLaunchKernelGGL(reduce_parts_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, p);
+  }
   return AWQ_OK;
 }
 
@@ -335,8 +392,19 @@ void launch_small(const GemmParams& p, bool zint, int n_waves, dim3 grid, hipStr
 
 }  // namespace
 
+// room for the partial sums of a product whose k is cut over workgroups (0: never cut)
+int64_t gemm_workspace_bytes(int64_t m, int64_t k, int64_t M) {
+  (void)k;
+  if (M <= 16 || (M <= 32 && m < 8192)) return 0;
+  const int64_t wgs = (m / 64) * ((M + kWideTokens - 1) / kWideTokens);
+  return wgs <= 128 ? 4 * M * m * 4 : 0;
+}
+
 int launch_gemm(const void* wq, const half_t* scale, const half_t* zp, int64_t m, int64_t k, const half_t* x,
-                half_t* y, int64_t M, int zp_integral, hipStream_t st) {
+                half_t* y, int64_t M, int zp_integral, int epilogue, const half_t* res, void* workspace,
+                int64_t workspace_bytes, hipStream_t st) {
+  AWQ_REQUIRE(epilogue == EPI_STORE || epilogue == EPI_GELU || (epilogue == EPI_RESIDUAL && res),
+              "epilogue must be store, GeLU or residual (with res)");
   AWQ_REQUIRE(m > 0 && m % 128 == 0 && k > 0 && k % 128 == 0, "m and k must be positive multiples of 128");
   AWQ_REQUIRE(M >= 1 && M <= (1 << 20), "M out of range");
   AWQ_REQUIRE(awq_group_period(m, k) == 1, "matrices whose scale group depends on the input index are not supported here");
@@ -353,6 +421,10 @@ int launch_gemm(const void* wq, const half_t* scale, const half_t* zp, int64_t m
   p.nblk = (int32_t)(k / AWQ_BLOCK_K);
   p.mg = (int32_t)(m / 128);
   p.kg = (int32_t)(k / 128);
+  p.epilogue = epilogue;
+  p.res = res;
+  p.kz = 1;
+  p.part = nullptr;
   // up to 16 tokens, and up to 32 on a matrix with few rows: the decode kernel's decomposition
   int g = 0;
   if (M <= 16 || (M <= 32 && m < 8192)) {
@@ -380,6 +452,17 @@ int launch_gemm(const void* wq, const half_t* scale, const half_t* zp, int64_t m
     if (tiles >= 128) {
       if (int rc = launch_wide<false>(p, zp_integral, st)) return rc;
     } else {
+      // few 64-row workgroups too (a matrix with few rows): cut k over 4 or 2 workgroups as well,
+      // when the caller brought room for the partial sums
+      const int64_t wgs = (m / 64) * ((M + kWideTokens - 1) / kWideTokens);
+      if (wgs <= 128 && workspace) {
+        for (int kz : {4, 2})
+          if (p.nblk % (16 * kz) == 0 && (int64_t)kz * M * m * 4 <= workspace_bytes) {
+            p.kz = kz;
+            p.part = (float*)workspace;
+            break;
+          }
+      }
       if (int rc = launch_wide<true>(p, zp_integral, st)) return rc;
     }
   }

@@ -481,10 +481,6 @@ bool plan_gemv(int64_t m, int64_t k, GemvPlan* out) {
     // at least 4 wavefronts: the fused norm sums with 256 threads
     if (groups / 4 >= 4 && (m / 16) * (groups / 4) >= 2048) break;
   }
-  if (const char* f = getenv("AWQ_DEV_G")) {
-    int g = atoi(f);
-    if (g >= 1 && nblk % g == 0 && (nblk / g) % 4 == 0 && nblk / g <= 64) *out = GemvPlan{g, (int)(nblk / g / 4)};
-  }
   return found;
 }
 
@@ -589,10 +585,6 @@ int launch_gemv(const LinearArgs& a, hipStream_t st) {
   // beyond that a workgroup walks several row groups and stages x once
   int64_t n_rg = a.m / 16, n_wg = n_rg;
   if (n_rg > 1024) n_wg = 1024;
-  if (const char* f = getenv("AWQ_DEV_WGS")) {
-    int64_t v = atoll(f);
-    if (v >= 1 && v < n_rg) n_wg = v;
-  }
   dim3 grid((unsigned)n_wg), block((unsigned)(plan.n_waves * 64));
   size_t lds = (size_t)a.k * 2 + (size_t)(a.k / AWQ_BLOCK_K / plan.g) * 16;  // x plus 16 bytes of skew per lane group
   switch (plan.g) {

@@ -205,9 +205,13 @@ int awq_gemv_fused(const awq_linear_args* args, void* stream);
  * are dequantised on load and contracted on the matrix cores with FP32
  * accumulation: within rounding noise of awq_gemv applied to each token, not
  * bit-identical to it.  Matrices whose scale group depends on the input index
- * (the 151936 x 4096 unembedding) are not supported. */
+ * (the 151936 x 4096 unembedding) are not supported.  workspace: NULL, or
+ * awq_gemm_workspace_bytes(m, k, M) bytes of device memory; with it, products
+ * with few output tiles also cut k over several workgroups (FP32 partial sums,
+ * added in a fixed order by a second launch). */
+int64_t awq_gemm_workspace_bytes(int64_t m, int64_t k, int64_t M);
 int awq_gemm(const void* repacked, const void* scale, const void* zp, int64_t m, int64_t k, const void* x, void* y,
-             int64_t M, int32_t zp_integral, void* stream);
+             int64_t M, int32_t zp_integral, void* workspace, void* stream);
 
 /* rmsNormKernel, Inference.cu:111-145.  n multiple of 256. */
 int awq_rmsnorm(const void* x, const void* gamma, void* out, int64_t n, float eps, void* stream);

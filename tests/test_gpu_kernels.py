@@ -461,13 +461,25 @@ def test_gemm_matches_fp32_accumulate_reference(awq, lib, oracle, torch_gpu, m, 
     d_y = torch.full((M, m), float("nan"), dtype=torch.float16, device="cuda")
     print("gemm", m, k, M, flush=True)
     awq.check(lib.awq_gemm(d_w.data_ptr(), d_s.data_ptr(), d_z.data_ptr(), m, k, d_x.data_ptr(), d_y.data_ptr(), M,
-                           1 if zp_int else 0, stream(torch)))
+                           1 if zp_int else 0, None, stream(torch)))
     torch.cuda.synchronize()
+    # with room for partial sums the product may cut k over several workgroups: same tolerance, and
+    # nothing changes where it does not (workspace size 0)
+    wsb = lib.awq_gemm_workspace_bytes(m, k, M)
+    d_ws = torch.zeros(max(wsb, 16), dtype=torch.uint8, device="cuda")
+    d_y2 = torch.full((M, m), float("nan"), dtype=torch.float16, device="cuda")
+    awq.check(lib.awq_gemm(d_w.data_ptr(), d_s.data_ptr(), d_z.data_ptr(), m, k, d_x.data_ptr(), d_y2.data_ptr(), M,
+                           1 if zp_int else 0, d_ws.data_ptr(), stream(torch)))
+    torch.cuda.synchronize()
+    got2 = d_y2.cpu().numpy()[sel].astype(np.float64)
+    if wsb == 0:
+        assert np.array_equal(d_y2.cpu().numpy().view(np.uint16), d_y.cpu().numpy().view(np.uint16))
     got = d_y.cpu().numpy()[sel].astype(np.float64)
     want = ref.astype(np.float64)
     denom = np.maximum(np.abs(want), 1e-2 * np.abs(want).max())
     assert np.all(np.isfinite(got))
     assert np.all(np.abs(got - want) <= 1e-2 * denom)
+    assert np.all(np.isfinite(got2)) and np.all(np.abs(got2 - want) <= 1e-2 * denom)
     # much tighter in practice: FP32 accumulation either way
     assert np.mean(d_y.cpu().numpy()[sel].view(np.uint16) == ref.view(np.uint16)) > 0.9
 
@@ -487,7 +499,7 @@ def test_gemm_one_hot_and_token_independence(awq, lib, torch_gpu):
         d_s, d_z, d_x = dev(torch, scale), dev(torch, zp), dev(torch, x)
         d_y = torch.zeros((M, m), dtype=torch.float16, device="cuda")
         awq.check(lib.awq_gemm(d_w.data_ptr(), d_s.data_ptr(), d_z.data_ptr(), m, k, d_x.data_ptr(), d_y.data_ptr(), M,
-                               1, stream(torch)))
+                               1, None, stream(torch)))
         torch.cuda.synchronize()
         y = d_y.cpu().numpy().astype(np.float64)
         expect = np.zeros((M, m))
@@ -495,4 +507,4 @@ def test_gemm_one_hot_and_token_independence(awq, lib, torch_gpu):
         assert np.array_equal(y, expect), p
     buf = torch.zeros(1 << 20, dtype=torch.uint8, device="cuda")
     b = buf.data_ptr()
-    assert lib.awq_gemm(b, b, b, 128 * 37, 512, b, b, 4, 1, None) != 0   # input-dependent scale groups: refused
+    assert lib.awq_gemm(b, b, b, 128 * 37, 512, b, b, 4, 1, None, None) != 0   # input-dependent scale groups: refused

@@ -152,3 +152,30 @@ def test_full_model_batched_prompt_tokens(awq, oracle, torch_gpu):
     assert same >= n_new // 2
     eng.close()
     oracle.awqo_model_destroy(model)
+
+
+def test_long_prompt_takes_the_rows_split_products(awq, oracle, torch_gpu):
+    """A 1027-token prompt at full width: every product of the layer has enough output tiles for the
+    rows-split workgroup shape (with the GeLU and residual epilogues), and the prompt spans the
+    short-sequence and the long-sequence attention launches of the batched pass."""
+    cfg = awq.make_config(n_layers=1, vocab=2048, max_pos=1100)
+    model = make_oracle_model(oracle, cfg)   # only as the host buffer of the weights here
+    eng = awq.QWen3AWQInfer.empty(cfg)
+    fill_pair(awq, oracle, cfg, 31, engine=eng, model=model, profile=awq.SYNTH_BALANCED)
+    oracle.awqo_model_destroy(model)
+    rng = np.random.default_rng(9)
+    prompt = rng.integers(0, cfg.vocab, 1027).tolist()
+    print("batched prompt pass, one full-width layer, P = 1027", flush=True)
+    eng.reset()
+    eng.prefill(prompt)
+    hid_seq = as_f32(eng.read_hidden()).copy()
+    tok_seq = eng.decode(4)
+    eng.reset()
+    eng.prefill(prompt, batched=True)
+    hid_bat = as_f32(eng.read_hidden()).copy()
+    tok_bat = eng.decode(4)
+    print("hidden: max |seq - batched| = %.5f at scale %.3f" % (np.abs(hid_seq - hid_bat).max(), np.abs(hid_seq).max()),
+          flush=True)
+    assert np.isfinite(hid_seq).all() and close(hid_seq, hid_bat)
+    assert tok_bat[0] == tok_seq[0]
+    eng.close()
