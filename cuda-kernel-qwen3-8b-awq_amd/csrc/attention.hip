@@ -17,7 +17,6 @@
 namespace {
 
 constexpr int kMaxChunks = 1024;    // 65536 positions
-constexpr int kLdsPositions = 8192; // scores kept in LDS up to this length
 constexpr int kLdsChunks = 32;      // chunk vectors kept in LDS up to this many chunks
 constexpr int kWaves = 16;   // wavefronts per workgroup of the decode variants
 constexpr int kThreads = kWaves * 64;
@@ -59,19 +58,18 @@ __device__ __forceinline__ float wave_tree_sum(float v) {
 // own query and output rows ([token][head][128]); it attends the positions the
 // prompt loop gives it (Inference.cu:1118 read before or after :1331):
 // max(pos, 1) when use_len_hi is 0, pos + 1 otherwise.
-// NW wavefronts; SCAP positions of scores and CCAP chunks (sums, and vectors
-// when LDS_CV) fit the LDS arrays.
-template <bool LDS_SCORES, bool LDS_CV, bool BATCH, int NW, int SCAP, int CCAP>
+// NW wavefronts; SCAP positions of scores and CCAP chunks (sums and vectors)
+// fit the LDS arrays.  Longer sequences take the split kernels further down.
+template <bool BATCH, int NW, int SCAP, int CCAP>
 __global__ __launch_bounds__(NW * 64) void attention_kernel(const half_t* __restrict__ q,
                                                              const half_t* __restrict__ kc,
                                                              const half_t* __restrict__ vc, half_t* __restrict__ ctx,
                                                              int64_t max_pos, int L_arg, const StepState* dyn,
-                                                             int use_len_hi, float* __restrict__ ws_scores,
-                                                             float* __restrict__ ws_cv, int max_chunks) {
+                                                             int use_len_hi) {
   __shared__ float cs[CCAP];
   __shared__ float wmax[NW];
-  __shared__ float s_lds[LDS_SCORES ? SCAP : 1];
-  __shared__ float cv_lds[LDS_CV ? CCAP * AWQ_HEAD_DIM : 1];
+  __shared__ float s[SCAP];
+  __shared__ float cv[CCAP * AWQ_HEAD_DIM];
   int L;
   if (BATCH) {
     const int pos = L_arg + blockIdx.y;
@@ -86,8 +84,6 @@ __global__ __launch_bounds__(NW * 64) void attention_kernel(const half_t* __rest
   const int tq = lane >> 4, dl = lane & 15;
   const half_t* kh = kc + (int64_t)head * max_pos * AWQ_HEAD_DIM;
   const half_t* vh = vc + (int64_t)head * max_pos * AWQ_HEAD_DIM;
-  float* s = LDS_SCORES ? s_lds : ws_scores + (int64_t)head * max_pos;
-  float* cv = LDS_CV ? cv_lds : ws_cv + (int64_t)head * max_chunks * AWQ_HEAD_DIM;
   const int nchunks = (L + 63) >> 6;
   const float scale = 1.0f / sqrtf((float)AWQ_HEAD_DIM);  // Inference.cu:218
 
@@ -199,12 +195,220 @@ __global__ __launch_bounds__(NW * 64) void attention_kernel(const half_t* __rest
   }
 }
 
+// ---------------------------------------------------------------------------
+// Long sequences: the same computation cut along the sequence, kSplit parts
+// (contiguous ranges of 64-position chunks) per head, so that a few hundred
+// workgroups stream the cache instead of one per head.  The summation orders
+// are unchanged -- every chunk is still summed by one wavefront, chunk results
+// are added in chunk order -- so the result is bit-identical to the one-kernel
+// path.  Four launches: scores and part maxima; exponentials and chunk sums;
+// chunk context vectors; their ordered sum.  Scores, chunk sums, chunk vectors
+// and part maxima live in the workspace.
+// ---------------------------------------------------------------------------
+constexpr int kSplit = 32;         // parts per head
+constexpr int kSplitWaves = 4;     // wavefronts per workgroup of the split kernels
+
+struct SplitArgs {
+  const half_t* q;
+  const half_t* kc;
+  const half_t* vc;
+  half_t* ctx;
+  int64_t max_pos;
+  int L_arg;
+  const StepState* dyn;
+  int use_len_hi;
+  float* scores;  // [head][max_pos]
+  float* cv;      // [head][max_chunks][128]
+  float* cs;      // [head][max_chunks]
+  float* pmax;    // [head][kSplit]
+  int max_chunks;
+};
+
+__device__ __forceinline__ int split_len(const SplitArgs& a) {
+  return a.dyn ? (a.use_len_hi ? a.dyn->len_hi : a.dyn->len_lo) : a.L_arg;
+}
+// chunk range [lo, hi) of part blockIdx.y
+__device__ __forceinline__ void split_range(int nchunks, int* lo, int* hi) {
+  const int per = (nchunks + kSplit - 1) / kSplit;
+  *lo = min((int)blockIdx.y * per, nchunks);
+  *hi = min(*lo + per, nchunks);
+}
+
+// scores (Inference.cu:202-226) of this part and their maximum (:229-233)
+__global__ __launch_bounds__(kSplitWaves * 64) void attn_scores_kernel(SplitArgs a) {
+  __shared__ float wmax[kSplitWaves];
+  const int L = split_len(a);
+  const int head = blockIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tq = lane >> 4, dl = lane & 15;
+  const half_t* kh = a.kc + (int64_t)head * a.max_pos * AWQ_HEAD_DIM;
+  float* s = a.scores + (int64_t)head * a.max_pos;
+  int c_lo, c_hi;
+  split_range((L + 63) >> 6, &c_lo, &c_hi);
+  const float scale = 1.0f / sqrtf((float)AWQ_HEAD_DIM);  // Inference.cu:218
+  float qf[8];
+  {
+    half8_t qv = *reinterpret_cast<const half8_t*>(a.q + head * AWQ_HEAD_DIM + 8 * dl);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) qf[i] = (float)qv[i];
+  }
+  float lmax = -1e9f;
+  const int q_hi = min(c_hi * 16, (L + 3) >> 2);
+  // eight groups of four positions per trip; the next trip's keys are in flight
+  // while this one's are multiplied
+  half8_t kv[8], kn[8];
+  auto load_keys = [&](int q0, half8_t (&dst)[8]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int t = 4 * (q0 + u * kSplitWaves) + tq;
+      if (q0 + u * kSplitWaves < q_hi && t < L)
+        dst[u] = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(kh + (int64_t)t * AWQ_HEAD_DIM + 8 * dl));
+    }
+  };
+  load_keys(c_lo * 16 + wave, kn);
+  for (int q0 = c_lo * 16 + wave; q0 < q_hi; q0 += 8 * kSplitWaves) {
+#pragma unroll
+    for (int u = 0; u < 8; ++u) kv[u] = kn[u];
+    load_keys(q0 + 8 * kSplitWaves, kn);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int t = 4 * (q0 + u * kSplitWaves) + tq;
+      const bool ok = q0 + u * kSplitWaves < q_hi && t < L;
+      float part = 0.0f;
+      if (ok) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) part = __builtin_fmaf(qf[i], (float)kv[u][i], part);
+      }
+      part = row16_tree_sum(part);
+      const float sc = part * scale;
+      if (ok) {
+        if (dl == 0) s[t] = sc;
+        lmax = fmaxf(lmax, sc);
+      }
+    }
+  }
+#pragma unroll
+  for (int mask = 1; mask < 64; mask <<= 1) lmax = fmaxf(lmax, __shfl_xor(lmax, mask, 64));
+  if (lane == 0) wmax[wave] = lmax;
+  __syncthreads();
+  if (tid == 0) {
+    float mx = wmax[0];
+#pragma unroll
+    for (int w = 1; w < kSplitWaves; ++w) mx = fmaxf(mx, wmax[w]);
+    a.pmax[head * kSplit + blockIdx.y] = mx;
+  }
+}
+
+// exponentials and chunk sums (Inference.cu:239-249), one wavefront per chunk
+__global__ __launch_bounds__(kSplitWaves * 64) void attn_exp_kernel(SplitArgs a) {
+  const int L = split_len(a);
+  const int head = blockIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  float* s = a.scores + (int64_t)head * a.max_pos;
+  int c_lo, c_hi;
+  split_range((L + 63) >> 6, &c_lo, &c_hi);
+  float mx = a.pmax[head * kSplit];
+#pragma unroll
+  for (int i = 1; i < kSplit; ++i) mx = fmaxf(mx, a.pmax[head * kSplit + i]);
+  for (int chunk = c_lo + wave; chunk < c_hi; chunk += kSplitWaves) {
+    const int t = (chunk << 6) + lane;
+    float e = 0.0f;
+    if (t < L) {
+      e = awq_expf(s[t] - mx);
+      s[t] = e;
+    }
+    e = wave_tree_sum(e);
+    if (lane == 0) a.cs[(int64_t)head * a.max_chunks + chunk] = e;
+  }
+}
+
+// weighted sums of V per chunk (Inference.cu:251-265), one wavefront per chunk
+__global__ __launch_bounds__(kSplitWaves * 64) void attn_pv_kernel(SplitArgs a) {
+  const int L = split_len(a);
+  const int head = blockIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tq = lane >> 4, dl = lane & 15;
+  const half_t* vh = a.vc + (int64_t)head * a.max_pos * AWQ_HEAD_DIM;
+  const float* s = a.scores + (int64_t)head * a.max_pos;
+  const float* cs = a.cs + (int64_t)head * a.max_chunks;
+  float* cv = a.cv + (int64_t)head * a.max_chunks * AWQ_HEAD_DIM;
+  const int nchunks = (L + 63) >> 6;
+  int c_lo, c_hi;
+  split_range(nchunks, &c_lo, &c_hi);
+  if (c_lo >= c_hi) return;
+  // the first chunk's values are requested before the (latency-bound) sum of the chunk sums
+  half8_t vv[16];
+  int chunk = c_lo + wave;
+  if (chunk < c_hi) {
+#pragma unroll
+    for (int nl = 0; nl < 16; ++nl) {
+      const int t = (chunk << 6) + 4 * nl + tq;
+      if (t < L) vv[nl] = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(vh + (int64_t)t * AWQ_HEAD_DIM + 8 * dl));
+    }
+  }
+  float Z = cs[0];
+  for (int c = 1; c < nchunks; ++c) Z += cs[c];
+  for (; chunk < c_hi; chunk += kSplitWaves) {
+    const int base = chunk << 6;
+    float acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
+#pragma unroll
+    for (int nl = 0; nl < 16; ++nl) {
+      const int t = base + 4 * nl + tq;
+      if (t < L) {
+        const float p = s[t] / Z;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] = __builtin_fmaf(p, (float)vv[nl][i], acc[i]);
+      }
+    }
+    // the next chunk's values while this one is reduced and stored
+    const int nxt = chunk + kSplitWaves;
+    if (nxt < c_hi) {
+#pragma unroll
+      for (int nl = 0; nl < 16; ++nl) {
+        const int t = (nxt << 6) + 4 * nl + tq;
+        if (t < L) vv[nl] = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(vh + (int64_t)t * AWQ_HEAD_DIM + 8 * dl));
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      acc[i] = xor_add(acc[i], 16);
+      acc[i] = xor_add(acc[i], 32);
+    }
+    if (tq == 0) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) cv[chunk * AWQ_HEAD_DIM + 8 * dl + i] = acc[i];
+    }
+  }
+}
+
+// chunk vectors added in chunk order (Inference.cu:259-265 runs over t in order)
+__global__ __launch_bounds__(AWQ_HEAD_DIM) void attn_sum_kernel(SplitArgs a) {
+  const int L = split_len(a);
+  const int head = blockIdx.x, tid = threadIdx.x;
+  const float* cv = a.cv + (int64_t)head * a.max_chunks * AWQ_HEAD_DIM;
+  const int nchunks = (L + 63) >> 6;
+  float out = cv[tid];
+  int c = 1;
+  for (; c + 16 <= nchunks; c += 16) {
+    float v[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) v[i] = cv[(c + i) * AWQ_HEAD_DIM + tid];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) out += v[i];
+  }
+  for (; c < nchunks; ++c) out += cv[c * AWQ_HEAD_DIM + tid];
+  a.ctx[head * AWQ_HEAD_DIM + tid] = (half_t)out;
+}
+
 }  // namespace
 
 static int64_t chunks_for(int64_t max_pos) { return (max_pos + 63) / 64; }
 
+// scores, chunk vectors, chunk sums, part maxima
 int64_t attention_workspace_bytes(int n_heads, int64_t max_pos) {
-  return (int64_t)n_heads * (max_pos + chunks_for(max_pos) * AWQ_HEAD_DIM) * 4;
+  return (int64_t)n_heads * (max_pos + chunks_for(max_pos) * (AWQ_HEAD_DIM + 1) + kSplit) * 4;
 }
 
 int launch_attention(const half_t* q, const half_t* kc, const half_t* vc, half_t* ctx, int n_heads, int64_t max_pos,
@@ -218,19 +422,32 @@ int launch_attention(const half_t* q, const half_t* kc, const half_t* vc, half_t
   // decides where the scores live); with a length known here, the length itself.
   const int64_t bound = dyn ? (len_bound > 0 ? len_bound : max_pos) : L;
   const int mc = (int)chunks_for(max_pos);
-  if (bound <= kLdsChunks * 64) {
-    hipLaunchKernelGGL((attention_kernel<true, true, false, kWaves, kLdsChunks * 64, kLdsChunks>), dim3(n_heads),
-                       dim3(kThreads), 0, st, q, kc, vc, ctx, max_pos,
-                       (int)L, dyn, use_len_hi, scores, cv, mc);
-  } else if (bound <= kLdsPositions) {
-    hipLaunchKernelGGL((attention_kernel<true, false, false, kWaves, kLdsPositions, kMaxChunks>), dim3(n_heads),
-                       dim3(kThreads), 0, st, q, kc, vc, ctx, max_pos,
-                       (int)L, dyn, use_len_hi, scores, cv, mc);
-  } else {
-    hipLaunchKernelGGL((attention_kernel<false, false, false, kWaves, 1, kMaxChunks>), dim3(n_heads),
-                       dim3(kThreads), 0, st, q, kc, vc, ctx,
-                       max_pos, (int)L, dyn, use_len_hi, scores, cv, mc);
+  if (bound > kLdsChunks * 64) {
+    // long sequences: cut along the sequence
+    SplitArgs a;
+    a.q = q;
+    a.kc = kc;
+    a.vc = vc;
+    a.ctx = ctx;
+    a.max_pos = max_pos;
+    a.L_arg = (int)L;
+    a.dyn = dyn;
+    a.use_len_hi = use_len_hi;
+    a.scores = scores;
+    a.cv = cv;
+    a.cs = cv + (int64_t)n_heads * mc * AWQ_HEAD_DIM;
+    a.pmax = a.cs + (int64_t)n_heads * mc;
+    a.max_chunks = mc;
+    const dim3 grid(n_heads, kSplit), block(kSplitWaves * 64);
+    hipLaunchKernelGGL(attn_scores_kernel, grid, block, 0, st, a);
+    hipLaunchKernelGGL(attn_exp_kernel, grid, block, 0, st, a);
+    hipLaunchKernelGGL(attn_pv_kernel, grid, block, 0, st, a);
+    hipLaunchKernelGGL(attn_sum_kernel, dim3(n_heads), dim3(AWQ_HEAD_DIM), 0, st, a);
+    AWQ_HIP_TRY(hipGetLastError());
+    return AWQ_OK;
   }
+  hipLaunchKernelGGL((attention_kernel<false, kWaves, kLdsChunks * 64, kLdsChunks>), dim3(n_heads), dim3(kThreads), 0,
+                     st, q, kc, vc, ctx, max_pos, (int)L, dyn, use_len_hi);
   AWQ_HIP_TRY(hipGetLastError());
   return AWQ_OK;
 }
@@ -245,15 +462,14 @@ int launch_attention_batch(const half_t* q, const half_t* kc, const half_t* vc, 
   AWQ_REQUIRE(ws != nullptr, "workspace required");
   // short prompts: small workgroups (4 wavefronts, 3 KiB of LDS), many of them per compute unit
   if (pos0 + M <= 256) {
-    hipLaunchKernelGGL((attention_kernel<true, true, true, 4, 256, 4>), dim3(n_heads, (unsigned)M), dim3(256), 0, st,
-                       q, kc, vc, ctx, max_pos, (int)pos0, nullptr, use_len_hi, nullptr, nullptr, 0);
+    hipLaunchKernelGGL((attention_kernel<true, 4, 256, 4>), dim3(n_heads, (unsigned)M), dim3(256), 0, st, q, kc, vc,
+                       ctx, max_pos, (int)pos0, nullptr, use_len_hi);
     AWQ_HIP_TRY(hipGetLastError());
     return AWQ_OK;
   }
   if (pos0 + M <= kLdsChunks * 64) {
-    hipLaunchKernelGGL((attention_kernel<true, true, true, kWaves, kLdsChunks * 64, kLdsChunks>),
-                       dim3(n_heads, (unsigned)M), dim3(kThreads), 0, st, q, kc, vc, ctx, max_pos, (int)pos0, nullptr,
-                       use_len_hi, nullptr, nullptr, 0);
+    hipLaunchKernelGGL((attention_kernel<true, kWaves, kLdsChunks * 64, kLdsChunks>), dim3(n_heads, (unsigned)M),
+                       dim3(kThreads), 0, st, q, kc, vc, ctx, max_pos, (int)pos0, nullptr, use_len_hi);
     AWQ_HIP_TRY(hipGetLastError());
     return AWQ_OK;
   }

@@ -255,6 +255,33 @@ def test_decode_attention_bit_exact(awq, lib, oracle, torch_gpu, L):
                                     ws.data_ptr(), stream(torch)) != 0
 
 
+@pytest.mark.parametrize("L", [2049, 3000, 9001, 20000])
+def test_decode_attention_long_sequences_bit_exact(awq, lib, oracle, torch_gpu, L):
+    """beyond 2048 positions the launches are cut along the sequence (32 parts per head); the
+    summation orders are those of the short path, so the oracle's bits must come out"""
+    torch = torch_gpu
+    nh, mp = 4, 20480
+    rng = np.random.default_rng(L)
+    q = rng.standard_normal(nh * 128).astype(np.float16)
+    kc = np.zeros((nh, mp, 128), dtype=np.float16)
+    vc = np.zeros((nh, mp, 128), dtype=np.float16)
+    kc[:, :L] = (0.3 * rng.standard_normal((nh, L, 128))).astype(np.float16)
+    vc[:, :L] = rng.standard_normal((nh, L, 128)).astype(np.float16)
+    kc[:, L:L + 3] = np.float16(1000.0)
+    vc[:, L:L + 3] = np.float16("inf")
+    ref = np.zeros(nh * 128, dtype=np.float16)
+    oracle.awqo_attention(ptr(q), ptr(kc), ptr(vc), ptr(ref), nh, mp, L, None)
+    d_q, d_k, d_v = dev(torch, q), dev(torch, kc), dev(torch, vc)
+    d_o = torch.zeros(nh * 128, dtype=torch.float16, device="cuda")
+    ws = torch.zeros(lib.awq_attention_workspace_bytes(nh, mp), dtype=torch.uint8, device="cuda")
+    print("attention, long sequence, L", L, flush=True)
+    for _ in range(2):   # the workspace holds the previous call's values the second time
+        awq.check(lib.awq_decode_attention(d_q.data_ptr(), d_k.data_ptr(), d_v.data_ptr(), d_o.data_ptr(), nh, mp, L,
+                                           ws.data_ptr(), stream(torch)))
+        torch.cuda.synchronize()
+        assert np.array_equal(d_o.cpu().numpy().view(np.uint16), ref.view(np.uint16))
+
+
 def test_gelu_all_fp16_values_and_residual(awq, lib, oracle, torch_gpu):
     torch = torch_gpu
     allh = np.arange(65536, dtype=np.uint16).view(np.float16)
