@@ -238,7 +238,7 @@ __global__ __launch_bounds__(256, KSPLIT ? 1 : 2) void gemm_wide_kernel(GemmPara
 #pragma unroll
     for (int h = 0; h < NH; ++h)
 #pragma unroll
-      for (int a = 0; a < kWideRP; ++a) wd[a][f][h] = __builtin_nontemporal_load(wp[a] + (int64_t)(f * NH + h) * 32);
+      for (int a = 0; a < kWideRP; ++a) wd[a][f][h] = KSPLIT ? __builtin_nontemporal_load(wp[a] + (int64_t)(f * NH + h) * 32) : wp[a][(int64_t)(f * NH + h) * 32];
 
   f32x16_t acc[kWideRP][kWideTT];
 #pragma unroll
@@ -268,7 +268,7 @@ __global__ __launch_bounds__(256, KSPLIT ? 1 : 2) void gemm_wide_kernel(GemmPara
       for (int a = 0; a < kWideRP; ++a) {
         wop[a][0] = dequant8<ZINT>(wd[a][f][h].x, sc, zz);
         wop[a][1] = dequant8<ZINT>(wd[a][f][h].y, sc, zz);
-        wd[a][f][h] = __builtin_nontemporal_load(wp[a] + (int64_t)(sn * NH + h) * 32);
+        wd[a][f][h] = KSPLIT ? __builtin_nontemporal_load(wp[a] + (int64_t)(sn * NH + h) * 32) : wp[a][(int64_t)(sn * NH + h) * 32];
       }
 #pragma unroll
       for (int t = 0; t < kWideTT; ++t) {
