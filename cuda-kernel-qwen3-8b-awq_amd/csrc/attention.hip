@@ -54,13 +54,9 @@ __device__ __forceinline__ float wave_tree_sum(float v) {
   return v;
 }
 
-// BATCH: blockIdx.y is a prompt token at position L_arg + blockIdx.y with its
-// own query and output rows ([token][head][128]); it attends the positions the
-// prompt loop gives it (Inference.cu:1118 read before or after :1331):
-// max(pos, 1) when use_len_hi is 0, pos + 1 otherwise.
 // NW wavefronts; SCAP positions of scores and CCAP chunks (sums and vectors)
 // fit the LDS arrays.  Longer sequences take the split kernels further down.
-template <bool BATCH, int NW, int SCAP, int CCAP>
+template <int NW, int SCAP, int CCAP>
 __global__ __launch_bounds__(NW * 64) void attention_kernel(const half_t* __restrict__ q,
                                                              const half_t* __restrict__ kc,
                                                              const half_t* __restrict__ vc, half_t* __restrict__ ctx,
@@ -70,15 +66,7 @@ __global__ __launch_bounds__(NW * 64) void attention_kernel(const half_t* __rest
   __shared__ float wmax[NW];
   __shared__ float s[SCAP];
   __shared__ float cv[CCAP * AWQ_HEAD_DIM];
-  int L;
-  if (BATCH) {
-    const int pos = L_arg + blockIdx.y;
-    L = use_len_hi ? pos + 1 : (pos > 1 ? pos : 1);
-    q += (int64_t)blockIdx.y * gridDim.x * AWQ_HEAD_DIM;
-    ctx += (int64_t)blockIdx.y * gridDim.x * AWQ_HEAD_DIM;
-  } else {
-    L = dyn ? (use_len_hi ? dyn->len_hi : dyn->len_lo) : L_arg;
-  }
+  const int L = dyn ? (use_len_hi ? dyn->len_hi : dyn->len_lo) : L_arg;
   const int head = blockIdx.x;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int tq = lane >> 4, dl = lane & 15;
@@ -446,39 +434,8 @@ int launch_attention(const half_t* q, const half_t* kc, const half_t* vc, half_t
     AWQ_HIP_TRY(hipGetLastError());
     return AWQ_OK;
   }
-  hipLaunchKernelGGL((attention_kernel<false, kWaves, kLdsChunks * 64, kLdsChunks>), dim3(n_heads), dim3(kThreads), 0,
+  hipLaunchKernelGGL((attention_kernel<kWaves, kLdsChunks * 64, kLdsChunks>), dim3(n_heads), dim3(kThreads), 0,
                      st, q, kc, vc, ctx, max_pos, (int)L, dyn, use_len_hi);
   AWQ_HIP_TRY(hipGetLastError());
-  return AWQ_OK;
-}
-
-// Attention of M consecutive prompt positions pos0 .. pos0+M-1, whose keys and
-// values are already in the cache.  While the longest attended length fits the
-// LDS variant all tokens go in one launch; beyond that, one launch per token.
-int launch_attention_batch(const half_t* q, const half_t* kc, const half_t* vc, half_t* ctx, int n_heads,
-                           int64_t max_pos, int64_t pos0, int64_t M, int use_len_hi, void* ws, hipStream_t st) {
-  AWQ_REQUIRE(n_heads > 0 && max_pos > 0 && max_pos <= (int64_t)kMaxChunks * 64, "max_pos must be in 1..65536");
-  AWQ_REQUIRE(M >= 1 && M <= 65535 && pos0 >= 0 && pos0 + M <= max_pos, "positions out of range");
-  AWQ_REQUIRE(ws != nullptr, "workspace required");
-  // short prompts: small workgroups (4 wavefronts, 3 KiB of LDS), many of them per compute unit
-  if (pos0 + M <= 256) {
-    hipLaunchKernelGGL((attention_kernel<true, 4, 256, 4>), dim3(n_heads, (unsigned)M), dim3(256), 0, st, q, kc, vc,
-                       ctx, max_pos, (int)pos0, nullptr, use_len_hi);
-    AWQ_HIP_TRY(hipGetLastError());
-    return AWQ_OK;
-  }
-  if (pos0 + M <= kLdsChunks * 64) {
-    hipLaunchKernelGGL((attention_kernel<true, kWaves, kLdsChunks * 64, kLdsChunks>), dim3(n_heads, (unsigned)M),
-                       dim3(kThreads), 0, st, q, kc, vc, ctx, max_pos, (int)pos0, nullptr, use_len_hi);
-    AWQ_HIP_TRY(hipGetLastError());
-    return AWQ_OK;
-  }
-  const int64_t H = (int64_t)n_heads * AWQ_HEAD_DIM;
-  for (int64_t t = 0; t < M; ++t) {
-    const int64_t pos = pos0 + t;
-    const int64_t L = use_len_hi ? pos + 1 : (pos > 1 ? pos : 1);
-    if (int rc = launch_attention(q + t * H, kc, vc, ctx + t * H, n_heads, max_pos, L, nullptr, 0, 0, ws, st))
-      return rc;
-  }
   return AWQ_OK;
 }

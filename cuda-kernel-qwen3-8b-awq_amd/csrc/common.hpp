@@ -122,8 +122,8 @@ int launch_rope_kv_append(const half_t* qkv, const half_t* cos_t, const half_t* 
 int64_t attention_workspace_bytes(int n_heads, int64_t max_pos);
 int launch_attention(const half_t* q, const half_t* kc, const half_t* vc, half_t* ctx, int n_heads, int64_t max_pos,
                      int64_t L, const StepState* dyn, int use_len_hi, int64_t len_bound, void* ws, hipStream_t st);
-int launch_attention_batch(const half_t* q, const half_t* kc, const half_t* vc, half_t* ctx, int n_heads,
-                           int64_t max_pos, int64_t pos0, int64_t M, int use_len_hi, void* ws, hipStream_t st);
+int launch_prefill_attention(const half_t* q, const half_t* kc, const half_t* vc, half_t* ctx, int n_heads,
+                             int64_t max_pos, int64_t pos0, int64_t M, int use_len_hi, hipStream_t st);
 int launch_embed_batch(const uint8_t* packed, const half_t* scale, const half_t* zp, int64_t hidden, int64_t vocab,
                        const int32_t* tokens_dev, int64_t M, half_t* out, hipStream_t st);
 int launch_rmsnorm_batch(const half_t* x, const half_t* gamma, half_t* out, int64_t n, int64_t M, float eps,

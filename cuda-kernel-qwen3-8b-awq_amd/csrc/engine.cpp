@@ -626,9 +626,9 @@ int enqueue_layer_batch(awq_engine* e, int l, int64_t pos0, int64_t M) {
   if (int rc = launch_rope_kv_append_batch(b.qkv, e->cos_t, e->sin_t, b.q, L.kcache, L.vcache, e->n_heads,
                                            e->cfg.max_pos, pos0, M, st))
     return rc;  // :1070-1103
-  if (int rc = launch_attention_batch(b.q, L.kcache, L.vcache, b.ctx, e->n_heads, e->cfg.max_pos, pos0, M, l >= 1,
-                                      e->attn_ws, st))
-    return rc;                                                         // :1110
+  if (int rc = launch_prefill_attention(b.q, L.kcache, L.vcache, b.ctx, e->n_heads, e->cfg.max_pos, pos0, M, l >= 1,
+                                        st))
+    return rc;  // :1110
   // :1128 Wo product, :1149 residual add in its epilogue
   if (int rc = gemm_of(e, L.wo, b.ctx, b.hidden, M, EPI_RESIDUAL, b.hidden)) return rc;
   if (int rc = launch_rmsnorm_batch(b.hidden, L.gamma, b.norm, H, M, e->cfg.eps, st)) return rc;  // :1163
@@ -931,6 +931,14 @@ extern "C" int awq_decode_attention(const void* q, const void* k_cache, const vo
   AWQ_REQUIRE(q && k_cache && v_cache && ctx, "NULL pointer");
   return launch_attention((const half_t*)q, (const half_t*)k_cache, (const half_t*)v_cache, (half_t*)ctx, n_heads,
                           max_pos, L, nullptr, 0, 0, workspace, (hipStream_t)stream);
+}
+
+extern "C" int awq_prefill_attention(const void* q, const void* k_cache, const void* v_cache, void* ctx,
+                                     int32_t n_heads, int64_t max_pos, int64_t pos0, int64_t n_tokens,
+                                     int32_t first_layer, void* stream) {
+  AWQ_REQUIRE(q && k_cache && v_cache && ctx, "NULL pointer");
+  return launch_prefill_attention((const half_t*)q, (const half_t*)k_cache, (const half_t*)v_cache, (half_t*)ctx,
+                                  n_heads, max_pos, pos0, n_tokens, first_layer ? 0 : 1, (hipStream_t)stream);
 }
 
 extern "C" int awq_residual_add(const void* a, const void* b, void* out, int64_t n, void* stream) {

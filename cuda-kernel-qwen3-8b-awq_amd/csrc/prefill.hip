@@ -85,6 +85,152 @@ __global__ __launch_bounds__(64) void rope_kv_batch_kernel(const half_t* __restr
   vc[dst + 1] = qkv[2 * H + e + 1];
 }
 
+
+// ---------------------------------------------------------------------------
+// Attention of a tile of 128 prompt positions of one head against the cache,
+// on the matrix cores: keys and values of 32 positions at a time go through
+// LDS once per workgroup instead of once per query.  Same mathematics as
+// attentionKernel's comments (Inference.cu:201-265) -- scores scaled by
+// 1/sqrt(128) after the dot product, softmax over the attended positions,
+// weighted sum of V -- in the usual streaming form (running maximum and sum,
+// context rescaled when the maximum moves; probabilities rounded to binary16
+// for the second product), so it agrees with the one-query kernel to rounding
+// noise, not bit for bit.  Every query is a column of the accumulators:
+//   S^T[key][query] = K[key][:] . Q[query][:]      v_mfma_f32_32x32x16_f16 x 8
+//   O^T[d][query]  += V^T[d][key] * P^T[key][query]  x 8 (4 tiles of d, 2 of keys)
+// so that a query's maximum, sum and rescaling stay inside one lane (plus its
+// partner lane + 32), and the probabilities a lane computed are exactly the
+// operand elements it has to supply to the second product.
+// ---------------------------------------------------------------------------
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+
+constexpr int kFaQueries = 128;   // per workgroup, 32 per wavefront
+constexpr int kFaKeys = 32;       // per step
+constexpr int kFaKStride = 136;   // halves per key row of the K tile (128 + 8 of padding)
+constexpr int kFaVStride = 36;    // halves per row of the transposed V tile (32 keys + 4 of padding)
+
+__global__ __launch_bounds__(256) void prefill_attention_kernel(const half_t* __restrict__ q,
+                                                                const half_t* __restrict__ kc,
+                                                                const half_t* __restrict__ vc,
+                                                                half_t* __restrict__ ctx, int64_t max_pos, int pos0,
+                                                                int M, int use_len_hi) {
+  __shared__ __attribute__((aligned(16))) half_t ks[kFaKeys * kFaKStride];
+  __shared__ __attribute__((aligned(16))) half_t vt[AWQ_HEAD_DIM * kFaVStride];
+  const int head = blockIdx.x, n_heads = gridDim.x;
+  const int H = n_heads * AWQ_HEAD_DIM;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 31, kh = lane >> 5;
+  const half_t* kh_ptr = kc + (int64_t)head * max_pos * AWQ_HEAD_DIM;
+  const half_t* vh_ptr = vc + (int64_t)head * max_pos * AWQ_HEAD_DIM;
+  // attended length of the query at position p (Inference.cu:1118 read before or after :1331)
+  auto len_of = [&](int p) { return use_len_hi ? p + 1 : (p > 1 ? p : 1); };
+  const int q_first = blockIdx.y * kFaQueries;
+  const int qi = q_first + wave * 32 + n;                 // this lane's query (a column)
+  const int qc = qi < M ? qi : M - 1;
+  const int Lq = len_of(pos0 + qc);
+  const int L_wg = len_of(pos0 + min(q_first + kFaQueries - 1, M - 1));      // lengths grow with the position
+  const int L_wave = len_of(pos0 + min(q_first + wave * 32 + 31, M - 1));
+
+  // the query's 128 components as the second operand of the 8 slices of the first product
+  half8_t qop[8];
+#pragma unroll
+  for (int s = 0; s < 8; ++s)
+    qop[s] = *reinterpret_cast<const half8_t*>(q + (int64_t)qc * H + head * AWQ_HEAD_DIM + 16 * s + 8 * kh);
+
+  f32x16_t o[4];
+#pragma unroll
+  for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) o[dt][i] = 0.0f;
+  float m_run = -1e30f, l_run = 0.0f;
+  // exp(x) = 2^(x log2 e); the scale of Inference.cu:218 folded into the same factor
+  const float scale2 = (1.0f / sqrtf((float)AWQ_HEAD_DIM)) * 1.44269504088896340736f;
+
+  for (int k0 = 0; k0 < L_wg; k0 += kFaKeys) {
+    __syncthreads();  // the previous tiles' readers are done
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int pc = tid + i * 256;
+      const int key = pc >> 4, part = pc & 15;
+      const int kg = k0 + key < L_wg ? k0 + key : L_wg - 1;  // rows past the end are masked below
+      const u32x4_t kv = *reinterpret_cast<const u32x4_t*>(kh_ptr + (int64_t)kg * AWQ_HEAD_DIM + part * 8);
+      const half8_t vv = *reinterpret_cast<const half8_t*>(vh_ptr + (int64_t)kg * AWQ_HEAD_DIM + part * 8);
+      *reinterpret_cast<u32x4_t*>(ks + key * kFaKStride + part * 8) = kv;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) vt[(part * 8 + e) * kFaVStride + key] = vv[e];
+    }
+    __syncthreads();
+    if (k0 >= L_wave) continue;  // nothing of this tile is attended by this wavefront's queries
+
+    f32x16_t sacc;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) sacc[i] = 0.0f;
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      const half8_t kop = *reinterpret_cast<const half8_t*>(ks + n * kFaKStride + 16 * s + 8 * kh);
+      sacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(kop, qop[s], sacc, 0, 0, 0);
+    }
+    // sacc[i] is the score of key k0 + 8 (i / 4) + 4 kh + i % 4 for this lane's query
+    float sv[16];
+    float mx = -1e30f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int key = k0 + 8 * (i >> 2) + 4 * kh + (i & 3);
+      sv[i] = key < Lq ? sacc[i] * scale2 : -1e30f;
+      mx = fmaxf(mx, sv[i]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m_run, mx);
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+    float rs = 0.0f;
+    half8_t pop[2];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int key = k0 + 8 * (i >> 2) + 4 * kh + (i & 3);
+      const float pe = key < Lq ? __builtin_amdgcn_exp2f(sv[i] - m_new) : 0.0f;
+      const half_t ph = (half_t)pe;
+      rs += (float)ph;  // the sum of what the second product really multiplies
+      pop[i >> 3][i & 7] = ph;
+    }
+    rs += __shfl_xor(rs, 32, 64);
+    l_run = l_run * alpha + rs;
+    m_run = m_new;
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
+    // second product: slice j takes keys 16 j + 8 (e / 4) + 4 kh + e % 4, e = 0..7, which are this
+    // lane's probabilities 8 j .. 8 j + 7
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+#pragma unroll
+      for (int dt = 0; dt < 4; ++dt) {
+        const half_t* vr = vt + (dt * 32 + n) * kFaVStride + 16 * j + 4 * kh;
+        const half4_t lo = *reinterpret_cast<const half4_t*>(vr);
+        const half4_t hi = *reinterpret_cast<const half4_t*>(vr + 8);
+        const half8_t vop = half8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vop, pop[j], o[dt], 0, 0, 0);
+      }
+    }
+  }
+  // o[dt][i] is component 32 dt + 8 (i / 4) + 4 kh + i % 4 of this lane's query
+  if (qi < M) {
+    const float inv = 1.0f / l_run;
+    half_t* out = ctx + (int64_t)qi * H + head * AWQ_HEAD_DIM;
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const half4_t v = half4_t{(half_t)(o[dt][4 * g] * inv), (half_t)(o[dt][4 * g + 1] * inv),
+                                  (half_t)(o[dt][4 * g + 2] * inv), (half_t)(o[dt][4 * g + 3] * inv)};
+        *reinterpret_cast<half4_t*>(out + dt * 32 + 8 * g + 4 * kh) = v;
+      }
+  }
+}
+
 }  // namespace
 
 int launch_embed_batch(const uint8_t* packed, const half_t* scale, const half_t* zp, int64_t hidden, int64_t vocab,
@@ -113,6 +259,16 @@ int launch_rope_kv_append_batch(const half_t* qkv, const half_t* cos_t, const ha
   AWQ_REQUIRE(M >= 1 && M <= 65535 && pos0 >= 0 && pos0 + M <= max_pos, "positions out of range");
   hipLaunchKernelGGL(rope_kv_batch_kernel, dim3((unsigned)n_heads, (unsigned)M), dim3(64), 0, st, qkv, cos_t, sin_t,
                      q_out, kc, vc, n_heads, max_pos, (int)pos0);
+  AWQ_HIP_TRY(hipGetLastError());
+  return AWQ_OK;
+}
+
+int launch_prefill_attention(const half_t* q, const half_t* kc, const half_t* vc, half_t* ctx, int n_heads,
+                             int64_t max_pos, int64_t pos0, int64_t M, int use_len_hi, hipStream_t st) {
+  AWQ_REQUIRE(n_heads > 0 && max_pos > 0, "n_heads and max_pos must be positive");
+  AWQ_REQUIRE(M >= 1 && M <= 65535 * kFaQueries && pos0 >= 0 && pos0 + M <= max_pos, "positions out of range");
+  hipLaunchKernelGGL(prefill_attention_kernel, dim3((unsigned)n_heads, (unsigned)((M + kFaQueries - 1) / kFaQueries)),
+                     dim3(256), 0, st, q, kc, vc, ctx, max_pos, (int)pos0, (int)M, use_len_hi);
   AWQ_HIP_TRY(hipGetLastError());
   return AWQ_OK;
 }

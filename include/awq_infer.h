@@ -228,6 +228,18 @@ int64_t awq_attention_workspace_bytes(int32_t n_heads, int64_t max_pos);
 int awq_decode_attention(const void* q, const void* k_cache, const void* v_cache, void* ctx, int32_t n_heads,
                          int64_t max_pos, int64_t L, void* workspace, void* stream);
 
+/* The same attention for n_tokens consecutive prompt positions pos0 ..
+ * pos0 + n_tokens - 1 at once (their keys and values already appended): q and
+ * ctx are [n_tokens][n_heads*128].  The token at position p attends p + 1
+ * positions, or, with first_layer != 0, max(p, 1): layer 0 of the prompt loop
+ * reads current_seq_len_ before it is updated (Inference.cu:1118 vs :1331).
+ * Keys and values go through LDS once per 128 queries and the products run on
+ * the matrix cores (streaming softmax, probabilities rounded to binary16), so
+ * the result agrees with awq_decode_attention to rounding noise, not bit for
+ * bit. */
+int awq_prefill_attention(const void* q, const void* k_cache, const void* v_cache, void* ctx, int32_t n_heads,
+                          int64_t max_pos, int64_t pos0, int64_t n_tokens, int32_t first_layer, void* stream);
+
 /* residual add lambda, Inference.cu:1149-1155: out = h(a + b); out may be a */
 int awq_residual_add(const void* a, const void* b, void* out, int64_t n, void* stream);
 

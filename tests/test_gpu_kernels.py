@@ -282,6 +282,40 @@ def test_decode_attention_long_sequences_bit_exact(awq, lib, oracle, torch_gpu, 
         assert np.array_equal(d_o.cpu().numpy().view(np.uint16), ref.view(np.uint16))
 
 
+@pytest.mark.parametrize("pos0,M,first_layer", [(0, 1, 1), (0, 37, 1), (0, 130, 0), (70, 150, 0), (2040, 40, 0), (5, 64, 1)])
+def test_prefill_attention_matches_the_one_query_path(awq, lib, oracle, torch_gpu, pos0, M, first_layer):
+    """attention of M prompt positions at once on the matrix cores against the oracle's one-query
+    attention with each token's own attended length; 1e-2 of the largest output magnitude"""
+    torch = torch_gpu
+    nh, mp = 4, 2112
+    rng = np.random.default_rng(pos0 * 1000 + M)
+    n_pos = pos0 + M
+    q = rng.standard_normal((M, nh * 128)).astype(np.float16)
+    kc = np.zeros((nh, mp, 128), dtype=np.float16)
+    vc = np.zeros((nh, mp, 128), dtype=np.float16)
+    kc[:, :n_pos] = (0.5 * rng.standard_normal((nh, n_pos, 128))).astype(np.float16)
+    vc[:, :n_pos] = rng.standard_normal((nh, n_pos, 128)).astype(np.float16)
+    ref = np.zeros((M, nh * 128), dtype=np.float16)
+    for t in range(M):
+        p = pos0 + t
+        L = max(p, 1) if first_layer else p + 1
+        row = np.zeros(nh * 128, dtype=np.float16)
+        oracle.awqo_attention(ptr(np.ascontiguousarray(q[t])), ptr(kc), ptr(vc), ptr(row), nh, mp, L, None)
+        ref[t] = row
+    d_q, d_k, d_v = dev(torch, q), dev(torch, kc), dev(torch, vc)
+    d_o = torch.full((M, nh * 128), float("nan"), dtype=torch.float16, device="cuda")
+    print("prefill attention", pos0, M, first_layer, flush=True)
+    awq.check(lib.awq_prefill_attention(d_q.data_ptr(), d_k.data_ptr(), d_v.data_ptr(), d_o.data_ptr(), nh, mp, pos0, M,
+                                        first_layer, stream(torch)))
+    torch.cuda.synchronize()
+    got = d_o.cpu().numpy().astype(np.float64)
+    want = ref.astype(np.float64)
+    assert np.all(np.isfinite(got))
+    assert np.abs(got - want).max() <= 1e-2 * np.abs(want).max()
+    assert lib.awq_prefill_attention(d_q.data_ptr(), d_k.data_ptr(), d_v.data_ptr(), d_o.data_ptr(), nh, mp, mp - 1, 2,
+                                     0, stream(torch)) != 0     # runs past max_pos
+
+
 def test_gelu_all_fp16_values_and_residual(awq, lib, oracle, torch_gpu):
     torch = torch_gpu
     allh = np.arange(65536, dtype=np.uint16).view(np.float16)
