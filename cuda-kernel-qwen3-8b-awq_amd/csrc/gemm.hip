@@ -9,9 +9,9 @@
 //
 // Same weight stream as the decode kernel: [16-row group][32-wide block][row][16 B],
 // dword c of a row holding elements 8c..8c+7 of the block.  Two kernels:
-//   few tokens   the decode kernel's decomposition, products on v_mfma_f32_16x16x32_f16
-//   many tokens  64 rows x 128 tokens per wavefront on v_mfma_f32_32x32x16_f16,
-//                tokens staged through LDS
+//   up to 4 tokens  the decode kernel's decomposition, products on v_mfma_f32_16x16x32_f16
+//   more tokens     64 rows x 32..128 tokens per wavefront on v_mfma_f32_32x32x16_f16,
+//                   tokens staged through LDS
 #include "common.hpp"
 
 #include <type_traits>
@@ -85,7 +85,7 @@ __device__ __forceinline__ half8_t dequant8(uint32_t v, half_t s, half_t z) {
   return half8_t{w0.x, w0.y, w1.x, w1.y, w2.x, w2.y, w3.x, w3.y};
 }
 
-// Few tokens (batched decode): the work is streaming the weights once, so the
+// Very few tokens (batched decode): the work is streaming the weights once, so the
 // decode kernel's decomposition is kept -- one workgroup per 16-row group, all
 // of k split over its wavefronts, lane (w, q, r) holding G whole blocks of row r
 // -- and only the dot products move to the matrix cores.  For a fixed b and
@@ -165,18 +165,22 @@ typedef uint32_t xvec_t __attribute__((ext_vector_type(4)));  // 16 bytes of tok
 typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 
 constexpr int kWideRP = 2;                              // 32-row pairs of row groups per wavefront
-constexpr int kWideTT = 4;                              // 32-token tiles per wavefront
+constexpr int kWideTT = 4;                              // 32-token tiles per wavefront (1 or 2 for few tokens, k split)
 constexpr int kWideTokens = 32 * kWideTT;               // 128
 constexpr int kWideNH = 2;                              // 32-wide blocks of k per step
 constexpr int kWideStride = 32 * kWideNH + 8;           // halves per token row of a tile in LDS (16 bytes of padding)
-constexpr int kWideSlot = kWideTokens * kWideStride;    // halves per token tile in LDS
-constexpr int kWideLdsRows = 2 * kWideSlot * 2;                          // bytes, rows split
-constexpr int kWideLdsK = 4 * kWideRP * kWideTT * 64 * 16 * 4;           // bytes, k split: the partial sums
+constexpr int wide_lds_bytes(bool ksplit, int tt) {
+  const int tiles = (ksplit ? 4 : 1) * 2 * (32 * tt) * kWideStride * 2;  // slots x double buffer x tile
+  const int sums = 4 * kWideRP * tt * 64 * 16 * 4;                       // k split: the partial sums
+  return ksplit && sums > tiles ? sums : tiles;
+}
 
-template <bool ZINT, bool KSPLIT, int EPI>
-__global__ __launch_bounds__(256, KSPLIT ? 1 : 2) void gemm_wide_kernel(GemmParams p) {
+template <bool ZINT, bool KSPLIT, int EPI, int TT>
+__global__ __launch_bounds__(256, (KSPLIT && TT == 4) ? 1 : 2) void gemm_wide_kernel(GemmParams p) {
+  constexpr int kTokens = 32 * TT;                   // tokens per workgroup
+  constexpr int kSlot = kTokens * kWideStride;       // halves per token tile in LDS
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  half_t* xs = reinterpret_cast<half_t*>(smem_raw);  // [2][NKB][128 tokens][kWideStride]
+  half_t* xs = reinterpret_cast<half_t*>(smem_raw);  // [2][NKB][32 TT tokens][kWideStride]
   constexpr int NKB = KSPLIT ? 4 : 1;
   constexpr int NH = kWideNH;
   const int tid = threadIdx.x, lane = tid & 63;
@@ -184,7 +188,7 @@ __global__ __launch_bounds__(256, KSPLIT ? 1 : 2) void gemm_wide_kernel(GemmPara
   const int n = lane & 31, kh = lane >> 5;
   const int rg0 = KSPLIT ? blockIdx.x * 4 : (blockIdx.x * 4 + wave) * 4;  // first of this wavefront's 4 row groups
   const bool rows_ok = rg0 * 16 < p.m;  // rows split: the last workgroup may hang over the edge
-  const int t0 = blockIdx.y * kWideTokens;
+  const int t0 = blockIdx.y * kTokens;
   // a step is NH blocks of k; the step count is even (checked by the launcher)
   const int steps = (KSPLIT ? p.nblk / (4 * p.kz) : p.nblk) / NH;
   // first block of this workgroup's chunk of k (k split only), then of this wavefront's quarter of it
@@ -201,7 +205,7 @@ __global__ __launch_bounds__(256, KSPLIT ? 1 : 2) void gemm_wide_kernel(GemmPara
   // before its use and written to LDS one step before.  The main loop has no
   // conditionals: loads past the end repeat the last tile (never used), tokens
   // past M repeat token M-1 (never stored).
-  constexpr int PCS = kWideTokens * 4 * NH;  // pieces per slot
+  constexpr int PCS = kTokens * 4 * NH;  // pieces per slot
   constexpr int PPT = NKB * PCS / 256;
   const half_t* xsrc[PPT];
   int xdst[PPT];
@@ -211,7 +215,7 @@ __global__ __launch_bounds__(256, KSPLIT ? 1 : 2) void gemm_wide_kernel(GemmPara
     const int j = pc / PCS, tok = (pc % PCS) / (4 * NH), part = pc % (4 * NH);
     const int tg = t0 + tok < p.M ? t0 + tok : p.M - 1;
     xsrc[i] = p.x + (int64_t)tg * p.k + (kb_wg + (KSPLIT ? j * steps * NH : 0)) * 32 + part * 8;
-    xdst[i] = j * kWideSlot + tok * kWideStride + part * 8;
+    xdst[i] = j * kSlot + tok * kWideStride + part * 8;
   }
   xvec_t xr0[PPT], xr1[PPT];  // two named register sets (an indexed array would live in scratch memory)
   auto load_x = [&](int s, xvec_t (&dst)[PPT]) __attribute__((always_inline)) {
@@ -221,7 +225,7 @@ __global__ __launch_bounds__(256, KSPLIT ? 1 : 2) void gemm_wide_kernel(GemmPara
   };
   auto store_x = [&](int buf, const xvec_t (&src)[PPT]) __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < PPT; ++i) *reinterpret_cast<xvec_t*>(xs + buf * NKB * kWideSlot + xdst[i]) = src[i];
+    for (int i = 0; i < PPT; ++i) *reinterpret_cast<xvec_t*>(xs + buf * NKB * kSlot + xdst[i]) = src[i];
   };
 
   // weights: row n of pair rp is row n % 16 of row group rg0 + 2 rp + n / 16; dwords 2kh, 2kh + 1 of its block
@@ -240,11 +244,11 @@ __global__ __launch_bounds__(256, KSPLIT ? 1 : 2) void gemm_wide_kernel(GemmPara
 #pragma unroll
       for (int a = 0; a < kWideRP; ++a) wd[a][f][h] = KSPLIT ? __builtin_nontemporal_load(wp[a] + (int64_t)(f * NH + h) * 32) : wp[a][(int64_t)(f * NH + h) * 32];
 
-  f32x16_t acc[kWideRP][kWideTT];
+  f32x16_t acc[kWideRP][TT];
 #pragma unroll
   for (int a = 0; a < kWideRP; ++a)
 #pragma unroll
-    for (int t = 0; t < kWideTT; ++t)
+    for (int t = 0; t < TT; ++t)
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[a][t][i] = 0.0f;
 
@@ -259,7 +263,7 @@ __global__ __launch_bounds__(256, KSPLIT ? 1 : 2) void gemm_wide_kernel(GemmPara
     if constexpr (f & 1) load_x(s + 2, xr1);
     else load_x(s + 2, xr0);
     __syncthreads();  // tile s is in buffer s & 1; the readers of tile s-1 are done
-    const half_t* xb = xs + ((s & 1) * NKB + slot) * kWideSlot + n * kWideStride + 16 * kh;
+    const half_t* xb = xs + ((s & 1) * NKB + slot) * kSlot + n * kWideStride + 16 * kh;
     const int sn = s + PF < steps ? s + PF : steps - 1;
 #pragma unroll
     for (int h = 0; h < NH; ++h) {
@@ -271,7 +275,7 @@ __global__ __launch_bounds__(256, KSPLIT ? 1 : 2) void gemm_wide_kernel(GemmPara
         wd[a][f][h] = KSPLIT ? __builtin_nontemporal_load(wp[a] + (int64_t)(sn * NH + h) * 32) : wp[a][(int64_t)(sn * NH + h) * 32];
       }
 #pragma unroll
-      for (int t = 0; t < kWideTT; ++t) {
+      for (int t = 0; t < TT; ++t) {
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
           // slice j: k = 8 (j + 2 kh) .. + 7 of block h
@@ -297,7 +301,7 @@ __global__ __launch_bounds__(256, KSPLIT ? 1 : 2) void gemm_wide_kernel(GemmPara
     for (int a = 0; a < kWideRP; ++a) {
       const int row = rg0 * 16 + a * 32 + n;
 #pragma unroll
-      for (int t = 0; t < kWideTT; ++t) {
+      for (int t = 0; t < TT; ++t) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
           const int tok = t0 + t * 32 + (i >> 2) * 8 + kh * 4 + (i & 3);
@@ -308,16 +312,16 @@ __global__ __launch_bounds__(256, KSPLIT ? 1 : 2) void gemm_wide_kernel(GemmPara
     return;
   }
   // k split: the four partial sums of every output meet in LDS (the token tiles
-  // are dead by now); wavefront w finishes token tile w
+  // are dead by now); wavefront w finishes quarter w of every accumulator tile
   float4_t* red = reinterpret_cast<float4_t*>(smem_raw);  // [wave][pair][tile][quarter][lane]
   __syncthreads();
 #pragma unroll
   for (int a = 0; a < kWideRP; ++a)
 #pragma unroll
-    for (int t = 0; t < kWideTT; ++t)
+    for (int t = 0; t < TT; ++t)
 #pragma unroll
       for (int i4 = 0; i4 < 4; ++i4)
-        red[(((wave * kWideRP + a) * kWideTT + t) * 4 + i4) * 64 + lane] =
+        red[(((wave * kWideRP + a) * TT + t) * 4 + i4) * 64 + lane] =
             float4_t{acc[a][t][4 * i4], acc[a][t][4 * i4 + 1], acc[a][t][4 * i4 + 2], acc[a][t][4 * i4 + 3]};
   __syncthreads();
   auto finish = [&](auto E) {
@@ -325,12 +329,12 @@ __global__ __launch_bounds__(256, KSPLIT ? 1 : 2) void gemm_wide_kernel(GemmPara
 #pragma unroll
     for (int a = 0; a < kWideRP; ++a) {
       const int row = rg0 * 16 + a * 32 + n;
-      const int t = wave;
+      const int i4 = wave;
 #pragma unroll
-      for (int i4 = 0; i4 < 4; ++i4) {
-        float4_t v = red[(((0 * kWideRP + a) * kWideTT + t) * 4 + i4) * 64 + lane];
+      for (int t = 0; t < TT; ++t) {
+        float4_t v = red[(((0 * kWideRP + a) * TT + t) * 4 + i4) * 64 + lane];
 #pragma unroll
-        for (int w = 1; w < 4; ++w) v += red[(((w * kWideRP + a) * kWideTT + t) * 4 + i4) * 64 + lane];
+        for (int w = 1; w < 4; ++w) v += red[(((w * kWideRP + a) * TT + t) * 4 + i4) * 64 + lane];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int tok = t0 + t * 32 + i4 * 8 + kh * 4 + i;
@@ -357,21 +361,24 @@ __global__ __launch_bounds__(256) void reduce_parts_kernel(GemmParams p) {
   with_epilogue(p, [&](auto E) { store_out<decltype(E)::value>(p, (int)(at / p.m), (int)(at % p.m), v); });
 }
 
-template <bool KSPLIT>
+// tokens per workgroup of the k-split shape: 32, 64 or 128
+int wide_tt(int64_t M) { return M <= 32 ? 1 : (M <= 64 ? 2 : 4); }
+
+template <bool KSPLIT, int TT>
 int launch_wide(const GemmParams& p, bool zint, hipStream_t st) {
   // the main loop takes two steps of two 32-wide blocks per trip (per quarter of k when k is split)
   AWQ_REQUIRE(p.nblk % (KSPLIT ? 16 * p.kz : 4) == 0, "k must be a multiple of 512");
-  const int lds = KSPLIT ? (kWideLdsK > 4 * kWideLdsRows ? kWideLdsK : 4 * kWideLdsRows) : kWideLdsRows;
-  static_assert(4 * kWideLdsRows <= 160 * 1024 && kWideLdsK <= 160 * 1024, "LDS of one compute unit");
+  constexpr int lds = wide_lds_bytes(KSPLIT, TT);
+  static_assert(lds <= 160 * 1024, "LDS of one compute unit");
   const unsigned gx = KSPLIT ? (unsigned)(p.m / 64) : (unsigned)((p.m + 255) / 256);
-  dim3 grid(gx, (unsigned)((p.M + kWideTokens - 1) / kWideTokens), KSPLIT ? (unsigned)p.kz : 1u);
+  dim3 grid(gx, (unsigned)((p.M + 32 * TT - 1) / (32 * TT)), KSPLIT ? (unsigned)p.kz : 1u);
   void (*kern)(GemmParams);
   if (p.epilogue == EPI_RESIDUAL)
-    kern = zint ? gemm_wide_kernel<true, KSPLIT, EPI_RESIDUAL> : gemm_wide_kernel<false, KSPLIT, EPI_RESIDUAL>;
+    kern = zint ? gemm_wide_kernel<true, KSPLIT, EPI_RESIDUAL, TT> : gemm_wide_kernel<false, KSPLIT, EPI_RESIDUAL, TT>;
   else if (p.epilogue == EPI_GELU)
-    kern = zint ? gemm_wide_kernel<true, KSPLIT, EPI_GELU> : gemm_wide_kernel<false, KSPLIT, EPI_GELU>;
+    kern = zint ? gemm_wide_kernel<true, KSPLIT, EPI_GELU, TT> : gemm_wide_kernel<false, KSPLIT, EPI_GELU, TT>;
   else
-    kern = zint ? gemm_wide_kernel<true, KSPLIT, EPI_STORE> : gemm_wide_kernel<false, KSPLIT, EPI_STORE>;
+    kern = zint ? gemm_wide_kernel<true, KSPLIT, EPI_STORE, TT> : gemm_wide_kernel<false, KSPLIT, EPI_STORE, TT>;
   if (lds > 65536) {
     // more LDS than a launch gets by default: raise this kernel's limit (per device; cheap, so every time)
     AWQ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds));
@@ -395,8 +402,9 @@ void launch_small(const GemmParams& p, bool zint, int n_waves, dim3 grid, hipStr
 // room for the partial sums of a product whose k is cut over workgroups (0: never cut)
 int64_t gemm_workspace_bytes(int64_t m, int64_t k, int64_t M) {
   (void)k;
-  if (M <= 16 || (M <= 32 && m < 8192)) return 0;
-  const int64_t wgs = (m / 64) * ((M + kWideTokens - 1) / kWideTokens);
+  if (M <= 4) return 0;
+  const int tokens = 32 * wide_tt(M);
+  const int64_t wgs = (m / 64) * ((M + tokens - 1) / tokens);
   return wgs <= 128 ? 4 * M * m * 4 : 0;
 }
 
@@ -425,9 +433,9 @@ int launch_gemm(const void* wq, const half_t* scale, const half_t* zp, int64_t m
   p.res = res;
   p.kz = 1;
   p.part = nullptr;
-  // up to 16 tokens, and up to 32 on a matrix with few rows: the decode kernel's decomposition
+  // up to 4 tokens: the decode kernel's decomposition (one 16-token operand tile, mostly padding)
   int g = 0;
-  if (M <= 16 || (M <= 32 && m < 8192)) {
+  if (M <= 4) {
     // lane groups of G blocks: (k/32)/G of them, a multiple of 4 and at most 64
     const int64_t nblk = k / AWQ_BLOCK_K;
     for (int c : {8, 4, 2, 1})
@@ -438,23 +446,23 @@ int launch_gemm(const void* wq, const half_t* scale, const half_t* zp, int64_t m
   }
   if (g) {
     const int n_waves = (int)(k / AWQ_BLOCK_K / g / 4);
-    const bool one = M <= 16;
-    dim3 grid((unsigned)(m / 16), (unsigned)((M + (one ? 15 : 63)) / (one ? 16 : 64)));
+    dim3 grid((unsigned)(m / 16), 1);
     switch (g) {
-      case 8: one ? launch_small<8, 1>(p, zp_integral, n_waves, grid, st) : launch_small<8, 4>(p, zp_integral, n_waves, grid, st); break;
-      case 4: one ? launch_small<4, 1>(p, zp_integral, n_waves, grid, st) : launch_small<4, 4>(p, zp_integral, n_waves, grid, st); break;
-      case 2: one ? launch_small<2, 1>(p, zp_integral, n_waves, grid, st) : launch_small<2, 4>(p, zp_integral, n_waves, grid, st); break;
-      default: one ? launch_small<1, 1>(p, zp_integral, n_waves, grid, st) : launch_small<1, 4>(p, zp_integral, n_waves, grid, st); break;
+      case 8: launch_small<8, 1>(p, zp_integral, n_waves, grid, st); break;
+      case 4: launch_small<4, 1>(p, zp_integral, n_waves, grid, st); break;
+      case 2: launch_small<2, 1>(p, zp_integral, n_waves, grid, st); break;
+      default: launch_small<1, 1>(p, zp_integral, n_waves, grid, st); break;
     }
   } else {
     // enough 256-row x 128-token tiles to fill half the device: rows split; otherwise k split
     const int64_t tiles = ((m + 255) / 256) * ((M + kWideTokens - 1) / kWideTokens);
     if (tiles >= 128) {
-      if (int rc = launch_wide<false>(p, zp_integral, st)) return rc;
+      if (int rc = launch_wide<false, 4>(p, zp_integral, st)) return rc;
     } else {
       // few 64-row workgroups too (a matrix with few rows): cut k over 4 or 2 workgroups as well,
       // when the caller brought room for the partial sums
-      const int64_t wgs = (m / 64) * ((M + kWideTokens - 1) / kWideTokens);
+      const int tt = wide_tt(M);
+      const int64_t wgs = (m / 64) * ((M + 32 * tt - 1) / (32 * tt));
       if (wgs <= 128 && workspace) {
         for (int kz : {4, 2})
           if (p.nblk % (16 * kz) == 0 && (int64_t)kz * M * m * 4 <= workspace_bytes) {
@@ -463,7 +471,10 @@ int launch_gemm(const void* wq, const half_t* scale, const half_t* zp, int64_t m
             break;
           }
       }
-      if (int rc = launch_wide<true>(p, zp_integral, st)) return rc;
+      if (int rc = tt == 1 ? launch_wide<true, 1>(p, zp_integral, st)
+                           : tt == 2 ? launch_wide<true, 2>(p, zp_integral, st)
+                                     : launch_wide<true, 4>(p, zp_integral, st))
+        return rc;
     }
   }
   AWQ_HIP_TRY(hipGetLastError());
