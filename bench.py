@@ -126,6 +126,23 @@ def main():
         kernels[name] = {"us": round(us, 3), "bytes": nbytes, "GBs": round(nbytes / us / 1e3, 1)}
         log("gemv %-8s %8.2f us/launch  %7.1f GB/s  (%.1f%% of peak)" % (name, us, nbytes / us / 1e3,
                                                                         nbytes / us / 1e3 / HBM_PEAK_GBS * 100))
+    # the same launches on ONE layer's matrices (25 MB, resident in the last-level cache): the
+    # cache-hot figure next to the rotating one above
+    hot_cfg = awq.make_config(n_layers=1, max_pos=64)
+    hot = awq.QWen3AWQInfer.empty(hot_cfg)
+    for layer, kind, part in awq.tensor_list(hot_cfg):
+        count = hot_cfg.part_count(kind, part)
+        nbytes = count if (part == awq.P_PACKED and kind != awq.T_GAMMA) else 2 * count
+        buf = (ctypes.c_uint8 * nbytes)()
+        awq.check(lib.awq_synth_fill_profile(profile, args.seed, layer, kind, part, buf, count))
+        hot.upload(layer, kind, part, buf, nbytes)
+    hot.finalize()
+    for name, kind in (("w1", awq.T_W1), ("wqkv", awq.T_WQKV), ("w2", awq.T_W2), ("wo", awq.T_WO)):
+        us, _ = hot.time_linear(kind, 400)
+        kernels[name]["us_cache_hot"] = round(us, 3)
+    hot.close()
+    log("cache-hot (one layer's matrices): " + ", ".join("%s %.2f us" % (n, kernels[n]["us_cache_hot"])
+                                                         for n in ("w1", "wqkv", "w2", "wo")))
     traffic = None
     tpath = os.path.join(ROOT, "profiles", "gemv_w1_traffic.json")
     if os.path.exists(tpath):
