@@ -57,14 +57,24 @@ __device__ __forceinline__ void with_epilogue(const GemmParams& p, F&& f) {
   else f(std::integral_constant<int, EPI_STORE>{});
 }
 
+// (x & mask) | 0x64006400 in one instruction; the three-operand encoding takes no
+// literal, so the mask travels in a scalar register and the exponent pattern in
+// a vector register
+__device__ __forceinline__ uint32_t and_or_magic(uint32_t x, uint32_t mask) {
+  uint32_t r;
+  const uint32_t magic = 0x64006400u;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "s"(mask), "v"(magic));
+  return r;
+}
+
 // 8 nibbles of one dword -> 8 binary16 weights in element order, h(h(q-z)*s)
 template <bool ZINT>
 __device__ __forceinline__ half8_t dequant8(uint32_t v, half_t s, half_t z) {
   const half2_t s2 = half2_t{s, s};
   const half2_t k16 = half2_t{(half_t)0.0625f, (half_t)0.0625f};
   const uint32_t v8 = v >> 8;
-  const half2_t lo0 = as_half2((v & 0x000f000fu) | 0x64006400u), hi0 = as_half2((v & 0x00f000f0u) | 0x64006400u);
-  const half2_t lo1 = as_half2((v8 & 0x000f000fu) | 0x64006400u), hi1 = as_half2((v8 & 0x00f000f0u) | 0x64006400u);
+  const half2_t lo0 = as_half2(and_or_magic(v, 0x000f000fu)), hi0 = as_half2(and_or_magic(v, 0x00f000f0u));
+  const half2_t lo1 = as_half2(and_or_magic(v8, 0x000f000fu)), hi1 = as_half2(and_or_magic(v8, 0x00f000f0u));
   half2_t u0, u1, u2, u3;
   if (ZINT) {
     const half_t a = -((half_t)1024.0f + z), b = -((half_t)64.0f + z);
@@ -274,10 +284,12 @@ __global__ __launch_bounds__(256, (KSPLIT && TT == 4) ? 1 : 2) void gemm_wide_ke
         wop[a][1] = dequant8<ZINT>(wd[a][f][h].y, sc, zz);
         wd[a][f][h] = KSPLIT ? __builtin_nontemporal_load(wp[a] + (int64_t)(sn * NH + h) * 32) : wp[a][(int64_t)(sn * NH + h) * 32];
       }
+      // slices outermost: an accumulator tile is touched again only after all the others (a
+      // matrix-core instruction that needs the previous result of its accumulator waits for it)
 #pragma unroll
-      for (int t = 0; t < TT; ++t) {
+      for (int j = 0; j < 2; ++j) {
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
+        for (int t = 0; t < TT; ++t) {
           // slice j: k = 8 (j + 2 kh) .. + 7 of block h
           const half8_t xop = *reinterpret_cast<const half8_t*>(xb + t * 32 * kWideStride + h * 32 + 8 * j);
 #pragma unroll
