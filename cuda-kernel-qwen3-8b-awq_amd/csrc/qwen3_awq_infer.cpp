@@ -23,3 +23,7 @@ std::vector<int> QWen3AWQInfer::generateResponse(const std::vector<int>& prompt_
   die_on(awq_generate(engine_, prompt.data(), (int32_t)prompt.size(), max_new_tokens, out.data()), "generateResponse");
   return std::vector<int>(out.begin(), out.end());
 }
+
+void QWen3AWQInfer::setBatchedPrefill(bool enabled) {
+  die_on(awq_set_prefill_mode(engine_, enabled ? 1 : 0), "setBatchedPrefill");
+}

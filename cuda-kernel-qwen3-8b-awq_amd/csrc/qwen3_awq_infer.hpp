@@ -20,6 +20,12 @@ class QWen3AWQInfer {
   // returns only the newly generated token IDs (Inference.cu:361-366)
   std::vector<int> generateResponse(const std::vector<int>& prompt_ids, int max_new_tokens);
 
+  // Not in the reference: send all prompt positions through each layer together
+  // (one W4A16 matrix product per weight matrix instead of one matrix-vector
+  // product per prompt token, Inference.cu:1304-1343).  Same state up to
+  // binary16 rounding noise; off by default.
+  void setBatchedPrefill(bool enabled);
+
  private:
   awq_engine* engine_;
 };
