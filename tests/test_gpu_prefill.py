@@ -179,3 +179,36 @@ def test_long_prompt_takes_the_rows_split_products(awq, oracle, torch_gpu):
     assert np.isfinite(hid_seq).all() and close(hid_seq, hid_bat)
     assert tok_bat[0] == tok_seq[0]
     eng.close()
+
+
+def test_maximum_sequence_length_one_layer(awq, oracle, torch_gpu):
+    """The reference's MAX_POSITION_EMBEDDINGS (40960, Inference.cu:39) on one full-width layer: a
+    40,950-token prompt through the batched pass and, token by token, through the bit-exact decode
+    kernels (attention cut along the sequence beyond 2048 positions), then generation up to the
+    last position; one more token is an error, not a cache overrun."""
+    cfg = awq.make_config(n_layers=1, vocab=2048, max_pos=40960)
+    model = make_oracle_model(oracle, cfg)   # only as the host buffer of the weights here
+    eng = awq.QWen3AWQInfer.empty(cfg)
+    fill_pair(awq, oracle, cfg, 40, engine=eng, model=model, profile=awq.SYNTH_BALANCED)
+    oracle.awqo_model_destroy(model)
+    rng = np.random.default_rng(40960)
+    prompt = rng.integers(0, cfg.vocab, 40950).tolist()
+    print("maximum sequence length: batched prompt pass", flush=True)
+    eng.reset()
+    eng.prefill(prompt, batched=True)
+    hid_bat = as_f32(eng.read_hidden()).copy()
+    tok_bat = eng.decode(10)            # positions 40950 .. 40959
+    with pytest.raises(awq.AwqError):
+        eng.decode(1)
+    print("maximum sequence length: token by token", flush=True)
+    eng.reset()
+    eng.prefill(prompt)
+    hid_seq = as_f32(eng.read_hidden()).copy()
+    tok_seq = eng.decode(10)
+    print("hidden: max |seq - batched| = %.5f at scale %.3f; tokens %s / %s" %
+          (np.abs(hid_seq - hid_bat).max(), np.abs(hid_seq).max(), tok_seq, tok_bat), flush=True)
+    assert np.isfinite(hid_seq).all() and close(hid_seq, hid_bat)
+    assert tok_seq[0] == tok_bat[0]
+    with pytest.raises(awq.AwqError):
+        eng.generateResponse(prompt, 11)   # 40950 + 11 > 40960
+    eng.close()
