@@ -147,7 +147,22 @@ __global__ __launch_bounds__(256) void fill_zero_kernel(uint32_t* p, int64_t n_w
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n_words; i += (int64_t)gridDim.x * 256) p[i] = 0;
 }
 
+__global__ __launch_bounds__(256) void copy_kernel(const uint32_t* __restrict__ src, uint32_t* __restrict__ dst,
+                                                   int64_t n_words) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n_words; i += (int64_t)gridDim.x * 256) dst[i] = src[i];
+}
+
 }  // namespace
+
+int launch_copy(const void* src, void* dst, int64_t bytes, hipStream_t st) {
+  AWQ_REQUIRE(bytes % 4 == 0 && bytes >= 0, "byte count must be a multiple of 4");
+  if (bytes == 0) return AWQ_OK;
+  int64_t words = bytes / 4, blocks = (words + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  hipLaunchKernelGGL(copy_kernel, dim3((unsigned)blocks), dim3(256), 0, st, (const uint32_t*)src, (uint32_t*)dst, words);
+  AWQ_HIP_TRY(hipGetLastError());
+  return AWQ_OK;
+}
 
 int launch_rmsnorm(const half_t* x, const half_t* gamma, half_t* out, int64_t n, float eps, hipStream_t st) {
   AWQ_REQUIRE(n > 0 && n % 256 == 0 && n < (1 << 30), "n must be a positive multiple of 256");

@@ -51,13 +51,15 @@ def test_small_model_sequence_crossing_2048_positions(awq, oracle, torch_gpu):
     oracle.awqo_model_destroy(model)
 
 
-@pytest.mark.parametrize("graph", [False, True])
-def test_small_model_tokens_and_state_identical(awq, oracle, torch_gpu, graph):
+@pytest.mark.parametrize("graph,flow", [(False, False), (True, False), (False, True), (True, True)])
+def test_small_model_tokens_and_state_identical(awq, oracle, torch_gpu, graph, flow):
+    """flow: the products after a layer's attention as dependent workgroup ranges of one launch"""
     cfg = awq.make_config(**SMALL)
     model = make_oracle_model(oracle, cfg)
     eng = awq.QWen3AWQInfer.empty(cfg)
     fill_pair(awq, oracle, cfg, 1234, engine=eng, model=model)
     eng.set_graph_mode(graph)
+    eng.set_flow_mode(flow)
     prompt = [3, 1000, 77, 512, 9]
     print("small model generate graph=", graph, flush=True)
     got = eng.generateResponse(prompt, 24)
@@ -222,7 +224,8 @@ def test_config2_one_decoder_layer_at_position_512(awq, lib, oracle, torch_gpu):
     oracle.awqo_model_destroy(model)
 
 
-def test_full_model_32_greedy_tokens_identical(awq, oracle, torch_gpu):
+@pytest.mark.parametrize("flow", [False, True])
+def test_full_model_32_greedy_tokens_identical(awq, oracle, torch_gpu, flow):
     """config 4 at reduced length: all 36 layers at the reference widths, random-init seeded weights, greedy
     decode of 32 tokens; ids, final hidden state and last logits must equal the CPU path bit for bit.
     Weights come from the balanced profile (include/awq_synth.h): with the benchmark's own distributions the
@@ -234,6 +237,7 @@ def test_full_model_32_greedy_tokens_identical(awq, oracle, torch_gpu):
     model = make_oracle_model(oracle, cfg)
     eng = awq.QWen3AWQInfer.empty(cfg)
     fill_pair(awq, oracle, cfg, 2025, engine=eng, model=model, profile=awq.SYNTH_BALANCED)
+    eng.set_flow_mode(flow)
     prompt = np.zeros(4, dtype=np.int32)
     awq.check(awq.load_library().awq_synth_tokens(2025, awq.SYNTH_STREAM_INPUT, ptr(prompt), prompt.size, cfg.vocab))
     print("36-layer model: 32 greedy tokens", flush=True)
