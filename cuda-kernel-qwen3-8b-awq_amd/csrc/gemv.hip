@@ -267,7 +267,10 @@ __device__ __forceinline__ int xs_index(int e) {
 // one by one: the first 16 dwords of the argument block are preloaded into
 // scalar registers at wavefront launch (see the build flags), which takes one
 // memory round trip off the start of the kernel.
-template <int G, bool ZINT, bool PERIODIC>
+// UFAST (periodic matrices only): the class length k/32/C when it is known at
+// compile time and divides G, so that a lane's G blocks are G/UFAST whole classes
+// whose constants it reads once per row group; 0 = look the class up per block.
+template <int G, bool ZINT, bool PERIODIC, int UFAST = 0>
 __global__ __launch_bounds__(1024) void gemv_kernel(const u32x4* __restrict__ wq, const half_t* __restrict__ x,
                                                     const half_t* __restrict__ gamma, const half_t* __restrict__ scale,
                                                     const half_t* __restrict__ zp, int32_t k, int32_t nblk,
@@ -275,9 +278,9 @@ __global__ __launch_bounds__(1024) void gemv_kernel(const u32x4* __restrict__ wq
                                                     GemvParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   half_t* xs = reinterpret_cast<half_t*>(smem);  // x in block order, k halves
-  __shared__ float red[16][16];
+  __shared__ float red[2][16][16];  // double-buffered: one barrier per row group
   __shared__ float nbuf[256];
-  __shared__ GroupConst gtab[PERIODIC ? 64 : 1];
+  __shared__ GroupConst gtab[2][PERIODIC ? 64 : 1];
   constexpr int MAXU = 8;  // 8-byte units of x a thread may hold in registers
 
   const int tid = threadIdx.x;
@@ -384,7 +387,15 @@ __global__ __launch_bounds__(1024) void gemv_kernel(const u32x4* __restrict__ wq
     if (tid + u * nthreads < total_units)
       *reinterpret_cast<uint2*>(xs + xs_index<G>(4 * (tid + u * nthreads))) = xu[u];
 
-  for (; rg < n_rg; rg += gridDim.x) {
+  // Group constants.  When the scale group depends on the input index it is
+  // constant within a class of blocks; the (at most 64) classes of a row group
+  // go through a table in LDS, filled one row group ahead.
+  if (PERIODIC && tid < C && rg < n_rg) {
+    int gi = (int)((((int64_t)tid * p.mg + (rg >> 3)) % p.kg) % p.mg);
+    gtab[0][tid] = make_group<ZINT>(scale[gi], zp[gi]);
+  }
+  __syncthreads();  // xs and the first table
+  for (int it = 0; rg < n_rg; rg += gridDim.x, ++it) {
     const int rg_next = rg + gridDim.x;
     if (rg_next < n_rg) {
       const u32x4* wpn = wq + ((int64_t)rg_next * nblk + blk0) * 16 + r;
@@ -392,36 +403,43 @@ __global__ __launch_bounds__(1024) void gemv_kernel(const u32x4* __restrict__ wq
       for (int b = 0; b < G; ++b) wn[b] = __builtin_nontemporal_load(wpn + b * 16);
     }
     // scale group of these 16 rows: row/128, then Inference.cu:90 with the index
-    // wrapped to the m/128 stored entries.  When the group depends on the input
-    // index it is constant within a class of blocks; the (at most 64) classes go
-    // through a table in LDS.
+    // wrapped to the m/128 stored entries
     const int a = rg >> 3;
     GroupConst g;
     if (!PERIODIC) {
       int gi = (a % p.kg) % p.mg;
       g = make_group<ZINT>(scale[gi], zp[gi]);
-    } else if (tid < C) {
-      int gi = (int)((((int64_t)tid * p.mg + a) % p.kg) % p.mg);
-      gtab[tid] = make_group<ZINT>(scale[gi], zp[gi]);
+    } else if (tid < C && rg_next < n_rg) {
+      // the next row group's table; its buffer was last read two barriers ago
+      int gi = (int)((((int64_t)tid * p.mg + (rg_next >> 3)) % p.kg) % p.mg);
+      gtab[(it + 1) & 1][tid] = make_group<ZINT>(scale[gi], zp[gi]);
     }
     int cls = 0, cls_left = 0;  // class of the next block and blocks left in it
     if (PERIODIC) {
       cls = blk0 / U;
       cls_left = U - (blk0 - cls * U);
     }
-    __syncthreads();  // xs (first pass), gtab, and the previous pass's use of red
-
     float bs[G];
+    if (PERIODIC && UFAST > 0) {
+      constexpr int NC = UFAST > 0 ? G / UFAST : 1;
+      GroupConst gc[NC];
 #pragma unroll
-    for (int b = 0; b < G; ++b) {
-      if (PERIODIC) {
-        g = gtab[cls];
-        if (--cls_left == 0) {
-          ++cls;
-          cls_left = U;
+      for (int c = 0; c < NC; ++c) gc[c] = gtab[it & 1][blk0 / UFAST + c];
+#pragma unroll
+      for (int b = 0; b < G; ++b)
+        bs[b] = block_dot<ZINT>(w[b], xs + xs_index<G>((blk0 + b) * AWQ_BLOCK_K), gc[UFAST > 0 ? b / UFAST : 0]);
+    } else {
+#pragma unroll
+      for (int b = 0; b < G; ++b) {
+        if (PERIODIC) {
+          g = gtab[it & 1][cls];
+          if (--cls_left == 0) {
+            ++cls;
+            cls_left = U;
+          }
         }
+        bs[b] = block_dot<ZINT>(w[b], xs + xs_index<G>((blk0 + b) * AWQ_BLOCK_K), g);
       }
-      bs[b] = block_dot<ZINT>(w[b], xs + xs_index<G>((blk0 + b) * AWQ_BLOCK_K), g);
     }
     // adjacent-pair tree: this lane's G blocks, then the four quarters of the
     // wavefront (consecutive block ranges), then the wavefronts
@@ -433,16 +451,20 @@ __global__ __launch_bounds__(1024) void gemv_kernel(const u32x4* __restrict__ wq
     float v = bs[0];
     v += __shfl_xor(v, 16, 64);
     v += __shfl_xor(v, 32, 64);
-    if (q == 0) red[wave][r] = v;
+    // The only barrier of the pass.  The 16 finishing lanes read this pass's
+    // buffer while the other wavefronts already multiply the next row group; the
+    // buffer is written again two passes on, after a barrier those lanes are part of.
+    float(*rd)[16] = red[it & 1];
+    if (q == 0) rd[wave][r] = v;
     __syncthreads();
     if (tid < 16) {
       int n = n_waves;
       while (n > 1 && (n & 1) == 0) {
         n >>= 1;
-        for (int i = 0; i < n; ++i) red[i][r] = red[2 * i][r] + red[2 * i + 1][r];
+        for (int i = 0; i < n; ++i) rd[i][r] = rd[2 * i][r] + rd[2 * i + 1][r];
       }
-      float tot = red[0][r];
-      for (int i = 1; i < n; ++i) tot += red[i][r];
+      float tot = rd[0][r];
+      for (int i = 1; i < n; ++i) tot += rd[i][r];
       epilogue(p, rg * 16 + r, r, tot);
     }
 #pragma unroll
@@ -792,6 +814,11 @@ bool plan_gemv(int64_t m, int64_t k, GemvPlan* out) {
 #define GEMV_HOT_ARGS p.wq, p.x, p.gamma, p.scale, p.zp, p.k, p.nblk, p.n_waves, p.m, p.prologue, p.C
 template <int G>
 void launch_g(const GemvParams& p, bool zint, bool periodic, dim3 grid, dim3 block, size_t lds, hipStream_t st) {
+  if (G == 8 && periodic && p.nblk / p.C == 4) {  // the unembedding: classes of 4 blocks
+    if (zint) hipLaunchKernelGGL((gemv_kernel<G, true, true, G == 8 ? 4 : 0>), grid, block, lds, st, GEMV_HOT_ARGS, p);
+    else hipLaunchKernelGGL((gemv_kernel<G, false, true, G == 8 ? 4 : 0>), grid, block, lds, st, GEMV_HOT_ARGS, p);
+    return;
+  }
   if (zint) {
     if (periodic) hipLaunchKernelGGL((gemv_kernel<G, true, true>), grid, block, lds, st, GEMV_HOT_ARGS, p);
     else hipLaunchKernelGGL((gemv_kernel<G, true, false>), grid, block, lds, st, GEMV_HOT_ARGS, p);
