@@ -139,3 +139,16 @@ def test_rope_tables_host_match_oracle(awq, lib, oracle):
     awq.check(lib.awq_rope_tables_host(ptr(a), ptr(b), mp))
     oracle.awqo_rope_tables(ptr(c), ptr(d), mp)
     assert np.array_equal(a.view(np.uint16), c.view(np.uint16)) and np.array_equal(b.view(np.uint16), d.view(np.uint16))
+
+
+def test_workspace_size_queries_need_no_gpu(lib):
+    """host-side arithmetic only: sizes of the scratch areas the kernel-level entry points take"""
+    assert lib.awq_gemv_workspace_bytes(4096, 4096) == 256
+    # a product with few output tiles may cut k over workgroups: room for 4 partial results
+    assert lib.awq_gemm_workspace_bytes(4096, 12288, 128) == 4 * 128 * 4096 * 4
+    assert lib.awq_gemm_workspace_bytes(12288, 4096, 2048) == 0     # plenty of tiles: never cut
+    assert lib.awq_gemm_workspace_bytes(4096, 4096, 4) == 0         # the few-token kernel
+    heads, max_pos = 32, 40960
+    chunks = (max_pos + 63) // 64
+    assert lib.awq_attention_workspace_bytes(heads, max_pos) == heads * (max_pos + chunks * 129 + 32) * 4
+    assert lib.awq_argmax_workspace_bytes(151936) > 0
