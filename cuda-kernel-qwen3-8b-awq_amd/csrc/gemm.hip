@@ -14,6 +14,7 @@
 //                   tokens staged through LDS
 #include "common.hpp"
 
+#include <atomic>
 #include <type_traits>
 
 namespace {
@@ -385,15 +386,27 @@ int launch_wide(const GemmParams& p, bool zint, hipStream_t st) {
   const unsigned gx = KSPLIT ? (unsigned)(p.m / 64) : (unsigned)((p.m + 255) / 256);
   dim3 grid(gx, (unsigned)((p.M + 32 * TT - 1) / (32 * TT)), KSPLIT ? (unsigned)p.kz : 1u);
   void (*kern)(GemmParams);
-  if (p.epilogue == EPI_RESIDUAL)
+  int variant;
+  if (p.epilogue == EPI_RESIDUAL) {
     kern = zint ? gemm_wide_kernel<true, KSPLIT, EPI_RESIDUAL, TT> : gemm_wide_kernel<false, KSPLIT, EPI_RESIDUAL, TT>;
-  else if (p.epilogue == EPI_GELU)
+    variant = zint ? 0 : 1;
+  } else if (p.epilogue == EPI_GELU) {
     kern = zint ? gemm_wide_kernel<true, KSPLIT, EPI_GELU, TT> : gemm_wide_kernel<false, KSPLIT, EPI_GELU, TT>;
-  else
+    variant = zint ? 2 : 3;
+  } else {
     kern = zint ? gemm_wide_kernel<true, KSPLIT, EPI_STORE, TT> : gemm_wide_kernel<false, KSPLIT, EPI_STORE, TT>;
+    variant = zint ? 4 : 5;
+  }
   if (lds > 65536) {
-    // more LDS than a launch gets by default: raise this kernel's limit (per device; cheap, so every time)
-    AWQ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+    // more LDS than a launch gets by default: raise this kernel's limit, once per device
+    static std::atomic<uint64_t> raised[6];
+    int dev = 0;
+    AWQ_HIP_TRY(hipGetDevice(&dev));
+    const uint64_t bit = 1ull << (dev & 63);
+    if (!(raised[variant].load(std::memory_order_relaxed) & bit)) {
+      AWQ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+      raised[variant].fetch_or(bit, std::memory_order_relaxed);
+    }
   }
   hipLaunchKernelGGL(kern, grid, dim3(256), lds, st, p);
   if (KSPLIT && p.kz > 1) {
