@@ -149,20 +149,33 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(const half_t* __
   // exp(x) = 2^(x log2 e); the scale of Inference.cu:218 folded into the same factor
   const float scale2 = (1.0f / sqrtf((float)AWQ_HEAD_DIM)) * 1.44269504088896340736f;
 
+  // this thread's two 16-byte pieces of the key tile and of the value tile: (key, part of its row)
+  u32x4_t kreg[2];
+  half8_t vreg[2];
+  auto load_tile = [&](int k0) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int pc = tid + i * 256;
+      const int key = pc >> 4, part = pc & 15;
+      const int kg = k0 + key < L_wg ? k0 + key : L_wg - 1;  // rows past the end are masked below
+      kreg[i] = *reinterpret_cast<const u32x4_t*>(kh_ptr + (int64_t)kg * AWQ_HEAD_DIM + part * 8);
+      vreg[i] = *reinterpret_cast<const half8_t*>(vh_ptr + (int64_t)kg * AWQ_HEAD_DIM + part * 8);
+    }
+  };
+  load_tile(0);
   for (int k0 = 0; k0 < L_wg; k0 += kFaKeys) {
     __syncthreads();  // the previous tiles' readers are done
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int pc = tid + i * 256;
       const int key = pc >> 4, part = pc & 15;
-      const int kg = k0 + key < L_wg ? k0 + key : L_wg - 1;  // rows past the end are masked below
-      const u32x4_t kv = *reinterpret_cast<const u32x4_t*>(kh_ptr + (int64_t)kg * AWQ_HEAD_DIM + part * 8);
-      const half8_t vv = *reinterpret_cast<const half8_t*>(vh_ptr + (int64_t)kg * AWQ_HEAD_DIM + part * 8);
-      *reinterpret_cast<u32x4_t*>(ks + key * kFaKStride + part * 8) = kv;
+      *reinterpret_cast<u32x4_t*>(ks + key * kFaKStride + part * 8) = kreg[i];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) vt[(part * 8 + e) * kFaVStride + key] = vv[e];
+      for (int e = 0; e < 8; ++e) vt[(part * 8 + e) * kFaVStride + key] = vreg[i][e];
     }
     __syncthreads();
+    // the next tile travels while this one is multiplied
+    if (k0 + kFaKeys < L_wg) load_tile(k0 + kFaKeys);
     if (k0 >= L_wave) continue;  // nothing of this tile is attended by this wavefront's queries
 
     f32x16_t sacc;
