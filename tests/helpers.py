@@ -119,9 +119,10 @@ def make_oracle_model(oracle, cfg):
     return oracle.awqo_model_create(ctypes.byref(ocfg))
 
 
-def fill_pair(awq, oracle, cfg, seed, engine=None, model=None, profile=0):
+def fill_pair(awq, oracle, cfg, seed, engine=None, model=None, profile=0, mutate=None):
     """Fill the oracle model's host arrays from the seeded generator and upload the very same
-    bytes to the engine."""
+    bytes to the engine.  mutate(layer, kind, part, address, count) may change a tensor in place
+    before it is uploaded."""
     lib = awq.load_library()
     for layer, kind, part in awq.tensor_list(cfg):
         count = cfg.part_count(kind, part)
@@ -130,6 +131,8 @@ def fill_pair(awq, oracle, cfg, seed, engine=None, model=None, profile=0):
         p = oracle.awqo_model_tensor(model, layer, kind, part, ctypes.byref(got))
         assert got.value == nbytes, (layer, kind, part, got.value, nbytes)
         awq.check(lib.awq_synth_fill_profile(profile, seed, layer, kind, part, p, count))
+        if mutate is not None:
+            mutate(layer, kind, part, p, count)
         if engine is not None:
             engine.upload(layer, kind, part, p, nbytes)
     if engine is not None:

@@ -266,3 +266,28 @@ def test_full_model_benchmark_distributions_overflow_identically(awq, oracle, to
     compare_state(awq, oracle, eng, model, cfg)
     eng.close()
     oracle.awqo_model_destroy(model)
+
+
+@pytest.mark.parametrize("flow", [False, True])
+def test_non_integral_zero_points_take_the_general_dequantisation(awq, oracle, torch_gpu, flow):
+    """AWQ zero-points are integers, which the kernels exploit (two exact operations instead of
+    three); a checkpoint with fractional zero-points must be detected at upload and still give the
+    oracle's bits through the general sequence"""
+    cfg = awq.make_config(**SMALL)
+    model = make_oracle_model(oracle, cfg)
+    eng = awq.QWen3AWQInfer.empty(cfg)
+
+    def fractional(layer, kind, part, address, count):
+        if part == awq.P_ZP and kind != awq.T_GAMMA:
+            z = np.ctypeslib.as_array(ctypes.cast(address, ctypes.POINTER(ctypes.c_uint16)), (count,)).view(np.float16)
+            z += np.float16(0.25) * ((np.arange(count) % 3) + 1).astype(np.float16)
+
+    fill_pair(awq, oracle, cfg, 4321, engine=eng, model=model, profile=awq.SYNTH_BALANCED, mutate=fractional)
+    eng.set_flow_mode(flow)
+    prompt = [9, 100, 1000]
+    print("fractional zero-points, flow =", flow, flush=True)
+    got = eng.generateResponse(prompt, 12)
+    assert got == oracle_generate(oracle, model, prompt, 12)
+    compare_state(awq, oracle, eng, model, cfg)
+    eng.close()
+    oracle.awqo_model_destroy(model)
