@@ -754,7 +754,7 @@ extern "C" int awq_prefill(awq_engine* e, const int32_t* prompt_ids, int32_t n_p
 namespace {
 
 constexpr int64_t kPrefillChunk = 1024;  // prompt positions per batched pass
-constexpr int64_t kGemmWsBytes = 64ll << 20;
+constexpr int64_t kGemmWsBytes = (64ll << 20) + 4096;  // header + partial sums (256 tiles, or 4 chunks of k for few rows)
 
 int ensure_prefill_buffers(awq_engine* e) {
   if (e->pb.chunk) return AWQ_OK;
@@ -767,6 +767,7 @@ int ensure_prefill_buffers(awq_engine* e) {
   if (int rc = dev_alloc(e, (void**)&e->pb.mid, C * I * 2)) return rc;
   if (int rc = dev_alloc(e, (void**)&e->pb.tokens, C * 4)) return rc;
   if (int rc = dev_alloc(e, &e->pb.gemm_ws, kGemmWsBytes)) return rc;
+  AWQ_HIP_TRY(hipMemset(e->pb.gemm_ws, 0, 4096));  // status word and hand-over counters start at zero
   e->pb.chunk = C;
   return AWQ_OK;
 }
@@ -832,6 +833,13 @@ extern "C" int awq_prefill_batched(awq_engine* e, const int32_t* prompt_ids, int
     AWQ_HIP_TRY(hipMemcpyAsync(e->hidden, e->pb.hidden + (M - 1) * H, (size_t)H * 2, hipMemcpyDeviceToDevice,
                                e->stream));
     AWQ_HIP_TRY(hipStreamSynchronize(e->stream));  // the token ids were read from the caller's buffer
+    int32_t gemm_status = 0;
+    AWQ_HIP_TRY(hipMemcpy(&gemm_status, e->pb.gemm_ws, 4, hipMemcpyDeviceToHost));
+    if (gemm_status != 0) {
+      AWQ_HIP_TRY(hipMemset(e->pb.gemm_ws, 0, 4096));
+      awq_set_error("a matrix product gave up waiting for partial sums of another workgroup");
+      return AWQ_ERR_HIP;
+    }
     e->current_seq_len = (int)(pos0 + M - 1);
     e->n_positions = (int)(pos0 + M);
   }

@@ -3,9 +3,12 @@
 // which is the reference's cublasGemmEx with n = M (ldb = k, ldc = m;
 // Inference.cu:1052-1065) applied to the same column-major reading of the
 // dequantised weights.  The weights stay packed int4 in memory and are turned
-// into binary16 in registers, bit-exactly as Inference.cu:102-104 rounds them;
-// the contraction runs on the matrix cores with FP32 accumulation, so results
-// agree with a sequential FP32 sum to rounding noise, not bit for bit.
+// into binary16 in registers; the contraction runs on the matrix cores with
+// FP32 accumulation, so results agree with a sequential FP32 sum to rounding
+// noise, not bit for bit.  The few-token kernel rounds every weight as
+// Inference.cu:102-104 does, h(h(q-z)*s); the many-token kernel multiplies
+// h(q-z), which is exact, and applies the row's scale to the FP32 sum (one
+// rounding fewer per weight than the reference).
 //
 // Same weight stream as the decode kernel: [16-row group][32-wide block][row][16 B],
 // dword c of a row holding elements 8c..8c+7 of the block.  Two kernels:
@@ -36,6 +39,9 @@ struct GemmParams {
   const half_t* res;    // EPI_RESIDUAL: [M][m], may be y itself
   int32_t kz;           // k is cut into kz chunks over blockIdx.z (k-split workgroups only)
   float* part;          // kz > 1: FP32 partial sums [kz][M][m], finished by reduce_parts_kernel
+  int32_t nr, n_tiles;  // rows split: 256-row blocks, tiles = row blocks x 128-token blocks (row block fastest)
+  int32_t* sk_head;     // rows split with handed-over sums: status word at [0], counters at [16 + workgroup]
+  float* sk_part;       // and one tile of FP32 sums per workgroup
 };
 
 // one finished output: the same epilogues as the decode kernel's.  The kind is
@@ -68,8 +74,9 @@ __device__ __forceinline__ uint32_t and_or_magic(uint32_t x, uint32_t mask) {
   return r;
 }
 
-// 8 nibbles of one dword -> 8 binary16 weights in element order, h(h(q-z)*s)
-template <bool ZINT>
+// 8 nibbles of one dword -> 8 binary16 weights in element order, h(h(q-z)*s);
+// SCALED = false stops at h(q-z) for a caller that multiplies its sums by s
+template <bool ZINT, bool SCALED = true>
 __device__ __forceinline__ half8_t dequant8(uint32_t v, half_t s, half_t z) {
   const half2_t s2 = half2_t{s, s};
   const half2_t k16 = half2_t{(half_t)0.0625f, (half_t)0.0625f};
@@ -92,6 +99,7 @@ __device__ __forceinline__ half8_t dequant8(uint32_t v, half_t s, half_t z) {
     u2 = (lo1 + m1024) + nz;
     u3 = __builtin_elementwise_fma(hi1, k16, m64) + nz;
   }
+  if (!SCALED) return half8_t{u0.x, u0.y, u1.x, u1.y, u2.x, u2.y, u3.x, u3.y};
   const half2_t w0 = u0 * s2, w1 = u1 * s2, w2 = u2 * s2, w3 = u3 * s2;
   return half8_t{w0.x, w0.y, w1.x, w1.y, w2.x, w2.y, w3.x, w3.y};
 }
@@ -166,9 +174,9 @@ __global__ __launch_bounds__(1024) void gemm_small_kernel(GemmParams p, int n_wa
 // j + 2 (kh = 1) of each row's 16 bytes, so that a lane's two weight dwords
 // (2kh, 2kh + 1) are adjacent in the weight stream.
 // Two workgroup shapes:
-//   rows split (KSPLIT = false): 4 wavefronts x 64 rows = 256 rows, one shared
+//   rows split: 4 wavefronts x 64 rows = 256 rows, one shared
 //     token tile per step; for products with many tiles.
-//   k split (KSPLIT = true): the 4 wavefronts share 64 rows and take a quarter
+//   k split: the 4 wavefronts share 64 rows and take a quarter
 //     of k each (a token tile of their own per step), partial sums meet in LDS;
 //     four times as many workgroups for products with few tiles.
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
@@ -186,8 +194,38 @@ constexpr int wide_lds_bytes(bool ksplit, int tt) {
   return ksplit && sums > tiles ? sums : tiles;
 }
 
-template <bool ZINT, bool KSPLIT, int EPI, int TT>
-__global__ __launch_bounds__(256, (KSPLIT && TT == 4) ? 1 : 2) void gemm_wide_kernel(GemmParams p) {
+// Rows split, work cut evenly: the steps of all tiles, in tile order, form one
+// sequence that is cut into gridDim.x equal ranges, one per workgroup, in units
+// of two steps.  A range covers the tail of one tile, whole tiles and the head
+// of another.  A workgroup whose piece of a tile does not reach the tile's last
+// step leaves its FP32 sums in its own slot of the workspace and counts itself
+// in at the workgroup that holds the last step; that one waits for the count,
+// adds the slots in workgroup order (a fixed order whatever the timing) and
+// writes the outputs.  Pieces are taken last tile first, so sums are handed
+// over early and collected late.  The collector has the highest index among a
+// tile's workgroups: with workgroups dispatched in index order, the ones it
+// waits for never wait themselves and are running or done.  The wait is
+// bounded all the same and reports through the status word.
+constexpr int kSkHeaderBytes = 4096;               // status word, then one counter per workgroup
+constexpr int kSkWgs = 256;                        // workgroups of a product whose work is cut evenly: one per compute unit
+constexpr int kSkTileFloats = 256 * kWideTokens;   // FP32 sums of one tile
+constexpr int kSkSpinLimit = 1 << 22;
+constexpr int kRowsSplitMinTiles = 128;            // fewer 256 x 128 tiles than this: k-split workgroups
+
+// the workgroup whose range holds step pair q, ranges being [b W / G, (b + 1) W / G)
+__device__ __forceinline__ int sk_wg_of(int64_t q, int64_t W, int G) {
+  int b = (int)(q * G / W);
+  while ((int64_t)(b + 1) * W / G <= q) ++b;
+  while ((int64_t)b * W / G > q) --b;
+  return b;
+}
+
+enum WideMode { WIDE_ROWS = 0, WIDE_K = 1, WIDE_ROWS_CUT = 2 };  // rows split (a tile per workgroup), k split, rows split with work cut evenly
+
+template <bool ZINT, int MODE, int EPI, int TT>
+__global__ __launch_bounds__(256, (MODE == WIDE_K && TT == 4) ? 1 : 2) void gemm_wide_kernel(GemmParams p) {
+  constexpr bool KSPLIT = MODE == WIDE_K;
+  constexpr bool CUT = MODE == WIDE_ROWS_CUT;
   constexpr int kTokens = 32 * TT;                   // tokens per workgroup
   constexpr int kSlot = kTokens * kWideStride;       // halves per token tile in LDS
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -197,170 +235,254 @@ __global__ __launch_bounds__(256, (KSPLIT && TT == 4) ? 1 : 2) void gemm_wide_ke
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n = lane & 31, kh = lane >> 5;
-  const int rg0 = KSPLIT ? blockIdx.x * 4 : (blockIdx.x * 4 + wave) * 4;  // first of this wavefront's 4 row groups
-  const bool rows_ok = rg0 * 16 < p.m;  // rows split: the last workgroup may hang over the edge
-  const int t0 = blockIdx.y * kTokens;
-  // a step is NH blocks of k; the step count is even (checked by the launcher)
-  const int steps = (KSPLIT ? p.nblk / (4 * p.kz) : p.nblk) / NH;
-  // first block of this workgroup's chunk of k (k split only), then of this wavefront's quarter of it
-  const int kb_wg = KSPLIT ? (int)blockIdx.z * 4 * steps * NH : 0;
-  const int kb_base = kb_wg + (KSPLIT ? wave * steps * NH : 0);
+  // a step is NH blocks of k; a tile (k split: this wavefront's quarter of this workgroup's chunk) has
+  // an even number of them (checked by the launcher)
+  const int tile_steps = (KSPLIT ? p.nblk / (4 * p.kz) : p.nblk) / NH;
   const int slot = KSPLIT ? wave : 0;
 
-  // the 64 rows share one scale group (rg0 is a multiple of 4, a group is 8 row groups)
-  const int gi = rows_ok ? ((rg0 >> 3) % p.kg) % p.mg : 0;
-  const half_t sc = p.scale[gi], zz = p.zp[gi];
+  // work cut evenly: this workgroup's range [lo, hi) of step pairs; otherwise one tile, whole
+  const int S2 = tile_steps / 2;
+  const int64_t W2 = (int64_t)p.n_tiles * S2;
+  const int64_t lo = CUT ? (int64_t)blockIdx.x * W2 / gridDim.x : 0;
+  const int64_t hi = CUT ? (int64_t)(blockIdx.x + 1) * W2 / gridDim.x : 1;
+  const int tile_first = CUT ? (int)(lo / S2) : 0;
+  int tile = CUT ? (int)((hi - 1) / S2) : (int)blockIdx.x;
 
-  // Token tile staging: piece = (slot, token, 16 bytes).  Two tiles are on their
-  // way in registers while a third is multiplied: a tile is requested two steps
-  // before its use and written to LDS one step before.  The main loop has no
-  // conditionals: loads past the end repeat the last tile (never used), tokens
-  // past M repeat token M-1 (never stored).
-  constexpr int PCS = kTokens * 4 * NH;  // pieces per slot
-  constexpr int PPT = NKB * PCS / 256;
-  const half_t* xsrc[PPT];
-  int xdst[PPT];
-#pragma unroll
-  for (int i = 0; i < PPT; ++i) {
-    const int pc = tid + i * 256;
-    const int j = pc / PCS, tok = (pc % PCS) / (4 * NH), part = pc % (4 * NH);
-    const int tg = t0 + tok < p.M ? t0 + tok : p.M - 1;
-    xsrc[i] = p.x + (int64_t)tg * p.k + (kb_wg + (KSPLIT ? j * steps * NH : 0)) * 32 + part * 8;
-    xdst[i] = j * kSlot + tok * kWideStride + part * 8;
-  }
-  xvec_t xr0[PPT], xr1[PPT];  // two named register sets (an indexed array would live in scratch memory)
-  auto load_x = [&](int s, xvec_t (&dst)[PPT]) __attribute__((always_inline)) {
-    const int sc_ = s < steps ? s : steps - 1;
-#pragma unroll
-    for (int i = 0; i < PPT; ++i) dst[i] = *reinterpret_cast<const xvec_t*>(xsrc[i] + sc_ * (32 * NH));
-  };
-  auto store_x = [&](int buf, const xvec_t (&src)[PPT]) __attribute__((always_inline)) {
-#pragma unroll
-    for (int i = 0; i < PPT; ++i) *reinterpret_cast<xvec_t*>(xs + buf * NKB * kSlot + xdst[i]) = src[i];
-  };
-
-  // weights: row n of pair rp is row n % 16 of row group rg0 + 2 rp + n / 16; dwords 2kh, 2kh + 1 of its block
-  const u32x2_t* wp[kWideRP];
-#pragma unroll
-  for (int a = 0; a < kWideRP; ++a) {
-    const int rg = rows_ok ? rg0 + 2 * a + (n >> 4) : 0;
-    wp[a] = reinterpret_cast<const u32x2_t*>(p.wq + (((int64_t)rg * p.nblk + kb_base) * 16 + (n & 15)) * 4 + 2 * kh);
-  }
-  constexpr int PF = 2;  // steps of weight dwords in flight
-  u32x2_t wd[kWideRP][PF][NH];
-#pragma unroll
-  for (int f = 0; f < PF; ++f)
-#pragma unroll
-    for (int h = 0; h < NH; ++h)
-#pragma unroll
-      for (int a = 0; a < kWideRP; ++a) wd[a][f][h] = KSPLIT ? __builtin_nontemporal_load(wp[a] + (int64_t)(f * NH + h) * 32) : wp[a][(int64_t)(f * NH + h) * 32];
-
-  f32x16_t acc[kWideRP][TT];
-#pragma unroll
-  for (int a = 0; a < kWideRP; ++a)
-#pragma unroll
-    for (int t = 0; t < TT; ++t)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) acc[a][t][i] = 0.0f;
-
-  load_x(0, xr0);
-  store_x(0, xr0);
-  load_x(1, xr1);
-  // one step; F is its index inside the unrolled pair (a compile-time constant)
-  auto step = [&](int s0, auto F) __attribute__((always_inline)) {
-    constexpr int f = decltype(F)::value;
-    const int s = s0 + f;
-    // tile s left these registers one step ago
-    if constexpr (f & 1) load_x(s + 2, xr1);
-    else load_x(s + 2, xr0);
-    __syncthreads();  // tile s is in buffer s & 1; the readers of tile s-1 are done
-    const half_t* xb = xs + ((s & 1) * NKB + slot) * kSlot + n * kWideStride + 16 * kh;
-    const int sn = s + PF < steps ? s + PF : steps - 1;
-#pragma unroll
-    for (int h = 0; h < NH; ++h) {
-      half8_t wop[kWideRP][2];
-#pragma unroll
-      for (int a = 0; a < kWideRP; ++a) {
-        wop[a][0] = dequant8<ZINT>(wd[a][f][h].x, sc, zz);
-        wop[a][1] = dequant8<ZINT>(wd[a][f][h].y, sc, zz);
-        wd[a][f][h] = KSPLIT ? __builtin_nontemporal_load(wp[a] + (int64_t)(sn * NH + h) * 32) : wp[a][(int64_t)(sn * NH + h) * 32];
-      }
-      // slices outermost: an accumulator tile is touched again only after all the others (a
-      // matrix-core instruction that needs the previous result of its accumulator waits for it)
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {
-#pragma unroll
-        for (int t = 0; t < TT; ++t) {
-          // slice j: k = 8 (j + 2 kh) .. + 7 of block h
-          const half8_t xop = *reinterpret_cast<const half8_t*>(xb + t * 32 * kWideStride + h * 32 + 8 * j);
-#pragma unroll
-          for (int a = 0; a < kWideRP; ++a)
-            acc[a][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xop, wop[a][j], acc[a][t], 0, 0, 0);
-        }
-      }
+  do {
+    // this piece: steps [s_lo, s_lo + steps) of the tile
+    int s_lo = 0, steps = tile_steps;
+    if (CUT) {
+      const int64_t q0 = (int64_t)tile * S2;
+      const int pb = (int)((lo > q0 ? lo : q0) - q0), pe = (int)((hi < q0 + S2 ? hi : q0 + S2) - q0);
+      s_lo = 2 * pb;
+      steps = 2 * (pe - pb);
     }
-    if constexpr (f & 1) store_x((s + 1) & 1, xr0);
-    else store_x((s + 1) & 1, xr1);
-  };
-  for (int s0 = 0; s0 < steps; s0 += 2) {
-    step(s0, std::integral_constant<int, 0>{});
-    step(s0, std::integral_constant<int, 1>{});
-  }
+    const int rb = KSPLIT ? (int)blockIdx.x : tile % p.nr;
+    const int tb = KSPLIT ? (int)blockIdx.y : tile / p.nr;
+    const int rg0 = KSPLIT ? rb * 4 : (rb * 4 + wave) * 4;  // first of this wavefront's 4 row groups
+    const bool rows_ok = rg0 * 16 < p.m;                    // rows split: the last tile may hang over the edge
+    const int t0 = tb * kTokens;
+    // first block of this workgroup's part of k, then of this wavefront's
+    const int kb_wg = KSPLIT ? (int)blockIdx.z * 4 * tile_steps * NH : s_lo * NH;
+    const int kb_base = kb_wg + (KSPLIT ? wave * tile_steps * NH : 0);
 
-  // acc[a][t][i] is D[token 32 t + 8 (i / 4) + 4 kh + i % 4][row 32 a + n]
-  if (!KSPLIT) {
-    if (!rows_ok) return;
+    // the 64 rows share one scale group (rg0 is a multiple of 4, a group is 8 row groups)
+    const int gi = rows_ok ? ((rg0 >> 3) % p.kg) % p.mg : 0;
+    const half_t sc = p.scale[gi], zz = p.zp[gi];
+
+    // Token tile staging: piece = (slot, token, 16 bytes).  Two tiles are on their
+    // way in registers while a third is multiplied: a tile is requested two steps
+    // before its use and written to LDS one step before.  The main loop has no
+    // conditionals: loads past the end repeat the last tile (never used), tokens
+    // past M repeat token M-1 (never stored).
+    constexpr int PCS = kTokens * 4 * NH;  // pieces per slot
+    constexpr int PPT = NKB * PCS / 256;
+    const half_t* xsrc[PPT];
+    int xdst[PPT];
+#pragma unroll
+    for (int i = 0; i < PPT; ++i) {
+      const int pc = tid + i * 256;
+      const int j = pc / PCS, tok = (pc % PCS) / (4 * NH), part = pc % (4 * NH);
+      const int tg = t0 + tok < p.M ? t0 + tok : p.M - 1;
+      xsrc[i] = p.x + (int64_t)tg * p.k + (kb_wg + (KSPLIT ? j * tile_steps * NH : 0)) * 32 + part * 8;
+      xdst[i] = j * kSlot + tok * kWideStride + part * 8;
+    }
+    xvec_t xr0[PPT], xr1[PPT];  // two named register sets (an indexed array would live in scratch memory)
+    auto load_x = [&](int s, xvec_t (&dst)[PPT]) __attribute__((always_inline)) {
+      const int sc_ = s < steps ? s : steps - 1;
+#pragma unroll
+      for (int i = 0; i < PPT; ++i) dst[i] = *reinterpret_cast<const xvec_t*>(xsrc[i] + sc_ * (32 * NH));
+    };
+    auto store_x = [&](int buf, const xvec_t (&src)[PPT]) __attribute__((always_inline)) {
+#pragma unroll
+      for (int i = 0; i < PPT; ++i) *reinterpret_cast<xvec_t*>(xs + buf * NKB * kSlot + xdst[i]) = src[i];
+    };
+
+    // weights: row n of pair rp is row n % 16 of row group rg0 + 2 rp + n / 16; dwords 2kh, 2kh + 1 of its block
+    const u32x2_t* wp[kWideRP];
 #pragma unroll
     for (int a = 0; a < kWideRP; ++a) {
-      const int row = rg0 * 16 + a * 32 + n;
-#pragma unroll
-      for (int t = 0; t < TT; ++t) {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int tok = t0 + t * 32 + (i >> 2) * 8 + kh * 4 + (i & 3);
-          if (tok < p.M) store_out<EPI>(p, tok, row, acc[a][t][i]);
-        }
-      }
+      const int rg = rows_ok ? rg0 + 2 * a + (n >> 4) : 0;
+      wp[a] = reinterpret_cast<const u32x2_t*>(p.wq + (((int64_t)rg * p.nblk + kb_base) * 16 + (n & 15)) * 4 + 2 * kh);
     }
-    return;
-  }
-  // k split: the four partial sums of every output meet in LDS (the token tiles
-  // are dead by now); wavefront w finishes quarter w of every accumulator tile
-  float4_t* red = reinterpret_cast<float4_t*>(smem_raw);  // [wave][pair][tile][quarter][lane]
-  __syncthreads();
+    constexpr int PF = 2;  // steps of weight dwords in flight
+    u32x2_t wd[kWideRP][PF][NH];
 #pragma unroll
-  for (int a = 0; a < kWideRP; ++a)
+    for (int f = 0; f < PF; ++f)
 #pragma unroll
-    for (int t = 0; t < TT; ++t)
+      for (int h = 0; h < NH; ++h)
 #pragma unroll
-      for (int i4 = 0; i4 < 4; ++i4)
-        red[(((wave * kWideRP + a) * TT + t) * 4 + i4) * 64 + lane] =
-            float4_t{acc[a][t][4 * i4], acc[a][t][4 * i4 + 1], acc[a][t][4 * i4 + 2], acc[a][t][4 * i4 + 3]};
-  __syncthreads();
-  auto finish = [&](auto E) {
-    constexpr int epi = decltype(E)::value;  // -1: this workgroup's chunk of k only, as FP32 partial sums
+        for (int a = 0; a < kWideRP; ++a) wd[a][f][h] = KSPLIT ? __builtin_nontemporal_load(wp[a] + (int64_t)(f * NH + h) * 32) : wp[a][(int64_t)(f * NH + h) * 32];
+
+    f32x16_t acc[kWideRP][TT];
 #pragma unroll
-    for (int a = 0; a < kWideRP; ++a) {
-      const int row = rg0 * 16 + a * 32 + n;
-      const int i4 = wave;
+    for (int a = 0; a < kWideRP; ++a)
 #pragma unroll
-      for (int t = 0; t < TT; ++t) {
-        float4_t v = red[(((0 * kWideRP + a) * TT + t) * 4 + i4) * 64 + lane];
+      for (int t = 0; t < TT; ++t)
 #pragma unroll
-        for (int w = 1; w < 4; ++w) v += red[(((w * kWideRP + a) * TT + t) * 4 + i4) * 64 + lane];
+        for (int i = 0; i < 16; ++i) acc[a][t][i] = 0.0f;
+
+    load_x(0, xr0);
+    store_x(0, xr0);
+    load_x(1, xr1);
+    // one step; F is its index inside the unrolled pair (a compile-time constant)
+    auto step = [&](int s0, auto F) __attribute__((always_inline)) {
+      constexpr int f = decltype(F)::value;
+      const int s = s0 + f;
+      // tile s left these registers one step ago
+      if constexpr (f & 1) load_x(s + 2, xr1);
+      else load_x(s + 2, xr0);
+      __syncthreads();  // tile s is in buffer s & 1; the readers of tile s-1 are done
+      const half_t* xb = xs + ((s & 1) * NKB + slot) * kSlot + n * kWideStride + 16 * kh;
+      const int sn = s + PF < steps ? s + PF : steps - 1;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int tok = t0 + t * 32 + i4 * 8 + kh * 4 + i;
-          if (tok < p.M) {
-            if (epi < 0) p.part[((int64_t)blockIdx.z * p.M + tok) * p.m + row] = v[i];
-            else store_out<(epi < 0 ? 0 : epi)>(p, tok, row, v[i]);
+      for (int h = 0; h < NH; ++h) {
+        half8_t wop[kWideRP][2];
+#pragma unroll
+        for (int a = 0; a < kWideRP; ++a) {
+          wop[a][0] = dequant8<ZINT, false>(wd[a][f][h].x, sc, zz);
+          wop[a][1] = dequant8<ZINT, false>(wd[a][f][h].y, sc, zz);
+          wd[a][f][h] = KSPLIT ? __builtin_nontemporal_load(wp[a] + (int64_t)(sn * NH + h) * 32) : wp[a][(int64_t)(sn * NH + h) * 32];
+        }
+        // slices outermost: an accumulator tile is touched again only after all the others (a
+        // matrix-core instruction that needs the previous result of its accumulator waits for it)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+#pragma unroll
+          for (int t = 0; t < TT; ++t) {
+            // slice j: k = 8 (j + 2 kh) .. + 7 of block h
+            const half8_t xop = *reinterpret_cast<const half8_t*>(xb + t * 32 * kWideStride + h * 32 + 8 * j);
+#pragma unroll
+            for (int a = 0; a < kWideRP; ++a)
+              acc[a][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xop, wop[a][j], acc[a][t], 0, 0, 0);
           }
         }
       }
+      if constexpr (f & 1) store_x((s + 1) & 1, xr0);
+      else store_x((s + 1) & 1, xr1);
+    };
+    for (int s0 = 0; s0 < steps; s0 += 2) {
+      step(s0, std::integral_constant<int, 0>{});
+      step(s0, std::integral_constant<int, 1>{});
     }
-  };
-  if (p.kz > 1) finish(std::integral_constant<int, -1>{});
-  else finish(std::integral_constant<int, EPI>{});
+
+    const float scf = (float)sc;  // the wavefront's rows share one scale: it multiplies the sums, not every weight
+    // acc[a][t][i] is D[token 32 t + 8 (i / 4) + 4 kh + i % 4][row 32 a + n]
+    if constexpr (!KSPLIT) {
+      typedef unsigned long long u64;
+      const int b = blockIdx.x;
+      // opaque to the compiler: the 64 slot addresses below are formed here, after the main loop, and
+      // not once before the tile loop (where they would sit in scratch memory across the main loop)
+      int tl = tid;
+      asm volatile("" : "+v"(tl));
+      if (CUT && s_lo + steps != tile_steps) {
+        // the tile's last step is elsewhere: hand the sums over, element (a, t, i) pairs [thread]
+        u64* mine = reinterpret_cast<u64*>(p.sk_part) + (int64_t)b * (kSkTileFloats / 2);
+#pragma unroll
+        for (int a = 0; a < kWideRP; ++a)
+#pragma unroll
+          for (int t = 0; t < TT; ++t)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+              const float2 v = float2{acc[a][t][2 * i], acc[a][t][2 * i + 1]};
+              __hip_atomic_store(mine + ((a * TT + t) * 8 + i) * 256 + tl, __builtin_bit_cast(u64, v), __ATOMIC_RELAXED,
+                                 __HIP_MEMORY_SCOPE_AGENT);
+            }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (tid == 0) {
+          const int owner = sk_wg_of((int64_t)(tile + 1) * S2 - 1, W2, gridDim.x);
+          __hip_atomic_fetch_add(p.sk_head + 16 + owner, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        continue;
+      }
+      if (CUT && s_lo != 0) {
+        // the tile's first steps were taken by workgroups first .. b - 1, one slot each
+        const int first = sk_wg_of((int64_t)tile * S2, W2, gridDim.x);
+        if (tid == 0) {
+          int spins = 0;
+          while (__hip_atomic_load(p.sk_head + 16 + b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < b - first) {
+            __builtin_amdgcn_s_sleep(4);
+            if (++spins > kSkSpinLimit) {
+              __hip_atomic_store(p.sk_head, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+              break;
+            }
+          }
+          __hip_atomic_store(p.sk_head + 16 + b, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
+        }
+        __syncthreads();
+        for (int c = first; c < b; ++c) {
+          const u64* theirs = reinterpret_cast<const u64*>(p.sk_part) + (int64_t)c * (kSkTileFloats / 2);
+#pragma unroll
+          for (int a = 0; a < kWideRP; ++a)
+#pragma unroll
+            for (int t = 0; t < TT; ++t) {
+#pragma unroll
+              for (int i = 0; i < 8; ++i) {
+                const float2 v = __builtin_bit_cast(
+                    float2, __hip_atomic_load(theirs + ((a * TT + t) * 8 + i) * 256 + tl, __ATOMIC_RELAXED,
+                                              __HIP_MEMORY_SCOPE_AGENT));
+                acc[a][t][2 * i] += v.x;
+                acc[a][t][2 * i + 1] += v.y;
+              }
+              __builtin_amdgcn_sched_barrier(0);  // 8 loads in flight, not all 64 (registers)
+            }
+        }
+      }
+      if (!rows_ok) continue;
+#pragma unroll
+      for (int a = 0; a < kWideRP; ++a) {
+        const int row = rg0 * 16 + a * 32 + n;
+#pragma unroll
+        for (int t = 0; t < TT; ++t) {
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            const int tok = t0 + t * 32 + (i >> 2) * 8 + kh * 4 + (i & 3);
+            if (tok < p.M) store_out<EPI>(p, tok, row, acc[a][t][i] * scf);
+          }
+        }
+      }
+    } else {
+      // k split: the four partial sums of every output meet in LDS (the token tiles
+      // are dead by now); wavefront w finishes quarter w of every accumulator tile
+      float4_t* red = reinterpret_cast<float4_t*>(smem_raw);  // [wave][pair][tile][quarter][lane]
+      __syncthreads();
+#pragma unroll
+      for (int a = 0; a < kWideRP; ++a)
+#pragma unroll
+        for (int t = 0; t < TT; ++t)
+#pragma unroll
+          for (int i4 = 0; i4 < 4; ++i4)
+            red[(((wave * kWideRP + a) * TT + t) * 4 + i4) * 64 + lane] =
+                float4_t{acc[a][t][4 * i4], acc[a][t][4 * i4 + 1], acc[a][t][4 * i4 + 2], acc[a][t][4 * i4 + 3]};
+      __syncthreads();
+      auto finish = [&](auto E) {
+        constexpr int epi = decltype(E)::value;  // -1: this workgroup's chunk of k only, as FP32 partial sums
+#pragma unroll
+        for (int a = 0; a < kWideRP; ++a) {
+          const int row = rg0 * 16 + a * 32 + n;
+          const int i4 = wave;
+#pragma unroll
+          for (int t = 0; t < TT; ++t) {
+            float4_t v = red[(((0 * kWideRP + a) * TT + t) * 4 + i4) * 64 + lane];
+#pragma unroll
+            for (int w = 1; w < 4; ++w) v += red[(((w * kWideRP + a) * TT + t) * 4 + i4) * 64 + lane];
+            v *= scf;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const int tok = t0 + t * 32 + i4 * 8 + kh * 4 + i;
+              if (tok < p.M) {
+                if (epi < 0) p.part[((int64_t)blockIdx.z * p.M + tok) * p.m + row] = v[i];
+                else store_out<(epi < 0 ? 0 : epi)>(p, tok, row, v[i]);
+              }
+            }
+          }
+        }
+      };
+      if (p.kz > 1) finish(std::integral_constant<int, -1>{});
+      else finish(std::integral_constant<int, EPI>{});
+    }
+  } while (CUT && --tile >= tile_first);
 }
 
 // k cut over several workgroups: the chunks' FP32 partial sums are added in
@@ -377,24 +499,25 @@ __global__ __launch_bounds__(256) void reduce_parts_kernel(GemmParams p) {
 // tokens per workgroup of the k-split shape: 32, 64 or 128
 int wide_tt(int64_t M) { return M <= 32 ? 1 : (M <= 64 ? 2 : 4); }
 
-template <bool KSPLIT, int TT>
-int launch_wide(const GemmParams& p, bool zint, hipStream_t st) {
+template <int MODE, int TT>
+int launch_wide(const GemmParams& p, bool zint, int n_wgs, hipStream_t st) {
+  constexpr bool KSPLIT = MODE == WIDE_K;
   // the main loop takes two steps of two 32-wide blocks per trip (per quarter of k when k is split)
-  AWQ_REQUIRE(p.nblk % (KSPLIT ? 16 * p.kz : 4) == 0, "k must be a multiple of 512");
+  AWQ_REQUIRE(p.nblk % (KSPLIT ? 16 * p.kz : 4) == 0, KSPLIT ? "k must be a multiple of 512" : "k must be a multiple of 128");
   constexpr int lds = wide_lds_bytes(KSPLIT, TT);
   static_assert(lds <= 160 * 1024, "LDS of one compute unit");
-  const unsigned gx = KSPLIT ? (unsigned)(p.m / 64) : (unsigned)((p.m + 255) / 256);
-  dim3 grid(gx, (unsigned)((p.M + 32 * TT - 1) / (32 * TT)), KSPLIT ? (unsigned)p.kz : 1u);
+  dim3 grid((unsigned)(p.m / 64), (unsigned)((p.M + 32 * TT - 1) / (32 * TT)), (unsigned)p.kz);
+  if (!KSPLIT) grid = dim3((unsigned)n_wgs);
   void (*kern)(GemmParams);
   int variant;
   if (p.epilogue == EPI_RESIDUAL) {
-    kern = zint ? gemm_wide_kernel<true, KSPLIT, EPI_RESIDUAL, TT> : gemm_wide_kernel<false, KSPLIT, EPI_RESIDUAL, TT>;
+    kern = zint ? gemm_wide_kernel<true, MODE, EPI_RESIDUAL, TT> : gemm_wide_kernel<false, MODE, EPI_RESIDUAL, TT>;
     variant = zint ? 0 : 1;
   } else if (p.epilogue == EPI_GELU) {
-    kern = zint ? gemm_wide_kernel<true, KSPLIT, EPI_GELU, TT> : gemm_wide_kernel<false, KSPLIT, EPI_GELU, TT>;
+    kern = zint ? gemm_wide_kernel<true, MODE, EPI_GELU, TT> : gemm_wide_kernel<false, MODE, EPI_GELU, TT>;
     variant = zint ? 2 : 3;
   } else {
-    kern = zint ? gemm_wide_kernel<true, KSPLIT, EPI_STORE, TT> : gemm_wide_kernel<false, KSPLIT, EPI_STORE, TT>;
+    kern = zint ? gemm_wide_kernel<true, MODE, EPI_STORE, TT> : gemm_wide_kernel<false, MODE, EPI_STORE, TT>;
     variant = zint ? 4 : 5;
   }
   if (lds > 65536) {
@@ -424,13 +547,15 @@ void launch_small(const GemmParams& p, bool zint, int n_waves, dim3 grid, hipStr
 
 }  // namespace
 
-// room for the partial sums of a product whose k is cut over workgroups (0: never cut)
+// room for a header and the partial sums of a product whose work is cut over workgroups (0: never cut)
 int64_t gemm_workspace_bytes(int64_t m, int64_t k, int64_t M) {
   (void)k;
   if (M <= 4) return 0;
+  const int64_t tiles = ((m + 255) / 256) * ((M + kWideTokens - 1) / kWideTokens);
+  if (tiles >= kRowsSplitMinTiles) return tiles * 3 <= kSkWgs * 2 ? kSkHeaderBytes + (int64_t)kSkWgs * kSkTileFloats * 4 : 0;
   const int tokens = 32 * wide_tt(M);
   const int64_t wgs = (m / 64) * ((M + tokens - 1) / tokens);
-  return wgs <= 128 ? 4 * M * m * 4 : 0;
+  return wgs <= 128 ? kSkHeaderBytes + 4 * M * m * 4 : 0;
 }
 
 int launch_gemm(const void* wq, const half_t* scale, const half_t* zp, int64_t m, int64_t k, const half_t* x,
@@ -458,6 +583,9 @@ int launch_gemm(const void* wq, const half_t* scale, const half_t* zp, int64_t m
   p.res = res;
   p.kz = 1;
   p.part = nullptr;
+  p.nr = p.n_tiles = 0;
+  p.sk_head = nullptr;
+  p.sk_part = nullptr;
   // up to 4 tokens: the decode kernel's decomposition (one 16-token operand tile, mostly padding)
   int g = 0;
   if (M <= 4) {
@@ -479,10 +607,30 @@ int launch_gemm(const void* wq, const half_t* scale, const half_t* zp, int64_t m
       default: launch_small<1, 1>(p, zp_integral, n_waves, grid, st); break;
     }
   } else {
-    // enough 256-row x 128-token tiles to fill half the device: rows split; otherwise k split
-    const int64_t tiles = ((m + 255) / 256) * ((M + kWideTokens - 1) / kWideTokens);
-    if (tiles >= 128) {
-      if (int rc = launch_wide<false, 4>(p, zp_integral, st)) return rc;
+    // enough 256-row x 128-token tiles: rows split; otherwise k split
+    const int64_t nr = (m + 255) / 256;
+    const int64_t tiles = nr * ((M + kWideTokens - 1) / kWideTokens);
+    // the partial sums start behind the header, whichever kernel writes them
+    char* ws_part = workspace ? (char*)workspace + kSkHeaderBytes : nullptr;
+    const int64_t part_bytes = workspace_bytes - kSkHeaderBytes;
+    if (tiles >= kRowsSplitMinTiles) {
+      AWQ_REQUIRE(tiles < (1ll << 31), "too many output tiles");
+      p.nr = (int32_t)nr;
+      p.n_tiles = (int32_t)tiles;
+      // One workgroup per tile.  When the tiles would leave a third of the compute units idle and
+      // the caller brought room for handed-over sums, the steps of all tiles are cut evenly over one
+      // workgroup per compute unit instead (measured on 4096 x 12288, 1024 tokens, 128 tiles: 172 -> 124 us;
+      // with 192 tiles the hand-over costs more than the idle units).
+      int64_t n_wgs = tiles;
+      const int64_t pairs = tiles * (p.nblk / kWideNH / 2);
+      if (workspace && tiles * 3 <= kSkWgs * 2 && pairs / 4 >= kSkWgs && kSkWgs * (int64_t)kSkTileFloats * 4 <= part_bytes) {
+        n_wgs = kSkWgs;
+        p.sk_head = (int32_t*)workspace;
+        p.sk_part = (float*)ws_part;
+      }
+      if (int rc = p.sk_part ? launch_wide<WIDE_ROWS_CUT, 4>(p, zp_integral, (int)n_wgs, st)
+                             : launch_wide<WIDE_ROWS, 4>(p, zp_integral, (int)n_wgs, st))
+        return rc;
     } else {
       // few 64-row workgroups too (a matrix with few rows): cut k over 4 or 2 workgroups as well,
       // when the caller brought room for the partial sums
@@ -490,15 +638,15 @@ int launch_gemm(const void* wq, const half_t* scale, const half_t* zp, int64_t m
       const int64_t wgs = (m / 64) * ((M + 32 * tt - 1) / (32 * tt));
       if (wgs <= 128 && workspace) {
         for (int kz : {4, 2})
-          if (p.nblk % (16 * kz) == 0 && (int64_t)kz * M * m * 4 <= workspace_bytes) {
+          if (p.nblk % (16 * kz) == 0 && (int64_t)kz * M * m * 4 <= part_bytes) {
             p.kz = kz;
-            p.part = (float*)workspace;
+            p.part = (float*)ws_part;
             break;
           }
       }
-      if (int rc = tt == 1 ? launch_wide<true, 1>(p, zp_integral, st)
-                           : tt == 2 ? launch_wide<true, 2>(p, zp_integral, st)
-                                     : launch_wide<true, 4>(p, zp_integral, st))
+      if (int rc = tt == 1 ? launch_wide<WIDE_K, 1>(p, zp_integral, 0, st)
+                           : tt == 2 ? launch_wide<WIDE_K, 2>(p, zp_integral, 0, st)
+                                     : launch_wide<WIDE_K, 4>(p, zp_integral, 0, st))
         return rc;
     }
   }

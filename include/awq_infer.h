@@ -215,9 +215,17 @@ int awq_gemv_fused(const awq_linear_args* args, void* stream);
  * accumulation: within rounding noise of awq_gemv applied to each token, not
  * bit-identical to it.  Matrices whose scale group depends on the input index
  * (the 151936 x 4096 unembedding) are not supported.  workspace: NULL, or
- * awq_gemm_workspace_bytes(m, k, M) bytes of device memory; with it, products
- * with few output tiles also cut k over several workgroups (FP32 partial sums,
- * added in a fixed order by a second launch). */
+ * awq_gemm_workspace_bytes(m, k, M) bytes of device memory whose first 4096
+ * bytes are zero before the first call (every call leaves them zero); with it,
+ * products with few output tiles also cut k over several workgroups (FP32
+ * partial sums, added in a fixed order whatever the timing, by a second launch
+ * or by the workgroup that holds a tile's last part of k).  That workgroup
+ * waits for the others; they have lower indices and never wait themselves, so
+ * the wait ends while the device dispatches workgroups in index order.  It is
+ * bounded all the same: should it expire, the first int32 of the workspace
+ * becomes 1 (read it after synchronising; the outputs are then wrong and the
+ * header must be zeroed again).  Calls that share a workspace must not
+ * overlap. */
 int64_t awq_gemm_workspace_bytes(int64_t m, int64_t k, int64_t M);
 int awq_gemm(const void* repacked, const void* scale, const void* zp, int64_t m, int64_t k, const void* x, void* y,
              int64_t M, int32_t zp_integral, void* workspace, void* stream);

@@ -502,7 +502,8 @@ def test_gemv_fused_norm_unembed_argmax(awq, lib, oracle, torch_gpu, m, k):
 # ----------------------------------------------------------------------------- W4A16 GEMM on the matrix cores
 @pytest.mark.parametrize("m,k,M,zp_int", [(256, 512, 3, True), (256, 512, 17, False), (384, 1536, 130, True),
                                           (12288, 4096, 16, True), (12288, 4096, 200, True), (4096, 12288, 64, False),
-                                          (4096, 12288, 128, True), (12288, 4096, 1030, True)])
+                                          (4096, 12288, 128, True), (12288, 4096, 1030, True),
+                                          (4096, 4096, 1024, True), (384, 3072, 8500, False)])
 def test_gemm_matches_fp32_accumulate_reference(awq, lib, oracle, torch_gpu, m, k, M, zp_int):
     """config 5: dequant-on-load MFMA product; 1e-2 relative against the sequential FP32-accumulate
     reference, and the weights it multiplies are the bit-exact dequantised ones (one-hot check below)"""
@@ -535,14 +536,29 @@ def test_gemm_matches_fp32_accumulate_reference(awq, lib, oracle, torch_gpu, m, 
     got2 = d_y2.cpu().numpy()[sel].astype(np.float64)
     if wsb == 0:
         assert np.array_equal(d_y2.cpu().numpy().view(np.uint16), d_y.cpu().numpy().view(np.uint16))
+    else:
+        # the header (status word, hand-over counters) is zero again, and a second product on the same
+        # workspace gives the same bits: partial sums are added in a fixed order
+        assert int(d_ws[:4096].to(torch.int32).sum().item()) == 0
+        d_y3 = torch.full((M, m), float("nan"), dtype=torch.float16, device="cuda")
+        awq.check(lib.awq_gemm(d_w.data_ptr(), d_s.data_ptr(), d_z.data_ptr(), m, k, d_x.data_ptr(), d_y3.data_ptr(),
+                               M, 1 if zp_int else 0, d_ws.data_ptr(), stream(torch)))
+        torch.cuda.synchronize()
+        assert np.array_equal(d_y3.cpu().numpy().view(np.uint16), d_y2.cpu().numpy().view(np.uint16))
+        assert int(d_ws[:4096].to(torch.int32).sum().item()) == 0
     got = d_y.cpu().numpy()[sel].astype(np.float64)
     want = ref.astype(np.float64)
-    denom = np.maximum(np.abs(want), 1e-2 * np.abs(want).max())
+    # 1e-2 relative; outputs smaller than the root mean square of all outputs are measured against that
+    # (a sum of 512..12288 terms that cancels to nearly nothing has no relative accuracy to speak of)
+    denom = np.maximum(np.abs(want), np.sqrt(np.mean(want * want)))
     assert np.all(np.isfinite(got))
     assert np.all(np.abs(got - want) <= 1e-2 * denom)
     assert np.all(np.isfinite(got2)) and np.all(np.abs(got2 - want) <= 1e-2 * denom)
-    # much tighter in practice: FP32 accumulation either way
-    assert np.mean(d_y.cpu().numpy()[sel].view(np.uint16) == ref.view(np.uint16)) > 0.9
+    # much tighter in practice (FP32 accumulation either way; the many-token kernel applies the scale
+    # to the sum instead of to every weight, one binary16 rounding fewer per weight than the oracle):
+    # 99% of the outputs within two binary16 roundings
+    assert np.percentile(np.abs(got - want) / denom, 99) <= 2.0 ** -10
+    assert np.percentile(np.abs(got2 - want) / denom, 99) <= 2.0 ** -10
 
 
 def test_gemm_one_hot_and_token_independence(awq, lib, torch_gpu):
