@@ -144,8 +144,11 @@ def test_rope_tables_host_match_oracle(awq, lib, oracle):
 def test_workspace_size_queries_need_no_gpu(lib):
     """host-side arithmetic only: sizes of the scratch areas the kernel-level entry points take"""
     assert lib.awq_gemv_workspace_bytes(4096, 4096) == 256
-    # a product with few output tiles may cut k over workgroups: room for 4 partial results
-    assert lib.awq_gemm_workspace_bytes(4096, 12288, 128) == 4 * 128 * 4096 * 4
+    # a product with few output tiles may cut k over workgroups: a 4096-byte header (status word,
+    # hand-over counters) and room for 4 partial results, or for one 256 x 128 tile of FP32 sums
+    # per compute unit
+    assert lib.awq_gemm_workspace_bytes(4096, 12288, 128) == 4096 + 4 * 128 * 4096 * 4
+    assert lib.awq_gemm_workspace_bytes(4096, 12288, 1024) == 4096 + 256 * 256 * 128 * 4
     assert lib.awq_gemm_workspace_bytes(12288, 4096, 2048) == 0     # plenty of tiles: never cut
     assert lib.awq_gemm_workspace_bytes(4096, 4096, 4) == 0         # the few-token kernel
     heads, max_pos = 32, 40960
