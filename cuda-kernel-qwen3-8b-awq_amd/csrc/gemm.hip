@@ -44,16 +44,31 @@ struct GemmParams {
   float* sk_part;       // and one tile of FP32 sums per workgroup
 };
 
+// exact-erf GeLU (Inference.cu:274-277) for the many-token kernels, whose sums are not bit-identical
+// to the decode path's anyway: erfc by Abramowitz & Stegun 7.1.26 (absolute error <= 1.5e-7, far
+// below the binary16 rounding of the result) on the hardware reciprocal and exponential, about a
+// fifth of the instructions of the bit-exact awq_gelu_f32 and free of branches.
+__device__ __forceinline__ float gelu_approx(float v) {
+  const float x = __builtin_fabsf(v) * 0.70710678f;
+  const float t = __builtin_amdgcn_rcpf(__builtin_fmaf(0.3275911f, x, 1.0f));
+  float q = __builtin_fmaf(t, 1.061405429f, -1.453152027f);
+  q = __builtin_fmaf(q, t, 1.421413741f);
+  q = __builtin_fmaf(q, t, -0.284496736f);
+  q = __builtin_fmaf(q, t, 0.254829592f);
+  const float erfc_abs = (q * t) * __builtin_amdgcn_exp2f((x * x) * -1.44269504f);  // 1 - erf(|v| / sqrt 2)
+  return (0.5f * v) * (v >= 0.0f ? 2.0f - erfc_abs : erfc_abs);                     // 1 + erf(v / sqrt 2)
+}
+
 // one finished output: the same epilogues as the decode kernel's.  The kind is
 // a template argument so that the fully unrolled output loops stay free of
 // branches (a branch inside them makes the accumulators an indexed array in
 // scratch memory).
-template <int EPI>
+template <int EPI, bool WIDE = false>
 __device__ __forceinline__ void store_out(const GemmParams& p, int tok, int row, float acc) {
   const int64_t at = (int64_t)tok * p.m + row;
   const half_t v = (half_t)acc;
   if (EPI == EPI_RESIDUAL) p.y[at] = p.res[at] + v;                          // Inference.cu:1149-1155
-  else if (EPI == EPI_GELU) p.y[at] = to_half_rn(awq_gelu_f32((float)v));    // Inference.cu:271-279
+  else if (EPI == EPI_GELU) p.y[at] = to_half_rn(WIDE ? gelu_approx((float)v) : awq_gelu_f32((float)v));  // Inference.cu:271-279
   else p.y[at] = v;
 }
 // f(integral_constant<int, kind>) for the kind in p.epilogue
@@ -189,7 +204,7 @@ constexpr int kWideTokens = 32 * kWideTT;               // 128
 constexpr int kWideNH = 2;                              // 32-wide blocks of k per step
 constexpr int kWideStride = 32 * kWideNH + 8;           // halves per token row of a tile in LDS (16 bytes of padding)
 constexpr int wide_lds_bytes(bool ksplit, int tt) {
-  const int tiles = (ksplit ? 4 : 1) * 2 * (32 * tt) * kWideStride * 2;  // slots x double buffer x tile
+  const int tiles = (ksplit ? 4 * 2 : 3) * (32 * tt) * kWideStride * 2;  // k split: slots x double buffer x tile; rows split: three tiles
   const int sums = 4 * kWideRP * tt * 64 * 16 * 4;                       // k split: the partial sums
   return ksplit && sums > tiles ? sums : tiles;
 }
@@ -322,48 +337,140 @@ __global__ __launch_bounds__(256, (MODE == WIDE_K && TT == 4) ? 1 : 2) void gemm
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[a][t][i] = 0.0f;
 
-    load_x(0, xr0);
-    store_x(0, xr0);
-    load_x(1, xr1);
-    // one step; F is its index inside the unrolled pair (a compile-time constant)
-    auto step = [&](int s0, auto F) __attribute__((always_inline)) {
-      constexpr int f = decltype(F)::value;
-      const int s = s0 + f;
-      // tile s left these registers one step ago
-      if constexpr (f & 1) load_x(s + 2, xr1);
-      else load_x(s + 2, xr0);
-      __syncthreads();  // tile s is in buffer s & 1; the readers of tile s-1 are done
-      const half_t* xb = xs + ((s & 1) * NKB + slot) * kSlot + n * kWideStride + 16 * kh;
-      const int sn = s + PF < steps ? s + PF : steps - 1;
+    if constexpr (!KSPLIT) {
+      // Software pipeline over quarter steps ("slices": 8 matrix-core instructions on one 16-wide
+      // piece of k).  While a slice is multiplied, the token operands of the next one are read from
+      // LDS and its weight operands are dequantised, so no instruction waits for a read issued just
+      // before it.  Three token tiles rotate through LDS: tile s + 1 is already visible during step
+      // s (the last slice of a step prepares the first of the next across the barrier) and tile
+      // s + 2 is written at the end of step s into the buffer tile s - 1 left before the barrier.
+      if (CUT) __syncthreads();  // the previous piece's readers are done
+      load_x(0, xr0);
+      store_x(0, xr0);
+      load_x(1, xr0);
+      store_x(1, xr0);
+      load_x(2, xr1);
+      half8_t xa[TT], xb_[TT], wa[kWideRP], wb[kWideRP];
+      const half_t* xlane = xs + n * kWideStride + 16 * kh;
+      auto read_x = [&](const half_t* tile, int h, int j, half8_t (&dst)[TT]) __attribute__((always_inline)) {
 #pragma unroll
-      for (int h = 0; h < NH; ++h) {
-        half8_t wop[kWideRP][2];
+        for (int t = 0; t < TT; ++t) dst[t] = *reinterpret_cast<const half8_t*>(tile + t * 32 * kWideStride + h * 32 + 8 * j);
+      };
+      auto mma = [&](const half8_t (&xo)[TT], const half8_t (&wo)[kWideRP]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int t = 0; t < TT; ++t)
+#pragma unroll
+          for (int a = 0; a < kWideRP; ++a) acc[a][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xo[t], wo[a], acc[a][t], 0, 0, 0);
+      };
+      // the order the scheduler is asked for inside a slice: one matrix-core instruction, then a few
+      // of the next slice's dequantisation instructions and one of its LDS reads
+      auto interleave = [&]() __attribute__((always_inline)) {
+#define AWQ_SLOT(valu, lds)                                        \
+  __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); /* matrix */  \
+  __builtin_amdgcn_sched_group_barrier(0x002, valu, 0);            \
+  __builtin_amdgcn_sched_group_barrier(0x100, lds, 0);
+        AWQ_SLOT(3, 1) AWQ_SLOT(3, 1) AWQ_SLOT(2, 1) AWQ_SLOT(2, 1)
+        AWQ_SLOT(2, 0) AWQ_SLOT(2, 0) AWQ_SLOT(2, 0) AWQ_SLOT(2, 0)
+#undef AWQ_SLOT
+      };
+      __syncthreads();
+      read_x(xlane, 0, 0, xa);
+#pragma unroll
+      for (int a = 0; a < kWideRP; ++a) wa[a] = dequant8<ZINT, false>(wd[a][0][0].x, sc, zz);
+      int buf = 0;  // s % 3
+      auto step = [&](int s0, auto F) __attribute__((always_inline)) {
+        constexpr int f = decltype(F)::value;
+        const int s = s0 + f;
+        if constexpr (f & 1) load_x(s + 3, xr1);
+        else load_x(s + 3, xr0);
+        __syncthreads();  // tile s + 1 is visible; the readers of tile s - 1 are done
+        const int buf1 = buf == 2 ? 0 : buf + 1, buf2 = buf1 == 2 ? 0 : buf1 + 1;
+        const half_t* cur = xlane + buf * kSlot;
+        const half_t* nxt = xlane + buf1 * kSlot;
+        const int sn = s + PF < steps ? s + PF : steps - 1;
+        // slice (h 0, j 0): prepare (0, 1)
+        read_x(cur, 0, 1, xb_);
 #pragma unroll
         for (int a = 0; a < kWideRP; ++a) {
-          wop[a][0] = dequant8<ZINT, false>(wd[a][f][h].x, sc, zz);
-          wop[a][1] = dequant8<ZINT, false>(wd[a][f][h].y, sc, zz);
-          wd[a][f][h] = KSPLIT ? __builtin_nontemporal_load(wp[a] + (int64_t)(sn * NH + h) * 32) : wp[a][(int64_t)(sn * NH + h) * 32];
+          wb[a] = dequant8<ZINT, false>(wd[a][f][0].y, sc, zz);
+          wd[a][f][0] = wp[a][(int64_t)(sn * NH + 0) * 32];
         }
-        // slices outermost: an accumulator tile is touched again only after all the others (a
-        // matrix-core instruction that needs the previous result of its accumulator waits for it)
+        mma(xa, wa);
+        interleave();
+        // slice (0, 1): prepare (1, 0)
+        read_x(cur, 1, 0, xa);
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
+        for (int a = 0; a < kWideRP; ++a) wa[a] = dequant8<ZINT, false>(wd[a][f][1].x, sc, zz);
+        mma(xb_, wb);
+        interleave();
+        // slice (1, 0): prepare (1, 1)
+        read_x(cur, 1, 1, xb_);
 #pragma unroll
-          for (int t = 0; t < TT; ++t) {
-            // slice j: k = 8 (j + 2 kh) .. + 7 of block h
-            const half8_t xop = *reinterpret_cast<const half8_t*>(xb + t * 32 * kWideStride + h * 32 + 8 * j);
+        for (int a = 0; a < kWideRP; ++a) {
+          wb[a] = dequant8<ZINT, false>(wd[a][f][1].y, sc, zz);
+          wd[a][f][1] = wp[a][(int64_t)(sn * NH + 1) * 32];
+        }
+        mma(xa, wa);
+        interleave();
+        // slice (1, 1): prepare (0, 0) of the next step
+        read_x(nxt, 0, 0, xa);
 #pragma unroll
-            for (int a = 0; a < kWideRP; ++a)
-              acc[a][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xop, wop[a][j], acc[a][t], 0, 0, 0);
+        for (int a = 0; a < kWideRP; ++a) wa[a] = dequant8<ZINT, false>(wd[a][f ^ 1][0].x, sc, zz);
+        mma(xb_, wb);
+        interleave();
+        if constexpr (f & 1) store_x(buf2, xr0);
+        else store_x(buf2, xr1);
+        buf = buf1;
+      };
+      for (int s0 = 0; s0 < steps; s0 += 2) {
+        step(s0, std::integral_constant<int, 0>{});
+        step(s0, std::integral_constant<int, 1>{});
+      }
+    } else {
+      load_x(0, xr0);
+      store_x(0, xr0);
+      load_x(1, xr1);
+      // one step; F is its index inside the unrolled pair (a compile-time constant)
+      auto step = [&](int s0, auto F) __attribute__((always_inline)) {
+        constexpr int f = decltype(F)::value;
+        const int s = s0 + f;
+        // tile s left these registers one step ago
+        if constexpr (f & 1) load_x(s + 2, xr1);
+        else load_x(s + 2, xr0);
+        __syncthreads();  // tile s is in buffer s & 1; the readers of tile s-1 are done
+        const half_t* xb = xs + ((s & 1) * NKB + slot) * kSlot + n * kWideStride + 16 * kh;
+        const int sn = s + PF < steps ? s + PF : steps - 1;
+  #pragma unroll
+        for (int h = 0; h < NH; ++h) {
+          half8_t wop[kWideRP][2];
+  #pragma unroll
+          for (int a = 0; a < kWideRP; ++a) {
+            wop[a][0] = dequant8<ZINT, false>(wd[a][f][h].x, sc, zz);
+            wop[a][1] = dequant8<ZINT, false>(wd[a][f][h].y, sc, zz);
+            wd[a][f][h] = KSPLIT ? __builtin_nontemporal_load(wp[a] + (int64_t)(sn * NH + h) * 32) : wp[a][(int64_t)(sn * NH + h) * 32];
+          }
+          // slices outermost: an accumulator tile is touched again only after all the others (a
+          // matrix-core instruction that needs the previous result of its accumulator waits for it)
+  #pragma unroll
+          for (int j = 0; j < 2; ++j) {
+  #pragma unroll
+            for (int t = 0; t < TT; ++t) {
+              // slice j: k = 8 (j + 2 kh) .. + 7 of block h
+              const half8_t xop = *reinterpret_cast<const half8_t*>(xb + t * 32 * kWideStride + h * 32 + 8 * j);
+  #pragma unroll
+              for (int a = 0; a < kWideRP; ++a)
+                acc[a][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xop, wop[a][j], acc[a][t], 0, 0, 0);
+            }
           }
         }
+        if constexpr (f & 1) store_x((s + 1) & 1, xr0);
+        else store_x((s + 1) & 1, xr1);
+      };
+      for (int s0 = 0; s0 < steps; s0 += 2) {
+        step(s0, std::integral_constant<int, 0>{});
+        step(s0, std::integral_constant<int, 1>{});
       }
-      if constexpr (f & 1) store_x((s + 1) & 1, xr0);
-      else store_x((s + 1) & 1, xr1);
-    };
-    for (int s0 = 0; s0 < steps; s0 += 2) {
-      step(s0, std::integral_constant<int, 0>{});
-      step(s0, std::integral_constant<int, 1>{});
+
     }
 
     const float scf = (float)sc;  // the wavefront's rows share one scale: it multiplies the sums, not every weight
@@ -438,7 +545,7 @@ __global__ __launch_bounds__(256, (MODE == WIDE_K && TT == 4) ? 1 : 2) void gemm
 #pragma unroll
           for (int i = 0; i < 16; ++i) {
             const int tok = t0 + t * 32 + (i >> 2) * 8 + kh * 4 + (i & 3);
-            if (tok < p.M) store_out<EPI>(p, tok, row, acc[a][t][i] * scf);
+            if (tok < p.M) store_out<EPI, true>(p, tok, row, acc[a][t][i] * scf);
           }
         }
       }
@@ -473,7 +580,7 @@ __global__ __launch_bounds__(256, (MODE == WIDE_K && TT == 4) ? 1 : 2) void gemm
               const int tok = t0 + t * 32 + i4 * 8 + kh * 4 + i;
               if (tok < p.M) {
                 if (epi < 0) p.part[((int64_t)blockIdx.z * p.M + tok) * p.m + row] = v[i];
-                else store_out<(epi < 0 ? 0 : epi)>(p, tok, row, v[i]);
+                else store_out<(epi < 0 ? 0 : epi), true>(p, tok, row, v[i]);
               }
             }
           }
@@ -493,7 +600,7 @@ __global__ __launch_bounds__(256) void reduce_parts_kernel(GemmParams p) {
   if (at >= total) return;
   float v = p.part[at];
   for (int z = 1; z < p.kz; ++z) v += p.part[(int64_t)z * total + at];
-  with_epilogue(p, [&](auto E) { store_out<decltype(E)::value>(p, (int)(at / p.m), (int)(at % p.m), v); });
+  with_epilogue(p, [&](auto E) { store_out<decltype(E)::value, true>(p, (int)(at / p.m), (int)(at % p.m), v); });
 }
 
 // tokens per workgroup of the k-split shape: 32, 64 or 128
