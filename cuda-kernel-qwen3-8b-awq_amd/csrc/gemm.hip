@@ -296,7 +296,8 @@ __global__ __launch_bounds__(256, (MODE == WIDE_K && TT == 4) ? 1 : 2) void gemm
     int xdst[PPT];
 #pragma unroll
     for (int i = 0; i < PPT; ++i) {
-      const int pc = tid + i * 256;
+      // k split: every wavefront stages its own slot (nobody else reads it: no workgroup barrier in the main loop)
+      const int pc = KSPLIT ? wave * PCS + lane + i * 64 : tid + i * 256;
       const int j = pc / PCS, tok = (pc % PCS) / (4 * NH), part = pc % (4 * NH);
       const int tg = t0 + tok < p.M ? t0 + tok : p.M - 1;
       xsrc[i] = p.x + (int64_t)tg * p.k + (kb_wg + (KSPLIT ? j * tile_steps * NH : 0)) * 32 + part * 8;
@@ -337,140 +338,130 @@ __global__ __launch_bounds__(256, (MODE == WIDE_K && TT == 4) ? 1 : 2) void gemm
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[a][t][i] = 0.0f;
 
-    if constexpr (!KSPLIT) {
-      // Software pipeline over quarter steps ("slices": 8 matrix-core instructions on one 16-wide
-      // piece of k).  While a slice is multiplied, the token operands of the next one are read from
-      // LDS and its weight operands are dequantised, so no instruction waits for a read issued just
-      // before it.  Three token tiles rotate through LDS: tile s + 1 is already visible during step
-      // s (the last slice of a step prepares the first of the next across the barrier) and tile
-      // s + 2 is written at the end of step s into the buffer tile s - 1 left before the barrier.
-      if (CUT) __syncthreads();  // the previous piece's readers are done
-      load_x(0, xr0);
-      store_x(0, xr0);
+    // Software pipeline over quarter steps ("slices": 2 TT matrix-core instructions on one 16-wide
+    // piece of k).  While a slice is multiplied, the token operands of the next one are read from
+    // LDS and its weight operands are dequantised, so no instruction waits for a read issued just
+    // before it; the last slice of a step prepares the first of the next.
+    //   rows split: three token tiles rotate through LDS.  Tile s + 1 is already visible during
+    //     step s and tile s + 2 is written at the end of step s into the buffer that tile s - 1
+    //     left before the step's barrier.
+    //   k split: a wavefront stages its own slot and nobody else reads it, so there is no workgroup
+    //     barrier; its LDS instructions execute in order, which lets two tiles do: tile s + 1 is
+    //     written before the last slice of step s reads it.
+    constexpr int NBUF = KSPLIT ? 2 : 3;
+    auto publish = [&]() __attribute__((always_inline)) {
+      if constexpr (KSPLIT) {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the writes have left the queue
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      } else {
+        __syncthreads();
+      }
+    };
+    auto wload = [&](int a, int64_t blk) __attribute__((always_inline)) {
+      return KSPLIT ? __builtin_nontemporal_load(wp[a] + blk * 32) : wp[a][blk * 32];
+    };
+    if (CUT) __syncthreads();  // the previous piece's readers are done
+    load_x(0, xr0);
+    store_x(0, xr0);
+    if constexpr (KSPLIT) {
+      load_x(1, xr1);
+    } else {
       load_x(1, xr0);
       store_x(1, xr0);
       load_x(2, xr1);
-      half8_t xa[TT], xb_[TT], wa[kWideRP], wb[kWideRP];
-      const half_t* xlane = xs + n * kWideStride + 16 * kh;
-      auto read_x = [&](const half_t* tile, int h, int j, half8_t (&dst)[TT]) __attribute__((always_inline)) {
+    }
+    half8_t xa[TT], xb_[TT], wa[kWideRP], wb[kWideRP];
+    const half_t* xlane = xs + slot * kSlot + n * kWideStride + 16 * kh;
+    auto read_x = [&](const half_t* tile, int h, int j, half8_t (&dst)[TT]) __attribute__((always_inline)) {
 #pragma unroll
-        for (int t = 0; t < TT; ++t) dst[t] = *reinterpret_cast<const half8_t*>(tile + t * 32 * kWideStride + h * 32 + 8 * j);
-      };
-      auto mma = [&](const half8_t (&xo)[TT], const half8_t (&wo)[kWideRP]) __attribute__((always_inline)) {
+      for (int t = 0; t < TT; ++t) dst[t] = *reinterpret_cast<const half8_t*>(tile + t * 32 * kWideStride + h * 32 + 8 * j);
+    };
+    auto mma = [&](const half8_t (&xo)[TT], const half8_t (&wo)[kWideRP]) __attribute__((always_inline)) {
 #pragma unroll
-        for (int t = 0; t < TT; ++t)
+      for (int t = 0; t < TT; ++t)
 #pragma unroll
-          for (int a = 0; a < kWideRP; ++a) acc[a][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xo[t], wo[a], acc[a][t], 0, 0, 0);
-      };
-      // the order the scheduler is asked for inside a slice: one matrix-core instruction, then a few
-      // of the next slice's dequantisation instructions and one of its LDS reads
-      auto interleave = [&]() __attribute__((always_inline)) {
+        for (int a = 0; a < kWideRP; ++a) acc[a][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xo[t], wo[a], acc[a][t], 0, 0, 0);
+    };
+    // the order the scheduler is asked for inside a slice: one matrix-core instruction, then a few
+    // of the next slice's dequantisation instructions and one of its LDS reads
+    auto interleave = [&]() __attribute__((always_inline)) {
 #define AWQ_SLOT(valu, lds)                                        \
   __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); /* matrix */  \
   __builtin_amdgcn_sched_group_barrier(0x002, valu, 0);            \
   __builtin_amdgcn_sched_group_barrier(0x100, lds, 0);
+      if constexpr (TT == 4) {
         AWQ_SLOT(3, 1) AWQ_SLOT(3, 1) AWQ_SLOT(2, 1) AWQ_SLOT(2, 1)
         AWQ_SLOT(2, 0) AWQ_SLOT(2, 0) AWQ_SLOT(2, 0) AWQ_SLOT(2, 0)
+      } else if constexpr (TT == 2) {
+        AWQ_SLOT(5, 1) AWQ_SLOT(5, 1) AWQ_SLOT(4, 0) AWQ_SLOT(4, 0)
+      } else {
+        AWQ_SLOT(9, 1) AWQ_SLOT(9, 0)
+      }
 #undef AWQ_SLOT
-      };
-      __syncthreads();
-      read_x(xlane, 0, 0, xa);
+    };
+    publish();
+    read_x(xlane, 0, 0, xa);
 #pragma unroll
-      for (int a = 0; a < kWideRP; ++a) wa[a] = dequant8<ZINT, false>(wd[a][0][0].x, sc, zz);
-      int buf = 0;  // s % 3
-      auto step = [&](int s0, auto F) __attribute__((always_inline)) {
-        constexpr int f = decltype(F)::value;
-        const int s = s0 + f;
-        if constexpr (f & 1) load_x(s + 3, xr1);
-        else load_x(s + 3, xr0);
-        __syncthreads();  // tile s + 1 is visible; the readers of tile s - 1 are done
-        const int buf1 = buf == 2 ? 0 : buf + 1, buf2 = buf1 == 2 ? 0 : buf1 + 1;
-        const half_t* cur = xlane + buf * kSlot;
-        const half_t* nxt = xlane + buf1 * kSlot;
-        const int sn = s + PF < steps ? s + PF : steps - 1;
-        // slice (h 0, j 0): prepare (0, 1)
-        read_x(cur, 0, 1, xb_);
+    for (int a = 0; a < kWideRP; ++a) wa[a] = dequant8<ZINT, false>(wd[a][0][0].x, sc, zz);
+    int buf = 0;  // s % NBUF
+    auto step = [&](int s0, auto F) __attribute__((always_inline)) {
+      constexpr int f = decltype(F)::value;
+      const int s = s0 + f;
+      // the tile that left these registers one step ago
+      if constexpr (f & 1) load_x(s + NBUF, xr1);
+      else load_x(s + NBUF, xr0);
+      if constexpr (!KSPLIT) __syncthreads();  // tile s + 1 is visible; the readers of tile s - 1 are done
+      const int buf1 = buf == NBUF - 1 ? 0 : buf + 1, buf2 = buf1 == NBUF - 1 ? 0 : buf1 + 1;
+      const half_t* cur = xlane + buf * NKB * kSlot;
+      const half_t* nxt = xlane + buf1 * NKB * kSlot;
+      const int sn = s + PF < steps ? s + PF : steps - 1;
+      // slice (h 0, j 0): prepare (0, 1)
+      read_x(cur, 0, 1, xb_);
 #pragma unroll
-        for (int a = 0; a < kWideRP; ++a) {
-          wb[a] = dequant8<ZINT, false>(wd[a][f][0].y, sc, zz);
-          wd[a][f][0] = wp[a][(int64_t)(sn * NH + 0) * 32];
-        }
-        mma(xa, wa);
-        interleave();
-        // slice (0, 1): prepare (1, 0)
-        read_x(cur, 1, 0, xa);
+      for (int a = 0; a < kWideRP; ++a) {
+        wb[a] = dequant8<ZINT, false>(wd[a][f][0].y, sc, zz);
+        wd[a][f][0] = wload(a, (int64_t)(sn * NH + 0));
+      }
+      mma(xa, wa);
+      interleave();
+      // slice (0, 1): prepare (1, 0)
+      read_x(cur, 1, 0, xa);
 #pragma unroll
-        for (int a = 0; a < kWideRP; ++a) wa[a] = dequant8<ZINT, false>(wd[a][f][1].x, sc, zz);
-        mma(xb_, wb);
-        interleave();
-        // slice (1, 0): prepare (1, 1)
-        read_x(cur, 1, 1, xb_);
+      for (int a = 0; a < kWideRP; ++a) wa[a] = dequant8<ZINT, false>(wd[a][f][1].x, sc, zz);
+      mma(xb_, wb);
+      interleave();
+      // slice (1, 0): prepare (1, 1)
+      read_x(cur, 1, 1, xb_);
 #pragma unroll
-        for (int a = 0; a < kWideRP; ++a) {
-          wb[a] = dequant8<ZINT, false>(wd[a][f][1].y, sc, zz);
-          wd[a][f][1] = wp[a][(int64_t)(sn * NH + 1) * 32];
-        }
-        mma(xa, wa);
-        interleave();
-        // slice (1, 1): prepare (0, 0) of the next step
-        read_x(nxt, 0, 0, xa);
+      for (int a = 0; a < kWideRP; ++a) {
+        wb[a] = dequant8<ZINT, false>(wd[a][f][1].y, sc, zz);
+        wd[a][f][1] = wload(a, (int64_t)(sn * NH + 1));
+      }
+      mma(xa, wa);
+      interleave();
+      if constexpr (KSPLIT) {
+        // tile s + 1 goes to the other buffer now, ahead of the read below
+        if constexpr (f & 1) store_x(buf1, xr0);
+        else store_x(buf1, xr1);
+        publish();
+      }
+      // slice (1, 1): prepare (0, 0) of the next step
+      read_x(nxt, 0, 0, xa);
 #pragma unroll
-        for (int a = 0; a < kWideRP; ++a) wa[a] = dequant8<ZINT, false>(wd[a][f ^ 1][0].x, sc, zz);
-        mma(xb_, wb);
-        interleave();
+      for (int a = 0; a < kWideRP; ++a) wa[a] = dequant8<ZINT, false>(wd[a][f ^ 1][0].x, sc, zz);
+      mma(xb_, wb);
+      interleave();
+      if constexpr (!KSPLIT) {
         if constexpr (f & 1) store_x(buf2, xr0);
         else store_x(buf2, xr1);
-        buf = buf1;
-      };
-      for (int s0 = 0; s0 < steps; s0 += 2) {
-        step(s0, std::integral_constant<int, 0>{});
-        step(s0, std::integral_constant<int, 1>{});
       }
-    } else {
-      load_x(0, xr0);
-      store_x(0, xr0);
-      load_x(1, xr1);
-      // one step; F is its index inside the unrolled pair (a compile-time constant)
-      auto step = [&](int s0, auto F) __attribute__((always_inline)) {
-        constexpr int f = decltype(F)::value;
-        const int s = s0 + f;
-        // tile s left these registers one step ago
-        if constexpr (f & 1) load_x(s + 2, xr1);
-        else load_x(s + 2, xr0);
-        __syncthreads();  // tile s is in buffer s & 1; the readers of tile s-1 are done
-        const half_t* xb = xs + ((s & 1) * NKB + slot) * kSlot + n * kWideStride + 16 * kh;
-        const int sn = s + PF < steps ? s + PF : steps - 1;
-  #pragma unroll
-        for (int h = 0; h < NH; ++h) {
-          half8_t wop[kWideRP][2];
-  #pragma unroll
-          for (int a = 0; a < kWideRP; ++a) {
-            wop[a][0] = dequant8<ZINT, false>(wd[a][f][h].x, sc, zz);
-            wop[a][1] = dequant8<ZINT, false>(wd[a][f][h].y, sc, zz);
-            wd[a][f][h] = KSPLIT ? __builtin_nontemporal_load(wp[a] + (int64_t)(sn * NH + h) * 32) : wp[a][(int64_t)(sn * NH + h) * 32];
-          }
-          // slices outermost: an accumulator tile is touched again only after all the others (a
-          // matrix-core instruction that needs the previous result of its accumulator waits for it)
-  #pragma unroll
-          for (int j = 0; j < 2; ++j) {
-  #pragma unroll
-            for (int t = 0; t < TT; ++t) {
-              // slice j: k = 8 (j + 2 kh) .. + 7 of block h
-              const half8_t xop = *reinterpret_cast<const half8_t*>(xb + t * 32 * kWideStride + h * 32 + 8 * j);
-  #pragma unroll
-              for (int a = 0; a < kWideRP; ++a)
-                acc[a][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xop, wop[a][j], acc[a][t], 0, 0, 0);
-            }
-          }
-        }
-        if constexpr (f & 1) store_x((s + 1) & 1, xr0);
-        else store_x((s + 1) & 1, xr1);
-      };
-      for (int s0 = 0; s0 < steps; s0 += 2) {
-        step(s0, std::integral_constant<int, 0>{});
-        step(s0, std::integral_constant<int, 1>{});
-      }
-
+      buf = buf1;
+    };
+    for (int s0 = 0; s0 < steps; s0 += 2) {
+      step(s0, std::integral_constant<int, 0>{});
+      step(s0, std::integral_constant<int, 1>{});
     }
 
     const float scf = (float)sc;  // the wavefront's rows share one scale: it multiplies the sums, not every weight
