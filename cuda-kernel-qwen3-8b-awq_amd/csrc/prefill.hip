@@ -27,42 +27,60 @@ __global__ __launch_bounds__(256) void embed_batch_kernel(const uint8_t* __restr
   out[(int64_t)blockIdx.y * hidden + idx] = d * scale[g];
 }
 
-// rmsNormKernel, Inference.cu:111-145, one workgroup per token
+// rmsNormKernel, Inference.cu:111-145, one workgroup per token: 16-byte loads, the
+// sum of squares through wavefront shuffles and one LDS exchange
 __global__ __launch_bounds__(256) void rmsnorm_batch_kernel(const half_t* __restrict__ x,
                                                             const half_t* __restrict__ gamma,
                                                             half_t* __restrict__ out, int n, float eps) {
-  __shared__ float buf[256];
+  __shared__ float wsum[4];
   const int tid = threadIdx.x;
-  x += (int64_t)blockIdx.x * n;
-  out += (int64_t)blockIdx.x * n;
+  const half8_t* xv = reinterpret_cast<const half8_t*>(x + (int64_t)blockIdx.x * n);
+  const half8_t* gv = reinterpret_cast<const half8_t*>(gamma);
+  half8_t* ov = reinterpret_cast<half8_t*>(out + (int64_t)blockIdx.x * n);
+  const int chunks = n >> 3;
+  constexpr int kKeep = 4;  // chunks a thread keeps in registers (n <= 8192: all of them)
+  half8_t held[kKeep];
   float acc = 0.0f;
-  for (int i = tid; i < n; i += 256) {
-    const float v = (float)x[i];
-    acc = __builtin_fmaf(v, v, acc);
+#pragma unroll
+  for (int c = 0; c < kKeep; ++c) {
+    const int at = tid + c * 256;
+    if (at < chunks) {
+      held[c] = xv[at];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc = __builtin_fmaf((float)held[c][e], (float)held[c][e], acc);
+    }
   }
-  buf[tid] = acc;
+  for (int at = tid + kKeep * 256; at < chunks; at += 256) {
+    const half8_t v = xv[at];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc = __builtin_fmaf((float)v[e], (float)v[e], acc);
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+  if ((tid & 63) == 0) wsum[tid >> 6] = acc;
   __syncthreads();
-  for (int stride = 128; stride > 0; stride >>= 1) {
-    if (tid < stride) buf[tid] += buf[tid + stride];
-    __syncthreads();
+  const float total = (wsum[0] + wsum[1]) + (wsum[2] + wsum[3]);
+  const half_t sc = (half_t)awq_rsqrtf(total / (float)n + eps);
+  const half8_t sc8 = half8_t{sc, sc, sc, sc, sc, sc, sc, sc};
+#pragma unroll
+  for (int c = 0; c < kKeep; ++c) {
+    const int at = tid + c * 256;
+    if (at < chunks) ov[at] = (held[c] * sc8) * gv[at];
   }
-  const half_t sc = (half_t)awq_rsqrtf(buf[0] / (float)n + eps);
-  for (int i = tid; i < n; i += 256) {
-    const half_t t = x[i] * sc;
-    out[i] = t * gamma[i];
-  }
+  for (int at = tid + kKeep * 256; at < chunks; at += 256) ov[at] = (xv[at] * sc8) * gv[at];
 }
 
 // QKV split, rotary on Q and K, KV append (Inference.cu:1070-1103, 150-177) for
-// token blockIdx.y at position pos0 + blockIdx.y; one workgroup per head.
-__global__ __launch_bounds__(64) void rope_kv_batch_kernel(const half_t* __restrict__ qkv,
+// token blockIdx.y at position pos0 + blockIdx.y; one wavefront per head, four heads per workgroup.
+__global__ __launch_bounds__(256) void rope_kv_batch_kernel(const half_t* __restrict__ qkv,
                                                            const half_t* __restrict__ cos_t,
                                                            const half_t* __restrict__ sin_t,
                                                            half_t* __restrict__ q_out, half_t* __restrict__ kc,
                                                            half_t* __restrict__ vc, int n_heads, int64_t max_pos,
                                                            int pos0) {
   const int tok = blockIdx.y, pos = pos0 + tok;
-  const int hd = blockIdx.x, i = threadIdx.x;
+  const int hd = blockIdx.x * 4 + (threadIdx.x >> 6), i = threadIdx.x & 63;
+  if (hd >= n_heads) return;
   const int H = n_heads * AWQ_HEAD_DIM;
   qkv += (int64_t)tok * 3 * H;
   q_out += (int64_t)tok * H;
@@ -270,7 +288,7 @@ int launch_rope_kv_append_batch(const half_t* qkv, const half_t* cos_t, const ha
                                 hipStream_t st) {
   AWQ_REQUIRE(n_heads > 0 && max_pos > 0, "n_heads and max_pos must be positive");
   AWQ_REQUIRE(M >= 1 && M <= 65535 && pos0 >= 0 && pos0 + M <= max_pos, "positions out of range");
-  hipLaunchKernelGGL(rope_kv_batch_kernel, dim3((unsigned)n_heads, (unsigned)M), dim3(64), 0, st, qkv, cos_t, sin_t,
+  hipLaunchKernelGGL(rope_kv_batch_kernel, dim3((unsigned)((n_heads + 3) / 4), (unsigned)M), dim3(256), 0, st, qkv, cos_t, sin_t,
                      q_out, kc, vc, n_heads, max_pos, (int)pos0);
   AWQ_HIP_TRY(hipGetLastError());
   return AWQ_OK;
