@@ -753,7 +753,7 @@ extern "C" int awq_prefill(awq_engine* e, const int32_t* prompt_ids, int32_t n_p
 
 namespace {
 
-constexpr int64_t kPrefillChunk = 1024;  // prompt positions per batched pass
+constexpr int64_t kPrefillChunk = 1280;  // prompt positions per batched pass
 constexpr int64_t kGemmWsBytes = (64ll << 20) + 4096;  // header + partial sums (256 tiles, or 4 chunks of k for few rows)
 
 int ensure_prefill_buffers(awq_engine* e) {
@@ -821,8 +821,12 @@ extern "C" int awq_prefill_batched(awq_engine* e, const int32_t* prompt_ids, int
   if (n_prompt == 0) return AWQ_OK;
   if (int rc = ensure_prefill_buffers(e)) return rc;
   const int64_t H = e->cfg.hidden;
-  for (int64_t off = 0; off < n_prompt; off += e->pb.chunk) {
-    const int64_t M = std::min<int64_t>(e->pb.chunk, n_prompt - off), pos0 = e->n_positions;
+  for (int64_t off = 0, M = 0; off < n_prompt; off += M) {
+    // equal passes rather than full ones and a small rest (whole 128-token tiles each): 4096 positions
+    // go as 4 x 1024, not 3 x 1280 + 256
+    const int64_t rest = n_prompt - off, passes = (rest + e->pb.chunk - 1) / e->pb.chunk;
+    M = std::min<int64_t>(rest, std::min<int64_t>(e->pb.chunk, ((rest + passes - 1) / passes + 127) / 128 * 128));
+    const int64_t pos0 = e->n_positions;
     AWQ_HIP_TRY(hipMemcpyAsync(e->pb.tokens, prompt_ids + off, (size_t)M * 4, hipMemcpyHostToDevice, e->stream));
     if (int rc = launch_embed_batch(e->embed.packed, e->embed.scale, e->embed.zp, H, e->cfg.vocab, e->pb.tokens, M,
                                     e->pb.hidden, e->stream))

@@ -156,8 +156,9 @@ def test_full_model_batched_prompt_tokens(awq, oracle, torch_gpu):
 
 def test_long_prompt_takes_the_rows_split_products(awq, oracle, torch_gpu):
     """A 1027-token prompt at full width: every product of the layer has enough output tiles for the
-    rows-split workgroup shape (with the GeLU and residual epilogues), and the prompt spans the
-    short-sequence and the long-sequence attention launches of the batched pass."""
+    rows-split workgroup shapes (Wqkv and W1 a tile per workgroup, Wo and W2 with their 144 tiles cut
+    evenly over 256 workgroups that hand FP32 sums over; GeLU and residual epilogues), and the prompt
+    spans the short-sequence and the long-sequence attention launches of the batched pass."""
     cfg = awq.make_config(n_layers=1, vocab=2048, max_pos=1100)
     model = make_oracle_model(oracle, cfg)   # only as the host buffer of the weights here
     eng = awq.QWen3AWQInfer.empty(cfg)
