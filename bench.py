@@ -156,6 +156,14 @@ def main():
                 "frac": round(w1["GBs"] / HBM_PEAK_GBS, 4), "traffic": traffic,
                 "bytes_per_launch": w1["bytes"], "us_per_launch": w1["us"], "all_shapes": kernels}
 
+    # ---- the prompt pass's product on the matrix cores: w1 shape, 2048 tokens (config 5) ---------
+    w4a16 = importlib.import_module("cuda-kernel-qwen3-8b-awq_amd.bench_w4a16")
+    g = w4a16.measure((2048,), ("w1",))["shapes"]["w1"]["M=2048"]
+    prefill_gemm = {"workload": "W4A16 product 12288 x 4096 (int4 g=128) x 2048 tokens, 12 rotating matrices",
+                    "bound": "mfma", "achieved": g["TFLOPs"], "peak": 2500.0, "unit": "TFLOP/s",
+                    "frac": g["mfma_frac"], "us_per_launch": g["us"]}
+    log("gemm w1 x 2048 tokens: %.1f us, %.0f TFLOP/s (%.1f%% of 2.5 PFLOP/s)" % (g["us"], g["TFLOPs"], 100 * g["mfma_frac"]))
+
     # ---- CPU oracle on this host's cores, bounded sample; and token identity on that sample ------
     cpu = None
     tokens_match = None
@@ -192,6 +200,7 @@ def main():
         "step_hbm_frac": round(step_bytes * tok_s / (HBM_PEAK_GBS * 1e9), 4),
         "greedy_tokens_identical_to_cpu": tokens_match,
         "prompt_pass_ms": prefill_ms,
+        "prefill_gemm": prefill_gemm,
         "roofline": roofline,
         "cpu_baseline": cpu,
     }

@@ -22,10 +22,11 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 sys.path.insert(0, ROOT)
 
 
-def main():
-    tokens = (1, 4, 16, 64, 128, 512, 2048)
-    if len(sys.argv) > 1:
-        tokens = tuple(int(v) for v in sys.argv[1].split(","))
+ALL_SHAPES = (("w1", (12288, 4096)), ("w2", (4096, 12288)))
+
+
+def measure(tokens, shapes=("w1", "w2")):
+    """Time the products for the given token counts on the named shapes; returns the result dictionary."""
     import numpy as np
     import torch
     awq = importlib.import_module("cuda-kernel-qwen3-8b-awq_amd")
@@ -33,7 +34,9 @@ def main():
     st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     out = {"mfma_peak_tflops": 2500.0, "hbm_peak_gbs": 8000.0, "shapes": {}}
     n_mat = 12  # 12 x 25 MB = 300 MB working set, above the 256 MB last-level cache
-    for name, (m, k) in (("w1", (12288, 4096)), ("w2", (4096, 12288))):
+    for name, (m, k) in ALL_SHAPES:
+        if name not in shapes:
+            continue
         mats = []
         for i in range(n_mat):
             host = np.zeros(m * k // 2, dtype=np.uint8)
@@ -80,12 +83,20 @@ def main():
             res["M=%d" % M] = {"us": round(us, 2), "TFLOPs": round(flops / us / 1e6, 2),
                                "mfma_frac": round(flops / us / 1e6 / 2500.0, 4), "GBs": round(nbytes / us / 1e3, 1),
                                "hbm_frac": round(nbytes / us / 1e3 / 8000.0, 4),
-                               "kernel": "gemv (VALU, bit-exact order)" if M == 1 else "gemm (MFMA 16x16x32 f16)"}
+                               "kernel": "gemv (VALU, bit-exact order)" if M == 1 else
+                                         ("gemm (MFMA 16x16x32 f16)" if M <= 4 else "gemm (MFMA 32x32x16 f16)")}
             print(name, "M=%d" % M, res["M=%d" % M], file=sys.stderr, flush=True)
         out["shapes"][name] = res
         del mats
         torch.cuda.empty_cache()
-    print(json.dumps(out))
+    return out
+
+
+def main():
+    tokens = (1, 4, 16, 64, 128, 512, 2048)
+    if len(sys.argv) > 1:
+        tokens = tuple(int(v) for v in sys.argv[1].split(","))
+    print(json.dumps(measure(tokens)))
 
 
 if __name__ == "__main__":
