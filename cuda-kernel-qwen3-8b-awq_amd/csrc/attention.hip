@@ -310,8 +310,15 @@ __global__ __launch_bounds__(kSplitWaves * 64) void attn_exp_kernel(SplitArgs a)
   }
 }
 
-// weighted sums of V per chunk (Inference.cu:251-265), one wavefront per chunk
+// weighted sums of V per chunk (Inference.cu:251-265), one wavefront per chunk.
+// The normaliser Z is the ordered sum of all chunk sums: they go through LDS
+// once per workgroup (every thread then adds them in order from broadcast reads;
+// read straight from memory the same loop cost tens of microseconds per
+// wavefront).  A lane divides one probability of the chunk and the lanes exchange
+// them; the values stream in two halves so that loads stay in flight while the
+// other half is multiplied.
 __global__ __launch_bounds__(kSplitWaves * 64) void attn_pv_kernel(SplitArgs a) {
+  extern __shared__ float zs[];  // the chunk sums of this head
   const int L = split_len(a);
   const int head = blockIdx.x;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -324,41 +331,52 @@ __global__ __launch_bounds__(kSplitWaves * 64) void attn_pv_kernel(SplitArgs a) 
   int c_lo, c_hi;
   split_range(nchunks, &c_lo, &c_hi);
   if (c_lo >= c_hi) return;
-  // the first chunk's values are requested before the (latency-bound) sum of the chunk sums
-  half8_t vv[16];
-  int chunk = c_lo + wave;
-  if (chunk < c_hi) {
+  half8_t va[8], vb[8];
+  auto load_half = [&](int chunk, int half, half8_t (&dst)[8]) __attribute__((always_inline)) {
 #pragma unroll
-    for (int nl = 0; nl < 16; ++nl) {
-      const int t = (chunk << 6) + 4 * nl + tq;
-      if (t < L) vv[nl] = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(vh + (int64_t)t * AWQ_HEAD_DIM + 8 * dl));
+    for (int u = 0; u < 8; ++u) {
+      const int t = (chunk << 6) + 4 * (8 * half + u) + tq;
+      if (chunk < c_hi && t < L)
+        dst[u] = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(vh + (int64_t)t * AWQ_HEAD_DIM + 8 * dl));
     }
-  }
-  float Z = cs[0];
-  for (int c = 1; c < nchunks; ++c) Z += cs[c];
+  };
+  int chunk = c_lo + wave;
+  // this wavefront's first exponentials and values are requested before the sum of the chunk sums
+  float e_lane = (chunk < c_hi && (chunk << 6) + lane < L) ? s[(chunk << 6) + lane] : 0.0f;
+  load_half(chunk, 0, va);
+  load_half(chunk, 1, vb);
+  for (int c = tid; c < nchunks; c += kSplitWaves * 64) zs[c] = cs[c];
+  __syncthreads();
+  float Z = zs[0];
+  for (int c = 1; c < nchunks; ++c) Z += zs[c];
   for (; chunk < c_hi; chunk += kSplitWaves) {
     const int base = chunk << 6;
+    const float p_lane = e_lane / Z;  // probability of position base + lane
+    const int nxt = chunk + kSplitWaves;
+    e_lane = (nxt < c_hi && (nxt << 6) + lane < L) ? s[(nxt << 6) + lane] : 0.0f;
     float acc[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
 #pragma unroll
-    for (int nl = 0; nl < 16; ++nl) {
-      const int t = base + 4 * nl + tq;
+    for (int u = 0; u < 8; ++u) {
+      const int t = base + 4 * u + tq;
+      const float pr = __shfl(p_lane, 4 * u + tq, 64);
       if (t < L) {
-        const float p = s[t] / Z;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) acc[i] = __builtin_fmaf(p, (float)vv[nl][i], acc[i]);
+        for (int i = 0; i < 8; ++i) acc[i] = __builtin_fmaf(pr, (float)va[u][i], acc[i]);
       }
     }
-    // the next chunk's values while this one is reduced and stored
-    const int nxt = chunk + kSplitWaves;
-    if (nxt < c_hi) {
+    load_half(nxt, 0, va);
 #pragma unroll
-      for (int nl = 0; nl < 16; ++nl) {
-        const int t = (nxt << 6) + 4 * nl + tq;
-        if (t < L) vv[nl] = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(vh + (int64_t)t * AWQ_HEAD_DIM + 8 * dl));
+    for (int u = 0; u < 8; ++u) {
+      const int t = base + 4 * (8 + u) + tq;
+      const float pr = __shfl(p_lane, 4 * (8 + u) + tq, 64);
+      if (t < L) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] = __builtin_fmaf(pr, (float)vb[u][i], acc[i]);
       }
     }
+    load_half(nxt, 1, vb);
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       acc[i] = xor_add(acc[i], 16);
@@ -371,23 +389,41 @@ __global__ __launch_bounds__(kSplitWaves * 64) void attn_pv_kernel(SplitArgs a) 
   }
 }
 
-// chunk vectors added in chunk order (Inference.cu:259-265 runs over t in order)
-__global__ __launch_bounds__(AWQ_HEAD_DIM) void attn_sum_kernel(SplitArgs a) {
+// chunk vectors added in chunk order (Inference.cu:259-265 runs over t in order).
+// The additions of one output element are a sequential chain, but the loads
+// need not be: 16 wavefronts per head (8 stages x 2 halves of the 128 elements)
+// each request up to 80 consecutive chunks of their half at once, then stage
+// after stage continues the running sums, which pass through LDS.
+constexpr int kSumStages = 8;
+constexpr int kSumRows = 80;  // chunks per stage and round
+__global__ __launch_bounds__(kSumStages * 2 * 64) void attn_sum_kernel(SplitArgs a) {
+  __shared__ float run[AWQ_HEAD_DIM];
   const int L = split_len(a);
   const int head = blockIdx.x, tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int stage = wave >> 1, col = (wave & 1) * 64 + lane;
   const float* cv = a.cv + (int64_t)head * a.max_chunks * AWQ_HEAD_DIM;
   const int nchunks = (L + 63) >> 6;
-  float out = cv[tid];
-  int c = 1;
-  for (; c + 16 <= nchunks; c += 16) {
-    float v[16];
+  for (int c0 = 0; c0 < nchunks; c0 += kSumStages * kSumRows) {
+    const int first = c0 + stage * kSumRows;
+    const int count = min(kSumRows, nchunks - first);  // <= 0: nothing for this stage
+    float v[kSumRows];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) v[i] = cv[(c + i) * AWQ_HEAD_DIM + tid];
+    for (int i = 0; i < kSumRows; ++i)
+      if (i < count) v[i] = cv[(int64_t)(first + i) * AWQ_HEAD_DIM + col];
+    for (int s = 0; s < kSumStages; ++s) {
+      if (s == stage && count > 0) {
+        // chunk 0 starts the sum (0 + x would turn a -0 into +0)
+        float out = first == 0 ? v[0] : run[col];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) out += v[i];
+        for (int i = 0; i < kSumRows; ++i)
+          if (i < count && first + i > 0) out += v[i];
+        run[col] = out;
+      }
+      __syncthreads();
+    }
   }
-  for (; c < nchunks; ++c) out += cv[c * AWQ_HEAD_DIM + tid];
-  a.ctx[head * AWQ_HEAD_DIM + tid] = (half_t)out;
+  if (stage == 0) a.ctx[head * AWQ_HEAD_DIM + col] = (half_t)run[col];
 }
 
 }  // namespace
@@ -426,11 +462,12 @@ int launch_attention(const half_t* q, const half_t* kc, const half_t* vc, half_t
     a.cs = cv + (int64_t)n_heads * mc * AWQ_HEAD_DIM;
     a.pmax = a.cs + (int64_t)n_heads * mc;
     a.max_chunks = mc;
+    AWQ_REQUIRE((int64_t)mc * 4 <= 65536, "sequence too long for the chunk-sum buffer in LDS");
     const dim3 grid(n_heads, kSplit), block(kSplitWaves * 64);
     hipLaunchKernelGGL(attn_scores_kernel, grid, block, 0, st, a);
     hipLaunchKernelGGL(attn_exp_kernel, grid, block, 0, st, a);
-    hipLaunchKernelGGL(attn_pv_kernel, grid, block, 0, st, a);
-    hipLaunchKernelGGL(attn_sum_kernel, dim3(n_heads), dim3(AWQ_HEAD_DIM), 0, st, a);
+    hipLaunchKernelGGL(attn_pv_kernel, grid, block, (size_t)a.max_chunks * 4, st, a);
+    hipLaunchKernelGGL(attn_sum_kernel, dim3(n_heads), dim3(kSumStages * 2 * 64), 0, st, a);
     AWQ_HIP_TRY(hipGetLastError());
     return AWQ_OK;
   }
