@@ -61,7 +61,7 @@ def main():
     from helpers import fill_pair, make_oracle_model, ptr
     import oracle_lib
 
-    max_pos = max(512, args.prompt_len + args.warmup + args.steps + 8)
+    max_pos = max(640, args.prompt_len + args.warmup + args.steps + 8)
     cfg = awq.make_config(n_layers=args.layers, max_pos=max_pos)
     oracle = oracle_lib.load() if args.cpu_steps > 0 else None
 
@@ -156,6 +156,28 @@ def main():
                 "frac": round(w1["GBs"] / HBM_PEAK_GBS, 4), "traffic": traffic,
                 "bytes_per_launch": w1["bytes"], "us_per_launch": w1["us"], "all_shapes": kernels}
 
+    # ---- one layer with about 512 cached positions (config 2): decode steps after a 512-token prompt,
+    #      the unembedding's launch subtracted, divided by the layer count -------------------------
+    p512 = np.zeros(512, dtype=np.int32)
+    awq.check(lib.awq_synth_tokens(args.seed + 1, awq.SYNTH_STREAM_INPUT, ptr(p512), p512.size, cfg.vocab))
+    eng.reset()
+    eng.prefill(p512.tolist(), batched=True)
+    eng.decode(8)
+    torch.cuda.synchronize()
+    t3 = time.perf_counter()
+    eng.decode(64)
+    torch.cuda.synchronize()
+    step_us = (time.perf_counter() - t3) * 1e6 / 64
+    layer_us = (step_us - kernels["unembed"]["us"]) / cfg.n_layers
+    L_mid = 512 + 8 + 32
+    layer_bytes = per_layer + 1024 + 8192 + 2 * cfg.hidden * 2 * L_mid + 16384
+    layer_cfg2 = {"workload": "one layer (RMSNorm, Wqkv + rotary + KV append, attention, Wo, W1 + GeLU, W2), "
+                              "attended length 520..584", "us": round(layer_us, 2), "bytes": int(layer_bytes),
+                  "GBs": round(layer_bytes / layer_us / 1e3, 1),
+                  "hbm_frac": round(layer_bytes / layer_us / 1e3 / HBM_PEAK_GBS, 4)}
+    log("one layer at ~%d positions: %.1f us, %.0f GB/s (%.1f%% of peak)" %
+        (L_mid, layer_us, layer_cfg2["GBs"], 100 * layer_cfg2["hbm_frac"]))
+
     # ---- the prompt pass's product on the matrix cores: w1 shape, 2048 tokens (config 5) ---------
     w4a16 = importlib.import_module("cuda-kernel-qwen3-8b-awq_amd.bench_w4a16")
     g = w4a16.measure((2048,), ("w1",))["shapes"]["w1"]["M=2048"]
@@ -200,6 +222,7 @@ def main():
         "step_hbm_frac": round(step_bytes * tok_s / (HBM_PEAK_GBS * 1e9), 4),
         "greedy_tokens_identical_to_cpu": tokens_match,
         "prompt_pass_ms": prefill_ms,
+        "layer_512_positions": layer_cfg2,
         "prefill_gemm": prefill_gemm,
         "roofline": roofline,
         "cpu_baseline": cpu,
