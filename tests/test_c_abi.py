@@ -155,3 +155,14 @@ def test_workspace_size_queries_need_no_gpu(lib):
     chunks = (max_pos + 63) // 64
     assert lib.awq_attention_workspace_bytes(heads, max_pos) == heads * (max_pos + chunks * 129 + 32) * 4
     assert lib.awq_argmax_workspace_bytes(151936) > 0
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """the benchmark measures one GPU; asking for more ends with a message, before anything touches a device"""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                       timeout=120)
+    assert r.returncode != 0
+    assert "ONE GPU" in r.stderr and r.stdout.strip() == ""
