@@ -204,9 +204,10 @@ constexpr int kWideTokens = 32 * kWideTT;               // 128
 constexpr int kWideNH = 2;                              // 32-wide blocks of k per step
 constexpr int kWideStride = 32 * kWideNH + 8;           // halves per token row of a tile in LDS (16 bytes of padding)
 constexpr int wide_lds_bytes(bool ksplit, int tt) {
-  const int tiles = (ksplit ? 4 * 2 : 3) * (32 * tt) * kWideStride * 2;  // k split: slots x double buffer x tile; rows split: three tiles
-  const int sums = 4 * kWideRP * tt * 64 * 16 * 4;                       // k split: the partial sums
-  return ksplit && sums > tiles ? sums : tiles;
+  if (!ksplit) return 0;  // rows split: three static tiles
+  const int tiles = 4 * 2 * (32 * tt) * kWideStride * 2;  // slots x double buffer x tile
+  const int sums = 4 * kWideRP * tt * 64 * 16 * 4;        // the partial sums
+  return sums > tiles ? sums : tiles;
 }
 
 // Rows split, work cut evenly: the steps of all tiles, in tile order, form one
@@ -321,7 +322,10 @@ __global__ __launch_bounds__(256, (MODE == WIDE_K && TT == 4) ? 1 : 2) void gemm
       const int rg = rows_ok ? rg0 + 2 * a + (n >> 4) : 0;
       wp[a] = reinterpret_cast<const u32x2_t*>(p.wq + (((int64_t)rg * p.nblk + kb_base) * 16 + (n & 15)) * 4 + 2 * kh);
     }
-    constexpr int PF = 2;  // steps of weight dwords in flight
+    // steps of weight dwords in registers.  Rows split: three sets, so that the set a step frees is
+    // requested again at the very start of the next step, ahead of the token tile's requests: the wait
+    // for the tile at the end of a step then covers no younger load.
+    constexpr int PF = KSPLIT ? 2 : 3;
     u32x2_t wd[kWideRP][PF][NH];
 #pragma unroll
     for (int f = 0; f < PF; ++f)
@@ -338,130 +342,245 @@ __global__ __launch_bounds__(256, (MODE == WIDE_K && TT == 4) ? 1 : 2) void gemm
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[a][t][i] = 0.0f;
 
-    // Software pipeline over quarter steps ("slices": 2 TT matrix-core instructions on one 16-wide
-    // piece of k).  While a slice is multiplied, the token operands of the next one are read from
-    // LDS and its weight operands are dequantised, so no instruction waits for a read issued just
-    // before it; the last slice of a step prepares the first of the next.
-    //   rows split: three token tiles rotate through LDS.  Tile s + 1 is already visible during
-    //     step s and tile s + 2 is written at the end of step s into the buffer that tile s - 1
-    //     left before the step's barrier.
-    //   k split: a wavefront stages its own slot and nobody else reads it, so there is no workgroup
-    //     barrier; its LDS instructions execute in order, which lets two tiles do: tile s + 1 is
-    //     written before the last slice of step s reads it.
-    constexpr int NBUF = KSPLIT ? 2 : 3;
-    auto publish = [&]() __attribute__((always_inline)) {
-      if constexpr (KSPLIT) {
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the writes have left the queue
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-      } else {
-        __syncthreads();
+    if constexpr (!KSPLIT) {
+      // Rows split: the token tile of a step goes from memory straight into LDS
+      // (global_load_lds_dwordx4: lane l of a wavefront instruction lands at base + 16 l), no
+      // staging registers and no LDS writes.  A tile is [32 TT tokens][64 k] halves, 128 bytes per
+      // token and unpadded; the eight 16-byte pieces of token row r sit at positions c ^ (r & 7), so
+      // that the eight lanes that read the same piece of eight consecutive rows hit all 32 banks.
+      // Three tiles rotate: during step s the requests for tile s + 2 are in flight (issued behind
+      // the step's barrier, which the readers of tile s - 1 have passed), tile s is multiplied and
+      // the last slice reads the first operands of tile s + 1.  The three tiles are three arrays so
+      // that the compiler can tell which LDS reads a pending request may alias: it waits for the
+      // requests only at the next barrier.  Same software pipeline over quarter steps as below.
+      typedef __attribute__((address_space(1))) const void* gptr_t;
+      typedef __attribute__((address_space(3))) void* lptr_t;
+      constexpr int kTile = kTokens * 64;  // halves
+      __shared__ __attribute__((aligned(16))) half_t tile_a[kTile];
+      __shared__ __attribute__((aligned(16))) half_t tile_b[kTile];
+      __shared__ __attribute__((aligned(16))) half_t tile_c[kTile];
+      // requests: instruction i of this wavefront covers token rows (wave TT + i) 8 .. + 7
+      const int piece = (lane & 7) ^ ((lane >> 3) & 7);  // piece of k this lane fetches for its row
+      const half_t* src[TT];
+#pragma unroll
+      for (int i = 0; i < TT; ++i) {
+        const int tok = t0 + (wave * TT + i) * 8 + (lane >> 3);
+        src[i] = p.x + (int64_t)(tok < p.M ? tok : p.M - 1) * p.k + kb_wg * 32 + piece * 8;
       }
-    };
-    auto wload = [&](int a, int64_t blk) __attribute__((always_inline)) {
-      return KSPLIT ? __builtin_nontemporal_load(wp[a] + blk * 32) : wp[a][blk * 32];
-    };
-    if (CUT) __syncthreads();  // the previous piece's readers are done
-    load_x(0, xr0);
-    store_x(0, xr0);
-    if constexpr (KSPLIT) {
-      load_x(1, xr1);
-    } else {
-      load_x(1, xr0);
-      store_x(1, xr0);
-      load_x(2, xr1);
-    }
-    half8_t xa[TT], xb_[TT], wa[kWideRP], wb[kWideRP];
-    const half_t* xlane = xs + slot * kSlot + n * kWideStride + 16 * kh;
-    auto read_x = [&](const half_t* tile, int h, int j, half8_t (&dst)[TT]) __attribute__((always_inline)) {
+      auto request = [&](half_t* tile, int s) __attribute__((always_inline)) {
+        const int sc_ = s < steps ? s : steps - 1;  // past the end: the last tile again, never used
 #pragma unroll
-      for (int t = 0; t < TT; ++t) dst[t] = *reinterpret_cast<const half8_t*>(tile + t * 32 * kWideStride + h * 32 + 8 * j);
-    };
-    auto mma = [&](const half8_t (&xo)[TT], const half8_t (&wo)[kWideRP]) __attribute__((always_inline)) {
+        for (int i = 0; i < TT; ++i)
+          __builtin_amdgcn_global_load_lds((gptr_t)(src[i] + sc_ * (32 * NH)), (lptr_t)(tile + (wave * TT + i) * 8 * 64), 16, 0, 0);
+      };
+      // operands: lane (n, kh) reads piece 4 h + 2 kh + j of token row 32 t + n
+      const int swz = (2 * kh) ^ (n & 7);
+      auto read_x = [&](const half_t* tile, int h, int j, half8_t (&dst)[TT]) __attribute__((always_inline)) {
+        const half_t* at = tile + n * 64 + (((4 * h + j) ^ swz) << 3);
 #pragma unroll
-      for (int t = 0; t < TT; ++t)
+        for (int t = 0; t < TT; ++t) dst[t] = *reinterpret_cast<const half8_t*>(at + t * 32 * 64);
+      };
+      auto mma = [&](const half8_t (&xo)[TT], const half8_t (&wo)[kWideRP]) __attribute__((always_inline)) {
 #pragma unroll
-        for (int a = 0; a < kWideRP; ++a) acc[a][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xo[t], wo[a], acc[a][t], 0, 0, 0);
-    };
-    // the order the scheduler is asked for inside a slice: one matrix-core instruction, then a few
-    // of the next slice's dequantisation instructions and one of its LDS reads
-    auto interleave = [&]() __attribute__((always_inline)) {
+        for (int t = 0; t < TT; ++t)
+#pragma unroll
+          for (int a = 0; a < kWideRP; ++a) acc[a][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xo[t], wo[a], acc[a][t], 0, 0, 0);
+      };
+      auto interleave = [&]() __attribute__((always_inline)) {
 #define AWQ_SLOT(valu, lds)                                        \
   __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); /* matrix */  \
   __builtin_amdgcn_sched_group_barrier(0x002, valu, 0);            \
   __builtin_amdgcn_sched_group_barrier(0x100, lds, 0);
-      if constexpr (TT == 4) {
+        static_assert(TT == 4, "slot pattern of the rows-split shape");
         AWQ_SLOT(3, 1) AWQ_SLOT(3, 1) AWQ_SLOT(2, 1) AWQ_SLOT(2, 1)
         AWQ_SLOT(2, 0) AWQ_SLOT(2, 0) AWQ_SLOT(2, 0) AWQ_SLOT(2, 0)
-      } else if constexpr (TT == 2) {
-        AWQ_SLOT(5, 1) AWQ_SLOT(5, 1) AWQ_SLOT(4, 0) AWQ_SLOT(4, 0)
-      } else {
-        AWQ_SLOT(9, 1) AWQ_SLOT(9, 0)
-      }
 #undef AWQ_SLOT
-    };
-    publish();
-    read_x(xlane, 0, 0, xa);
+      };
+      half8_t xa[TT], xb_[TT], wa[kWideRP], wb[kWideRP];
+      if (CUT) __syncthreads();  // the previous piece's readers are done
+      request(tile_a, 0);
+      request(tile_b, 1);
+      __syncthreads();
+      read_x(tile_a, 0, 0, xa);
 #pragma unroll
-    for (int a = 0; a < kWideRP; ++a) wa[a] = dequant8<ZINT, false>(wd[a][0][0].x, sc, zz);
-    int buf = 0;  // s % NBUF
-    auto step = [&](int s0, auto F) __attribute__((always_inline)) {
-      constexpr int f = decltype(F)::value;
-      const int s = s0 + f;
-      // the tile that left these registers one step ago
-      if constexpr (f & 1) load_x(s + NBUF, xr1);
-      else load_x(s + NBUF, xr0);
-      if constexpr (!KSPLIT) __syncthreads();  // tile s + 1 is visible; the readers of tile s - 1 are done
-      const int buf1 = buf == NBUF - 1 ? 0 : buf + 1, buf2 = buf1 == NBUF - 1 ? 0 : buf1 + 1;
-      const half_t* cur = xlane + buf * NKB * kSlot;
-      const half_t* nxt = xlane + buf1 * NKB * kSlot;
-      const int sn = s + PF < steps ? s + PF : steps - 1;
-      // slice (h 0, j 0): prepare (0, 1)
-      read_x(cur, 0, 1, xb_);
+      for (int a = 0; a < kWideRP; ++a) wa[a] = dequant8<ZINT, false>(wd[a][0][0].x, sc, zz);
+      // one step; B = s % 3 picks the tile and the weight register set
+      auto step = [&](int s, auto B) __attribute__((always_inline)) {
+        constexpr int bi = decltype(B)::value, b1 = (bi + 1) % 3, b2 = (bi + 2) % 3;
+        half_t* const cur = bi == 0 ? tile_a : (bi == 1 ? tile_b : tile_c);
+        half_t* const nxt = bi == 0 ? tile_b : (bi == 1 ? tile_c : tile_a);
+        half_t* const tgt = bi == 0 ? tile_c : (bi == 1 ? tile_a : tile_b);
+        // everything this wavefront requested a step ago has arrived (said here, so that no wait for a
+        // register lands behind the new requests below)
+        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+        __syncthreads();  // tile s + 1 has landed and is visible; the readers of tile s - 1 are done
+        const int sn = s + 2 < steps ? s + 2 : steps - 1;
 #pragma unroll
-      for (int a = 0; a < kWideRP; ++a) {
-        wb[a] = dequant8<ZINT, false>(wd[a][f][0].y, sc, zz);
-        wd[a][f][0] = wload(a, (int64_t)(sn * NH + 0));
+        for (int h = 0; h < NH; ++h)
+#pragma unroll
+          for (int a = 0; a < kWideRP; ++a) wd[a][b2][h] = wp[a][(int64_t)(sn * NH + h) * 32];
+        request(tgt, s + 2);
+        __builtin_amdgcn_sched_barrier(0);  // the requests stay here, a whole step ahead of the wait for them
+        // slice (h 0, j 0): prepare (0, 1)
+        read_x(cur, 0, 1, xb_);
+#pragma unroll
+        for (int a = 0; a < kWideRP; ++a) wb[a] = dequant8<ZINT, false>(wd[a][bi][0].y, sc, zz);
+        mma(xa, wa);
+        interleave();
+        // slice (0, 1): prepare (1, 0)
+        read_x(cur, 1, 0, xa);
+#pragma unroll
+        for (int a = 0; a < kWideRP; ++a) wa[a] = dequant8<ZINT, false>(wd[a][bi][1].x, sc, zz);
+        mma(xb_, wb);
+        interleave();
+        // slice (1, 0): prepare (1, 1)
+        read_x(cur, 1, 1, xb_);
+#pragma unroll
+        for (int a = 0; a < kWideRP; ++a) wb[a] = dequant8<ZINT, false>(wd[a][bi][1].y, sc, zz);
+        mma(xa, wa);
+        interleave();
+        // slice (1, 1): prepare (0, 0) of the next step
+        read_x(nxt, 0, 0, xa);
+#pragma unroll
+        for (int a = 0; a < kWideRP; ++a) wa[a] = dequant8<ZINT, false>(wd[a][b1][0].x, sc, zz);
+        mma(xb_, wb);
+        interleave();
+      };
+      using I0 = std::integral_constant<int, 0>;
+      using I1 = std::integral_constant<int, 1>;
+      using I2 = std::integral_constant<int, 2>;
+      for (int s0 = 0; s0 < steps; s0 += 3) {
+        step(s0, I0{});
+        if (s0 + 1 < steps) step(s0 + 1, I1{});
+        if (s0 + 2 < steps) step(s0 + 2, I2{});
       }
-      mma(xa, wa);
-      interleave();
-      // slice (0, 1): prepare (1, 0)
-      read_x(cur, 1, 0, xa);
-#pragma unroll
-      for (int a = 0; a < kWideRP; ++a) wa[a] = dequant8<ZINT, false>(wd[a][f][1].x, sc, zz);
-      mma(xb_, wb);
-      interleave();
-      // slice (1, 0): prepare (1, 1)
-      read_x(cur, 1, 1, xb_);
-#pragma unroll
-      for (int a = 0; a < kWideRP; ++a) {
-        wb[a] = dequant8<ZINT, false>(wd[a][f][1].y, sc, zz);
-        wd[a][f][1] = wload(a, (int64_t)(sn * NH + 1));
-      }
-      mma(xa, wa);
-      interleave();
+    } else {
+      // Software pipeline over quarter steps ("slices": 2 TT matrix-core instructions on one 16-wide
+      // piece of k).  While a slice is multiplied, the token operands of the next one are read from
+      // LDS and its weight operands are dequantised, so no instruction waits for a read issued just
+      // before it; the last slice of a step prepares the first of the next.
+      //   rows split: three token tiles rotate through LDS.  Tile s + 1 is already visible during
+      //     step s and tile s + 2 is written at the end of step s into the buffer that tile s - 1
+      //     left before the step's barrier.
+      //   k split: a wavefront stages its own slot and nobody else reads it, so there is no workgroup
+      //     barrier; its LDS instructions execute in order, which lets two tiles do: tile s + 1 is
+      //     written before the last slice of step s reads it.
+      constexpr int NBUF = KSPLIT ? 2 : 3;
+      auto publish = [&]() __attribute__((always_inline)) {
+        if constexpr (KSPLIT) {
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+          __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the writes have left the queue
+          __builtin_amdgcn_wave_barrier();
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        } else {
+          __syncthreads();
+        }
+      };
+      auto wload = [&](int a, int64_t blk) __attribute__((always_inline)) {
+        return KSPLIT ? __builtin_nontemporal_load(wp[a] + blk * 32) : wp[a][blk * 32];
+      };
+      if (CUT) __syncthreads();  // the previous piece's readers are done
+      load_x(0, xr0);
+      store_x(0, xr0);
       if constexpr (KSPLIT) {
-        // tile s + 1 goes to the other buffer now, ahead of the read below
-        if constexpr (f & 1) store_x(buf1, xr0);
-        else store_x(buf1, xr1);
-        publish();
+        load_x(1, xr1);
+      } else {
+        load_x(1, xr0);
+        store_x(1, xr0);
+        load_x(2, xr1);
       }
-      // slice (1, 1): prepare (0, 0) of the next step
-      read_x(nxt, 0, 0, xa);
-#pragma unroll
-      for (int a = 0; a < kWideRP; ++a) wa[a] = dequant8<ZINT, false>(wd[a][f ^ 1][0].x, sc, zz);
-      mma(xb_, wb);
-      interleave();
-      if constexpr (!KSPLIT) {
-        if constexpr (f & 1) store_x(buf2, xr0);
-        else store_x(buf2, xr1);
+      half8_t xa[TT], xb_[TT], wa[kWideRP], wb[kWideRP];
+      const half_t* xlane = xs + slot * kSlot + n * kWideStride + 16 * kh;
+      auto read_x = [&](const half_t* tile, int h, int j, half8_t (&dst)[TT]) __attribute__((always_inline)) {
+  #pragma unroll
+        for (int t = 0; t < TT; ++t) dst[t] = *reinterpret_cast<const half8_t*>(tile + t * 32 * kWideStride + h * 32 + 8 * j);
+      };
+      auto mma = [&](const half8_t (&xo)[TT], const half8_t (&wo)[kWideRP]) __attribute__((always_inline)) {
+  #pragma unroll
+        for (int t = 0; t < TT; ++t)
+  #pragma unroll
+          for (int a = 0; a < kWideRP; ++a) acc[a][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xo[t], wo[a], acc[a][t], 0, 0, 0);
+      };
+      // the order the scheduler is asked for inside a slice: one matrix-core instruction, then a few
+      // of the next slice's dequantisation instructions and one of its LDS reads
+      auto interleave = [&]() __attribute__((always_inline)) {
+  #define AWQ_SLOT(valu, lds)                                        \
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); /* matrix */  \
+    __builtin_amdgcn_sched_group_barrier(0x002, valu, 0);            \
+    __builtin_amdgcn_sched_group_barrier(0x100, lds, 0);
+        if constexpr (TT == 4) {
+          AWQ_SLOT(3, 1) AWQ_SLOT(3, 1) AWQ_SLOT(2, 1) AWQ_SLOT(2, 1)
+          AWQ_SLOT(2, 0) AWQ_SLOT(2, 0) AWQ_SLOT(2, 0) AWQ_SLOT(2, 0)
+        } else if constexpr (TT == 2) {
+          AWQ_SLOT(5, 1) AWQ_SLOT(5, 1) AWQ_SLOT(4, 0) AWQ_SLOT(4, 0)
+        } else {
+          AWQ_SLOT(9, 1) AWQ_SLOT(9, 0)
+        }
+  #undef AWQ_SLOT
+      };
+      publish();
+      read_x(xlane, 0, 0, xa);
+  #pragma unroll
+      for (int a = 0; a < kWideRP; ++a) wa[a] = dequant8<ZINT, false>(wd[a][0][0].x, sc, zz);
+      int buf = 0;  // s % NBUF
+      auto step = [&](int s0, auto F) __attribute__((always_inline)) {
+        constexpr int f = decltype(F)::value;
+        const int s = s0 + f;
+        // the tile that left these registers one step ago
+        if constexpr (f & 1) load_x(s + NBUF, xr1);
+        else load_x(s + NBUF, xr0);
+        if constexpr (!KSPLIT) __syncthreads();  // tile s + 1 is visible; the readers of tile s - 1 are done
+        const int buf1 = buf == NBUF - 1 ? 0 : buf + 1, buf2 = buf1 == NBUF - 1 ? 0 : buf1 + 1;
+        const half_t* cur = xlane + buf * NKB * kSlot;
+        const half_t* nxt = xlane + buf1 * NKB * kSlot;
+        const int sn = s + PF < steps ? s + PF : steps - 1;
+        // slice (h 0, j 0): prepare (0, 1)
+        read_x(cur, 0, 1, xb_);
+  #pragma unroll
+        for (int a = 0; a < kWideRP; ++a) {
+          wb[a] = dequant8<ZINT, false>(wd[a][f][0].y, sc, zz);
+          wd[a][f][0] = wload(a, (int64_t)(sn * NH + 0));
+        }
+        mma(xa, wa);
+        interleave();
+        // slice (0, 1): prepare (1, 0)
+        read_x(cur, 1, 0, xa);
+  #pragma unroll
+        for (int a = 0; a < kWideRP; ++a) wa[a] = dequant8<ZINT, false>(wd[a][f][1].x, sc, zz);
+        mma(xb_, wb);
+        interleave();
+        // slice (1, 0): prepare (1, 1)
+        read_x(cur, 1, 1, xb_);
+  #pragma unroll
+        for (int a = 0; a < kWideRP; ++a) {
+          wb[a] = dequant8<ZINT, false>(wd[a][f][1].y, sc, zz);
+          wd[a][f][1] = wload(a, (int64_t)(sn * NH + 1));
+        }
+        mma(xa, wa);
+        interleave();
+        if constexpr (KSPLIT) {
+          // tile s + 1 goes to the other buffer now, ahead of the read below
+          if constexpr (f & 1) store_x(buf1, xr0);
+          else store_x(buf1, xr1);
+          publish();
+        }
+        // slice (1, 1): prepare (0, 0) of the next step
+        read_x(nxt, 0, 0, xa);
+  #pragma unroll
+        for (int a = 0; a < kWideRP; ++a) wa[a] = dequant8<ZINT, false>(wd[a][f ^ 1][0].x, sc, zz);
+        mma(xb_, wb);
+        interleave();
+        if constexpr (!KSPLIT) {
+          if constexpr (f & 1) store_x(buf2, xr0);
+          else store_x(buf2, xr1);
+        }
+        buf = buf1;
+      };
+      for (int s0 = 0; s0 < steps; s0 += 2) {
+        step(s0, std::integral_constant<int, 0>{});
+        step(s0, std::integral_constant<int, 1>{});
       }
-      buf = buf1;
-    };
-    for (int s0 = 0; s0 < steps; s0 += 2) {
-      step(s0, std::integral_constant<int, 0>{});
-      step(s0, std::integral_constant<int, 1>{});
+
     }
 
     const float scf = (float)sc;  // the wavefront's rows share one scale: it multiplies the sums, not every weight
