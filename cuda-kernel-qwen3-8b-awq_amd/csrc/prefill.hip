@@ -189,7 +189,9 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(const half_t* __
       const int key = pc >> 4, part = pc & 15;
       *reinterpret_cast<u32x4_t*>(ks + key * kFaKStride + part * 8) = kreg[i];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) vt[(part * 8 + e) * kFaVStride + key] = vreg[i][e];
+      // the 8 rows of a part are rotated by 4 (part + part / 8) keys: without it the 16 parts of a
+      // wavefront's store hit two banks, with it all 32
+      for (int e = 0; e < 8; ++e) vt[(part * 8 + e) * kFaVStride + ((key + 4 * (part + (part >> 3))) & 31)] = vreg[i][e];
     }
     __syncthreads();
     // the next tile travels while this one is multiplied
@@ -229,19 +231,23 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(const half_t* __
     rs += __shfl_xor(rs, 32, 64);
     l_run = l_run * alpha + rs;
     m_run = m_new;
+    // once the running maxima have settled (most tiles), alpha is 1 in every lane
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
 #pragma unroll
-    for (int dt = 0; dt < 4; ++dt)
+      for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
+        for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
+    }
     // second product: slice j takes keys 16 j + 8 (e / 4) + 4 kh + e % 4, e = 0..7, which are this
     // lane's probabilities 8 j .. 8 j + 7
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
 #pragma unroll
       for (int dt = 0; dt < 4; ++dt) {
-        const half_t* vr = vt + (dt * 32 + n) * kFaVStride + 16 * j + 4 * kh;
-        const half4_t lo = *reinterpret_cast<const half4_t*>(vr);
-        const half4_t hi = *reinterpret_cast<const half4_t*>(vr + 8);
+        const half_t* vr = vt + (dt * 32 + n) * kFaVStride;
+        const int rot = 4 * (((dt * 32 + n) >> 3) + ((dt * 32 + n) >> 6));  // the row's rotation, a multiple of 4 keys
+        const half4_t lo = *reinterpret_cast<const half4_t*>(vr + ((16 * j + 4 * kh + rot) & 31));
+        const half4_t hi = *reinterpret_cast<const half4_t*>(vr + ((16 * j + 4 * kh + 8 + rot) & 31));
         const half8_t vop = half8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
         o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vop, pop[j], o[dt], 0, 0, 0);
       }
