@@ -7,7 +7,8 @@
   * M = 1 through the decode kernel, M = 4, 16, 64, 128, 512 through the MFMA kernels: microseconds,
     algorithmic GB/s and the fraction of the 8 TB/s HBM peak.
 
-An optional argument lists the token counts to run, e.g. 128,2048.
+An optional argument lists the token counts to run, e.g. 128,2048; a second one the shapes (w1,w2,wo;
+wo is the 4096 x 4096 attention output matrix).
 
 Weights rotate over several distinct matrices so that they come from HBM, not from cache.
 Prints one JSON object.  Run on the GPU box: python cuda-kernel-qwen3-8b-awq_amd/bench_w4a16.py
@@ -22,7 +23,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 sys.path.insert(0, ROOT)
 
 
-ALL_SHAPES = (("w1", (12288, 4096)), ("w2", (4096, 12288)))
+ALL_SHAPES = (("w1", (12288, 4096)), ("w2", (4096, 12288)), ("wo", (4096, 4096)))
 
 
 def measure(tokens, shapes=("w1", "w2")):
@@ -96,7 +97,8 @@ def main():
     tokens = (1, 4, 16, 64, 128, 512, 2048)
     if len(sys.argv) > 1:
         tokens = tuple(int(v) for v in sys.argv[1].split(","))
-    print(json.dumps(measure(tokens)))
+    shapes = tuple(sys.argv[2].split(",")) if len(sys.argv) > 2 else ("w1", "w2")
+    print(json.dumps(measure(tokens, shapes)))
 
 
 if __name__ == "__main__":

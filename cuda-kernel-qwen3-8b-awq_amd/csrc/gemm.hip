@@ -226,7 +226,7 @@ constexpr int kSkHeaderBytes = 4096;               // status word, then one coun
 constexpr int kSkWgs = 256;                        // workgroups of a product whose work is cut evenly: one per compute unit
 constexpr int kSkTileFloats = 256 * kWideTokens;   // FP32 sums of one tile
 constexpr int kSkSpinLimit = 1 << 22;
-constexpr int kRowsSplitMinTiles = 128;            // fewer 256 x 128 tiles than this: k-split workgroups
+constexpr int kRowsSplitMinTiles = 80;             // fewer 256 x 128 tiles than this: k-split workgroups
 
 // the workgroup whose range holds step pair q, ranges being [b W / G, (b + 1) W / G)
 __device__ __forceinline__ int sk_wg_of(int64_t q, int64_t W, int G) {
@@ -391,9 +391,13 @@ __global__ __launch_bounds__(256, (MODE == WIDE_K && TT == 4) ? 1 : 2) void gemm
   __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); /* matrix */  \
   __builtin_amdgcn_sched_group_barrier(0x002, valu, 0);            \
   __builtin_amdgcn_sched_group_barrier(0x100, lds, 0);
-        static_assert(TT == 4, "slot pattern of the rows-split shape");
-        AWQ_SLOT(3, 1) AWQ_SLOT(3, 1) AWQ_SLOT(2, 1) AWQ_SLOT(2, 1)
-        AWQ_SLOT(2, 0) AWQ_SLOT(2, 0) AWQ_SLOT(2, 0) AWQ_SLOT(2, 0)
+        static_assert(TT == 4 || TT == 2, "slot patterns of the rows-split shapes");
+        if constexpr (TT == 4) {
+          AWQ_SLOT(3, 1) AWQ_SLOT(3, 1) AWQ_SLOT(2, 1) AWQ_SLOT(2, 1)
+          AWQ_SLOT(2, 0) AWQ_SLOT(2, 0) AWQ_SLOT(2, 0) AWQ_SLOT(2, 0)
+        } else {
+          AWQ_SLOT(5, 1) AWQ_SLOT(5, 1) AWQ_SLOT(4, 0) AWQ_SLOT(4, 0)
+        }
 #undef AWQ_SLOT
       };
       half8_t xa[TT], xb_[TT], wa[kWideRP], wb[kWideRP];
@@ -764,15 +768,38 @@ void launch_small(const GemmParams& p, bool zint, int n_waves, dim3 grid, hipStr
 
 }  // namespace
 
+// Which workgroup shape a many-token product takes (measured on the three matrix shapes of the
+// model, 128 to 4096 tokens):
+//   fewer than 80 tiles of 256 rows x 128 tokens          k split
+//   tiles would leave a third of the compute units idle:
+//     k <= 4096 and at least 160 tiles of 64 tokens       rows split, 64 tokens per workgroup (no hand-over;
+//                                                         the attention output matrix at 640..1024 tokens: -25 %)
+//     otherwise, with a workspace                          rows split, work cut evenly: two aligned pieces per
+//                                                         tile up to 128 tiles, 256 equal ranges above
+//   otherwise                                              rows split, a tile per workgroup
+enum WidePlan { PLAN_K, PLAN_ROWS, PLAN_ROWS_64, PLAN_ROWS_CUT };
+static WidePlan plan_wide(int64_t m, int64_t k, int64_t M, bool has_workspace) {
+  const int64_t nr = (m + 255) / 256;
+  const int64_t tiles = nr * ((M + kWideTokens - 1) / kWideTokens), tiles64 = nr * ((M + 63) / 64);
+  if (tiles < kRowsSplitMinTiles) return PLAN_K;
+  if (tiles * 3 > kSkWgs * 2) return PLAN_ROWS;
+  if (k <= 4096 && tiles64 >= 160) return PLAN_ROWS_64;
+  const int64_t pairs = tiles * (k / AWQ_BLOCK_K / kWideNH / 2);
+  return has_workspace && pairs / 4 >= kSkWgs ? PLAN_ROWS_CUT : PLAN_ROWS;
+}
+
 // room for a header and the partial sums of a product whose work is cut over workgroups (0: never cut)
 int64_t gemm_workspace_bytes(int64_t m, int64_t k, int64_t M) {
-  (void)k;
   if (M <= 4) return 0;
-  const int64_t tiles = ((m + 255) / 256) * ((M + kWideTokens - 1) / kWideTokens);
-  if (tiles >= kRowsSplitMinTiles) return tiles * 3 <= kSkWgs * 2 ? kSkHeaderBytes + (int64_t)kSkWgs * kSkTileFloats * 4 : 0;
-  const int tokens = 32 * wide_tt(M);
-  const int64_t wgs = (m / 64) * ((M + tokens - 1) / tokens);
-  return wgs <= 128 ? kSkHeaderBytes + 4 * M * m * 4 : 0;
+  switch (plan_wide(m, k, M, true)) {
+    case PLAN_ROWS_CUT: return kSkHeaderBytes + (int64_t)kSkWgs * kSkTileFloats * 4;
+    case PLAN_K: {
+      const int tokens = 32 * wide_tt(M);
+      const int64_t wgs = (m / 64) * ((M + tokens - 1) / tokens);
+      return wgs <= 128 ? kSkHeaderBytes + 4 * M * m * 4 : 0;
+    }
+    default: return 0;
+  }
 }
 
 int launch_gemm(const void* wq, const half_t* scale, const half_t* zp, int64_t m, int64_t k, const half_t* x,
@@ -824,30 +851,29 @@ int launch_gemm(const void* wq, const half_t* scale, const half_t* zp, int64_t m
       default: launch_small<1, 1>(p, zp_integral, n_waves, grid, st); break;
     }
   } else {
-    // enough 256-row x 128-token tiles: rows split; otherwise k split
     const int64_t nr = (m + 255) / 256;
     const int64_t tiles = nr * ((M + kWideTokens - 1) / kWideTokens);
     // the partial sums start behind the header, whichever kernel writes them
     char* ws_part = workspace ? (char*)workspace + kSkHeaderBytes : nullptr;
     const int64_t part_bytes = workspace_bytes - kSkHeaderBytes;
-    if (tiles >= kRowsSplitMinTiles) {
-      AWQ_REQUIRE(tiles < (1ll << 31), "too many output tiles");
+    const bool room = workspace && kSkWgs * (int64_t)kSkTileFloats * 4 <= part_bytes;
+    const WidePlan plan = plan_wide(m, k, M, room);
+    if (plan != PLAN_K) {
+      AWQ_REQUIRE(tiles < (1ll << 30), "too many output tiles");
       p.nr = (int32_t)nr;
       p.n_tiles = (int32_t)tiles;
-      // One workgroup per tile.  When the tiles would leave a third of the compute units idle and
-      // the caller brought room for handed-over sums, the steps of all tiles are cut evenly over one
-      // workgroup per compute unit instead (measured on 4096 x 12288, 1024 tokens, 128 tiles: 172 -> 124 us;
-      // with 192 tiles the hand-over costs more than the idle units).
-      int64_t n_wgs = tiles;
-      const int64_t pairs = tiles * (p.nblk / kWideNH / 2);
-      if (workspace && tiles * 3 <= kSkWgs * 2 && pairs / 4 >= kSkWgs && kSkWgs * (int64_t)kSkTileFloats * 4 <= part_bytes) {
-        n_wgs = kSkWgs;
+      int rc;
+      if (plan == PLAN_ROWS_64) {
+        p.n_tiles = (int32_t)(nr * ((M + 63) / 64));
+        rc = launch_wide<WIDE_ROWS, 2>(p, zp_integral, p.n_tiles, st);
+      } else if (plan == PLAN_ROWS_CUT) {
         p.sk_head = (int32_t*)workspace;
         p.sk_part = (float*)ws_part;
+        rc = launch_wide<WIDE_ROWS_CUT, 4>(p, zp_integral, (int)(2 * tiles <= kSkWgs ? 2 * tiles : kSkWgs), st);
+      } else {
+        rc = launch_wide<WIDE_ROWS, 4>(p, zp_integral, (int)tiles, st);
       }
-      if (int rc = p.sk_part ? launch_wide<WIDE_ROWS_CUT, 4>(p, zp_integral, (int)n_wgs, st)
-                             : launch_wide<WIDE_ROWS, 4>(p, zp_integral, (int)n_wgs, st))
-        return rc;
+      if (rc) return rc;
     } else {
       // few 64-row workgroups too (a matrix with few rows): cut k over 4 or 2 workgroups as well,
       // when the caller brought room for the partial sums

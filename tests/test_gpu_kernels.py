@@ -503,10 +503,15 @@ def test_gemv_fused_norm_unembed_argmax(awq, lib, oracle, torch_gpu, m, k):
 @pytest.mark.parametrize("m,k,M,zp_int", [(256, 512, 3, True), (256, 512, 17, False), (384, 1536, 130, True),
                                           (12288, 4096, 16, True), (12288, 4096, 200, True), (4096, 12288, 64, False),
                                           (4096, 12288, 128, True), (12288, 4096, 1030, True),
-                                          (4096, 4096, 1024, True), (384, 3072, 8500, False)])
+                                          (4096, 4096, 1024, True), (4096, 12288, 1024, True),
+                                          (4096, 12288, 640, True), (384, 6144, 8500, False)])
 def test_gemm_matches_fp32_accumulate_reference(awq, lib, oracle, torch_gpu, m, k, M, zp_int):
     """config 5: dequant-on-load MFMA product; 1e-2 relative against the sequential FP32-accumulate
-    reference, and the weights it multiplies are the bit-exact dequantised ones (one-hot check below)"""
+    reference, and the weights it multiplies are the bit-exact dequantised ones (one-hot check below).
+    The shapes cover every workgroup shape: few tokens (3), k split (17, 64, 128, 130 tokens; k also cut
+    over workgroups for 4096 x 12288 x 128), rows split with 64 tokens per workgroup (12288 x 4096 x 200,
+    4096 x 4096 x 1024), a tile per workgroup (1030 tokens), and work cut evenly with handed-over sums:
+    two aligned pieces per tile (4096 x 12288 x 1024 and x 640) and 256 unequal ranges (384 x 6144 x 8500)"""
     torch = torch_gpu
     rng = np.random.default_rng(m + k + M)
     packed, scale, zp = rand_awq(rng, m, k, zp_int=zp_int)
