@@ -772,18 +772,22 @@ void launch_small(const GemmParams& p, bool zint, int n_waves, dim3 grid, hipStr
 // model, 128 to 4096 tokens):
 //   fewer than 80 tiles of 256 rows x 128 tokens          k split
 //   tiles would leave a third of the compute units idle:
-//     k <= 4096 and at least 160 tiles of 64 tokens       rows split, 64 tokens per workgroup (no hand-over;
+//     k <= 4096 and at least 128 tiles of 64 tokens       rows split, 64 tokens per workgroup (no hand-over;
 //                                                         the attention output matrix at 640..1024 tokens: -25 %)
 //     otherwise, with a workspace                          rows split, work cut evenly: two aligned pieces per
 //                                                         tile up to 128 tiles, 256 equal ranges above
 //   otherwise                                              rows split, a tile per workgroup
 enum WidePlan { PLAN_K, PLAN_ROWS, PLAN_ROWS_64, PLAN_ROWS_CUT };
+// k split: k also cut over 2-4 workgroups (second launch adds the chunks) when the 64-row workgroups
+// are few; with 65..128 of them only for long k (4096 x 4096 at 256 tokens: 29 us with, 23 us without;
+// 4096 x 12288: 48 us with, 58 us without)
+static bool k_cut_pays(int64_t wgs, int64_t k) { return wgs <= 64 || (wgs <= 128 && k >= 8192); }
 static WidePlan plan_wide(int64_t m, int64_t k, int64_t M, bool has_workspace) {
   const int64_t nr = (m + 255) / 256;
   const int64_t tiles = nr * ((M + kWideTokens - 1) / kWideTokens), tiles64 = nr * ((M + 63) / 64);
   if (tiles < kRowsSplitMinTiles) return PLAN_K;
   if (tiles * 3 > kSkWgs * 2) return PLAN_ROWS;
-  if (k <= 4096 && tiles64 >= 160) return PLAN_ROWS_64;
+  if (k <= 4096 && tiles64 >= 128) return PLAN_ROWS_64;
   const int64_t pairs = tiles * (k / AWQ_BLOCK_K / kWideNH / 2);
   return has_workspace && pairs / 4 >= kSkWgs ? PLAN_ROWS_CUT : PLAN_ROWS;
 }
@@ -796,7 +800,7 @@ int64_t gemm_workspace_bytes(int64_t m, int64_t k, int64_t M) {
     case PLAN_K: {
       const int tokens = 32 * wide_tt(M);
       const int64_t wgs = (m / 64) * ((M + tokens - 1) / tokens);
-      return wgs <= 128 ? kSkHeaderBytes + 4 * M * m * 4 : 0;
+      return k_cut_pays(wgs, k) ? kSkHeaderBytes + 4 * M * m * 4 : 0;
     }
     default: return 0;
   }
@@ -879,7 +883,7 @@ int launch_gemm(const void* wq, const half_t* scale, const half_t* zp, int64_t m
       // when the caller brought room for the partial sums
       const int tt = wide_tt(M);
       const int64_t wgs = (m / 64) * ((M + 32 * tt - 1) / (32 * tt));
-      if (wgs <= 128 && workspace) {
+      if (k_cut_pays(wgs, k) && workspace) {
         for (int kz : {4, 2})
           if (p.nblk % (16 * kz) == 0 && (int64_t)kz * M * m * 4 <= part_bytes) {
             p.kz = kz;
