@@ -566,6 +566,58 @@ def test_gemm_matches_fp32_accumulate_reference(awq, lib, oracle, torch_gpu, m, 
     assert np.percentile(np.abs(got2 - want) / denom, 99) <= 2.0 ** -10
 
 
+def _random_gemm_shapes(n, seed):
+    """(m, k, M): multiples of 128 / 512 whose scale group does not depend on the input index"""
+    rng = np.random.default_rng(seed)
+    out = []
+    while len(out) < n:
+        a, r = int(rng.integers(1, 25)), int(rng.choice([1, 2, 3, 4]))
+        mg, kg = (a * r, a) if rng.random() < 0.5 else (a, a * r)
+        kg = max(4, kg - kg % 4)            # k a multiple of 512
+        if not (mg % kg == 0 or kg % mg == 0) or mg > 96 or kg > 96:
+            continue
+        if not any(kg % g == 0 and kg // g <= 16 for g in (8, 4, 2, 1)):
+            continue                        # the weight stream's lane groups (shared with the decode kernel)
+        M = int(rng.choice([rng.integers(5, 130), rng.integers(130, 700), rng.integers(700, 2600)]))
+        out.append((128 * mg, 128 * kg, M))
+    return out
+
+
+@pytest.mark.parametrize("m,k,M", _random_gemm_shapes(24, 20240607))
+def test_gemm_random_shapes_match_torch_fp32(awq, lib, torch_gpu, m, k, M):
+    """every workgroup shape the planner can pick, on random matrix shapes and token counts, against an
+    FP32 product of the bit-exactly dequantised weights (awq_dequant, itself pinned against the oracle):
+    1e-2 relative as above, with and without a workspace"""
+    torch = torch_gpu
+    rng = np.random.default_rng(m * 31 + k * 7 + M)
+    zp_int = bool(rng.integers(0, 2))
+    packed, scale, zp = rand_awq(rng, m, k, zp_int=zp_int)
+    d_in, d_s, d_z = dev(torch, packed), dev(torch, scale), dev(torch, zp)
+    d_dq = torch.zeros(m * k, dtype=torch.float16, device="cuda")
+    awq.check(lib.awq_dequant(d_in.data_ptr(), d_s.data_ptr(), d_z.data_ptr(), d_dq.data_ptr(), m, k, m // 128,
+                              stream(torch)))
+    d_w = torch.zeros(m * k // 2, dtype=torch.uint8, device="cuda")
+    awq.check(lib.awq_linear_repack(d_in.data_ptr(), d_w.data_ptr(), m, k, stream(torch)))
+    d_x = torch.from_numpy(rng.standard_normal((M, k)).astype(np.float16)).cuda()
+    # the reference reads the row-major dequantised buffer column-major: W(i, j) = dq[i + j m]
+    want = (d_x.float() @ d_dq.view(k, m).float()).double().cpu().numpy()
+    denom = np.maximum(np.abs(want), np.sqrt(np.mean(want * want)))
+    for use_ws in (False, True):
+        wsb = lib.awq_gemm_workspace_bytes(m, k, M) if use_ws else 0
+        d_ws = torch.zeros(max(wsb, 16), dtype=torch.uint8, device="cuda")
+        d_y = torch.full((M, m), float("nan"), dtype=torch.float16, device="cuda")
+        print("gemm", m, k, M, "workspace", wsb, flush=True)
+        awq.check(lib.awq_gemm(d_w.data_ptr(), d_s.data_ptr(), d_z.data_ptr(), m, k, d_x.data_ptr(), d_y.data_ptr(), M,
+                               1 if zp_int else 0, d_ws.data_ptr() if wsb else None, stream(torch)))
+        torch.cuda.synchronize()
+        got = d_y.double().cpu().numpy()
+        assert np.all(np.isfinite(got))
+        assert np.all(np.abs(got - want) <= 1e-2 * denom)
+        assert np.percentile(np.abs(got - want) / denom, 99) <= 2.0 ** -9
+        if wsb:
+            assert int(d_ws[:4096].to(torch.int32).sum().item()) == 0
+
+
 def test_gemm_one_hot_and_token_independence(awq, lib, torch_gpu):
     torch = torch_gpu
     m, k, M = 256, 512, 20
