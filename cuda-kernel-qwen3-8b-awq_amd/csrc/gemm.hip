@@ -239,7 +239,7 @@ __device__ __forceinline__ int sk_wg_of(int64_t q, int64_t W, int G) {
 enum WideMode { WIDE_ROWS = 0, WIDE_K = 1, WIDE_ROWS_CUT = 2 };  // rows split (a tile per workgroup), k split, rows split with work cut evenly
 
 template <bool ZINT, int MODE, int EPI, int TT>
-__global__ __launch_bounds__(256, (MODE == WIDE_K && TT == 4) ? 1 : 2) void gemm_wide_kernel(GemmParams p) {
+__global__ __launch_bounds__(256, (MODE == WIDE_K && TT == 4) ? 1 : ((MODE == WIDE_ROWS && TT == 2) ? 3 : 2)) void gemm_wide_kernel(GemmParams p) {
   constexpr bool KSPLIT = MODE == WIDE_K;
   constexpr bool CUT = MODE == WIDE_ROWS_CUT;
   constexpr int kTokens = 32 * TT;                   // tokens per workgroup
@@ -784,6 +784,8 @@ void launch_small(const GemmParams& p, bool zint, int n_waves, dim3 grid, hipStr
 //                                                         the attention output matrix at 640..1024 tokens: -25 %)
 //     otherwise, with a workspace                          rows split, work cut evenly: two aligned pieces per
 //                                                         tile up to 128 tiles, 256 equal ranges above
+//   257..384 tiles, k <= 4096                              rows split, 64 tokens per workgroup, three workgroups per
+//                                                         compute unit in one round instead of two uneven rounds
 //   otherwise                                              rows split, a tile per workgroup
 enum WidePlan { PLAN_K, PLAN_ROWS, PLAN_ROWS_64, PLAN_ROWS_CUT };
 // k split: k also cut over 2-4 workgroups (second launch adds the chunks) when the 64-row workgroups
@@ -794,6 +796,9 @@ static WidePlan plan_wide(int64_t m, int64_t k, int64_t M, bool has_workspace) {
   const int64_t nr = (m + 255) / 256;
   const int64_t tiles = nr * ((M + kWideTokens - 1) / kWideTokens), tiles64 = nr * ((M + 63) / 64);
   if (tiles < kRowsSplitMinTiles) return PLAN_K;
+  // 257..384 tiles would run as two uneven rounds of two workgroups per compute unit; as 64-token tiles
+  // they are one round of three (12288 x 4096 at 704..1024 tokens: -5 to -11 %)
+  if (k <= 4096 && tiles > kSkWgs && tiles64 <= 3 * kSkWgs) return PLAN_ROWS_64;
   if (tiles * 3 > kSkWgs * 2) return PLAN_ROWS;
   if (k <= 4096 && tiles64 >= 128) return PLAN_ROWS_64;
   const int64_t pairs = tiles * (k / AWQ_BLOCK_K / kWideNH / 2);
