@@ -83,6 +83,7 @@ SIGNATURES = {
     "awq_gemv_workspace_bytes": (_i64, [_i64, _i64]),
     "awq_gemv": (ctypes.c_int, [_vp, _vp, _vp, _i64, _i64, _vp, _vp, _i32, _vp, _vp]),
     "awq_gemm_workspace_bytes": (_i64, [_i64, _i64, _i64]),
+    "awq_gemm_plan": (_i32, [_i64, _i64, _i64, _i32]),
     "awq_gemm": (ctypes.c_int, [_vp, _vp, _vp, _i64, _i64, _vp, _vp, _i64, _i32, _vp, _vp]),
     "awq_rmsnorm": (ctypes.c_int, [_vp, _vp, _vp, _i64, _f32, _vp]),
     "awq_rope_kv_append": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i64, _i64, _vp]),

@@ -114,6 +114,7 @@ int launch_repack(const uint8_t* in, void* out, int64_t m, int64_t k, hipStream_
 int64_t gemv_workspace_bytes(int64_t m, int64_t k);
 int launch_gemv(const LinearArgs& a, hipStream_t st);
 int64_t gemm_workspace_bytes(int64_t m, int64_t k, int64_t M);
+int gemm_plan(int64_t m, int64_t k, int64_t M, int has_workspace);
 // Several dependent products in one launch (gemv.hip): role i + 1 consumes what
 // role i produced.  All roles take k_unit inputs per workgroup; a role with
 // k = S * k_unit is cut into S slices.

@@ -1069,6 +1069,9 @@ extern "C" int awq_gemv(const void* repacked, const void* scale, const void* zp,
 }
 
 extern "C" int64_t awq_gemm_workspace_bytes(int64_t m, int64_t k, int64_t M) { return gemm_workspace_bytes(m, k, M); }
+extern "C" int awq_gemm_plan(int64_t m, int64_t k, int64_t M, int has_workspace) {
+  return gemm_plan(m, k, M, has_workspace);
+}
 
 extern "C" int awq_gemm(const void* repacked, const void* scale, const void* zp, int64_t m, int64_t k, const void* x,
                         void* y, int64_t M, int32_t zp_integral, void* workspace, void* stream) {

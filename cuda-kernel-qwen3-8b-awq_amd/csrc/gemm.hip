@@ -806,6 +806,18 @@ static WidePlan plan_wide(int64_t m, int64_t k, int64_t M, bool has_workspace) {
 }
 
 // room for a header and the partial sums of a product whose work is cut over workgroups (0: never cut)
+// the shape awq_gemm takes for a product (diagnostics and tests): 0 few tokens, 1 k split, 2 rows split
+// with a tile per workgroup, 3 rows split with 64 tokens per workgroup, 4 rows split with the work cut evenly
+int gemm_plan(int64_t m, int64_t k, int64_t M, int has_workspace) {
+  if (M <= 4) return 0;
+  switch (plan_wide(m, k, M, has_workspace != 0)) {
+    case PLAN_K: return 1;
+    case PLAN_ROWS: return 2;
+    case PLAN_ROWS_64: return 3;
+    default: return 4;
+  }
+}
+
 int64_t gemm_workspace_bytes(int64_t m, int64_t k, int64_t M) {
   if (M <= 4) return 0;
   switch (plan_wide(m, k, M, true)) {

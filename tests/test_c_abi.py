@@ -166,3 +166,23 @@ def test_bench_refuses_more_than_one_gpu():
                        timeout=120)
     assert r.returncode != 0
     assert "ONE GPU" in r.stderr and r.stdout.strip() == ""
+
+
+def test_gemm_plan_for_the_model_matrices(lib):
+    """the workgroup shape awq_gemm picks (host arithmetic): the measured rules, on the model's matrices"""
+    K_SPLIT, ROWS, ROWS_64, ROWS_CUT = 1, 2, 3, 4
+    w1, w2, wo = (12288, 4096), (4096, 12288), (4096, 4096)
+    plan = lambda shape, M, ws=1: lib.awq_gemm_plan(shape[0], shape[1], M, ws)
+    assert plan(w1, 1) == 0 and plan(w1, 4) == 0
+    assert [plan(w1, M) for M in (5, 64, 128)] == [K_SPLIT] * 3
+    assert [plan(w1, M) for M in (256, 384)] == [ROWS_64] * 2           # 96..144 tiles: units would idle
+    assert [plan(w1, M) for M in (512, 640)] == [ROWS] * 2              # 192..240 tiles, one per unit
+    assert [plan(w1, M) for M in (704, 1024)] == [ROWS_64] * 2          # 288..384 tiles: three per unit in one round
+    assert [plan(w1, M) for M in (1280, 2048, 4096)] == [ROWS] * 3
+    assert [plan(w2, M) for M in (128, 512)] == [K_SPLIT] * 2
+    assert [plan(w2, M) for M in (640, 1024, 1280)] == [ROWS_CUT] * 3   # long k, 80..160 tiles
+    assert plan(w2, 1024, 0) == ROWS                                    # no workspace: no hand-over
+    assert [plan(w2, M) for M in (2048, 4096)] == [ROWS] * 2
+    assert [plan(wo, M) for M in (128, 512)] == [K_SPLIT] * 2
+    assert [plan(wo, M) for M in (576, 1024, 1280)] == [ROWS_64] * 3
+    assert plan(wo, 2048) == ROWS and plan(wo, 2560) == ROWS_64 and plan(wo, 4096) == ROWS
