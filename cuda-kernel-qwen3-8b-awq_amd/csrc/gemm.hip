@@ -459,59 +459,41 @@ __global__ __launch_bounds__(256, (MODE == WIDE_K && TT == 4) ? 1 : ((MODE == WI
         if (s0 + 2 < steps) step(s0 + 2, I2{});
       }
     } else {
-      // Software pipeline over quarter steps ("slices": 2 TT matrix-core instructions on one 16-wide
-      // piece of k).  While a slice is multiplied, the token operands of the next one are read from
-      // LDS and its weight operands are dequantised, so no instruction waits for a read issued just
-      // before it; the last slice of a step prepares the first of the next.
-      //   rows split: three token tiles rotate through LDS.  Tile s + 1 is already visible during
-      //     step s and tile s + 2 is written at the end of step s into the buffer that tile s - 1
-      //     left before the step's barrier.
-      //   k split: a wavefront stages its own slot and nobody else reads it, so there is no workgroup
-      //     barrier; its LDS instructions execute in order, which lets two tiles do: tile s + 1 is
-      //     written before the last slice of step s reads it.
-      constexpr int NBUF = KSPLIT ? 2 : 3;
+      // k split: the same software pipeline over quarter steps.  A wavefront stages its own slot
+      // (through registers: two tiles in flight) and nobody else reads it, so there is no workgroup
+      // barrier; its LDS instructions execute in order, which lets two tiles do: tile s + 1 is written
+      // before the last slice of step s reads it.
       auto publish = [&]() __attribute__((always_inline)) {
-        if constexpr (KSPLIT) {
-          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-          __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the writes have left the queue
-          __builtin_amdgcn_wave_barrier();
-          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        } else {
-          __syncthreads();
-        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the writes have left the queue
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
       };
       auto wload = [&](int a, int64_t blk) __attribute__((always_inline)) {
-        return KSPLIT ? __builtin_nontemporal_load(wp[a] + blk * 32) : wp[a][blk * 32];
+        return __builtin_nontemporal_load(wp[a] + blk * 32);
       };
-      if (CUT) __syncthreads();  // the previous piece's readers are done
       load_x(0, xr0);
       store_x(0, xr0);
-      if constexpr (KSPLIT) {
-        load_x(1, xr1);
-      } else {
-        load_x(1, xr0);
-        store_x(1, xr0);
-        load_x(2, xr1);
-      }
+      load_x(1, xr1);
       half8_t xa[TT], xb_[TT], wa[kWideRP], wb[kWideRP];
       const half_t* xlane = xs + slot * kSlot + n * kWideStride + 16 * kh;
       auto read_x = [&](const half_t* tile, int h, int j, half8_t (&dst)[TT]) __attribute__((always_inline)) {
-  #pragma unroll
+#pragma unroll
         for (int t = 0; t < TT; ++t) dst[t] = *reinterpret_cast<const half8_t*>(tile + t * 32 * kWideStride + h * 32 + 8 * j);
       };
       auto mma = [&](const half8_t (&xo)[TT], const half8_t (&wo)[kWideRP]) __attribute__((always_inline)) {
-  #pragma unroll
+#pragma unroll
         for (int t = 0; t < TT; ++t)
-  #pragma unroll
+#pragma unroll
           for (int a = 0; a < kWideRP; ++a) acc[a][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xo[t], wo[a], acc[a][t], 0, 0, 0);
       };
       // the order the scheduler is asked for inside a slice: one matrix-core instruction, then a few
       // of the next slice's dequantisation instructions and one of its LDS reads
       auto interleave = [&]() __attribute__((always_inline)) {
-  #define AWQ_SLOT(valu, lds)                                        \
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); /* matrix */  \
-    __builtin_amdgcn_sched_group_barrier(0x002, valu, 0);            \
-    __builtin_amdgcn_sched_group_barrier(0x100, lds, 0);
+#define AWQ_SLOT(valu, lds)                                        \
+  __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); /* matrix */  \
+  __builtin_amdgcn_sched_group_barrier(0x002, valu, 0);            \
+  __builtin_amdgcn_sched_group_barrier(0x100, lds, 0);
         if constexpr (TT == 4) {
           AWQ_SLOT(3, 1) AWQ_SLOT(3, 1) AWQ_SLOT(2, 1) AWQ_SLOT(2, 1)
           AWQ_SLOT(2, 0) AWQ_SLOT(2, 0) AWQ_SLOT(2, 0) AWQ_SLOT(2, 0)
@@ -520,27 +502,26 @@ __global__ __launch_bounds__(256, (MODE == WIDE_K && TT == 4) ? 1 : ((MODE == WI
         } else {
           AWQ_SLOT(9, 1) AWQ_SLOT(9, 0)
         }
-  #undef AWQ_SLOT
+#undef AWQ_SLOT
       };
       publish();
       read_x(xlane, 0, 0, xa);
-  #pragma unroll
+#pragma unroll
       for (int a = 0; a < kWideRP; ++a) wa[a] = dequant8<ZINT, false>(wd[a][0][0].x, sc, zz);
-      int buf = 0;  // s % NBUF
+      // one step; F is its index inside the unrolled pair (a compile-time constant): tile s is in
+      // buffer F, tile s + 1 goes to the other one
       auto step = [&](int s0, auto F) __attribute__((always_inline)) {
         constexpr int f = decltype(F)::value;
         const int s = s0 + f;
         // the tile that left these registers one step ago
-        if constexpr (f & 1) load_x(s + NBUF, xr1);
-        else load_x(s + NBUF, xr0);
-        if constexpr (!KSPLIT) __syncthreads();  // tile s + 1 is visible; the readers of tile s - 1 are done
-        const int buf1 = buf == NBUF - 1 ? 0 : buf + 1, buf2 = buf1 == NBUF - 1 ? 0 : buf1 + 1;
-        const half_t* cur = xlane + buf * NKB * kSlot;
-        const half_t* nxt = xlane + buf1 * NKB * kSlot;
+        if constexpr (f & 1) load_x(s + 2, xr1);
+        else load_x(s + 2, xr0);
+        const half_t* cur = xlane + f * NKB * kSlot;
+        const half_t* nxt = xlane + (f ^ 1) * NKB * kSlot;
         const int sn = s + PF < steps ? s + PF : steps - 1;
         // slice (h 0, j 0): prepare (0, 1)
         read_x(cur, 0, 1, xb_);
-  #pragma unroll
+#pragma unroll
         for (int a = 0; a < kWideRP; ++a) {
           wb[a] = dequant8<ZINT, false>(wd[a][f][0].y, sc, zz);
           wd[a][f][0] = wload(a, (int64_t)(sn * NH + 0));
@@ -549,42 +530,34 @@ __global__ __launch_bounds__(256, (MODE == WIDE_K && TT == 4) ? 1 : ((MODE == WI
         interleave();
         // slice (0, 1): prepare (1, 0)
         read_x(cur, 1, 0, xa);
-  #pragma unroll
+#pragma unroll
         for (int a = 0; a < kWideRP; ++a) wa[a] = dequant8<ZINT, false>(wd[a][f][1].x, sc, zz);
         mma(xb_, wb);
         interleave();
         // slice (1, 0): prepare (1, 1)
         read_x(cur, 1, 1, xb_);
-  #pragma unroll
+#pragma unroll
         for (int a = 0; a < kWideRP; ++a) {
           wb[a] = dequant8<ZINT, false>(wd[a][f][1].y, sc, zz);
           wd[a][f][1] = wload(a, (int64_t)(sn * NH + 1));
         }
         mma(xa, wa);
         interleave();
-        if constexpr (KSPLIT) {
-          // tile s + 1 goes to the other buffer now, ahead of the read below
-          if constexpr (f & 1) store_x(buf1, xr0);
-          else store_x(buf1, xr1);
-          publish();
-        }
+        // tile s + 1 goes to the other buffer now, ahead of the read below
+        if constexpr (f & 1) store_x(0, xr0);
+        else store_x(1, xr1);
+        publish();
         // slice (1, 1): prepare (0, 0) of the next step
         read_x(nxt, 0, 0, xa);
-  #pragma unroll
+#pragma unroll
         for (int a = 0; a < kWideRP; ++a) wa[a] = dequant8<ZINT, false>(wd[a][f ^ 1][0].x, sc, zz);
         mma(xb_, wb);
         interleave();
-        if constexpr (!KSPLIT) {
-          if constexpr (f & 1) store_x(buf2, xr0);
-          else store_x(buf2, xr1);
-        }
-        buf = buf1;
       };
       for (int s0 = 0; s0 < steps; s0 += 2) {
         step(s0, std::integral_constant<int, 0>{});
         step(s0, std::integral_constant<int, 1>{});
       }
-
     }
 
     const float scf = (float)sc;  // the wavefront's rows share one scale: it multiplies the sums, not every weight
