@@ -323,12 +323,15 @@ __global__ __launch_bounds__(1024) void gemv_kernel(const u32x4* __restrict__ wq
       }
     }
   }
-  // x first, and alone: once every wavefront of the device has its 8 KiB of
+  // x first, and almost alone: once every wavefront of the device has its 8 KiB of
   // weight loads in flight, a small load of x (an L2 hit) waits microseconds in
-  // the same queues.  So the weight stream starts only when x has arrived.
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  // the same queues.  So only the first weight block is requested along with x
+  // (it brings the stream's first round trip forward: +2.8 % tokens/s over none;
+  // two blocks +2.4 %, four +0.6 %) and the rest starts when x has arrived.
+  w[0] = __builtin_nontemporal_load(wp);
+  asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
 #pragma unroll
-  for (int b = 0; b < G; ++b) w[b] = __builtin_nontemporal_load(wp + b * 16);
+  for (int b = 1; b < G; ++b) w[b] = __builtin_nontemporal_load(wp + b * 16);
   if (norm) {
     // rmsNormKernel, Inference.cu:111-145: 256 strided fma partial sums over the
     // natural order, the stride-halving tree, then two binary16 multiplies.
