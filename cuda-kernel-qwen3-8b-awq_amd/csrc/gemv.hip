@@ -187,11 +187,11 @@ struct GemvParams {
 };
 
 // the 16 finished rows of a workgroup; r = lane = row % 16, lanes 0..15 of wavefront 0
-__device__ __forceinline__ void epilogue(const GemvParams& p, int row, int r, float acc) {
+__device__ __forceinline__ void epilogue(const GemvParams& p, int row, int r, float acc, half_t res) {
   half_t v = (half_t)acc;
   switch (p.epilogue) {
     case EPI_RESIDUAL:  // Inference.cu:1149-1155
-      p.y[row] = p.res[row] + v;
+      p.y[row] = res + v;
       return;
     case EPI_GELU:  // Inference.cu:271-279
       p.y[row] = to_half_rn(awq_gelu_f32((float)v));
@@ -405,6 +405,10 @@ __global__ __launch_bounds__(1024) void gemv_kernel(const u32x4* __restrict__ wq
 #pragma unroll
       for (int b = 0; b < G; ++b) wn[b] = __builtin_nontemporal_load(wpn + b * 16);
     }
+    // the residual row is requested before the pass multiplies: the end of the
+    // launch then does not wait for one more round trip to memory
+    half_t res = (half_t)0.0f;
+    if (tid < 16 && p.epilogue == EPI_RESIDUAL) res = p.res[rg * 16 + r];
     // scale group of these 16 rows: row/128, then Inference.cu:90 with the index
     // wrapped to the m/128 stored entries
     const int a = rg >> 3;
@@ -468,7 +472,7 @@ __global__ __launch_bounds__(1024) void gemv_kernel(const u32x4* __restrict__ wq
       }
       float tot = rd[0][r];
       for (int i = 1; i < n; ++i) tot += rd[i][r];
-      epilogue(p, rg * 16 + r, r, tot);
+      epilogue(p, rg * 16 + r, r, tot, res);
     }
 #pragma unroll
     for (int b = 0; b < G; ++b) w[b] = wn[b];
@@ -744,7 +748,7 @@ __global__ __launch_bounds__(256) void flow_kernel(FlowParams p) {
     gp.pos = p.pos;
     gp.max_pos = p.max_pos;
     gp.dyn = p.dyn;
-    epilogue(gp, row, r, tot);
+    epilogue(gp, row, r, tot, (half_t)0.0f);
   } else {
     half_t out = hv;
     if (R.epilogue == EPI_RESIDUAL) {
