@@ -109,7 +109,8 @@ int awq_set_flow_mode(awq_engine* e, int enabled);
 /* Measurement aid with no counterpart in the reference: runs the engine's own
  * fused-linear launch of `kind` (AWQ_T_WQKV/WO/W1/W2/UNEMBED) over every
  * layer's resident matrix, n_rounds times, between two HIP events on the
- * engine's stream.  Returns the mean launch duration and the algorithmic bytes
+ * engine's stream (a round is captured once and replayed as a graph, the way
+ * the decode step issues these launches).  Returns the mean launch duration and the algorithmic bytes
  * of one launch (packed weights + scales + zero-points + input + output).
  * Resets the sequence. */
 int awq_time_linear(awq_engine* e, int kind, int32_t n_rounds, float* avg_us_per_launch, int64_t* bytes_per_launch);
