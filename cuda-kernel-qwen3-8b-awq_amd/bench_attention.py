@@ -17,7 +17,7 @@ vc = torch.randn(H, MP, 128, dtype=torch.float16, device="cuda")
 q = torch.randn(H * 128, dtype=torch.float16, device="cuda")
 ctx = torch.empty(H * 128, dtype=torch.float16, device="cuda")
 ws = torch.zeros(lib.awq_attention_workspace_bytes(H, MP), dtype=torch.uint8, device="cuda")
-for L in (128, 256, 512, 768, 1024, 1536, 2048, 4096, 8192, 16384, 40960):
+for L in (128, 256, 512, 768, 1024, 1536, 1792, 2000, 2048, 4096, 8192, 16384, 40960):
     def run():
         awq.check(lib.awq_decode_attention(q.data_ptr(), kc.data_ptr(), vc.data_ptr(), ctx.data_ptr(), H, MP, L, ws.data_ptr(), st))
     for _ in range(3): run()

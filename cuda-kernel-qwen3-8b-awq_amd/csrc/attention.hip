@@ -153,14 +153,17 @@ __global__ __launch_bounds__(NW * 64) void attention_kernel(const half_t* __rest
         if (t < L) vv[nl] = *reinterpret_cast<const half8_t*>(vh + (int64_t)t * AWQ_HEAD_DIM + 8 * dl);
       }
     }
+    // one division per position (lane = position in the chunk), handed to the 16 lanes that
+    // multiply that position's values
+    const float p_lane = base + lane < L ? s[base + lane] / Z : 0.0f;
     float acc[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
 #pragma unroll
     for (int nl = 0; nl < 16; ++nl) {
       const int t = base + 4 * nl + tq;
+      const float p = __shfl(p_lane, 4 * nl + tq, 64);
       if (t < L) {
-        const float p = s[t] / Z;
 #pragma unroll
         for (int i = 0; i < 8; ++i) acc[i] = __builtin_fmaf(p, (float)vv[nl][i], acc[i]);
       }
@@ -446,7 +449,8 @@ int launch_attention(const half_t* q, const half_t* kc, const half_t* vc, half_t
   // decides where the scores live); with a length known here, the length itself.
   const int64_t bound = dyn ? (len_bound > 0 ? len_bound : max_pos) : L;
   const int mc = (int)chunks_for(max_pos);
-  if (bound > kLdsChunks * 64) {
+  static_assert(kAttnOneWorkgroupMax <= kLdsChunks * 64, "the one-workgroup kernel keeps its scores in LDS");
+  if (bound > kAttnOneWorkgroupMax) {
     // long sequences: cut along the sequence
     SplitArgs a;
     a.q = q;

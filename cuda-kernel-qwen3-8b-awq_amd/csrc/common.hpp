@@ -163,6 +163,12 @@ int launch_gemm(const void* wq, const half_t* scale, const half_t* zp, int64_t m
 int launch_rmsnorm(const half_t* x, const half_t* gamma, half_t* out, int64_t n, float eps, hipStream_t st);
 int launch_rope_kv_append(const half_t* qkv, const half_t* cos_t, const half_t* sin_t, half_t* q_out, half_t* kc,
                           half_t* vc, int n_heads, int64_t max_pos, int64_t pos, const StepState* dyn, hipStream_t st);
+// Attended lengths up to this bound take one workgroup per head (a handful of
+// memory round trips, 32 compute units); longer ones the four launches cut
+// along the sequence (15 us floor, all compute units).  Measured in the decode
+// loop, where the cache comes from HBM every step: 539 against 502 tok/s at
+// 508..772 positions, 458 against 490 at 908..1172, 378 against 475 at 1708..1972.
+constexpr int64_t kAttnOneWorkgroupMax = 832;
 int64_t attention_workspace_bytes(int n_heads, int64_t max_pos);
 int launch_attention(const half_t* q, const half_t* kc, const half_t* vc, half_t* ctx, int n_heads, int64_t max_pos,
                      int64_t L, const StepState* dyn, int use_len_hi, int64_t len_bound, void* ws, hipStream_t st);

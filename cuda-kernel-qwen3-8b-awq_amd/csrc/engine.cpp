@@ -447,7 +447,7 @@ int run_step(awq_engine* e, bool gen, StepState s) {
   // the attention launch is specialised by an upper bound of the attended
   // length (one workgroup per head with its scores in LDS, or the launches cut
   // along the sequence); one captured graph per bound
-  static const int64_t kBounds[2] = {2048, 1 << 30};
+  static const int64_t kBounds[2] = {kAttnOneWorkgroupMax, 1 << 30};
   int bucket = 0;
   while (s.len_hi > kBounds[bucket]) ++bucket;
   const int64_t len_bound = kBounds[bucket] < e->cfg.max_pos ? kBounds[bucket] : e->cfg.max_pos;
