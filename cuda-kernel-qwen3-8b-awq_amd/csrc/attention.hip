@@ -392,6 +392,79 @@ __global__ __launch_bounds__(kSplitWaves * 64) void attn_pv_kernel(SplitArgs a) 
   }
 }
 
+// The two kernels above as one launch, for sequences of at most kMergedMax
+// positions: every workgroup computes the head's exponentials and chunk sums
+// for itself (at most 16 exponentials per thread: cheaper than a launch), keeps
+// those of its own chunks in LDS and goes on to their weighted sums.  A chunk is
+// still summed by one wavefront with position = lane and the chunk sums are
+// added in order, so the bits are those of the separate launches.
+constexpr int kMergedMax = 4096;
+constexpr int kMergedChunks = kMergedMax / 64;
+constexpr int kMergedOwn = (kMergedChunks + kSplit - 1) / kSplit;  // chunks per part
+__global__ __launch_bounds__(kSplitWaves * 64) void attn_exp_pv_kernel(SplitArgs a) {
+  __shared__ float zs[kMergedChunks];
+  __shared__ float es[kMergedOwn * 64];
+  const int L = split_len(a);
+  const int head = blockIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tq = lane >> 4, dl = lane & 15;
+  const half_t* vh = a.vc + (int64_t)head * a.max_pos * AWQ_HEAD_DIM;
+  const float* s = a.scores + (int64_t)head * a.max_pos;
+  float* cv = a.cv + (int64_t)head * a.max_chunks * AWQ_HEAD_DIM;
+  const int nchunks = (L + 63) >> 6;
+  int c_lo, c_hi;
+  split_range(nchunks, &c_lo, &c_hi);
+  if (c_lo >= c_hi) return;  // the whole workgroup
+  // the values of this wavefront's chunk travel while the exponentials are computed
+  half8_t vv[16];
+  const int chunk = c_lo + wave;  // at most one chunk per wavefront: kMergedOwn <= kSplitWaves
+  if (chunk < c_hi) {
+#pragma unroll
+    for (int nl = 0; nl < 16; ++nl) {
+      const int t = (chunk << 6) + 4 * nl + tq;
+      if (t < L) vv[nl] = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(vh + (int64_t)t * AWQ_HEAD_DIM + 8 * dl));
+    }
+  }
+  float mx = a.pmax[head * kSplit];
+#pragma unroll
+  for (int i = 1; i < kSplit; ++i) mx = fmaxf(mx, a.pmax[head * kSplit + i]);
+  for (int c = wave; c < nchunks; c += kSplitWaves) {
+    const int t = (c << 6) + lane;
+    float e = 0.0f;
+    if (t < L) e = awq_expf(s[t] - mx);
+    if (c >= c_lo && c < c_hi) es[(c - c_lo) * 64 + lane] = e;
+    e = wave_tree_sum(e);
+    if (lane == 0) zs[c] = e;
+  }
+  __syncthreads();
+  if (chunk >= c_hi) return;
+  float Z = zs[0];
+  for (int c = 1; c < nchunks; ++c) Z += zs[c];
+  const int base = chunk << 6;
+  const float p_lane = base + lane < L ? es[(chunk - c_lo) * 64 + lane] / Z : 0.0f;
+  float acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
+#pragma unroll
+  for (int nl = 0; nl < 16; ++nl) {
+    const int t = base + 4 * nl + tq;
+    const float pr = __shfl(p_lane, 4 * nl + tq, 64);
+    if (t < L) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[i] = __builtin_fmaf(pr, (float)vv[nl][i], acc[i]);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    acc[i] = xor_add(acc[i], 16);
+    acc[i] = xor_add(acc[i], 32);
+  }
+  if (tq == 0) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) cv[chunk * AWQ_HEAD_DIM + 8 * dl + i] = acc[i];
+  }
+}
+
 // chunk vectors added in chunk order (Inference.cu:259-265 runs over t in order).
 // The additions of one output element are a sequential chain, but the loads
 // need not be: 16 wavefronts per head (8 stages x 2 halves of the 128 elements)
@@ -450,6 +523,7 @@ int launch_attention(const half_t* q, const half_t* kc, const half_t* vc, half_t
   const int64_t bound = dyn ? (len_bound > 0 ? len_bound : max_pos) : L;
   const int mc = (int)chunks_for(max_pos);
   static_assert(kAttnOneWorkgroupMax <= kLdsChunks * 64, "the one-workgroup kernel keeps its scores in LDS");
+  static_assert(kAttnMergedMax == kMergedMax && kMergedOwn <= kSplitWaves, "one chunk per wavefront in the merged launch");
   if (bound > kAttnOneWorkgroupMax) {
     // long sequences: cut along the sequence
     SplitArgs a;
@@ -469,8 +543,12 @@ int launch_attention(const half_t* q, const half_t* kc, const half_t* vc, half_t
     AWQ_REQUIRE((int64_t)mc * 4 <= 65536, "sequence too long for the chunk-sum buffer in LDS");
     const dim3 grid(n_heads, kSplit), block(kSplitWaves * 64);
     hipLaunchKernelGGL(attn_scores_kernel, grid, block, 0, st, a);
-    hipLaunchKernelGGL(attn_exp_kernel, grid, block, 0, st, a);
-    hipLaunchKernelGGL(attn_pv_kernel, grid, block, (size_t)a.max_chunks * 4, st, a);
+    if (bound <= kMergedMax) {
+      hipLaunchKernelGGL(attn_exp_pv_kernel, grid, block, 0, st, a);
+    } else {
+      hipLaunchKernelGGL(attn_exp_kernel, grid, block, 0, st, a);
+      hipLaunchKernelGGL(attn_pv_kernel, grid, block, (size_t)a.max_chunks * 4, st, a);
+    }
     hipLaunchKernelGGL(attn_sum_kernel, dim3(n_heads), dim3(kSumStages * 2 * 64), 0, st, a);
     AWQ_HIP_TRY(hipGetLastError());
     return AWQ_OK;

@@ -164,11 +164,15 @@ int launch_rmsnorm(const half_t* x, const half_t* gamma, half_t* out, int64_t n,
 int launch_rope_kv_append(const half_t* qkv, const half_t* cos_t, const half_t* sin_t, half_t* q_out, half_t* kc,
                           half_t* vc, int n_heads, int64_t max_pos, int64_t pos, const StepState* dyn, hipStream_t st);
 // Attended lengths up to this bound take one workgroup per head (a handful of
-// memory round trips, 32 compute units); longer ones the four launches cut
-// along the sequence (15 us floor, all compute units).  Measured in the decode
-// loop, where the cache comes from HBM every step: 539 against 502 tok/s at
-// 508..772 positions, 458 against 490 at 908..1172, 378 against 475 at 1708..1972.
-constexpr int64_t kAttnOneWorkgroupMax = 832;
+// memory round trips, 32 compute units); longer ones the launches cut along
+// the sequence (three kernel boundaries, all compute units).  Measured in the
+// decode loop, where the cache comes from HBM every step: one workgroup per
+// head 539 tok/s at 508..772 positions, 458 at 908..1172, 378 at 1708..1972;
+// cut along the sequence 502, 510 and 480.
+constexpr int64_t kAttnOneWorkgroupMax = 704;
+// Up to this bound the cut path takes three launches instead of four (the
+// exponentials are recomputed by every workgroup of a head).
+constexpr int64_t kAttnMergedMax = 4096;
 int64_t attention_workspace_bytes(int n_heads, int64_t max_pos);
 int launch_attention(const half_t* q, const half_t* kc, const half_t* vc, half_t* ctx, int n_heads, int64_t max_pos,
                      int64_t L, const StepState* dyn, int use_len_hi, int64_t len_bound, void* ws, hipStream_t st);

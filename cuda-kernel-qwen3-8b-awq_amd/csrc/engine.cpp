@@ -158,7 +158,7 @@ struct awq_engine {
   int n_generated = 0;
   bool finalized = false;
   bool graph_mode = true;
-  hipGraphExec_t graphs[2][2] = {{nullptr, nullptr}, {nullptr, nullptr}};  // [prompt|gen][length bound]
+  hipGraphExec_t graphs[2][3] = {{nullptr, nullptr, nullptr}, {nullptr, nullptr, nullptr}};  // [prompt|gen][length bound]
   // activations of the batched prompt pass, [chunk][n] each; allocated at first use
   struct {
     half_t *hidden = nullptr, *norm = nullptr, *qkv = nullptr, *q = nullptr, *ctx = nullptr, *mid = nullptr;
@@ -447,7 +447,7 @@ int run_step(awq_engine* e, bool gen, StepState s) {
   // the attention launch is specialised by an upper bound of the attended
   // length (one workgroup per head with its scores in LDS, or the launches cut
   // along the sequence); one captured graph per bound
-  static const int64_t kBounds[2] = {kAttnOneWorkgroupMax, 1 << 30};
+  static const int64_t kBounds[3] = {kAttnOneWorkgroupMax, kAttnMergedMax, 1 << 30};
   int bucket = 0;
   while (s.len_hi > kBounds[bucket]) ++bucket;
   const int64_t len_bound = kBounds[bucket] < e->cfg.max_pos ? kBounds[bucket] : e->cfg.max_pos;
