@@ -394,11 +394,11 @@ __global__ __launch_bounds__(kSplitWaves * 64) void attn_pv_kernel(SplitArgs a) 
 
 // The two kernels above as one launch, for sequences of at most kMergedMax
 // positions: every workgroup computes the head's exponentials and chunk sums
-// for itself (at most 16 exponentials per thread: cheaper than a launch), keeps
+// for itself (at most 8 exponentials per thread: cheaper than a launch), keeps
 // those of its own chunks in LDS and goes on to their weighted sums.  A chunk is
 // still summed by one wavefront with position = lane and the chunk sums are
 // added in order, so the bits are those of the separate launches.
-constexpr int kMergedMax = 4096;
+constexpr int kMergedMax = 2048;
 constexpr int kMergedChunks = kMergedMax / 64;
 constexpr int kMergedOwn = (kMergedChunks + kSplit - 1) / kSplit;  // chunks per part
 __global__ __launch_bounds__(kSplitWaves * 64) void attn_exp_pv_kernel(SplitArgs a) {

@@ -255,10 +255,10 @@ def test_decode_attention_bit_exact(awq, lib, oracle, torch_gpu, L):
                                     ws.data_ptr(), stream(torch)) != 0
 
 
-@pytest.mark.parametrize("L", [705, 1000, 2049, 4096, 4097, 9001, 20000])
+@pytest.mark.parametrize("L", [705, 1000, 2048, 2049, 4097, 9001, 20000])
 def test_decode_attention_long_sequences_bit_exact(awq, lib, oracle, torch_gpu, L):
     """beyond 704 positions the launches are cut along the sequence (32 parts per head, some of them
-    empty while the sequence has fewer than 32 chunks; three launches up to 4096 positions, four beyond);
+    empty while the sequence has fewer than 32 chunks; three launches up to 2048 positions, four beyond);
     the summation orders are those of the short
     path, so the oracle's bits must come out"""
     torch = torch_gpu
