@@ -21,7 +21,7 @@ vcs = [torch.randn(H, MP, 128, dtype=torch.float16, device="cuda") for _ in rang
 q = torch.randn(H * 128, dtype=torch.float16, device="cuda")
 ctx = torch.empty(H * 128, dtype=torch.float16, device="cuda")
 ws = torch.zeros(lib.awq_attention_workspace_bytes(H, MP), dtype=torch.uint8, device="cuda")
-for L in (128, 256, 512, 704, 705, 1024, 1536, 2048, 2049, 4096, 8192, 16384, 40960):
+for L in (128, 256, 512, 576, 577, 768, 1024, 1025, 1536, 2048, 2049, 4096, 8192, 16384, 40960):
     def run(i):
         awq.check(lib.awq_decode_attention(q.data_ptr(), kcs[i % NL].data_ptr(), vcs[i % NL].data_ptr(), ctx.data_ptr(),
                                            H, MP, L, ws.data_ptr(), st))

@@ -20,6 +20,7 @@ constexpr int kMaxChunks = 1024;    // 65536 positions
 constexpr int kLdsChunks = 32;      // chunk vectors kept in LDS up to this many chunks
 constexpr int kWaves = 16;   // wavefronts per workgroup of the decode variants
 constexpr int kThreads = kWaves * 64;
+constexpr int kSplit = 32;   // parts per head when the sequence is cut over several workgroups
 
 // v + (value of lane ^ mask) inside a row of 16 lanes.  After the xor-1 and
 // xor-2 steps all four lanes of a quad hold the same sum, so mirroring inside
@@ -56,12 +57,16 @@ __device__ __forceinline__ float wave_tree_sum(float v) {
 
 // NW wavefronts; SCAP positions of scores and CCAP chunks (sums and vectors)
 // fit the LDS arrays.  Longer sequences take the split kernels further down.
-template <int NW, int SCAP, int CCAP>
+// FROM_SCORES: the scores and the maxima of their kSplit parts were left in memory
+// by attn_scores_kernel (all compute units stream the keys); this launch does the
+// rest of the head.
+template <int NW, int SCAP, int CCAP, bool FROM_SCORES = false>
 __global__ __launch_bounds__(NW * 64) void attention_kernel(const half_t* __restrict__ q,
                                                              const half_t* __restrict__ kc,
                                                              const half_t* __restrict__ vc, half_t* __restrict__ ctx,
                                                              int64_t max_pos, int L_arg, const StepState* dyn,
-                                                             int use_len_hi) {
+                                                             int use_len_hi, const float* __restrict__ scores_g,
+                                                             const float* __restrict__ pmax_g) {
   __shared__ float cs[CCAP];
   __shared__ float wmax[NW];
   __shared__ float s[SCAP];
@@ -75,6 +80,23 @@ __global__ __launch_bounds__(NW * 64) void attention_kernel(const half_t* __rest
   const int nchunks = (L + 63) >> 6;
   const float scale = 1.0f / sqrtf((float)AWQ_HEAD_DIM);  // Inference.cu:218
 
+  half8_t vv[16];
+  float mx;
+  if constexpr (FROM_SCORES) {
+    // the values of this wavefront's first chunk travel while the scores arrive
+    if (wave < nchunks) {
+#pragma unroll
+      for (int nl = 0; nl < 16; ++nl) {
+        const int t = (wave << 6) + 4 * nl + tq;
+        if (t < L) vv[nl] = *reinterpret_cast<const half8_t*>(vh + (int64_t)t * AWQ_HEAD_DIM + 8 * dl);
+      }
+    }
+    for (int t = tid; t < L; t += NW * 64) s[t] = scores_g[(int64_t)head * max_pos + t];
+    mx = pmax_g[head * kSplit];
+#pragma unroll
+    for (int i = 1; i < kSplit; ++i) mx = fmaxf(mx, pmax_g[head * kSplit + i]);
+    __syncthreads();
+  } else {
   float qf[8];
   {
     half8_t qv = *reinterpret_cast<const half8_t*>(q + head * AWQ_HEAD_DIM + 8 * dl);
@@ -86,7 +108,6 @@ __global__ __launch_bounds__(NW * 64) void attention_kernel(const half_t* __rest
   // positions go round the wavefronts, six groups' loads in flight.  The values
   // of this wavefront's first chunk are requested right behind the first keys,
   // so that both arrive in one memory round trip.
-  half8_t vv[16];
   float lmax = -1e9f;
   const int nquads = (L + 3) >> 2;
   for (int q0 = wave; q0 < nquads; q0 += 6 * NW) {
@@ -123,9 +144,10 @@ __global__ __launch_bounds__(NW * 64) void attention_kernel(const half_t* __rest
   for (int mask = 1; mask < 64; mask <<= 1) lmax = fmaxf(lmax, __shfl_xor(lmax, mask, 64));
   if (lane == 0) wmax[wave] = lmax;
   __syncthreads();
-  float mx = wmax[0];
+  mx = wmax[0];
 #pragma unroll
   for (int w = 1; w < NW; ++w) mx = fmaxf(mx, wmax[w]);
+  }
 
   // exponentials and their sum (Inference.cu:239-249), one wavefront per chunk
   for (int chunk = wave; chunk < nchunks; chunk += NW) {
@@ -196,7 +218,6 @@ __global__ __launch_bounds__(NW * 64) void attention_kernel(const half_t* __rest
 // chunk context vectors; their ordered sum.  Scores, chunk sums, chunk vectors
 // and part maxima live in the workspace.
 // ---------------------------------------------------------------------------
-constexpr int kSplit = 32;         // parts per head
 constexpr int kSplitWaves = 4;     // wavefronts per workgroup of the split kernels
 
 struct SplitArgs {
@@ -524,6 +545,7 @@ int launch_attention(const half_t* q, const half_t* kc, const half_t* vc, half_t
   const int mc = (int)chunks_for(max_pos);
   static_assert(kAttnOneWorkgroupMax <= kLdsChunks * 64, "the one-workgroup kernel keeps its scores in LDS");
   static_assert(kAttnMergedMax == kMergedMax && kMergedOwn <= kSplitWaves, "one chunk per wavefront in the merged launch");
+  static_assert(kAttnTwoLaunchMax <= kWaves * 64 && kAttnTwoLaunchMax <= kLdsChunks * 64, "one chunk per wavefront after the scores launch");
   if (bound > kAttnOneWorkgroupMax) {
     // long sequences: cut along the sequence
     SplitArgs a;
@@ -543,6 +565,13 @@ int launch_attention(const half_t* q, const half_t* kc, const half_t* vc, half_t
     AWQ_REQUIRE((int64_t)mc * 4 <= 65536, "sequence too long for the chunk-sum buffer in LDS");
     const dim3 grid(n_heads, kSplit), block(kSplitWaves * 64);
     hipLaunchKernelGGL(attn_scores_kernel, grid, block, 0, st, a);
+    if (bound <= kAttnTwoLaunchMax) {
+      // the rest of the head in one workgroup: at most one chunk per wavefront
+      hipLaunchKernelGGL((attention_kernel<kWaves, kLdsChunks * 64, kLdsChunks, true>), dim3(n_heads), dim3(kThreads), 0,
+                         st, q, kc, vc, ctx, max_pos, (int)L, dyn, use_len_hi, a.scores, a.pmax);
+      AWQ_HIP_TRY(hipGetLastError());
+      return AWQ_OK;
+    }
     if (bound <= kMergedMax) {
       hipLaunchKernelGGL(attn_exp_pv_kernel, grid, block, 0, st, a);
     } else {
@@ -554,7 +583,7 @@ int launch_attention(const half_t* q, const half_t* kc, const half_t* vc, half_t
     return AWQ_OK;
   }
   hipLaunchKernelGGL((attention_kernel<kWaves, kLdsChunks * 64, kLdsChunks>), dim3(n_heads), dim3(kThreads), 0,
-                     st, q, kc, vc, ctx, max_pos, (int)L, dyn, use_len_hi);
+                     st, q, kc, vc, ctx, max_pos, (int)L, dyn, use_len_hi, (const float*)nullptr, (const float*)nullptr);
   AWQ_HIP_TRY(hipGetLastError());
   return AWQ_OK;
 }

@@ -163,17 +163,24 @@ int launch_gemm(const void* wq, const half_t* scale, const half_t* zp, int64_t m
 int launch_rmsnorm(const half_t* x, const half_t* gamma, half_t* out, int64_t n, float eps, hipStream_t st);
 int launch_rope_kv_append(const half_t* qkv, const half_t* cos_t, const half_t* sin_t, half_t* q_out, half_t* kc,
                           half_t* vc, int n_heads, int64_t max_pos, int64_t pos, const StepState* dyn, hipStream_t st);
-// Attended lengths up to this bound take one workgroup per head (a handful of
-// memory round trips, 32 compute units); longer ones the launches cut along
-// the sequence (three kernel boundaries, all compute units).  Measured in the
-// decode loop, where the cache comes from HBM every step: one workgroup per
-// head 539 tok/s at 508..772 positions, 458 at 908..1172, 378 at 1708..1972;
-// cut along the sequence 502, 510 and 480.
-constexpr int64_t kAttnOneWorkgroupMax = 704;
-// Up to this bound the cut path takes three launches instead of four (the
-// exponentials are recomputed by every workgroup of a head; a part is one chunk
-// of 64 positions).  15.6 against 17.6 us at 1024 positions, even at 2048,
-// 29.1 against 26.6 us at 4096.
+// How the decode attention is launched, by an upper bound of the attended length
+// (measured in the decode loop of the 36-layer model, where every layer's cache
+// comes from HBM, and with bench_attention.py):
+//   <= kAttnOneWorkgroupMax  one workgroup per head does everything: a handful of
+//        memory round trips on 32 compute units (6 us at 256, 12.4 us at 704 positions);
+//   <= kAttnTwoLaunchMax     the keys are streamed by all compute units (scores and part
+//        maxima to memory), a second launch with one workgroup per head does the rest,
+//        one 64-position chunk per wavefront (11 us at 705, 12.8 us at 1024 positions;
+//        with two chunks per wavefront 24 us at 1536);
+//   <= kAttnMergedMax        three launches: scores; exponentials, chunk sums and chunk
+//        vectors per part (the exponentials are recomputed by every workgroup of a
+//        head); ordered sum (17.7 us at 1536, 20.1 us at 2048 positions);
+//   beyond                   four launches (26.5 us at 4096; three would take 29.1 us).
+// Tokens per second over 264 decode steps, one workgroup per head against the cut
+// path: 582 / 567 at 258..522 positions, 556 / 557 at 408..672, 539 / 523 at 708..972
+// (before the two-launch form: 513), 458 / 510 at 908..1172, 378 / 480 at 1708..1972.
+constexpr int64_t kAttnOneWorkgroupMax = 576;
+constexpr int64_t kAttnTwoLaunchMax = 1024;
 constexpr int64_t kAttnMergedMax = 2048;
 int64_t attention_workspace_bytes(int n_heads, int64_t max_pos);
 int launch_attention(const half_t* q, const half_t* kc, const half_t* vc, half_t* ctx, int n_heads, int64_t max_pos,

@@ -158,7 +158,7 @@ struct awq_engine {
   int n_generated = 0;
   bool finalized = false;
   bool graph_mode = true;
-  hipGraphExec_t graphs[2][3] = {{nullptr, nullptr, nullptr}, {nullptr, nullptr, nullptr}};  // [prompt|gen][length bound]
+  hipGraphExec_t graphs[2][4] = {{nullptr, nullptr, nullptr, nullptr}, {nullptr, nullptr, nullptr, nullptr}};  // [prompt|gen][length bound]
   // activations of the batched prompt pass, [chunk][n] each; allocated at first use
   struct {
     half_t *hidden = nullptr, *norm = nullptr, *qkv = nullptr, *q = nullptr, *ctx = nullptr, *mid = nullptr;
@@ -444,10 +444,10 @@ int build_graph(awq_engine* e, bool gen, int64_t len_bound, hipGraphExec_t* out)
 int run_step(awq_engine* e, bool gen, StepState s) {
   s.epoch = ++e->epoch;
   if (int rc = launch_set_state(e->d_state, s, e->stream)) return rc;
-  // the attention launch is specialised by an upper bound of the attended
-  // length (one workgroup per head with its scores in LDS, or the launches cut
-  // along the sequence); one captured graph per bound
-  static const int64_t kBounds[3] = {kAttnOneWorkgroupMax, kAttnMergedMax, 1 << 30};
+  // the attention launches are specialised by an upper bound of the attended
+  // length (one workgroup per head, or two to four launches cut along the
+  // sequence); one captured graph per bound
+  static const int64_t kBounds[4] = {kAttnOneWorkgroupMax, kAttnTwoLaunchMax, kAttnMergedMax, 1 << 30};
   int bucket = 0;
   while (s.len_hi > kBounds[bucket]) ++bucket;
   const int64_t len_bound = kBounds[bucket] < e->cfg.max_pos ? kBounds[bucket] : e->cfg.max_pos;
