@@ -167,36 +167,40 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(const half_t* __
   // exp(x) = 2^(x log2 e); the scale of Inference.cu:218 folded into the same factor
   const float scale2 = (1.0f / sqrtf((float)AWQ_HEAD_DIM)) * 1.44269504088896340736f;
 
-  // this thread's two 16-byte pieces of the key tile and of the value tile: (key, part of its row)
-  u32x4_t kreg[2];
-  half8_t vreg[2];
-  auto load_tile = [&](int k0) __attribute__((always_inline)) {
+  // this thread's two 16-byte pieces of the key tile and of the value tile: (key, part of its row).
+  // Two tiles are on their way at any time (register sets A and B): with one, a step lasted as long
+  // as a trip to memory, which is longer than its arithmetic.
+  struct TileRegs {
+    u32x4_t k[2];
+    half8_t v[2];
+  };
+  auto load_tile = [&](int k0, TileRegs& r) __attribute__((always_inline)) {
+    if (k0 >= L_wg) return;
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int pc = tid + i * 256;
       const int key = pc >> 4, part = pc & 15;
       const int kg = k0 + key < L_wg ? k0 + key : L_wg - 1;  // rows past the end are masked below
-      kreg[i] = *reinterpret_cast<const u32x4_t*>(kh_ptr + (int64_t)kg * AWQ_HEAD_DIM + part * 8);
-      vreg[i] = *reinterpret_cast<const half8_t*>(vh_ptr + (int64_t)kg * AWQ_HEAD_DIM + part * 8);
+      r.k[i] = *reinterpret_cast<const u32x4_t*>(kh_ptr + (int64_t)kg * AWQ_HEAD_DIM + part * 8);
+      r.v[i] = *reinterpret_cast<const half8_t*>(vh_ptr + (int64_t)kg * AWQ_HEAD_DIM + part * 8);
     }
   };
-  load_tile(0);
-  for (int k0 = 0; k0 < L_wg; k0 += kFaKeys) {
+  auto step = [&](int k0, TileRegs& r) __attribute__((always_inline)) {
     __syncthreads();  // the previous tiles' readers are done
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int pc = tid + i * 256;
       const int key = pc >> 4, part = pc & 15;
-      *reinterpret_cast<u32x4_t*>(ks + key * kFaKStride + part * 8) = kreg[i];
+      *reinterpret_cast<u32x4_t*>(ks + key * kFaKStride + part * 8) = r.k[i];
 #pragma unroll
       // the 8 rows of a part are rotated by 4 (part + part / 8) keys: without it the 16 parts of a
       // wavefront's store hit two banks, with it all 32
-      for (int e = 0; e < 8; ++e) vt[(part * 8 + e) * kFaVStride + ((key + 4 * (part + (part >> 3))) & 31)] = vreg[i][e];
+      for (int e = 0; e < 8; ++e) vt[(part * 8 + e) * kFaVStride + ((key + 4 * (part + (part >> 3))) & 31)] = r.v[i][e];
     }
     __syncthreads();
-    // the next tile travels while this one is multiplied
-    if (k0 + kFaKeys < L_wg) load_tile(k0 + kFaKeys);
-    if (k0 >= L_wave) continue;  // nothing of this tile is attended by this wavefront's queries
+    // the tile after the next travels while this one and the next are multiplied
+    load_tile(k0 + 2 * kFaKeys, r);
+    if (k0 >= L_wave) return;  // nothing of this tile is attended by this wavefront's queries
 
     f32x16_t sacc;
 #pragma unroll
@@ -252,6 +256,13 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(const half_t* __
         o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vop, pop[j], o[dt], 0, 0, 0);
       }
     }
+  };
+  TileRegs ra, rb;
+  load_tile(0, ra);
+  load_tile(kFaKeys, rb);
+  for (int k0 = 0; k0 < L_wg; k0 += 2 * kFaKeys) {
+    step(k0, ra);
+    if (k0 + kFaKeys < L_wg) step(k0 + kFaKeys, rb);
   }
   // o[dt][i] is component 32 dt + 8 (i / 4) + 4 kh + i % 4 of this lane's query
   if (qi < M) {
