@@ -61,7 +61,7 @@ def main():
     from helpers import fill_pair, make_oracle_model, ptr
     import oracle_lib
 
-    max_pos = max(640, args.prompt_len + args.warmup + args.steps + 8)
+    max_pos = max(2176, args.prompt_len + args.warmup + args.steps + 8)
     cfg = awq.make_config(n_layers=args.layers, max_pos=max_pos)
     oracle = oracle_lib.load() if args.cpu_steps > 0 else None
 
@@ -178,6 +178,24 @@ def main():
     log("one layer at ~%d positions: %.1f us, %.0f GB/s (%.1f%% of peak)" %
         (L_mid, layer_us, layer_cfg2["GBs"], 100 * layer_cfg2["hbm_frac"]))
 
+    # ---- the decode rate with a longer context: 64 steps after a batched 2040-token prompt (the
+    #      attention takes three, then four launches cut along the sequence there) ---------------
+    p2k = np.zeros(2040, dtype=np.int32)
+    awq.check(lib.awq_synth_tokens(args.seed + 2, awq.SYNTH_STREAM_INPUT, ptr(p2k), p2k.size, cfg.vocab))
+    eng.reset()
+    torch.cuda.synchronize()
+    t4 = time.perf_counter()
+    eng.prefill(p2k.tolist(), batched=True)
+    prompt_2k_ms = (time.perf_counter() - t4) * 1e3
+    eng.decode(4)
+    torch.cuda.synchronize()
+    t5 = time.perf_counter()
+    eng.decode(64)
+    torch.cuda.synchronize()
+    long_context = {"attended_positions": "2044..2108", "tok_s": round(64 / (time.perf_counter() - t5), 1),
+                    "prompt_pass_ms_2040_tokens": round(prompt_2k_ms, 2)}
+    log("decode at ~2k positions: %.1f tok/s; 2040-token prompt %.1f ms" % (long_context["tok_s"], prompt_2k_ms))
+
     # ---- the prompt pass's product on the matrix cores: w1 shape, 2048 tokens (config 5) ---------
     w4a16 = importlib.import_module("cuda-kernel-qwen3-8b-awq_amd.bench_w4a16")
     g = w4a16.measure((2048,), ("w1",))["shapes"]["w1"]["M=2048"]
@@ -223,6 +241,7 @@ def main():
         "greedy_tokens_identical_to_cpu": tokens_match,
         "prompt_pass_ms": prefill_ms,
         "layer_512_positions": layer_cfg2,
+        "long_context": long_context,
         "prefill_gemm": prefill_gemm,
         "roofline": roofline,
         "cpu_baseline": cpu,

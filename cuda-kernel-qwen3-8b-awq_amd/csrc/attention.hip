@@ -64,8 +64,9 @@ template <int NW, int SCAP, int CCAP, bool FROM_SCORES = false>
 __global__ __launch_bounds__(NW * 64) void attention_kernel(const half_t* __restrict__ q,
                                                              const half_t* __restrict__ kc,
                                                              const half_t* __restrict__ vc, half_t* __restrict__ ctx,
-                                                             int64_t max_pos, int L_arg, const StepState* dyn,
-                                                             int use_len_hi, const float* __restrict__ scores_g,
+                                                             KvLayout lay, int L_arg, const StepState* dyn,
+                                                             int use_len_hi, int64_t max_pos,
+                                                             const float* __restrict__ scores_g,
                                                              const float* __restrict__ pmax_g) {
   __shared__ float cs[CCAP];
   __shared__ float wmax[NW];
@@ -75,8 +76,8 @@ __global__ __launch_bounds__(NW * 64) void attention_kernel(const half_t* __rest
   const int head = blockIdx.x;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int tq = lane >> 4, dl = lane & 15;
-  const half_t* kh = kc + (int64_t)head * max_pos * AWQ_HEAD_DIM;
-  const half_t* vh = vc + (int64_t)head * max_pos * AWQ_HEAD_DIM;
+  const half_t* kh = kc;
+  const half_t* vh = vc;
   const int nchunks = (L + 63) >> 6;
   const float scale = 1.0f / sqrtf((float)AWQ_HEAD_DIM);  // Inference.cu:218
 
@@ -88,7 +89,7 @@ __global__ __launch_bounds__(NW * 64) void attention_kernel(const half_t* __rest
 #pragma unroll
       for (int nl = 0; nl < 16; ++nl) {
         const int t = (wave << 6) + 4 * nl + tq;
-        if (t < L) vv[nl] = *reinterpret_cast<const half8_t*>(vh + (int64_t)t * AWQ_HEAD_DIM + 8 * dl);
+        if (t < L) vv[nl] = *reinterpret_cast<const half8_t*>(vh + kv_row(lay, head, t) + 8 * dl);
       }
     }
     for (int t = tid; t < L; t += NW * 64) s[t] = scores_g[(int64_t)head * max_pos + t];
@@ -115,13 +116,13 @@ __global__ __launch_bounds__(NW * 64) void attention_kernel(const half_t* __rest
 #pragma unroll
     for (int u = 0; u < 6; ++u) {
       const int t = 4 * (q0 + u * NW) + tq;
-      if (t < L) kv[u] = *reinterpret_cast<const half8_t*>(kh + (int64_t)t * AWQ_HEAD_DIM + 8 * dl);
+      if (t < L) kv[u] = *reinterpret_cast<const half8_t*>(kh + kv_row(lay, head, t) + 8 * dl);
     }
     if (q0 == wave && wave < nchunks) {
 #pragma unroll
       for (int nl = 0; nl < 16; ++nl) {
         const int t = (wave << 6) + 4 * nl + tq;
-        if (t < L) vv[nl] = *reinterpret_cast<const half8_t*>(vh + (int64_t)t * AWQ_HEAD_DIM + 8 * dl);
+        if (t < L) vv[nl] = *reinterpret_cast<const half8_t*>(vh + kv_row(lay, head, t) + 8 * dl);
       }
     }
 #pragma unroll
@@ -172,7 +173,7 @@ __global__ __launch_bounds__(NW * 64) void attention_kernel(const half_t* __rest
 #pragma unroll
       for (int nl = 0; nl < 16; ++nl) {
         const int t = base + 4 * nl + tq;
-        if (t < L) vv[nl] = *reinterpret_cast<const half8_t*>(vh + (int64_t)t * AWQ_HEAD_DIM + 8 * dl);
+        if (t < L) vv[nl] = *reinterpret_cast<const half8_t*>(vh + kv_row(lay, head, t) + 8 * dl);
       }
     }
     // one division per position (lane = position in the chunk), handed to the 16 lanes that
@@ -226,6 +227,7 @@ struct SplitArgs {
   const half_t* vc;
   half_t* ctx;
   int64_t max_pos;
+  KvLayout kv;
   int L_arg;
   const StepState* dyn;
   int use_len_hi;
@@ -253,7 +255,8 @@ __global__ __launch_bounds__(kSplitWaves * 64) void attn_scores_kernel(SplitArgs
   const int head = blockIdx.x;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int tq = lane >> 4, dl = lane & 15;
-  const half_t* kh = a.kc + (int64_t)head * a.max_pos * AWQ_HEAD_DIM;
+  const half_t* kh = a.kc;
+  const KvLayout lay = a.kv;
   float* s = a.scores + (int64_t)head * a.max_pos;
   int c_lo, c_hi;
   split_range((L + 63) >> 6, &c_lo, &c_hi);
@@ -274,7 +277,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void attn_scores_kernel(SplitArgs
     for (int u = 0; u < 8; ++u) {
       const int t = 4 * (q0 + u * kSplitWaves) + tq;
       if (q0 + u * kSplitWaves < q_hi && t < L)
-        dst[u] = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(kh + (int64_t)t * AWQ_HEAD_DIM + 8 * dl));
+        dst[u] = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(kh + kv_row(lay, head, t) + 8 * dl));
     }
   };
   load_keys(c_lo * 16 + wave, kn);
@@ -347,7 +350,8 @@ __global__ __launch_bounds__(kSplitWaves * 64) void attn_pv_kernel(SplitArgs a) 
   const int head = blockIdx.x;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int tq = lane >> 4, dl = lane & 15;
-  const half_t* vh = a.vc + (int64_t)head * a.max_pos * AWQ_HEAD_DIM;
+  const half_t* vh = a.vc;
+  const KvLayout lay = a.kv;
   const float* s = a.scores + (int64_t)head * a.max_pos;
   const float* cs = a.cs + (int64_t)head * a.max_chunks;
   float* cv = a.cv + (int64_t)head * a.max_chunks * AWQ_HEAD_DIM;
@@ -361,7 +365,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void attn_pv_kernel(SplitArgs a) 
     for (int u = 0; u < 8; ++u) {
       const int t = (chunk << 6) + 4 * (8 * half + u) + tq;
       if (chunk < c_hi && t < L)
-        dst[u] = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(vh + (int64_t)t * AWQ_HEAD_DIM + 8 * dl));
+        dst[u] = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(vh + kv_row(lay, head, t) + 8 * dl));
     }
   };
   int chunk = c_lo + wave;
@@ -429,7 +433,8 @@ __global__ __launch_bounds__(kSplitWaves * 64) void attn_exp_pv_kernel(SplitArgs
   const int head = blockIdx.x;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int tq = lane >> 4, dl = lane & 15;
-  const half_t* vh = a.vc + (int64_t)head * a.max_pos * AWQ_HEAD_DIM;
+  const half_t* vh = a.vc;
+  const KvLayout lay = a.kv;
   const float* s = a.scores + (int64_t)head * a.max_pos;
   float* cv = a.cv + (int64_t)head * a.max_chunks * AWQ_HEAD_DIM;
   const int nchunks = (L + 63) >> 6;
@@ -443,7 +448,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void attn_exp_pv_kernel(SplitArgs
 #pragma unroll
     for (int nl = 0; nl < 16; ++nl) {
       const int t = (chunk << 6) + 4 * nl + tq;
-      if (t < L) vv[nl] = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(vh + (int64_t)t * AWQ_HEAD_DIM + 8 * dl));
+      if (t < L) vv[nl] = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(vh + kv_row(lay, head, t) + 8 * dl));
     }
   }
   float mx = a.pmax[head * kSplit];
@@ -533,7 +538,8 @@ int64_t attention_workspace_bytes(int n_heads, int64_t max_pos) {
 }
 
 int launch_attention(const half_t* q, const half_t* kc, const half_t* vc, half_t* ctx, int n_heads, int64_t max_pos,
-                     int64_t L, const StepState* dyn, int use_len_hi, int64_t len_bound, void* ws, hipStream_t st) {
+                     KvLayout kv, int64_t L, const StepState* dyn, int use_len_hi, int64_t len_bound, void* ws,
+                     hipStream_t st) {
   AWQ_REQUIRE(n_heads > 0 && max_pos > 0 && max_pos <= (int64_t)kMaxChunks * 64, "max_pos must be in 1..65536");
   AWQ_REQUIRE(dyn || (L >= 1 && L <= max_pos), "attended length out of range");
   AWQ_REQUIRE(ws != nullptr, "workspace required");
@@ -554,6 +560,7 @@ int launch_attention(const half_t* q, const half_t* kc, const half_t* vc, half_t
     a.vc = vc;
     a.ctx = ctx;
     a.max_pos = max_pos;
+    a.kv = kv;
     a.L_arg = (int)L;
     a.dyn = dyn;
     a.use_len_hi = use_len_hi;
@@ -568,7 +575,7 @@ int launch_attention(const half_t* q, const half_t* kc, const half_t* vc, half_t
     if (bound <= kAttnTwoLaunchMax) {
       // the rest of the head in one workgroup: at most one chunk per wavefront
       hipLaunchKernelGGL((attention_kernel<kWaves, kLdsChunks * 64, kLdsChunks, true>), dim3(n_heads), dim3(kThreads), 0,
-                         st, q, kc, vc, ctx, max_pos, (int)L, dyn, use_len_hi, a.scores, a.pmax);
+                         st, q, kc, vc, ctx, kv, (int)L, dyn, use_len_hi, max_pos, a.scores, a.pmax);
       AWQ_HIP_TRY(hipGetLastError());
       return AWQ_OK;
     }
@@ -583,7 +590,7 @@ int launch_attention(const half_t* q, const half_t* kc, const half_t* vc, half_t
     return AWQ_OK;
   }
   hipLaunchKernelGGL((attention_kernel<kWaves, kLdsChunks * 64, kLdsChunks>), dim3(n_heads), dim3(kThreads), 0,
-                     st, q, kc, vc, ctx, max_pos, (int)L, dyn, use_len_hi, (const float*)nullptr, (const float*)nullptr);
+                     st, q, kc, vc, ctx, kv, (int)L, dyn, use_len_hi, max_pos, (const float*)nullptr, (const float*)nullptr);
   AWQ_HIP_TRY(hipGetLastError());
   return AWQ_OK;
 }

@@ -45,6 +45,26 @@ void awq_set_error(const std::string& msg);
     }                                                                \
   } while (0)
 
+// Where row (head, position) of a key or value cache starts, in binary16 elements:
+//   head * head_stride + (position >> shift) * block_stride + (position % 2^shift) * 128.
+//   head major: [head][max_pos][128], the reference's arrangement (Inference.cu:676)
+//     and that of the kernel-level entry points;
+//   blocked: [position / 64][head][position % 64][128], the engine's own.  The rows
+//     a step touches are then a prefix of the layer's cache whatever max_pos is, and
+//     a head's 64 consecutive positions are still 16 KB in one piece.  Head major
+//     they are n_heads islands max_pos * 256 bytes apart.
+struct KvLayout {
+  int32_t head_stride;
+  int32_t block_stride;
+  int32_t shift;
+};
+inline KvLayout kv_head_major(int64_t max_pos) { return KvLayout{(int32_t)(max_pos * 128), 0, 30}; }
+inline KvLayout kv_blocked(int n_heads) { return KvLayout{64 * 128, n_heads * 64 * 128, 6}; }
+__host__ __device__ inline int64_t kv_row(const KvLayout& kv, int head, int pos) {
+  return (int64_t)head * kv.head_stride + (int64_t)(pos >> kv.shift) * kv.block_stride +
+         (int64_t)(pos & ((1 << kv.shift) - 1)) * 128;
+}
+
 // Values that change from step to step live in device memory so that a
 // captured graph can be replayed unchanged: kernels read them from here.
 struct StepState {
@@ -90,6 +110,7 @@ struct LinearArgs {
   int32_t hidden = 0;
   int32_t pos = 0;
   int64_t max_pos = 0;
+  KvLayout kv = {0, 0, 0};
   const StepState* dyn = nullptr;     // pos / out_index come from here when set
   unsigned long long* best = nullptr;  // EPI_ARGMAX: zero between launches
   int32_t* out_token = nullptr;
@@ -154,6 +175,7 @@ struct FlowLaunch {
   int32_t hidden = 0;
   int32_t pos = 0;
   int64_t max_pos = 0;
+  KvLayout kv = {0, 0, 0};
 };
 bool flow_supported(int64_t hidden, int64_t inter);
 int launch_flow(const FlowLaunch& f, hipStream_t st);
@@ -162,7 +184,8 @@ int launch_gemm(const void* wq, const half_t* scale, const half_t* zp, int64_t m
                 int64_t workspace_bytes, hipStream_t st);
 int launch_rmsnorm(const half_t* x, const half_t* gamma, half_t* out, int64_t n, float eps, hipStream_t st);
 int launch_rope_kv_append(const half_t* qkv, const half_t* cos_t, const half_t* sin_t, half_t* q_out, half_t* kc,
-                          half_t* vc, int n_heads, int64_t max_pos, int64_t pos, const StepState* dyn, hipStream_t st);
+                          half_t* vc, int n_heads, int64_t max_pos, KvLayout kv, int64_t pos, const StepState* dyn,
+                          hipStream_t st);
 // How the decode attention is launched, by an upper bound of the attended length
 // (measured in the decode loop of the 36-layer model, where every layer's cache
 // comes from HBM, and with bench_attention.py):
@@ -184,16 +207,17 @@ constexpr int64_t kAttnTwoLaunchMax = 1024;
 constexpr int64_t kAttnMergedMax = 2048;
 int64_t attention_workspace_bytes(int n_heads, int64_t max_pos);
 int launch_attention(const half_t* q, const half_t* kc, const half_t* vc, half_t* ctx, int n_heads, int64_t max_pos,
-                     int64_t L, const StepState* dyn, int use_len_hi, int64_t len_bound, void* ws, hipStream_t st);
+                     KvLayout kv, int64_t L, const StepState* dyn, int use_len_hi, int64_t len_bound, void* ws,
+                     hipStream_t st);
 int launch_prefill_attention(const half_t* q, const half_t* kc, const half_t* vc, half_t* ctx, int n_heads,
-                             int64_t max_pos, int64_t pos0, int64_t M, int use_len_hi, hipStream_t st);
+                             int64_t max_pos, KvLayout kv, int64_t pos0, int64_t M, int use_len_hi, hipStream_t st);
 int launch_embed_batch(const uint8_t* packed, const half_t* scale, const half_t* zp, int64_t hidden, int64_t vocab,
                        const int32_t* tokens_dev, int64_t M, half_t* out, hipStream_t st);
 int launch_rmsnorm_batch(const half_t* x, const half_t* gamma, half_t* out, int64_t n, int64_t M, float eps,
                          hipStream_t st);
 int launch_rope_kv_append_batch(const half_t* qkv, const half_t* cos_t, const half_t* sin_t, half_t* q_out,
-                                half_t* kc, half_t* vc, int n_heads, int64_t max_pos, int64_t pos0, int64_t M,
-                                hipStream_t st);
+                                half_t* kc, half_t* vc, int n_heads, int64_t max_pos, KvLayout kv, int64_t pos0,
+                                int64_t M, hipStream_t st);
 int launch_residual(const half_t* a, const half_t* b, half_t* out, int64_t n, hipStream_t st);
 int launch_gelu(half_t* x, int64_t n, hipStream_t st);
 int64_t argmax_workspace_bytes(int64_t n);

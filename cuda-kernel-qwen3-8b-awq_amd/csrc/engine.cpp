@@ -265,6 +265,7 @@ int enqueue_wqkv(awq_engine* e, int l) {
   a.v_cache = L.vcache;
   a.hidden = e->cfg.hidden;
   a.max_pos = e->cfg.max_pos;
+  a.kv = kv_blocked(e->n_heads);
   return launch_gemv(a, e->stream);
 }
 
@@ -345,6 +346,7 @@ int enqueue_flow(awq_engine* e, int l, int idx) {
     f.v_cache = N.vcache;
     f.hidden = (int32_t)H;
     f.max_pos = e->cfg.max_pos;
+    f.kv = kv_blocked(e->n_heads);
     f.n_roles = 4;
     zint = zint && N.wqkv.zp_integral;
   }
@@ -356,7 +358,8 @@ int enqueue_layer(awq_engine* e, int l, int use_len_hi, int64_t len_bound) {
   LayerDev& L = e->layers[l];
   hipStream_t st = e->stream;
   if (int rc = enqueue_wqkv(e, l)) return rc;
-  if (int rc = launch_attention(e->q, L.kcache, L.vcache, e->ctx, e->n_heads, e->cfg.max_pos, 0, e->d_state,
+  if (int rc = launch_attention(e->q, L.kcache, L.vcache, e->ctx, e->n_heads, e->cfg.max_pos,
+                                kv_blocked(e->n_heads), 0, e->d_state,
                                 use_len_hi, len_bound, e->attn_ws, st))
     return rc;  // :1110
   {  // :1128-1155 Wo product and residual add; input and output are distinct
@@ -410,6 +413,7 @@ int enqueue_step_body(awq_engine* e, bool gen, int64_t len_bound) {
     int idx = 0;  // which buffer of the ring holds the layer's input
     for (int l = 0; l < e->cfg.n_layers; ++l) {
       if (int rc = launch_attention(e->q, e->layers[l].kcache, e->layers[l].vcache, e->ctx, e->n_heads, e->cfg.max_pos,
+                                    kv_blocked(e->n_heads),
                                     0, e->d_state, l >= split, len_bound, e->attn_ws, e->stream))
         return rc;  // :1110
       if (int rc = enqueue_flow(e, l, idx)) return rc;
@@ -504,7 +508,9 @@ extern "C" int awq_create_empty(const awq_config* cfg_in, awq_engine** out) {
     return rc;
   };
   const int64_t H = cfg.hidden, I = cfg.inter, V = cfg.vocab;
-  const int64_t kv_bytes = (int64_t)e->n_heads * cfg.max_pos * AWQ_HEAD_DIM * 2;  // Inference.cu:676
+  // Inference.cu:676; the rows are kept in blocks of 64 positions here (see KvLayout), so whole blocks
+  // are allocated
+  const int64_t kv_bytes = (int64_t)e->n_heads * ((cfg.max_pos + 63) / 64 * 64) * AWQ_HEAD_DIM * 2;
   for (int l = 0; l < cfg.n_layers; ++l) {
     LayerDev& L = e->layers[l];
     if (int rc = alloc_linear(ep, L.wqkv, AWQ_T_WQKV)) return fail(rc);
@@ -618,7 +624,7 @@ extern "C" int awq_finalize(awq_engine* e) {
     AWQ_HIP_TRY(hipMemcpy(e->sin_t, s.data(), s.size() * 2, hipMemcpyHostToDevice));
   }
   // zero the KV caches (Inference.cu:431-437) and the self-resetting workspaces
-  const int64_t kv_bytes = (int64_t)e->n_heads * e->cfg.max_pos * AWQ_HEAD_DIM * 2;
+  const int64_t kv_bytes = (int64_t)e->n_heads * ((e->cfg.max_pos + 63) / 64 * 64) * AWQ_HEAD_DIM * 2;
   for (auto& L : e->layers) {
     if (int rc = launch_fill_zero(L.kcache, kv_bytes, st)) return rc;
     if (int rc = launch_fill_zero(L.vcache, kv_bytes, st)) return rc;
@@ -788,9 +794,10 @@ int enqueue_layer_batch(awq_engine* e, int l, int64_t pos0, int64_t M) {
   if (int rc = launch_rmsnorm_batch(b.hidden, L.gamma, b.norm, H, M, e->cfg.eps, st)) return rc;  // :1040
   if (int rc = gemm_of(e, L.wqkv, b.norm, b.qkv, M)) return rc;                                    // :1052
   if (int rc = launch_rope_kv_append_batch(b.qkv, e->cos_t, e->sin_t, b.q, L.kcache, L.vcache, e->n_heads,
-                                           e->cfg.max_pos, pos0, M, st))
+                                           e->cfg.max_pos, kv_blocked(e->n_heads), pos0, M, st))
     return rc;  // :1070-1103
-  if (int rc = launch_prefill_attention(b.q, L.kcache, L.vcache, b.ctx, e->n_heads, e->cfg.max_pos, pos0, M, l >= 1,
+  if (int rc = launch_prefill_attention(b.q, L.kcache, L.vcache, b.ctx, e->n_heads, e->cfg.max_pos,
+                                        kv_blocked(e->n_heads), pos0, M, l >= 1,
                                         st))
     return rc;  // :1110
   // :1128 Wo product, :1149 residual add in its epilogue
@@ -946,6 +953,7 @@ extern "C" int awq_time_linear(awq_engine* e, int kind, int32_t n_rounds, float*
           a.v_cache = e->layers[l].vcache;
           a.hidden = e->cfg.hidden;
           a.max_pos = e->cfg.max_pos;
+          a.kv = kv_blocked(e->n_heads);
           break;
         case AWQ_T_WO:
           a = linear_args(e, t, e->ctx, e->hidden);
@@ -1068,6 +1076,7 @@ extern "C" int awq_gemv_fused(const awq_linear_args* u, void* stream) {
   a.hidden = u->hidden;
   a.pos = (int32_t)u->pos;
   a.max_pos = u->max_pos;
+  a.kv = kv_head_major(u->max_pos);
   a.out_token = (int32_t*)u->out_token;
   return launch_gemv(a, (hipStream_t)stream);
 }
@@ -1117,7 +1126,7 @@ extern "C" int awq_rope_kv_append(const void* qkv, const void* cos_t, const void
                                   void* v_cache, int32_t n_heads, int64_t max_pos, int64_t pos, void* stream) {
   AWQ_REQUIRE(qkv && cos_t && sin_t && q_out && k_cache && v_cache, "NULL pointer");
   return launch_rope_kv_append((const half_t*)qkv, (const half_t*)cos_t, (const half_t*)sin_t, (half_t*)q_out,
-                               (half_t*)k_cache, (half_t*)v_cache, n_heads, max_pos, pos, nullptr,
+                               (half_t*)k_cache, (half_t*)v_cache, n_heads, max_pos, kv_head_major(max_pos), pos, nullptr,
                                (hipStream_t)stream);
 }
 
@@ -1129,7 +1138,7 @@ extern "C" int awq_decode_attention(const void* q, const void* k_cache, const vo
                                     int64_t max_pos, int64_t L, void* workspace, void* stream) {
   AWQ_REQUIRE(q && k_cache && v_cache && ctx, "NULL pointer");
   return launch_attention((const half_t*)q, (const half_t*)k_cache, (const half_t*)v_cache, (half_t*)ctx, n_heads,
-                          max_pos, L, nullptr, 0, 0, workspace, (hipStream_t)stream);
+                          max_pos, kv_head_major(max_pos), L, nullptr, 0, 0, workspace, (hipStream_t)stream);
 }
 
 extern "C" int awq_prefill_attention(const void* q, const void* k_cache, const void* v_cache, void* ctx,
@@ -1137,7 +1146,8 @@ extern "C" int awq_prefill_attention(const void* q, const void* k_cache, const v
                                      int32_t first_layer, void* stream) {
   AWQ_REQUIRE(q && k_cache && v_cache && ctx, "NULL pointer");
   return launch_prefill_attention((const half_t*)q, (const half_t*)k_cache, (const half_t*)v_cache, (half_t*)ctx,
-                                  n_heads, max_pos, pos0, n_tokens, first_layer ? 0 : 1, (hipStream_t)stream);
+                                  n_heads, max_pos, kv_head_major(max_pos), pos0, n_tokens, first_layer ? 0 : 1,
+                                  (hipStream_t)stream);
 }
 
 extern "C" int awq_residual_add(const void* a, const void* b, void* out, int64_t n, void* stream) {

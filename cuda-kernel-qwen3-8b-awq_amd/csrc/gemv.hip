@@ -180,7 +180,7 @@ struct GemvParams {
   half_t* v_cache;
   int32_t hidden;
   int32_t pos;
-  int64_t max_pos;
+  KvLayout kv;
   const StepState* dyn;
   // EPI_ARGMAX
   unsigned long long* best;
@@ -222,7 +222,7 @@ __device__ __forceinline__ void epilogue(const GemvParams& p, int row, int r, fl
         p.y[rr] = out;
       } else {
         half_t* cache = sec == 1 ? p.k_cache : p.v_cache;
-        cache[((int64_t)(rr >> 7) * p.max_pos + pos) * AWQ_HEAD_DIM + d] = out;
+        cache[kv_row(p.kv, rr >> 7, pos) + d] = out;
       }
       return;
     }
@@ -557,7 +557,7 @@ struct FlowParams {
   half_t* v_cache;
   int32_t hidden;
   int32_t pos;
-  int64_t max_pos;
+  KvLayout kv;
 };
 
 constexpr int kFlowSpinLimit = 1 << 18;  // polls (each about 0.1 us apart) before a wait gives up
@@ -746,7 +746,7 @@ __global__ __launch_bounds__(256) void flow_kernel(FlowParams p) {
     gp.v_cache = p.v_cache;
     gp.hidden = p.hidden;
     gp.pos = p.pos;
-    gp.max_pos = p.max_pos;
+    gp.kv = p.kv;
     gp.dyn = p.dyn;
     epilogue(gp, row, r, tot, (half_t)0.0f);
   } else {
@@ -886,7 +886,7 @@ int launch_gemv(const LinearArgs& a, hipStream_t st) {
   AWQ_REQUIRE(a.epilogue != EPI_RESIDUAL || a.res, "residual epilogue needs res");
   if (a.epilogue == EPI_QKV_ROPE) {
     AWQ_REQUIRE(a.cos_t && a.sin_t && a.k_cache && a.v_cache && a.hidden > 0 && a.m == 3 * (int64_t)a.hidden &&
-                    a.hidden % AWQ_HEAD_DIM == 0 && a.max_pos > 0,
+                    a.hidden % AWQ_HEAD_DIM == 0 && a.max_pos > 0 && a.kv.head_stride > 0,
                 "QKV epilogue needs rotary tables, caches and m == 3*hidden");
     AWQ_REQUIRE(a.dyn || (a.pos >= 0 && a.pos < a.max_pos), "pos out of range");
   }
@@ -915,7 +915,7 @@ int launch_gemv(const LinearArgs& a, hipStream_t st) {
   p.v_cache = a.v_cache;
   p.hidden = a.hidden;
   p.pos = a.pos;
-  p.max_pos = a.max_pos;
+  p.kv = a.kv;
   p.dyn = a.dyn;
   p.best = a.best;
   const bool periodic = p.C > 1;
@@ -1002,7 +1002,7 @@ int launch_flow(const FlowLaunch& f, hipStream_t st) {
   p.v_cache = f.v_cache;
   p.hidden = f.hidden;
   p.pos = f.pos;
-  p.max_pos = f.max_pos;
+  p.kv = f.kv;
   const dim3 grid((unsigned)first), block(256);
   void (*kern)(FlowParams);
   const bool z = f.zp_integral != 0;

@@ -35,13 +35,13 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const half_t* __restrict__
 __global__ __launch_bounds__(64) void rope_kv_kernel(const half_t* __restrict__ qkv, const half_t* __restrict__ cos_t,
                                                      const half_t* __restrict__ sin_t, half_t* __restrict__ q_out,
                                                      half_t* __restrict__ kc, half_t* __restrict__ vc, int n_heads,
-                                                     int64_t max_pos, int pos_arg, const StepState* dyn) {
+                                                     KvLayout kv, int pos_arg, const StepState* dyn) {
   const int pos = dyn ? dyn->pos : pos_arg;
   const int hd = blockIdx.x, i = threadIdx.x;
   const int H = n_heads * AWQ_HEAD_DIM;
   const half_t c = cos_t[(int64_t)pos * 64 + i], s = sin_t[(int64_t)pos * 64 + i];
   const int e = hd * AWQ_HEAD_DIM + 2 * i;
-  const int64_t dst = ((int64_t)hd * max_pos + pos) * AWQ_HEAD_DIM + 2 * i;
+  const int64_t dst = kv_row(kv, hd, pos) + 2 * i;
   {
     half_t a = qkv[e], b = qkv[e + 1];
     half_t ac = a * c, bs = b * s, as = a * s, bc = b * c;
@@ -172,12 +172,12 @@ int launch_rmsnorm(const half_t* x, const half_t* gamma, half_t* out, int64_t n,
 }
 
 int launch_rope_kv_append(const half_t* qkv, const half_t* cos_t, const half_t* sin_t, half_t* q_out, half_t* kc,
-                          half_t* vc, int n_heads, int64_t max_pos, int64_t pos, const StepState* dyn,
+                          half_t* vc, int n_heads, int64_t max_pos, KvLayout kv, int64_t pos, const StepState* dyn,
                           hipStream_t st) {
   AWQ_REQUIRE(n_heads > 0 && max_pos > 0, "n_heads and max_pos must be positive");
   AWQ_REQUIRE(dyn || (pos >= 0 && pos < max_pos), "pos out of range");
   hipLaunchKernelGGL(rope_kv_kernel, dim3(n_heads), dim3(64), 0, st, qkv, cos_t, sin_t, q_out, kc, vc, n_heads,
-                     max_pos, (int)pos, dyn);
+                     kv, (int)pos, dyn);
   AWQ_HIP_TRY(hipGetLastError());
   return AWQ_OK;
 }

@@ -76,7 +76,7 @@ __global__ __launch_bounds__(256) void rope_kv_batch_kernel(const half_t* __rest
                                                            const half_t* __restrict__ cos_t,
                                                            const half_t* __restrict__ sin_t,
                                                            half_t* __restrict__ q_out, half_t* __restrict__ kc,
-                                                           half_t* __restrict__ vc, int n_heads, int64_t max_pos,
+                                                           half_t* __restrict__ vc, int n_heads, KvLayout kv,
                                                            int pos0) {
   const int tok = blockIdx.y, pos = pos0 + tok;
   const int hd = blockIdx.x * 4 + (threadIdx.x >> 6), i = threadIdx.x & 63;
@@ -86,7 +86,7 @@ __global__ __launch_bounds__(256) void rope_kv_batch_kernel(const half_t* __rest
   q_out += (int64_t)tok * H;
   const half_t c = cos_t[(int64_t)pos * 64 + i], s = sin_t[(int64_t)pos * 64 + i];
   const int e = hd * AWQ_HEAD_DIM + 2 * i;
-  const int64_t dst = ((int64_t)hd * max_pos + pos) * AWQ_HEAD_DIM + 2 * i;
+  const int64_t dst = kv_row(kv, hd, pos) + 2 * i;
   {
     const half_t a = qkv[e], b = qkv[e + 1];
     const half_t ac = a * c, bs = b * s, as = a * s, bc = b * c;
@@ -132,7 +132,7 @@ constexpr int kFaVStride = 36;    // halves per row of the transposed V tile (32
 __global__ __launch_bounds__(256) void prefill_attention_kernel(const half_t* __restrict__ q,
                                                                 const half_t* __restrict__ kc,
                                                                 const half_t* __restrict__ vc,
-                                                                half_t* __restrict__ ctx, int64_t max_pos, int pos0,
+                                                                half_t* __restrict__ ctx, KvLayout kv, int pos0,
                                                                 int M, int use_len_hi) {
   __shared__ __attribute__((aligned(16))) half_t ks[kFaKeys * kFaKStride];
   __shared__ __attribute__((aligned(16))) half_t vt[AWQ_HEAD_DIM * kFaVStride];
@@ -141,8 +141,8 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(const half_t* __
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n = lane & 31, kh = lane >> 5;
-  const half_t* kh_ptr = kc + (int64_t)head * max_pos * AWQ_HEAD_DIM;
-  const half_t* vh_ptr = vc + (int64_t)head * max_pos * AWQ_HEAD_DIM;
+  const half_t* kh_ptr = kc;
+  const half_t* vh_ptr = vc;
   // attended length of the query at position p (Inference.cu:1118 read before or after :1331)
   auto len_of = [&](int p) { return use_len_hi ? p + 1 : (p > 1 ? p : 1); };
   const int q_first = blockIdx.y * kFaQueries;
@@ -181,8 +181,8 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(const half_t* __
       const int pc = tid + i * 256;
       const int key = pc >> 4, part = pc & 15;
       const int kg = k0 + key < L_wg ? k0 + key : L_wg - 1;  // rows past the end are masked below
-      r.k[i] = *reinterpret_cast<const u32x4_t*>(kh_ptr + (int64_t)kg * AWQ_HEAD_DIM + part * 8);
-      r.v[i] = *reinterpret_cast<const half8_t*>(vh_ptr + (int64_t)kg * AWQ_HEAD_DIM + part * 8);
+      r.k[i] = *reinterpret_cast<const u32x4_t*>(kh_ptr + kv_row(kv, head, kg) + part * 8);
+      r.v[i] = *reinterpret_cast<const half8_t*>(vh_ptr + kv_row(kv, head, kg) + part * 8);
     }
   };
   auto step = [&](int k0, TileRegs& r) __attribute__((always_inline)) {
@@ -301,22 +301,22 @@ int launch_rmsnorm_batch(const half_t* x, const half_t* gamma, half_t* out, int6
 }
 
 int launch_rope_kv_append_batch(const half_t* qkv, const half_t* cos_t, const half_t* sin_t, half_t* q_out,
-                                half_t* kc, half_t* vc, int n_heads, int64_t max_pos, int64_t pos0, int64_t M,
-                                hipStream_t st) {
+                                half_t* kc, half_t* vc, int n_heads, int64_t max_pos, KvLayout kv, int64_t pos0,
+                                int64_t M, hipStream_t st) {
   AWQ_REQUIRE(n_heads > 0 && max_pos > 0, "n_heads and max_pos must be positive");
   AWQ_REQUIRE(M >= 1 && M <= 65535 && pos0 >= 0 && pos0 + M <= max_pos, "positions out of range");
   hipLaunchKernelGGL(rope_kv_batch_kernel, dim3((unsigned)((n_heads + 3) / 4), (unsigned)M), dim3(256), 0, st, qkv, cos_t, sin_t,
-                     q_out, kc, vc, n_heads, max_pos, (int)pos0);
+                     q_out, kc, vc, n_heads, kv, (int)pos0);
   AWQ_HIP_TRY(hipGetLastError());
   return AWQ_OK;
 }
 
 int launch_prefill_attention(const half_t* q, const half_t* kc, const half_t* vc, half_t* ctx, int n_heads,
-                             int64_t max_pos, int64_t pos0, int64_t M, int use_len_hi, hipStream_t st) {
+                             int64_t max_pos, KvLayout kv, int64_t pos0, int64_t M, int use_len_hi, hipStream_t st) {
   AWQ_REQUIRE(n_heads > 0 && max_pos > 0, "n_heads and max_pos must be positive");
   AWQ_REQUIRE(M >= 1 && M <= 65535 * kFaQueries && pos0 >= 0 && pos0 + M <= max_pos, "positions out of range");
   hipLaunchKernelGGL(prefill_attention_kernel, dim3((unsigned)n_heads, (unsigned)((M + kFaQueries - 1) / kFaQueries)),
-                     dim3(256), 0, st, q, kc, vc, ctx, max_pos, (int)pos0, (int)M, use_len_hi);
+                     dim3(256), 0, st, q, kc, vc, ctx, kv, (int)pos0, (int)M, use_len_hi);
   AWQ_HIP_TRY(hipGetLastError());
   return AWQ_OK;
 }
