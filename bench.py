@@ -37,6 +37,7 @@ def main():
     ap.add_argument("--layers", type=int, default=36, help="debug only: fewer layers make the result invalid")
     ap.add_argument("--prompt-len", type=int, default=128)
     ap.add_argument("--seed", type=int, default=2024)
+    ap.add_argument("--max-pos", type=int, default=40960, help="positions the key/value cache is allocated for")
     ap.add_argument("--cpu-prompt", type=int, default=16, help="prompt length of the CPU sample")
     ap.add_argument("--cpu-steps", type=int, default=112, help="generated tokens of the CPU sample (0 = skip)")
     ap.add_argument("--no-graph", action="store_true")
@@ -61,8 +62,9 @@ def main():
     from helpers import fill_pair, make_oracle_model, ptr
     import oracle_lib
 
-    max_pos = max(2176, args.prompt_len + args.warmup + args.steps + 8)
-    cfg = awq.make_config(n_layers=args.layers, max_pos=max_pos)
+    # the reference's sequence capacity (MAX_SEQ_LEN, Inference.cu:39): 24 GB of key/value cache
+    cfg = awq.make_config(n_layers=args.layers, max_pos=args.max_pos)
+    assert args.max_pos >= max(2176, args.prompt_len + args.warmup + args.steps + 8)
     oracle = oracle_lib.load() if args.cpu_steps > 0 else None
 
     profile = awq.SYNTH_BALANCED if args.profile == "balanced" else awq.SYNTH_SPEC
@@ -70,7 +72,8 @@ def main():
     eng = awq.QWen3AWQInfer.empty(cfg)
     if oracle is not None:
         # the checker owns the host copy of the weights; the engine gets the same bytes
-        model = make_oracle_model(oracle, cfg)
+        # (with room for its own sample only: its cache lives in host memory)
+        model = make_oracle_model(oracle, awq.make_config(n_layers=args.layers, max_pos=args.cpu_prompt + args.cpu_steps + 8))
         fill_pair(awq, oracle, cfg, args.seed, engine=eng, model=model, profile=profile)
     else:
         model = None
@@ -235,7 +238,7 @@ def main():
                                "intermediate 12288, vocab 151936, int4 g=128; %d-token prompt, batch-1 greedy decode"
                                % (cfg.n_layers, args.prompt_len),
                    "attended_positions": "%d..%d" % (args.prompt_len + args.warmup, args.prompt_len + args.warmup + args.steps),
-                   "graph": not args.no_graph, "flow_launches": args.flow},
+                   "max_pos": cfg.max_pos, "graph": not args.no_graph, "flow_launches": args.flow},
         "step_algorithmic_bytes": int(step_bytes),
         "step_hbm_frac": round(step_bytes * tok_s / (HBM_PEAK_GBS * 1e9), 4),
         "greedy_tokens_identical_to_cpu": tokens_match,
