@@ -759,7 +759,9 @@ extern "C" int awq_prefill(awq_engine* e, const int32_t* prompt_ids, int32_t n_p
 
 namespace {
 
-constexpr int64_t kPrefillChunk = 1280;  // prompt positions per batched pass
+constexpr int64_t kPrefillChunk = 1280;      // prompt positions per batched pass
+constexpr int64_t kPrefillLongChunk = 1024;  // ... of a sequence longer than kPrefillLongFrom
+constexpr int64_t kPrefillLongFrom = 4096;
 constexpr int64_t kGemmWsBytes = (64ll << 20) + 4096;  // header + partial sums (256 tiles, or 4 chunks of k for few rows)
 
 int ensure_prefill_buffers(awq_engine* e) {
@@ -830,9 +832,17 @@ extern "C" int awq_prefill_batched(awq_engine* e, const int32_t* prompt_ids, int
   const int64_t H = e->cfg.hidden;
   for (int64_t off = 0, M = 0; off < n_prompt; off += M) {
     // equal passes rather than full ones and a small rest (whole 128-token tiles each): 4096 positions
-    // go as 4 x 1024, not 3 x 1280 + 256
-    const int64_t rest = n_prompt - off, passes = (rest + e->pb.chunk - 1) / e->pb.chunk;
-    M = std::min<int64_t>(rest, std::min<int64_t>(e->pb.chunk, ((rest + passes - 1) / passes + 127) / 128 * 128));
+    // go as 4 x 1024, not 3 x 1280 + 256.  Sequences beyond kPrefillLongFrom positions take at most
+    // 1024 per pass: the prompt attention has one workgroup of 128 queries per compute unit, so 1280
+    // positions x 32 heads are 320 workgroups and two rounds where 1024 are one (1.27 ms per launch at
+    // 15,000 cached positions against 0.5 ms), which by then outweighs the products' better tile
+    // count at 1280 (8192 tokens: 201 -> 166 ms, 30,000: 1.48 -> 1.11 s; 2560 tokens stay at
+    // 2 x 1280: 41 ms, not 47).
+    const int64_t rest = n_prompt - off;
+    const int64_t chunk = e->n_positions + rest > kPrefillLongFrom ? std::min<int64_t>(e->pb.chunk, kPrefillLongChunk)
+                                                                  : e->pb.chunk;
+    const int64_t passes = (rest + chunk - 1) / chunk;
+    M = std::min<int64_t>(rest, std::min<int64_t>(chunk, ((rest + passes - 1) / passes + 127) / 128 * 128));
     const int64_t pos0 = e->n_positions;
     AWQ_HIP_TRY(hipMemcpyAsync(e->pb.tokens, prompt_ids + off, (size_t)M * 4, hipMemcpyHostToDevice, e->stream));
     if (int rc = launch_embed_batch(e->embed.packed, e->embed.scale, e->embed.zp, H, e->cfg.vocab, e->pb.tokens, M,
