@@ -127,7 +127,8 @@ typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 constexpr int kFaQueries = 128;   // per workgroup, 32 per wavefront
 constexpr int kFaKeys = 32;       // per step
 constexpr int kFaKStride = 136;   // halves per key row of the K tile (128 + 8 of padding)
-constexpr int kFaVStride = 36;    // halves per row of the transposed V tile (32 keys + 4 of padding)
+constexpr int kFaVStride = 144;   // halves per key row of the V tile (128 + 16: four consecutive rows start 8 banks apart)
+typedef short short4_t __attribute__((ext_vector_type(4)));
 
 __global__ __launch_bounds__(256) void prefill_attention_kernel(const half_t* __restrict__ q,
                                                                 const half_t* __restrict__ kc,
@@ -135,7 +136,7 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(const half_t* __
                                                                 half_t* __restrict__ ctx, KvLayout kv, int pos0,
                                                                 int M, int use_len_hi) {
   __shared__ __attribute__((aligned(16))) half_t ks[kFaKeys * kFaKStride];
-  __shared__ __attribute__((aligned(16))) half_t vt[AWQ_HEAD_DIM * kFaVStride];
+  __shared__ __attribute__((aligned(16))) half_t vs[kFaKeys * kFaVStride];
   const int head = blockIdx.x, n_heads = gridDim.x;
   const int H = n_heads * AWQ_HEAD_DIM;
   const int tid = threadIdx.x, lane = tid & 63;
@@ -151,6 +152,7 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(const half_t* __
   const int Lq = len_of(pos0 + qc);
   const int L_wg = len_of(pos0 + min(q_first + kFaQueries - 1, M - 1));      // lengths grow with the position
   const int L_wave = len_of(pos0 + min(q_first + wave * 32 + 31, M - 1));
+  const int L_wave_min = len_of(pos0 + min(q_first + wave * 32, M - 1));  // the shortest range among its queries
 
   // the query's 128 components as the second operand of the 8 slices of the first product
   half8_t qop[8];
@@ -192,10 +194,7 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(const half_t* __
       const int pc = tid + i * 256;
       const int key = pc >> 4, part = pc & 15;
       *reinterpret_cast<u32x4_t*>(ks + key * kFaKStride + part * 8) = r.k[i];
-#pragma unroll
-      // the 8 rows of a part are rotated by 4 (part + part / 8) keys: without it the 16 parts of a
-      // wavefront's store hit two banks, with it all 32
-      for (int e = 0; e < 8; ++e) vt[(part * 8 + e) * kFaVStride + ((key + 4 * (part + (part >> 3))) & 31)] = r.v[i][e];
+      *reinterpret_cast<half8_t*>(vs + key * kFaVStride + part * 8) = r.v[i];
     }
     __syncthreads();
     // the tile after the next travels while this one and the next are multiplied
@@ -210,27 +209,31 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(const half_t* __
       const half8_t kop = *reinterpret_cast<const half8_t*>(ks + n * kFaKStride + 16 * s + 8 * kh);
       sacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(kop, qop[s], sacc, 0, 0, 0);
     }
-    // sacc[i] is the score of key k0 + 8 (i / 4) + 4 kh + i % 4 for this lane's query
-    float sv[16];
+    // sacc[i] is the score of key k0 + 8 (i / 4) + 4 kh + i % 4 for this lane's query.  A tile that
+    // lies wholly inside the attended range of every query of the wavefront (nearly all tiles of a
+    // long prompt) needs no masks; the scale goes into the exponent's multiply-add.
+    const bool masked = k0 + kFaKeys > L_wave_min;  // same for the whole wavefront
     float mx = -1e30f;
+    if (masked) {
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int key = k0 + 8 * (i >> 2) + 4 * kh + (i & 3);
-      sv[i] = key < Lq ? sacc[i] * scale2 : -1e30f;
-      mx = fmaxf(mx, sv[i]);
+      for (int i = 0; i < 16; ++i) {
+        const int key = k0 + 8 * (i >> 2) + 4 * kh + (i & 3);
+        sacc[i] = key < Lq ? sacc[i] : -1e30f;  // 2^(scale * -1e30 - m) is 0
+      }
     }
+#pragma unroll
+    for (int i = 0; i < 16; ++i) mx = fmaxf(mx, sacc[i]);
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float m_new = fmaxf(m_run, mx);
+    // (a tile in which none of this query's keys is attended leaves the maximum where it was)
+    const float m_new = fmaxf(m_run, mx > -1e29f ? mx * scale2 : -1e30f);
     const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
     float rs = 0.0f;
     half8_t pop[2];
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-      const int key = k0 + 8 * (i >> 2) + 4 * kh + (i & 3);
-      const float pe = key < Lq ? __builtin_amdgcn_exp2f(sv[i] - m_new) : 0.0f;
-      const half_t ph = (half_t)pe;
-      rs += (float)ph;  // the sum of what the second product really multiplies
-      pop[i >> 3][i & 7] = ph;
+      const float pe = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[i], scale2, -m_new));
+      rs += pe;
+      pop[i >> 3][i & 7] = (half_t)pe;
     }
     rs += __shfl_xor(rs, 32, 64);
     l_run = l_run * alpha + rs;
@@ -243,16 +246,23 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(const half_t* __
         for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
     }
     // second product: slice j takes keys 16 j + 8 (e / 4) + 4 kh + e % 4, e = 0..7, which are this
-    // lane's probabilities 8 j .. 8 j + 7
+    // lane's probabilities 8 j .. 8 j + 7.  Its first operand is V transposed: component 32 dt + n of
+    // four consecutive keys per 8-byte half.  The transposing LDS read delivers exactly that from the
+    // tile as it came from memory: within 16 lanes, lane i receives element i % 4 of the 8-byte pieces
+    // that lanes i / 4, i / 4 + 4, i / 4 + 8, i / 4 + 12 point at -- so lane L points at the row of key
+    // L / 4 of the four, components 4 (L % 4) .. + 3 of the group's sixteen.
+    const int L16 = lane & 15;
+    const half_t* vlane = vs + (4 * kh + (L16 >> 2)) * kFaVStride + 16 * ((lane >> 4) & 1) + 4 * (L16 & 3);
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
 #pragma unroll
       for (int dt = 0; dt < 4; ++dt) {
-        const half_t* vr = vt + (dt * 32 + n) * kFaVStride;
-        const int rot = 4 * (((dt * 32 + n) >> 3) + ((dt * 32 + n) >> 6));  // the row's rotation, a multiple of 4 keys
-        const half4_t lo = *reinterpret_cast<const half4_t*>(vr + ((16 * j + 4 * kh + rot) & 31));
-        const half4_t hi = *reinterpret_cast<const half4_t*>(vr + ((16 * j + 4 * kh + 8 + rot) & 31));
-        const half8_t vop = half8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        const half_t* vp = vlane + 16 * j * kFaVStride + dt * 32;
+        const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((short4_t __attribute__((address_space(3)))*)vp);
+        const short4_t hi =
+            __builtin_amdgcn_ds_read_tr16_b64_v4i16((short4_t __attribute__((address_space(3)))*)(vp + 8 * kFaVStride));
+        const half4_t lh = __builtin_bit_cast(half4_t, lo), hh = __builtin_bit_cast(half4_t, hi);
+        const half8_t vop = half8_t{lh[0], lh[1], lh[2], lh[3], hh[0], hh[1], hh[2], hh[3]};
         o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vop, pop[j], o[dt], 0, 0, 0);
       }
     }
