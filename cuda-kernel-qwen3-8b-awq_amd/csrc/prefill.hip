@@ -130,7 +130,7 @@ constexpr int kFaKStride = 136;   // halves per key row of the K tile (128 + 8 o
 constexpr int kFaVStride = 144;   // halves per key row of the V tile (128 + 16: four consecutive rows start 8 banks apart)
 typedef short short4_t __attribute__((ext_vector_type(4)));
 
-__global__ __launch_bounds__(256) void prefill_attention_kernel(const half_t* __restrict__ q,
+__global__ __launch_bounds__(256, 2) void prefill_attention_kernel(const half_t* __restrict__ q,
                                                                 const half_t* __restrict__ kc,
                                                                 const half_t* __restrict__ vc,
                                                                 half_t* __restrict__ ctx, KvLayout kv, int pos0,
