@@ -833,11 +833,10 @@ extern "C" int awq_prefill_batched(awq_engine* e, const int32_t* prompt_ids, int
   for (int64_t off = 0, M = 0; off < n_prompt; off += M) {
     // equal passes rather than full ones and a small rest (whole 128-token tiles each): 4096 positions
     // go as 4 x 1024, not 3 x 1280 + 256.  Sequences beyond kPrefillLongFrom positions take at most
-    // 1024 per pass: the prompt attention has one workgroup of 128 queries per compute unit, so 1280
-    // positions x 32 heads are 320 workgroups and two rounds where 1024 are one (1.27 ms per launch at
-    // 15,000 cached positions against 0.5 ms), which by then outweighs the products' better tile
-    // count at 1280 (8192 tokens: 201 -> 166 ms, 30,000: 1.48 -> 1.11 s; 2560 tokens stay at
-    // 2 x 1280: 41 ms, not 47).
+    // 1024 per pass: deep in a long prompt the attention dominates, and 1024 positions x 32 heads
+    // are 256 of its workgroups (one per compute unit) where 1280 are 320, which outweighs the
+    // products' better tile count at 1280 (8192 tokens: 159 -> 146 ms, 30,000: 0.93 -> 0.89 s;
+    // 2560 tokens stay at 2 x 1280).
     const int64_t rest = n_prompt - off;
     const int64_t chunk = e->n_positions + rest > kPrefillLongFrom ? std::min<int64_t>(e->pb.chunk, kPrefillLongChunk)
                                                                   : e->pb.chunk;
