@@ -135,8 +135,8 @@ __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(const half_t*
                                                                 const half_t* __restrict__ vc,
                                                                 half_t* __restrict__ ctx, KvLayout kv, int pos0,
                                                                 int M, int use_len_hi) {
-  __shared__ __attribute__((aligned(16))) half_t ks[kFaKeys * kFaKStride];
-  __shared__ __attribute__((aligned(16))) half_t vs[kFaKeys * kFaVStride];
+  __shared__ __attribute__((aligned(16))) half_t ks2[2 * kFaKeys * kFaKStride];
+  __shared__ __attribute__((aligned(16))) half_t vs2[2 * kFaKeys * kFaVStride];
   const int head = blockIdx.x, n_heads = gridDim.x;
   const int H = n_heads * AWQ_HEAD_DIM;
   const int tid = threadIdx.x, lane = tid & 63;
@@ -176,6 +176,7 @@ __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(const half_t*
     u32x4_t k[2];
     half8_t v[2];
   };
+  TileRegs ra, rb;
   auto load_tile = [&](int k0, TileRegs& r) __attribute__((always_inline)) {
     if (k0 >= L_wg) return;
 #pragma unroll
@@ -187,19 +188,29 @@ __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(const half_t*
       r.v[i] = *reinterpret_cast<const half8_t*>(vh_ptr + kv_row(kv, head, kg) + part * 8);
     }
   };
-  auto step = [&](int k0, TileRegs& r) __attribute__((always_inline)) {
+  // both register sets go to LDS between one pair of barriers (two tiles of 32 keys per step)
+  auto stage = [&](int k0) __attribute__((always_inline)) {
     __syncthreads();  // the previous tiles' readers are done
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int pc = tid + i * 256;
       const int key = pc >> 4, part = pc & 15;
-      *reinterpret_cast<u32x4_t*>(ks + key * kFaKStride + part * 8) = r.k[i];
-      *reinterpret_cast<half8_t*>(vs + key * kFaVStride + part * 8) = r.v[i];
+      *reinterpret_cast<u32x4_t*>(ks2 + key * kFaKStride + part * 8) = ra.k[i];
+      *reinterpret_cast<half8_t*>(vs2 + key * kFaVStride + part * 8) = ra.v[i];
+      if (k0 + kFaKeys < L_wg) {
+        *reinterpret_cast<u32x4_t*>(ks2 + (kFaKeys + key) * kFaKStride + part * 8) = rb.k[i];
+        *reinterpret_cast<half8_t*>(vs2 + (kFaKeys + key) * kFaVStride + part * 8) = rb.v[i];
+      }
     }
     __syncthreads();
-    // the tile after the next travels while this one and the next are multiplied
-    load_tile(k0 + 2 * kFaKeys, r);
+    // the next two tiles travel while these are multiplied
+    load_tile(k0 + 2 * kFaKeys, ra);
+    load_tile(k0 + 3 * kFaKeys, rb);
+  };
+  auto step = [&](int k0, int half) __attribute__((always_inline)) {
     if (k0 >= L_wave) return;  // nothing of this tile is attended by this wavefront's queries
+    const half_t* ks = ks2 + half * kFaKeys * kFaKStride;
+    const half_t* vs = vs2 + half * kFaKeys * kFaVStride;
 
     f32x16_t sacc;
 #pragma unroll
@@ -267,12 +278,12 @@ __global__ __launch_bounds__(256, 2) void prefill_attention_kernel(const half_t*
       }
     }
   };
-  TileRegs ra, rb;
   load_tile(0, ra);
   load_tile(kFaKeys, rb);
   for (int k0 = 0; k0 < L_wg; k0 += 2 * kFaKeys) {
-    step(k0, ra);
-    if (k0 + kFaKeys < L_wg) step(k0 + kFaKeys, rb);
+    stage(k0);
+    step(k0, 0);
+    if (k0 + kFaKeys < L_wg) step(k0 + kFaKeys, 1);
   }
   // o[dt][i] is component 32 dt + 8 (i / 4) + 4 kh + i % 4 of this lane's query
   if (qi < M) {
