@@ -202,6 +202,8 @@ int launch_rope_kv_append(const half_t* qkv, const half_t* cos_t, const half_t* 
 // Tokens per second over 264 decode steps, one workgroup per head against the cut
 // path: 582 / 567 at 258..522 positions, 556 / 557 at 408..672, 539 / 523 at 708..972
 // (before the two-launch form: 513), 458 / 510 at 908..1172, 378 / 480 at 1708..1972.
+// With the cache in blocks of 64 positions: 590 / 566 at 258..522, 569 / 561 at 358..622,
+// 547 / 555 at 458..722 -- the two forms meet near 540 positions.
 constexpr int64_t kAttnOneWorkgroupMax = 576;
 constexpr int64_t kAttnTwoLaunchMax = 1024;
 constexpr int64_t kAttnMergedMax = 2048;
