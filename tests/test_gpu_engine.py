@@ -51,6 +51,38 @@ def test_small_model_sequence_crossing_the_attention_switch(awq, oracle, torch_g
     oracle.awqo_model_destroy(model)
 
 
+def test_results_do_not_depend_on_the_cache_capacity(awq, torch_gpu):
+    """the engine keeps its key/value rows in blocks of 64 positions per head; whatever capacity the
+    cache is allocated for (not a multiple of 64, the reference's 40,960), a sequence that crosses a
+    block boundary gives the same tokens, hidden state and logits, prompt token by token or batched"""
+    results = []
+    for max_pos in (150, 1024, 40960):
+        cfg = awq.make_config(n_layers=2, hidden=512, inter=512, vocab=1024, max_pos=max_pos)
+        eng = awq.QWen3AWQInfer.empty(cfg)
+        lib = awq.load_library()
+        for layer, kind, part in awq.tensor_list(cfg):
+            count = cfg.part_count(kind, part)
+            nbytes = count if (part == awq.P_PACKED and kind != awq.T_GAMMA) else 2 * count
+            buf = (ctypes.c_uint8 * nbytes)()
+            awq.check(lib.awq_synth_fill_profile(awq.SYNTH_BALANCED, 7, layer, kind, part, buf, count))
+            eng.upload(layer, kind, part, buf, nbytes)
+        eng.finalize()
+        rng = np.random.default_rng(11)
+        prompt = rng.integers(0, cfg.vocab, 100).tolist()
+        for batched in (False, True):
+            eng.set_prefill_mode(batched)
+            print("cache capacity", max_pos, "batched prompt", batched, flush=True)
+            toks = eng.generateResponse(prompt, 40)
+            results.append((max_pos, batched, toks, np.ctypeslib.as_array(eng.read_hidden()).copy(),
+                            np.ctypeslib.as_array(eng.read_logits()).copy()))
+        eng.close()
+    for batched in (False, True):
+        same = [r for r in results if r[1] == batched]
+        for r in same[1:]:
+            assert r[2] == same[0][2]
+            assert np.array_equal(r[3], same[0][3]) and np.array_equal(r[4], same[0][4])
+
+
 @pytest.mark.parametrize("graph,flow", [(False, False), (True, False), (False, True), (True, True)])
 def test_small_model_tokens_and_state_identical(awq, oracle, torch_gpu, graph, flow):
     """flow: the products after a layer's attention as dependent workgroup ranges of one launch"""
