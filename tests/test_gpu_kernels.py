@@ -507,7 +507,13 @@ def test_gemv_fused_norm_unembed_argmax(awq, lib, oracle, torch_gpu, m, k):
                                           (12288, 4096, 16, True), (12288, 4096, 200, True), (4096, 12288, 64, False),
                                           (4096, 12288, 128, True), (12288, 4096, 1030, True),
                                           (4096, 4096, 1024, True), (4096, 12288, 1024, True),
-                                          (4096, 12288, 640, True), (384, 6144, 8500, False)])
+                                          (4096, 12288, 640, True), (384, 6144, 8500, False),
+                                          # config 5's own points: the 2048-token prefill product and the
+                                          # decode-batch sweep M = 1, 4, 16, 64 on the w1 and w2 shapes
+                                          (12288, 4096, 2048, True), (4096, 12288, 2048, True),
+                                          (12288, 4096, 1, True), (4096, 12288, 1, True),
+                                          (12288, 4096, 4, True), (4096, 12288, 4, True),
+                                          (4096, 12288, 16, True), (12288, 4096, 64, True)])
 def test_gemm_matches_fp32_accumulate_reference(awq, lib, oracle, torch_gpu, m, k, M, zp_int):
     """config 5: dequant-on-load MFMA product; 1e-2 relative against the sequential FP32-accumulate
     reference, and the weights it multiplies are the bit-exact dequantised ones (one-hot check below).
