@@ -41,8 +41,6 @@ def main():
     ap.add_argument("--cpu-prompt", type=int, default=16, help="prompt length of the CPU sample")
     ap.add_argument("--cpu-steps", type=int, default=112, help="generated tokens of the CPU sample (0 = skip)")
     ap.add_argument("--no-graph", action="store_true")
-    ap.add_argument("--flow", action="store_true",
-                    help="the products after a layer's attention as dependent workgroup ranges of one launch")
     ap.add_argument("--profile", choices=["balanced", "spec"], default="balanced",
                     help="value distributions of the synthetic weights (include/awq_synth.h); 'spec' overflows "
                          "binary16 by layer 3 and decodes token 0 forever, so the default keeps activations finite")
@@ -85,7 +83,6 @@ def main():
             eng.upload(layer, kind, part, buf, nbytes)
         eng.finalize()
     eng.set_graph_mode(not args.no_graph)
-    eng.set_flow_mode(args.flow)
     log("weights generated, uploaded and reordered in %.1f s" % (time.time() - t0))
 
     prompt = np.zeros(args.prompt_len, dtype=np.int32)
@@ -238,7 +235,7 @@ def main():
                                "intermediate 12288, vocab 151936, int4 g=128; %d-token prompt, batch-1 greedy decode"
                                % (cfg.n_layers, args.prompt_len),
                    "attended_positions": "%d..%d" % (args.prompt_len + args.warmup, args.prompt_len + args.warmup + args.steps),
-                   "max_pos": cfg.max_pos, "graph": not args.no_graph, "flow_launches": args.flow},
+                   "max_pos": cfg.max_pos, "graph": not args.no_graph},
         "step_algorithmic_bytes": int(step_bytes),
         "step_hbm_frac": round(step_bytes * tok_s / (HBM_PEAK_GBS * 1e9), 4),
         "greedy_tokens_identical_to_cpu": tokens_match,

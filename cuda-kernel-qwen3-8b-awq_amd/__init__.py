@@ -69,7 +69,6 @@ SIGNATURES = {
     "awq_read_hidden": (ctypes.c_int, [_vp, _vp]),
     "awq_read_logits": (ctypes.c_int, [_vp, _vp]),
     "awq_set_graph_mode": (ctypes.c_int, [_vp, ctypes.c_int]),
-    "awq_set_flow_mode": (ctypes.c_int, [_vp, ctypes.c_int]),
     "awq_time_linear": (ctypes.c_int, [_vp, ctypes.c_int, _i32, ctypes.POINTER(_f32), ctypes.POINTER(_i64)]),
     "awq_destroy": (None, [_vp]),
     "awq_write_weight_dir": (ctypes.c_int, [ctypes.c_char_p, _cfgp, _u64]),
@@ -252,10 +251,6 @@ class QWen3AWQInfer:
 
     def set_graph_mode(self, enabled):
         check(self._lib.awq_set_graph_mode(self._h, 1 if enabled else 0))
-
-    def set_flow_mode(self, enabled):
-        """Dependent products of a layer in one launch (default) or one launch per product."""
-        check(self._lib.awq_set_flow_mode(self._h, 1 if enabled else 0))
 
     def read_hidden(self):
         buf = (ctypes.c_uint16 * self.config.hidden)()

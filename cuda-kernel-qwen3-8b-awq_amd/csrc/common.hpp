@@ -74,7 +74,6 @@ struct StepState {
   int32_t token;      // token to embed at the start of the step, -1 = keep the hidden state
   int32_t out_index;  // where the sampled token goes in the output array
   int32_t sample;     // 1 = run the sampler at the end of the step
-  int32_t epoch;      // steps since the flow counters were zeroed (1-based)
 };
 
 // what the fused linear kernel does to its input and its output
@@ -136,49 +135,6 @@ int64_t gemv_workspace_bytes(int64_t m, int64_t k);
 int launch_gemv(const LinearArgs& a, hipStream_t st);
 int64_t gemm_workspace_bytes(int64_t m, int64_t k, int64_t M);
 int gemm_plan(int64_t m, int64_t k, int64_t M, int has_workspace);
-// Several dependent products in one launch (gemv.hip): role i + 1 consumes what
-// role i produced.  All roles take k_unit inputs per workgroup; a role with
-// k = S * k_unit is cut into S slices.
-struct FlowRoleArgs {
-  const void* wq = nullptr;
-  const half_t* scale = nullptr;
-  const half_t* zp = nullptr;
-  const half_t* x = nullptr;
-  const half_t* gamma = nullptr;   // fused RMSNorm when set
-  half_t* y = nullptr;
-  const half_t* res = nullptr;
-  float* part = nullptr;           // [k / k_unit][m] when k > k_unit
-  int64_t m = 0, k = 0;
-  int epilogue = EPI_STORE;
-  int x_fresh = 0, res_fresh = 0;  // written by an earlier role of the same launch
-  int wait = 0;                    // wait for the previous role
-  int32_t* wait_ready = nullptr;   // its ready words, [64][16]
-  int32_t* pre_ready = nullptr;    // ready words of the role before that: the weights are requested after it
-  int32_t* done_grp = nullptr;     // [ceil(m/256)][16] counters per 16 row groups, a cache line each
-  int32_t* done_cnt = nullptr;     // completion counter of this role and
-  int32_t* done_ready = nullptr;   // the ready words it publishes, [64][16]
-  int32_t* rg_cnt = nullptr;       // [m/16] when k > k_unit
-};
-struct FlowLaunch {
-  FlowRoleArgs role[4];
-  int n_roles = 0;
-  int64_t k_unit = 0;
-  int zp_integral = 0;
-  const StepState* dyn = nullptr;
-  int32_t epoch = 0;               // when dyn is null
-  int32_t* err = nullptr;
-  float eps = 0.0f;
-  const half_t* cos_t = nullptr;   // EPI_QKV_ROPE role
-  const half_t* sin_t = nullptr;
-  half_t* k_cache = nullptr;
-  half_t* v_cache = nullptr;
-  int32_t hidden = 0;
-  int32_t pos = 0;
-  int64_t max_pos = 0;
-  KvLayout kv = {0, 0, 0};
-};
-bool flow_supported(int64_t hidden, int64_t inter);
-int launch_flow(const FlowLaunch& f, hipStream_t st);
 int launch_gemm(const void* wq, const half_t* scale, const half_t* zp, int64_t m, int64_t k, const half_t* x,
                 half_t* y, int64_t M, int zp_integral, int epilogue, const half_t* res, void* workspace,
                 int64_t workspace_bytes, hipStream_t st);

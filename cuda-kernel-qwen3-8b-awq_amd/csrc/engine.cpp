@@ -167,21 +167,6 @@ struct awq_engine {
     int64_t chunk = 0;
   } pb;
   bool batched_prefill = false;
-  // dependent products of a layer in one launch (flow_kernel): completion counters
-  // [layer][3 + hidden/16], error flag, partial sums of the sliced w2 product
-  bool flow_ok = false;    // the shapes fit
-  bool flow_mode = false;  // and the caller wants it (measured slower than one launch per product: off)
-  int32_t* flow_cnt = nullptr;
-  int32_t* flow_err = nullptr;
-  float* flow_part = nullptr;
-  // Hidden state of the flow launches: input, after Wo, after W2 are three
-  // different buffers, rotating from layer to layer (ring[0] is `hidden`).  A
-  // vector written inside a launch is then read for the first time after it
-  // was written, so no cache of another XCD can hold an older copy of it, and
-  // ordinary (L2-cached) loads may read it.
-  half_t* ring[3] = {nullptr, nullptr, nullptr};
-  int64_t flow_stride = 0;
-  int32_t epoch = 0;       // steps since the counters were zeroed
   std::vector<void*> allocations;
 };
 
@@ -269,91 +254,6 @@ int enqueue_wqkv(awq_engine* e, int l) {
   return launch_gemv(a, e->stream);
 }
 
-// Everything of layer l after its attention, and the Wqkv product of layer l + 1,
-// as the roles of one flow launch: Wo (+residual), W1 (norm, GeLU), W2 (+residual),
-// next Wqkv (norm, rotary, KV append).
-int enqueue_flow(awq_engine* e, int l, int idx) {
-  LayerDev& L = e->layers[l];
-  half_t* h_in = e->ring[idx];
-  half_t* h_mid = e->ring[(idx + 1) % 3];
-  half_t* h_out = e->ring[(idx + 2) % 3];
-  const int64_t H = e->cfg.hidden;
-  int32_t* cnt = e->flow_cnt + (int64_t)l * e->flow_stride;  // 3 role counters, H/16 slice counters,
-  int32_t* ready = cnt + 3 + H / 16;                         // 3 x 64 ready words, a cache line each
-  int32_t* grp = ready + 3 * 1024;                           // 3 x 64 group counters, a cache line each
-  FlowLaunch f;
-  f.k_unit = H;
-  f.dyn = e->d_state;
-  f.err = e->flow_err;
-  f.eps = e->cfg.eps;
-  auto fill = [&](FlowRoleArgs& r, const DevLinear& t, const half_t* x, half_t* y) {
-    r.wq = t.stream_order;
-    r.scale = t.scale;
-    r.zp = t.zp;
-    r.x = x;
-    r.y = y;
-    r.m = t.m;
-    r.k = t.k;
-  };
-  int zint = L.wo.zp_integral && L.w1.zp_integral && L.w2.zp_integral;
-  {  // :1128-1155
-    FlowRoleArgs& r = f.role[0];
-    fill(r, L.wo, e->ctx, h_mid);
-    r.epilogue = EPI_RESIDUAL;
-    r.res = h_in;
-    r.done_cnt = cnt + 0;
-    r.done_grp = grp + 0 * 1024;
-    r.done_ready = ready + 0 * 1024;
-  }
-  {  // :1163-1196
-    FlowRoleArgs& r = f.role[1];
-    fill(r, L.w1, h_mid, e->mid);
-    r.gamma = L.gamma;
-    r.epilogue = EPI_GELU;
-    r.wait = 1;
-    r.wait_ready = ready + 0 * 1024;
-    r.done_cnt = cnt + 1;
-    r.done_grp = grp + 1 * 1024;
-    r.done_ready = ready + 1 * 1024;
-  }
-  {  // :1201-1227
-    FlowRoleArgs& r = f.role[2];
-    fill(r, L.w2, e->mid, h_out);
-    r.epilogue = EPI_RESIDUAL;
-    r.res = h_mid;
-    r.part = e->flow_part;
-    r.rg_cnt = cnt + 3;
-    r.wait = 1;
-    r.wait_ready = ready + 1 * 1024;
-    r.pre_ready = ready + 0 * 1024;
-    r.done_cnt = cnt + 2;
-    r.done_grp = grp + 2 * 1024;
-    r.done_ready = ready + 2 * 1024;
-  }
-  f.n_roles = 3;
-  if (l + 1 < e->cfg.n_layers) {  // :1040-1103 of the next layer
-    LayerDev& N = e->layers[l + 1];
-    FlowRoleArgs& r = f.role[3];
-    fill(r, N.wqkv, h_out, e->q);
-    r.gamma = N.gamma;
-    r.epilogue = EPI_QKV_ROPE;
-    r.wait = 1;
-    r.wait_ready = ready + 2 * 1024;
-    r.pre_ready = ready + 1 * 1024;
-    f.cos_t = e->cos_t;
-    f.sin_t = e->sin_t;
-    f.k_cache = N.kcache;
-    f.v_cache = N.vcache;
-    f.hidden = (int32_t)H;
-    f.max_pos = e->cfg.max_pos;
-    f.kv = kv_blocked(e->n_heads);
-    f.n_roles = 4;
-    zint = zint && N.wqkv.zp_integral;
-  }
-  f.zp_integral = zint;
-  return launch_flow(f, e->stream);
-}
-
 int enqueue_layer(awq_engine* e, int l, int use_len_hi, int64_t len_bound) {
   LayerDev& L = e->layers[l];
   hipStream_t st = e->stream;
@@ -407,25 +307,8 @@ int enqueue_step_body(awq_engine* e, bool gen, int64_t len_bound) {
                             e->d_token, e->hidden, e->stream))
     return rc;
   const int split = gen ? e->cfg.split_idx : 1;
-  if (e->flow_ok && e->flow_mode) {
-    // two launches per layer: attention, then the layer's products and the next layer's Wqkv
-    if (int rc = enqueue_wqkv(e, 0)) return rc;
-    int idx = 0;  // which buffer of the ring holds the layer's input
-    for (int l = 0; l < e->cfg.n_layers; ++l) {
-      if (int rc = launch_attention(e->q, e->layers[l].kcache, e->layers[l].vcache, e->ctx, e->n_heads, e->cfg.max_pos,
-                                    kv_blocked(e->n_heads),
-                                    0, e->d_state, l >= split, len_bound, e->attn_ws, e->stream))
-        return rc;  // :1110
-      if (int rc = enqueue_flow(e, l, idx)) return rc;
-      idx = (idx + 2) % 3;
-    }
-    // the step's result belongs in `hidden` (the sampler, the next step and the readers look there)
-    if (idx != 0)
-      if (int rc = launch_copy(e->ring[idx], e->hidden, (int64_t)e->cfg.hidden * 2, e->stream)) return rc;
-  } else {
-    for (int l = 0; l < e->cfg.n_layers; ++l)
-      if (int rc = enqueue_layer(e, l, l >= split, len_bound)) return rc;
-  }
+  for (int l = 0; l < e->cfg.n_layers; ++l)
+    if (int rc = enqueue_layer(e, l, l >= split, len_bound)) return rc;
   if (gen) return enqueue_sample(e);
   return AWQ_OK;
 }
@@ -446,7 +329,6 @@ int build_graph(awq_engine* e, bool gen, int64_t len_bound, hipGraphExec_t* out)
 }
 
 int run_step(awq_engine* e, bool gen, StepState s) {
-  s.epoch = ++e->epoch;
   if (int rc = launch_set_state(e->d_state, s, e->stream)) return rc;
   // the attention launches are specialised by an upper bound of the attended
   // length (one workgroup per head, or two to four launches cut along the
@@ -537,15 +419,6 @@ extern "C" int awq_create_empty(const awq_config* cfg_in, awq_engine** out) {
   if (int rc = dev_alloc(ep, (void**)&e->d_state, sizeof(StepState))) return fail(rc);
   if (int rc = dev_alloc(ep, (void**)&e->d_token, 4)) return fail(rc);
   if (int rc = dev_alloc(ep, (void**)&e->d_out, (int64_t)cfg.max_pos * 4)) return fail(rc);
-  e->flow_ok = flow_supported(H, I);
-  e->flow_stride = 3 + H / 16 + 6 * 1024 + 13;  // counters, slice counters, ready words, group counters
-  e->flow_stride = (e->flow_stride + 15) / 16 * 16;
-  if (int rc = dev_alloc(ep, (void**)&e->flow_cnt, (int64_t)cfg.n_layers * e->flow_stride * 4)) return fail(rc);
-  if (int rc = dev_alloc(ep, (void**)&e->flow_err, 4)) return fail(rc);
-  if (int rc = dev_alloc(ep, (void**)&e->flow_part, (I / H + 1) * H * 4)) return fail(rc);
-  e->ring[0] = e->hidden;
-  if (int rc = dev_alloc(ep, (void**)&e->ring[1], H * 2)) return fail(rc);
-  if (int rc = dev_alloc(ep, (void**)&e->ring[2], H * 2)) return fail(rc);
   *out = e.release();
   return AWQ_OK;
 }
@@ -692,41 +565,7 @@ extern "C" int awq_reset(awq_engine* e) {
   e->n_positions = 0;
   e->n_generated = 0;
   if (int rc = launch_fill_zero(e->hidden, (int64_t)e->cfg.hidden * 2, e->stream)) return rc;
-  // the completion counters of the flow launches count steps since here
-  e->epoch = 0;
-  if (int rc = launch_fill_zero(e->flow_cnt, (int64_t)e->cfg.n_layers * e->flow_stride * 4, e->stream)) return rc;
-  if (int rc = launch_fill_zero(e->flow_err, 4, e->stream)) return rc;
   AWQ_HIP_TRY(hipStreamSynchronize(e->stream));
-  return AWQ_OK;
-}
-
-namespace {
-// after the stream has drained: did a wait inside a flow launch give up?
-int check_flow(awq_engine* e) {
-  if (!(e->flow_ok && e->flow_mode)) return AWQ_OK;
-  int32_t err = 0;
-  AWQ_HIP_TRY(hipMemcpy(&err, e->flow_err, 4, hipMemcpyDeviceToHost));
-  if (err) {
-    awq_set_error("a workgroup of a flow launch waited for its producers beyond the limit; results are invalid "
-                  "(awq_set_flow_mode(e, 0) selects one launch per product)");
-    return AWQ_ERR_HIP;
-  }
-  return AWQ_OK;
-}
-}  // namespace
-
-extern "C" int awq_set_flow_mode(awq_engine* e, int enabled) {
-  AWQ_REQUIRE(e != nullptr, "engine is NULL");
-  if ((enabled != 0) != e->flow_mode) {
-    // the captured graphs hold the other launch sequence
-    for (auto& row : e->graphs)
-      for (hipGraphExec_t& g : row)
-        if (g) {
-          AWQ_HIP_TRY(hipGraphExecDestroy(g));
-          g = nullptr;
-        }
-  }
-  e->flow_mode = enabled != 0;
   return AWQ_OK;
 }
 
@@ -754,7 +593,7 @@ extern "C" int awq_prefill(awq_engine* e, const int32_t* prompt_ids, int32_t n_p
     e->n_positions = t + 1;
   }
   AWQ_HIP_TRY(hipStreamSynchronize(e->stream));
-  return check_flow(e);
+  return AWQ_OK;
 }
 
 namespace {
@@ -898,7 +737,6 @@ extern "C" int awq_decode(awq_engine* e, int32_t n_steps, int32_t* out_ids) {
     e->n_generated += 1;
   }
   AWQ_HIP_TRY(hipStreamSynchronize(e->stream));
-  if (int rc = check_flow(e)) return rc;
   if (n_steps > 0)
     AWQ_HIP_TRY(hipMemcpy(out_ids, e->d_out + first, (size_t)n_steps * 4, hipMemcpyDeviceToHost));
   return AWQ_OK;

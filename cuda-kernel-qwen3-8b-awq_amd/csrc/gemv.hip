@@ -479,311 +479,6 @@ __global__ __launch_bounds__(1024) void gemv_kernel(const u32x4* __restrict__ wq
   }
 }
 
-// ---------------------------------------------------------------------------
-// Several dependent matrix-vector products in ONE launch ("flow" launch).
-//
-// The decode step is a chain of products in which every workgroup of one needs
-// all outputs of the previous one, and a kernel boundary costs about 4 us of
-// launch gap and cold first loads per link.  Here the links are workgroup
-// ranges ("roles") of a single grid, in dependency order.  A workgroup
-//   1. requests its weights (they do not depend on anything) -- but not before
-//      the role two links up the chain has finished: with every resident
-//      workgroup's 32 KiB of weights queued at once, the small loads of the
-//      vector a running role needs wait for microseconds behind them in the
-//      compute units' memory pipelines; gated like this, only the next role's
-//      weights stream while the current one computes,
-//   2. waits until the producer role has finished (one poller per workgroup,
-//      bounded).  Hundreds of workgroups polling one counter would queue at one
-//      memory channel and delay the very increments they wait for, so the
-//      producer whose increment completes the count publishes the epoch in 64
-//      "ready" words in 64 different cache lines and a consumer polls the one
-//      its id selects,
-//   3. reads its input vector past the non-coherent caches, computes exactly as
-//      gemv_kernel does (same blocks, same trees: bit-identical results),
-//   4. writes its outputs through to memory, waits for the writes, and adds 1
-//      to its own role's counter.
-// Why this cannot deadlock: workgroups are dispatched in increasing id order
-// (per XCD), a role only waits for roles with lower ids, so the lowest
-// unfinished workgroup is always resident and never has to wait.  Every wait is
-// bounded anyway: past the limit the error flag is set, all waits give up, the
-// grid drains and the host reports the failure.
-//
-// Every role here has k = 512 G inputs per workgroup (4 wavefronts, G blocks
-// per lane); a matrix with S times as many inputs (w2) is cut into S slices of
-// that size handled by S consecutive workgroups, whose FP32 partial sums the
-// last one adds in the canonical order (awq_tree_sum over the slices).
-// ---------------------------------------------------------------------------
-struct FlowRole {
-  const u32x4* wq;
-  const half_t* scale;
-  const half_t* zp;
-  const half_t* x;      // input vector, k halves
-  const half_t* gamma;  // fused RMSNorm when not null (single-slice roles only)
-  half_t* y;
-  const half_t* res;    // EPI_RESIDUAL
-  float* part;          // [slice][m] partial sums (n_slices > 1)
-  int32_t first_wg;     // first workgroup of the role
-  int32_t n_rg;         // m / 16
-  int32_t n_slices;     // k / (512 G)
-  int32_t nblk_total;   // k / 32
-  int32_t mg, kg;       // m / 128, k / 128
-  int32_t epilogue;
-  int32_t x_fresh;      // x is written by an earlier role of this launch
-  int32_t res_fresh;    // res likewise
-  int32_t wait;         // 1: wait for the ready words of the producer role
-  int32_t* wait_ready;  // [64][16] words, one per cache line
-  int32_t* pre_ready;   // ready words to wait for before the weights are requested (or null)
-  // Completion of this role: a counter per 16 row groups (a cache line each;
-  // hundreds of increments of ONE word serialise at about 12 ns apiece), the
-  // count of complete groups, and the ready words published by the workgroup
-  // whose increment completes the count.
-  int32_t* done_grp;
-  int32_t* done_cnt;
-  int32_t* done_ready;
-  int32_t* rg_cnt;      // [n_rg] slice counters (n_slices > 1)
-};
-constexpr int kFlowRoles = 4;
-struct FlowParams {
-  FlowRole role[kFlowRoles];
-  int32_t n_roles;
-  const StepState* dyn;
-  int32_t epoch_arg;  // used when dyn is null
-  int32_t* err;
-  float eps;
-  // EPI_QKV_ROPE
-  const half_t* cos_t;
-  const half_t* sin_t;
-  half_t* k_cache;
-  half_t* v_cache;
-  int32_t hidden;
-  int32_t pos;
-  KvLayout kv;
-};
-
-constexpr int kFlowSpinLimit = 1 << 18;  // polls (each about 0.1 us apart) before a wait gives up
-
-__device__ __forceinline__ int32_t flow_load(const int32_t* p) {
-  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-// true when the counter reached the target; false (and the error flag set) when the wait gave up
-__device__ __forceinline__ bool flow_wait(const int32_t* cnt, int32_t target, int32_t* err) {
-  int spins = 0;
-  while (flow_load(cnt) < target) {
-    __builtin_amdgcn_s_sleep(1);
-    ++spins;
-    if ((spins & 63) == 0 && (spins > kFlowSpinLimit || flow_load(err) != 0)) {
-      __hip_atomic_store(err, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      return false;
-    }
-  }
-  return true;
-}
-
-template <int G, bool ZINT>
-__global__ __launch_bounds__(256) void flow_kernel(FlowParams p) {
-  __shared__ __attribute__((aligned(16))) half_t xs[512 * G + 16 * 8];  // x in block order, skewed
-  __shared__ float red[4][16];
-  __shared__ float nbuf[256];
-  constexpr int K = 512 * G;     // inputs per workgroup
-  constexpr int NBLK = 16 * G;   // blocks per workgroup
-  constexpr int MAXU = (K / 4 + 255) / 256;
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int q = lane >> 4, r = lane & 15;
-  const int epoch = p.dyn ? p.dyn->epoch : p.epoch_arg;
-
-  int ri = 0;
-#pragma unroll
-  for (int i = 1; i < kFlowRoles; ++i)
-    if (i < p.n_roles && (int)blockIdx.x >= p.role[i].first_wg) ri = i;
-  const FlowRole& R = p.role[ri];
-  const int local = blockIdx.x - R.first_wg;
-  const int rg = local / R.n_slices, slice = local - rg * R.n_slices;
-  const int blk0 = (4 * wave + q) * G;
-
-  // 1. the weights
-  if (R.pre_ready) {
-    if (tid == 0) flow_wait(R.pre_ready + (blockIdx.x & 63) * 16, epoch, p.err);
-    __syncthreads();
-  }
-  const u32x4* wp = R.wq + ((int64_t)rg * R.nblk_total + slice * NBLK + blk0) * 16 + r;
-  u32x4 w[G];
-#pragma unroll
-  for (int b = 0; b < G; ++b) w[b] = __builtin_nontemporal_load(wp + b * 16);
-  const int gi = ((rg >> 3) % R.kg) % R.mg;
-  const GroupConst g = make_group<ZINT>(R.scale[gi], R.zp[gi]);
-
-  // 2. the producers
-  if (R.wait) {
-    if (tid == 0) flow_wait(R.wait_ready + (blockIdx.x & 63) * 16, epoch, p.err);
-    __syncthreads();
-  }
-
-  // 3. x (this workgroup's slice), normalised on the way when the norm is fused
-  const half_t* xin = R.x + slice * K;
-  const bool norm = R.gamma != nullptr;
-  uint2 xu[MAXU], gu[MAXU];
-#pragma unroll
-  for (int u = 0; u < MAXU; ++u) {
-    const int unit = tid + u * 256;
-    if (unit < K / 4) {
-      if (R.x_fresh) {
-        const unsigned long long v = __hip_atomic_load(reinterpret_cast<const unsigned long long*>(xin) + unit,
-                                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        xu[u] = __builtin_bit_cast(uint2, v);
-      } else {
-        xu[u] = reinterpret_cast<const uint2*>(xin)[unit];
-      }
-      if (norm) gu[u] = reinterpret_cast<const uint2*>(R.gamma)[unit];
-    }
-  }
-  if (norm) {
-    // rmsNormKernel, Inference.cu:111-145, exactly as in gemv_kernel
-    half_t* xn = xs;
-#pragma unroll
-    for (int u = 0; u < MAXU; ++u)
-      if (tid + u * 256 < K / 4) reinterpret_cast<uint2*>(xn)[tid + u * 256] = xu[u];
-    __syncthreads();
-    {
-      float acc = 0.0f;
-      for (int i = tid; i < K; i += 256) {
-        float v = (float)xn[i];
-        acc = __builtin_fmaf(v, v, acc);
-      }
-      nbuf[tid] = acc;
-    }
-    __syncthreads();
-    if (tid < 128) nbuf[tid] += nbuf[tid + 128];
-    __syncthreads();
-    if (tid < 64) {
-      float v = nbuf[tid] + nbuf[tid + 64];
-#pragma unroll
-      for (int stride = 32; stride > 0; stride >>= 1) v += __shfl_down(v, stride, 64);
-      if (tid == 0) nbuf[0] = v;
-    }
-    __syncthreads();
-    const half_t sc = (half_t)awq_rsqrtf(nbuf[0] / (float)K + p.eps);
-    const half2_t sc2 = half2_t{sc, sc};
-#pragma unroll
-    for (int u = 0; u < MAXU; ++u) {
-      if (tid + u * 256 < K / 4) {
-        half2_t t0 = as_half2(xu[u].x) * sc2, t1 = as_half2(xu[u].y) * sc2;
-        t0 = t0 * as_half2(gu[u].x);
-        t1 = t1 * as_half2(gu[u].y);
-        xu[u].x = __builtin_bit_cast(uint32_t, t0);
-        xu[u].y = __builtin_bit_cast(uint32_t, t1);
-      }
-    }
-    __syncthreads();  // everyone is done with the natural-order copy
-  }
-#pragma unroll
-  for (int u = 0; u < MAXU; ++u)
-    if (tid + u * 256 < K / 4) *reinterpret_cast<uint2*>(xs + xs_index<G>(4 * (tid + u * 256))) = xu[u];
-  __syncthreads();
-
-  float bs[G];
-#pragma unroll
-  for (int b = 0; b < G; ++b) bs[b] = block_dot<ZINT>(w[b], xs + xs_index<G>((blk0 + b) * AWQ_BLOCK_K), g);
-#pragma unroll
-  for (int n = G; n > 1; n >>= 1) {
-#pragma unroll
-    for (int i = 0; i < n / 2; ++i) bs[i] = bs[2 * i] + bs[2 * i + 1];
-  }
-  float v = bs[0];
-  v += __shfl_xor(v, 16, 64);
-  v += __shfl_xor(v, 32, 64);
-  if (q == 0) red[wave][r] = v;
-  __syncthreads();
-  if (tid >= 16) return;
-  float tot = (red[0][r] + red[1][r]) + (red[2][r] + red[3][r]);
-  const int row = rg * 16 + r;
-  const int m = R.n_rg * 16;
-
-  // 4. slices of one row group meet in the last one
-  if (R.n_slices > 1) {
-    if (slice < R.n_slices - 1) {
-      __hip_atomic_store(R.part + (int64_t)slice * m + row, tot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      if (r == 0) __hip_atomic_fetch_add(R.rg_cnt + rg, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      return;
-    }
-    if (r == 0) flow_wait(R.rg_cnt + rg, (R.n_slices - 1) * epoch, p.err);
-    // awq_tree_sum over the slices, with compile-time indices (at most 8 slices)
-    float pv[8];
-    int n = R.n_slices;
-#pragma unroll
-    for (int sl = 0; sl < 8; ++sl) {
-      pv[sl] = 0.0f;
-      if (sl < n - 1)
-        pv[sl] = __hip_atomic_load(R.part + (int64_t)sl * m + row, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      else if (sl == n - 1)
-        pv[sl] = tot;
-    }
-#pragma unroll
-    for (int lvl = 0; lvl < 3; ++lvl) {
-      if (n > 1 && (n & 1) == 0) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) pv[i] = pv[2 * i] + pv[2 * i + 1];
-        n >>= 1;
-      }
-    }
-    tot = pv[0];
-#pragma unroll
-    for (int i = 1; i < 8; ++i)
-      if (i < n) tot += pv[i];
-  }
-
-  // outputs: through to memory, then the role's counter
-  const half_t hv = (half_t)tot;
-  if (R.epilogue == EPI_QKV_ROPE) {
-    // consumed by the next launch (attention): ordinary stores, the epilogue of gemv_kernel
-    GemvParams gp;
-    gp.epilogue = EPI_QKV_ROPE;
-    gp.y = R.y;
-    gp.cos_t = p.cos_t;
-    gp.sin_t = p.sin_t;
-    gp.k_cache = p.k_cache;
-    gp.v_cache = p.v_cache;
-    gp.hidden = p.hidden;
-    gp.pos = p.pos;
-    gp.kv = p.kv;
-    gp.dyn = p.dyn;
-    epilogue(gp, row, r, tot, (half_t)0.0f);
-  } else {
-    half_t out = hv;
-    if (R.epilogue == EPI_RESIDUAL) {
-      half_t old;
-      if (R.res_fresh)
-        old = __builtin_bit_cast(half_t, __hip_atomic_load(reinterpret_cast<const unsigned short*>(R.res) + row,
-                                                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-      else
-        old = R.res[row];
-      out = old + hv;
-    } else if (R.epilogue == EPI_GELU) {
-      out = to_half_rn(awq_gelu_f32((float)hv));
-    }
-    __hip_atomic_store(reinterpret_cast<unsigned short*>(R.y) + row, __builtin_bit_cast(unsigned short, out),
-                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  if (R.done_cnt) {
-    int last = 0;
-    if (r == 0) {
-      const int grp = rg >> 4, n_grp = (R.n_rg + 15) >> 4;
-      const int grp_size = min(16, R.n_rg - grp * 16);
-      if (__hip_atomic_fetch_add(R.done_grp + grp * 16, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1 ==
-          grp_size * epoch)
-        last = __hip_atomic_fetch_add(R.done_cnt, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1 == n_grp * epoch;
-    }
-    last = __shfl(last, 0, 64);
-    if (last) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        __hip_atomic_store(R.done_ready + (r * 4 + i) * 16, epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-  }
-}
-
 // Inference.cu:1282-1290, last step: turn the best candidate into the token id
 __global__ void sample_finish_kernel(unsigned long long* best, int32_t* out_token, const StepState* dyn,
                                      int32_t* out_array) {
@@ -937,82 +632,5 @@ int launch_gemv(const LinearArgs& a, hipStream_t st) {
     hipLaunchKernelGGL(sample_finish_kernel, dim3(1), dim3(64), 0, st, a.best, a.out_token, a.dyn, a.out_array);
     AWQ_HIP_TRY(hipGetLastError());
   }
-  return AWQ_OK;
-}
-
-// ---- several dependent products in one launch --------------------------------
-bool flow_supported(int64_t hidden, int64_t inter) {
-  return (hidden == 512 || hidden == 1024 || hidden == 2048 || hidden == 4096) && inter % hidden == 0 &&
-         inter / hidden <= 8;
-}
-
-int launch_flow(const FlowLaunch& f, hipStream_t st) {
-  AWQ_REQUIRE(f.n_roles >= 1 && f.n_roles <= kFlowRoles, "1..4 roles");
-  AWQ_REQUIRE(f.k_unit == 512 || f.k_unit == 1024 || f.k_unit == 2048 || f.k_unit == 4096, "unsupported input width");
-  AWQ_REQUIRE(f.err != nullptr && (f.dyn || f.epoch > 0), "error flag and epoch required");
-  FlowParams p;
-  int first = 0;
-  for (int i = 0; i < f.n_roles; ++i) {
-    const FlowRoleArgs& a = f.role[i];
-    AWQ_REQUIRE(a.m > 0 && a.m % 128 == 0 && a.k % f.k_unit == 0 && a.k / f.k_unit >= 1 && a.k / f.k_unit <= 8,
-                "role shape does not fit the launch");
-    AWQ_REQUIRE(awq_group_period(a.m, a.k) == 1, "matrices whose scale group depends on the input index are not supported here");
-    AWQ_REQUIRE(a.gamma == nullptr || a.k == f.k_unit, "the fused norm needs the whole input in one workgroup");
-    AWQ_REQUIRE(a.k == f.k_unit || (a.part && a.rg_cnt), "a sliced role needs room for partial sums and counters");
-    AWQ_REQUIRE(a.epilogue != EPI_ARGMAX, "no sampling epilogue here");
-    AWQ_REQUIRE(a.epilogue != EPI_RESIDUAL || a.res, "residual epilogue needs res");
-    AWQ_REQUIRE(!a.wait || a.wait_ready, "ready words of the producer missing");
-    AWQ_REQUIRE(!a.done_cnt || (a.done_ready && a.done_grp), "ready words or group counters missing");
-    FlowRole& R = p.role[i];
-    R.wq = (const u32x4*)a.wq;
-    R.scale = a.scale;
-    R.zp = a.zp;
-    R.x = a.x;
-    R.gamma = a.gamma;
-    R.y = a.y;
-    R.res = a.res;
-    R.part = a.part;
-    R.first_wg = first;
-    R.n_rg = (int32_t)(a.m / 16);
-    R.n_slices = (int32_t)(a.k / f.k_unit);
-    R.nblk_total = (int32_t)(a.k / AWQ_BLOCK_K);
-    R.mg = (int32_t)(a.m / 128);
-    R.kg = (int32_t)(a.k / 128);
-    R.epilogue = a.epilogue;
-    R.x_fresh = a.x_fresh;
-    R.res_fresh = a.res_fresh;
-    R.wait = a.wait;
-    R.wait_ready = a.wait_ready;
-    R.pre_ready = a.pre_ready;
-    R.done_grp = a.done_grp;
-    R.done_cnt = a.done_cnt;
-    R.done_ready = a.done_ready;
-    R.rg_cnt = a.rg_cnt;
-    first += R.n_rg * R.n_slices;
-  }
-  for (int i = f.n_roles; i < kFlowRoles; ++i) p.role[i] = p.role[0];
-  p.n_roles = f.n_roles;
-  p.dyn = f.dyn;
-  p.epoch_arg = f.epoch;
-  p.err = f.err;
-  p.eps = f.eps;
-  p.cos_t = f.cos_t;
-  p.sin_t = f.sin_t;
-  p.k_cache = f.k_cache;
-  p.v_cache = f.v_cache;
-  p.hidden = f.hidden;
-  p.pos = f.pos;
-  p.kv = f.kv;
-  const dim3 grid((unsigned)first), block(256);
-  void (*kern)(FlowParams);
-  const bool z = f.zp_integral != 0;
-  switch (f.k_unit / 512) {
-    case 1: kern = z ? flow_kernel<1, true> : flow_kernel<1, false>; break;
-    case 2: kern = z ? flow_kernel<2, true> : flow_kernel<2, false>; break;
-    case 4: kern = z ? flow_kernel<4, true> : flow_kernel<4, false>; break;
-    default: kern = z ? flow_kernel<8, true> : flow_kernel<8, false>; break;
-  }
-  hipLaunchKernelGGL(kern, grid, block, 0, st, p);
-  AWQ_HIP_TRY(hipGetLastError());
   return AWQ_OK;
 }

@@ -97,15 +97,6 @@ int awq_read_logits(awq_engine* e, uint16_t* host_dst);
 /* 0: every op is its own launch; 1 (default): one captured graph per step */
 int awq_set_graph_mode(awq_engine* e, int enabled);
 
-/* One launch per product (0, the default), or, where the shapes allow it (1),
- * the products of a layer that follow its attention -- Wo, W1, W2 and the next
- * layer's Wqkv (Inference.cu:1128-1227, 1040-1103) -- as dependent workgroup
- * ranges of ONE launch that hand their vectors over through memory and
- * completion counters.  Same arithmetic, bit-identical results; on MI355X the
- * hand-over costs about as much as a kernel boundary, so it is not faster
- * (572 against 598 tok/s) and stays off.  No counterpart in the reference. */
-int awq_set_flow_mode(awq_engine* e, int enabled);
-
 /* Measurement aid with no counterpart in the reference: runs the engine's own
  * fused-linear launch of `kind` (AWQ_T_WQKV/WO/W1/W2/UNEMBED) over every
  * layer's resident matrix, n_rounds times, between two HIP events on the

@@ -83,15 +83,13 @@ def test_results_do_not_depend_on_the_cache_capacity(awq, torch_gpu):
             assert np.array_equal(r[3], same[0][3]) and np.array_equal(r[4], same[0][4])
 
 
-@pytest.mark.parametrize("graph,flow", [(False, False), (True, False), (False, True), (True, True)])
-def test_small_model_tokens_and_state_identical(awq, oracle, torch_gpu, graph, flow):
-    """flow: the products after a layer's attention as dependent workgroup ranges of one launch"""
+@pytest.mark.parametrize("graph", [False, True])
+def test_small_model_tokens_and_state_identical(awq, oracle, torch_gpu, graph):
     cfg = awq.make_config(**SMALL)
     model = make_oracle_model(oracle, cfg)
     eng = awq.QWen3AWQInfer.empty(cfg)
     fill_pair(awq, oracle, cfg, 1234, engine=eng, model=model)
     eng.set_graph_mode(graph)
-    eng.set_flow_mode(flow)
     prompt = [3, 1000, 77, 512, 9]
     print("small model generate graph=", graph, flush=True)
     got = eng.generateResponse(prompt, 24)
@@ -256,8 +254,7 @@ def test_config2_one_decoder_layer_at_position_512(awq, lib, oracle, torch_gpu):
     oracle.awqo_model_destroy(model)
 
 
-@pytest.mark.parametrize("flow", [False, True])
-def test_full_model_32_greedy_tokens_identical(awq, oracle, torch_gpu, flow):
+def test_full_model_32_greedy_tokens_identical(awq, oracle, torch_gpu):
     """config 4 at reduced length: all 36 layers at the reference widths, random-init seeded weights, greedy
     decode of 32 tokens; ids, final hidden state and last logits must equal the CPU path bit for bit.
     Weights come from the balanced profile (include/awq_synth.h): with the benchmark's own distributions the
@@ -269,7 +266,6 @@ def test_full_model_32_greedy_tokens_identical(awq, oracle, torch_gpu, flow):
     model = make_oracle_model(oracle, cfg)
     eng = awq.QWen3AWQInfer.empty(cfg)
     fill_pair(awq, oracle, cfg, 2025, engine=eng, model=model, profile=awq.SYNTH_BALANCED)
-    eng.set_flow_mode(flow)
     prompt = np.zeros(4, dtype=np.int32)
     awq.check(awq.load_library().awq_synth_tokens(2025, awq.SYNTH_STREAM_INPUT, ptr(prompt), prompt.size, cfg.vocab))
     print("36-layer model: 32 greedy tokens", flush=True)
@@ -300,8 +296,7 @@ def test_full_model_benchmark_distributions_overflow_identically(awq, oracle, to
     oracle.awqo_model_destroy(model)
 
 
-@pytest.mark.parametrize("flow", [False, True])
-def test_non_integral_zero_points_take_the_general_dequantisation(awq, oracle, torch_gpu, flow):
+def test_non_integral_zero_points_take_the_general_dequantisation(awq, oracle, torch_gpu):
     """AWQ zero-points are integers, which the kernels exploit (two exact operations instead of
     three); a checkpoint with fractional zero-points must be detected at upload and still give the
     oracle's bits through the general sequence"""
@@ -315,9 +310,8 @@ def test_non_integral_zero_points_take_the_general_dequantisation(awq, oracle, t
             z += np.float16(0.25) * ((np.arange(count) % 3) + 1).astype(np.float16)
 
     fill_pair(awq, oracle, cfg, 4321, engine=eng, model=model, profile=awq.SYNTH_BALANCED, mutate=fractional)
-    eng.set_flow_mode(flow)
     prompt = [9, 100, 1000]
-    print("fractional zero-points, flow =", flow, flush=True)
+    print("fractional zero-points", flush=True)
     got = eng.generateResponse(prompt, 12)
     assert got == oracle_generate(oracle, model, prompt, 12)
     compare_state(awq, oracle, eng, model, cfg)

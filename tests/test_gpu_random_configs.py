@@ -22,23 +22,22 @@ def _cases():
         vocab = int(rng.choice([256, 1024, 128 * 37, 128 * 9])) if hidden == 512 else int(rng.choice([512, 2048]))
         n_prompt = int(rng.choice([0, 1, 2, 7, 33, 70]))
         n_new = int(rng.integers(3, 12))
-        out.append((i, hidden, inter, n_layers, vocab, n_prompt, n_new, bool(i & 1), bool(i & 2)))
+        out.append((i, hidden, inter, n_layers, vocab, n_prompt, n_new, bool(i & 1)))
     return out
 
 
-@pytest.mark.parametrize("case,hidden,inter,n_layers,vocab,n_prompt,n_new,graph,flow", _cases())
+@pytest.mark.parametrize("case,hidden,inter,n_layers,vocab,n_prompt,n_new,graph", _cases())
 def test_random_shape_matches_oracle(awq, oracle, torch_gpu, case, hidden, inter, n_layers, vocab, n_prompt, n_new,
-                                     graph, flow):
+                                     graph):
     cfg = awq.make_config(n_layers=n_layers, hidden=hidden, inter=inter, vocab=vocab, max_pos=96,
                           split_idx=max(1, n_layers // 2))
     model = make_oracle_model(oracle, cfg)
     eng = awq.QWen3AWQInfer.empty(cfg)
     fill_pair(awq, oracle, cfg, 500 + case, engine=eng, model=model, profile=awq.SYNTH_BALANCED)
     eng.set_graph_mode(graph)
-    eng.set_flow_mode(flow)
     rng = np.random.default_rng(case)
     prompt = rng.integers(0, vocab, n_prompt).astype(np.int32)
-    print("random shape", case, hidden, inter, n_layers, vocab, n_prompt, n_new, graph, flow, flush=True)
+    print("random shape", case, hidden, inter, n_layers, vocab, n_prompt, n_new, graph, flush=True)
     got = eng.generateResponse(prompt.tolist(), n_new)
     ref = np.zeros(n_new, dtype=np.int32)
     assert oracle.awqo_model_generate(model, ptr(prompt) if n_prompt else None, n_prompt, n_new, ptr(ref)) == n_new
