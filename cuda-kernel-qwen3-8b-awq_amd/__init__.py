@@ -88,6 +88,7 @@ SIGNATURES = {
     "awq_rope_kv_append": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i64, _i64, _vp]),
     "awq_attention_workspace_bytes": (_i64, [_i32, _i64]),
     "awq_decode_attention": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i32, _i64, _i64, _vp, _vp]),
+    "awq_decode_attention_static": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i32, _i64, _i64, _vp]),
     "awq_prefill_attention": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i32, _i64, _i64, _i64, _i32, _vp]),
     "awq_residual_add": (ctypes.c_int, [_vp, _vp, _vp, _i64, _vp]),
     "awq_gelu": (ctypes.c_int, [_vp, _i64, _vp]),

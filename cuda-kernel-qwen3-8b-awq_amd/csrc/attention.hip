@@ -14,6 +14,8 @@
 // keys even for short sequences.  Context: one wavefront per chunk.
 #include "common.hpp"
 
+#include <mutex>
+
 namespace {
 
 constexpr int kMaxChunks = 1024;    // 65536 positions
@@ -537,11 +539,23 @@ int64_t attention_workspace_bytes(int n_heads, int64_t max_pos) {
   return (int64_t)n_heads * (max_pos + chunks_for(max_pos) * (AWQ_HEAD_DIM + 1) + kSplit) * 4;
 }
 
+// ws_pos: the number of positions the workspace is laid out for (the cache's own
+// max_pos for a workspace of attention_workspace_bytes(n_heads, max_pos))
+static int launch_attention_ws(const half_t* q, const half_t* kc, const half_t* vc, half_t* ctx, int n_heads,
+                               int64_t max_pos, KvLayout kv, int64_t L, const StepState* dyn, int use_len_hi,
+                               int64_t len_bound, void* ws, int64_t ws_pos, hipStream_t st);
+
 int launch_attention(const half_t* q, const half_t* kc, const half_t* vc, half_t* ctx, int n_heads, int64_t max_pos,
                      KvLayout kv, int64_t L, const StepState* dyn, int use_len_hi, int64_t len_bound, void* ws,
                      hipStream_t st) {
+  return launch_attention_ws(q, kc, vc, ctx, n_heads, max_pos, kv, L, dyn, use_len_hi, len_bound, ws, max_pos, st);
+}
+
+static int launch_attention_ws(const half_t* q, const half_t* kc, const half_t* vc, half_t* ctx, int n_heads,
+                               int64_t cache_pos, KvLayout kv, int64_t L, const StepState* dyn, int use_len_hi,
+                               int64_t len_bound, void* ws, int64_t max_pos, hipStream_t st) {
   AWQ_REQUIRE(n_heads > 0 && max_pos > 0 && max_pos <= (int64_t)kMaxChunks * 64, "max_pos must be in 1..65536");
-  AWQ_REQUIRE(dyn || (L >= 1 && L <= max_pos), "attended length out of range");
+  AWQ_REQUIRE(dyn || (L >= 1 && L <= max_pos && L <= cache_pos), "attended length out of range");
   AWQ_REQUIRE(ws != nullptr, "workspace required");
   float* scores = (float*)ws;
   float* cv = scores + (int64_t)n_heads * max_pos;
@@ -593,4 +607,47 @@ int launch_attention(const half_t* q, const half_t* kc, const half_t* vc, half_t
                      st, q, kc, vc, ctx, kv, (int)L, dyn, use_len_hi, max_pos, (const float*)nullptr, (const float*)nullptr);
   AWQ_HIP_TRY(hipGetLastError());
   return AWQ_OK;
+}
+
+// ---------------------------------------------------------------------------
+// The same attention for callers that cannot allocate (code under stream
+// capture, serving loops, harnesses that forbid hipMalloc): scores, part
+// maxima, chunk sums and chunk vectors live in a file-scope device array of
+// fixed size instead of a caller-provided workspace.  Each device holds its own
+// copy of the array at its own address, looked up once per device with
+// hipGetSymbolAddress; every call on a device shares it, so calls that may
+// overlap on one device race.  The kernels write every word before they read
+// it, so nothing needs clearing between calls.
+// ---------------------------------------------------------------------------
+constexpr int kStaticHeads = 32;
+constexpr int64_t kStaticPos = 8192;
+constexpr int64_t kStaticBytes =
+    (int64_t)kStaticHeads * (kStaticPos + (kStaticPos / 64) * (AWQ_HEAD_DIM + 1) + kSplit) * 4;  // 3,166,208 B
+static __device__ __align__(256) unsigned char scratch[kStaticBytes];
+
+static std::mutex g_scratch_mutex;
+static void* g_scratch_ptr[64];  // per device; null until its first call
+
+int launch_attention_static(const half_t* q, const half_t* kc, const half_t* vc, half_t* ctx, int n_heads,
+                            int64_t max_pos, int64_t L, hipStream_t st) {
+  AWQ_REQUIRE(n_heads >= 1 && n_heads <= kStaticHeads, "at most 32 heads fit the built-in scratch array");
+  AWQ_REQUIRE(L >= 1 && L <= kStaticPos, "at most 8192 attended positions fit the built-in scratch array");
+  AWQ_REQUIRE(max_pos >= L, "attended length exceeds the cache");
+  int dev = 0;
+  AWQ_HIP_TRY(hipGetDevice(&dev));
+  AWQ_REQUIRE(dev >= 0 && dev < 64, "device index out of range");
+  void* ws = nullptr;
+  {
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+      void* p = nullptr;
+      AWQ_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+      g_scratch_ptr[dev] = p;
+    }
+    ws = g_scratch_ptr[dev];
+  }
+  static_assert(kStaticBytes == (int64_t)kStaticHeads * (kStaticPos + ((kStaticPos + 63) / 64) * (AWQ_HEAD_DIM + 1) + kSplit) * 4,
+                "the array is attention_workspace_bytes(32, 8192)");
+  // the workspace is laid out for n_heads x kStaticPos positions whatever the cache's capacity
+  return launch_attention_ws(q, kc, vc, ctx, n_heads, max_pos, kv_head_major(max_pos), L, nullptr, 0, 0, ws, kStaticPos, st);
 }

@@ -167,6 +167,8 @@ int64_t attention_workspace_bytes(int n_heads, int64_t max_pos);
 int launch_attention(const half_t* q, const half_t* kc, const half_t* vc, half_t* ctx, int n_heads, int64_t max_pos,
                      KvLayout kv, int64_t L, const StepState* dyn, int use_len_hi, int64_t len_bound, void* ws,
                      hipStream_t st);
+int launch_attention_static(const half_t* q, const half_t* kc, const half_t* vc, half_t* ctx, int n_heads,
+                            int64_t max_pos, int64_t L, hipStream_t st);
 int launch_prefill_attention(const half_t* q, const half_t* kc, const half_t* vc, half_t* ctx, int n_heads,
                              int64_t max_pos, KvLayout kv, int64_t pos0, int64_t M, int use_len_hi, hipStream_t st);
 int launch_embed_batch(const uint8_t* packed, const half_t* scale, const half_t* zp, int64_t hidden, int64_t vocab,

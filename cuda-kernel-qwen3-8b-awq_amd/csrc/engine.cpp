@@ -988,6 +988,13 @@ extern "C" int awq_decode_attention(const void* q, const void* k_cache, const vo
                           max_pos, kv_head_major(max_pos), L, nullptr, 0, 0, workspace, (hipStream_t)stream);
 }
 
+extern "C" int awq_decode_attention_static(const void* q, const void* k_cache, const void* v_cache, void* ctx,
+                                           int32_t n_heads, int64_t max_pos, int64_t L, void* stream) {
+  AWQ_REQUIRE(q && k_cache && v_cache && ctx, "NULL pointer");
+  return launch_attention_static((const half_t*)q, (const half_t*)k_cache, (const half_t*)v_cache, (half_t*)ctx, n_heads,
+                                 max_pos, L, (hipStream_t)stream);
+}
+
 extern "C" int awq_prefill_attention(const void* q, const void* k_cache, const void* v_cache, void* ctx,
                                      int32_t n_heads, int64_t max_pos, int64_t pos0, int64_t n_tokens,
                                      int32_t first_layer, void* stream) {

@@ -246,6 +246,20 @@ int64_t awq_attention_workspace_bytes(int32_t n_heads, int64_t max_pos);
 int awq_decode_attention(const void* q, const void* k_cache, const void* v_cache, void* ctx, int32_t n_heads,
                          int64_t max_pos, int64_t L, void* workspace, void* stream);
 
+/* awq_decode_attention without a workspace argument and without any allocation.
+ * No counterpart in the reference: it is for callers that cannot allocate device
+ * memory (code under HIP stream capture, tight serving loops, harnesses that
+ * forbid hipMalloc).  The scores and partial sums live in a 3,166,208-byte device
+ * array inside the library, one copy per GPU, held until the process ends.
+ * Limits: n_heads <= 32 and L <= 8192 (max_pos, the cache's row capacity, may be
+ * larger); anything beyond is refused with AWQ_ERR_ARG.  Same kernels and same
+ * bits as awq_decode_attention.  All calls on one GPU share the array: calls
+ * that may overlap there (different streams, different threads) race.  The
+ * first call on a GPU looks the array's address up; make it outside stream
+ * capture. */
+int awq_decode_attention_static(const void* q, const void* k_cache, const void* v_cache, void* ctx, int32_t n_heads,
+                                int64_t max_pos, int64_t L, void* stream);
+
 /* The same attention for n_tokens consecutive prompt positions pos0 ..
  * pos0 + n_tokens - 1 at once (their keys and values already appended): q and
  * ctx are [n_tokens][n_heads*128].  The token at position p attends p + 1
