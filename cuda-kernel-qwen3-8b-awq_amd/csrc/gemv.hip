@@ -78,84 +78,60 @@ __global__ __launch_bounds__(256) void repack_kernel(const uint8_t* __restrict__
 
 // ---------------------------------------------------------------------------
 // fused dequant + matrix-vector product
+//
+// Arithmetic (awq_canon_math.h): per block of 32 inputs T = A + B, two fma
+// chains over the raw nibbles, then (T - z X) s with X the block's input sum.
+// A masked dword (v & 0x000f000f) is a pair of binary16 subnormals q * 2^-24,
+// (v & 0x00f000f0) a pair q * 2^-20; v_fma_mix_f32 widens them exactly, so a
+// weight costs one multiply-add and an eighth of (one shift + four ANDs): 13
+// instructions per 8 weights.  The powers of two are carried by the group
+// constants: chain A runs at 2^-24, chain B at 2^-20, T' = fma(A, 16, B) is
+// T * 2^-20 (exactly the rounding of A + B), and
+//     fma(-z * 2^-20, X, T') * (s * 2^20)  ==  fma(-z, X, T) * s   bit for bit
+// (every intermediate is a multiple of 2^-68 and far from the binary32
+// exponent limits, so the scalings commute with the roundings).
 // ---------------------------------------------------------------------------
 struct GroupConst {
-  half2_t s2;  // (s, s)
-  half2_t a2;  // integral zp: -(1024+z) twice; otherwise -z twice
-  half2_t b2;  // integral zp: -(64+z) twice; unused otherwise
+  float s;   // scale * 2^20
+  float zn;  // -zero_point * 2^-20
 };
 
-template <bool ZINT>
 __device__ __forceinline__ GroupConst make_group(half_t s, half_t z) {
-  GroupConst g;
-  g.s2 = half2_t{s, s};
-  if (ZINT) {
-    half_t a = -((half_t)1024.0f + z);  // exact: z is an integer in [0,1024]
-    half_t b = -((half_t)64.0f + z);
-    g.a2 = half2_t{a, a};
-    g.b2 = half2_t{b, b};
-  } else {
-    g.a2 = half2_t{-z, -z};
-    g.b2 = g.a2;
-  }
-  return g;
+  return GroupConst{(float)s * 1048576.0f, -(float)z * (1.0f / 1048576.0f)};
 }
 
-// (x & mask) | 0x64006400 in one instruction.  gfx950's three-operand encoding
-// takes no literal, so the mask travels in a scalar register and the exponent
-// pattern in a vector register.
-__device__ __forceinline__ uint32_t and_or_magic(uint32_t x, uint32_t mask) {
-  uint32_t r;
-  const uint32_t magic = 0x64006400u;
-  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "s"(mask), "v"(magic));
-  return r;
-}
-
-// two weights from the pair 1024+q (LOW) or 1024+16q (!LOW):
-//   h( h(q - z) * s )  exactly as Inference.cu:102-104 rounds it
-template <bool ZINT, bool LOW>
-__device__ __forceinline__ half2_t dq_pair(uint32_t word, const GroupConst& g) {
-  half2_t v = as_half2(and_or_magic(word, LOW ? 0x000f000fu : 0x00f000f0u));
-  const half2_t k16 = half2_t{(half_t)0.0625f, (half_t)0.0625f};
-  half2_t u;
-  if (ZINT) {
-    // (1024+q) - (1024+z) and (1024+16q)/16 - (64+z) are both q - z with no rounding
-    u = LOW ? (v + g.a2) : __builtin_elementwise_fma(v, k16, g.b2);
-  } else {
-    const half2_t m1024 = half2_t{(half_t)-1024.0f, (half_t)-1024.0f};
-    const half2_t m64 = half2_t{(half_t)-64.0f, (half_t)-64.0f};
-    half2_t q = LOW ? (v + m1024) : __builtin_elementwise_fma(v, k16, m64);  // q exactly
-    u = q + g.a2;                                                            // h(q - z)
-  }
-  return u * g.s2;
-}
-
-// one block: 32 weights of this lane's row against 32 inputs in LDS, a
-// sequential fma chain that starts from 0
-template <bool ZINT>
-__device__ __forceinline__ float block_dot(const u32x4& w, const half_t* xs, const GroupConst& g) {
+// T * 2^-20 of one block: 32 weights of this lane's row against 32 inputs in LDS
+__device__ __forceinline__ float block_dot(const u32x4& w, const half_t* xs) {
   const uint32_t d[4] = {w.x, w.y, w.z, w.w};
-  float acc = 0.0f;
+  float acc_a = 0.0f, acc_b = 0.0f;
 #pragma unroll
   for (int c = 0; c < 4; ++c) {
     const uint4 xv = *reinterpret_cast<const uint4*>(xs + 8 * c);
     const half2_t x0 = as_half2(xv.x), x1 = as_half2(xv.y), x2 = as_half2(xv.z), x3 = as_half2(xv.w);
     const uint32_t v = d[c], v8 = v >> 8;
-    const half2_t wa = dq_pair<ZINT, true>(v, g);
-    const half2_t wb = dq_pair<ZINT, false>(v, g);
-    const half2_t wc = dq_pair<ZINT, true>(v8, g);
-    const half2_t wd = dq_pair<ZINT, false>(v8, g);
-    acc = __builtin_fmaf((float)wa.x, (float)x0.x, acc);
-    acc = __builtin_fmaf((float)wa.y, (float)x0.y, acc);
-    acc = __builtin_fmaf((float)wb.x, (float)x1.x, acc);
-    acc = __builtin_fmaf((float)wb.y, (float)x1.y, acc);
-    acc = __builtin_fmaf((float)wc.x, (float)x2.x, acc);
-    acc = __builtin_fmaf((float)wc.y, (float)x2.y, acc);
-    acc = __builtin_fmaf((float)wd.x, (float)x3.x, acc);
-    acc = __builtin_fmaf((float)wd.y, (float)x3.y, acc);
+    const half2_t wa = as_half2(v & 0x000f000fu), wb = as_half2(v & 0x00f000f0u);
+    const half2_t wc = as_half2(v8 & 0x000f000fu), wd = as_half2(v8 & 0x00f000f0u);
+    acc_a = __builtin_fmaf((float)wa.x, (float)x0.x, acc_a);
+    acc_a = __builtin_fmaf((float)wa.y, (float)x0.y, acc_a);
+    acc_b = __builtin_fmaf((float)wb.x, (float)x1.x, acc_b);
+    acc_b = __builtin_fmaf((float)wb.y, (float)x1.y, acc_b);
+    acc_a = __builtin_fmaf((float)wc.x, (float)x2.x, acc_a);
+    acc_a = __builtin_fmaf((float)wc.y, (float)x2.y, acc_a);
+    acc_b = __builtin_fmaf((float)wd.x, (float)x3.x, acc_b);
+    acc_b = __builtin_fmaf((float)wd.y, (float)x3.y, acc_b);
   }
-  return acc;
+  return __builtin_fmaf(acc_a, 16.0f, acc_b);
 }
+
+// value of another lane of the same row of 16 (DPP: no LDS round trip)
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+constexpr int kDppXor1 = 0xB1;        // quad_perm:[1,0,3,2]
+constexpr int kDppXor2 = 0x4E;        // quad_perm:[2,3,0,1]
+constexpr int kDppHalfMirror = 0x141; // lane i <-> 7 - i within 8
+constexpr int kDppRor4 = 0x124, kDppRor8 = 0x128;
 
 struct GemvParams {
   const u32x4* wq;
@@ -260,28 +236,35 @@ __device__ __forceinline__ int xs_index(int e) {
 
 // A workgroup takes row groups blockIdx.x, blockIdx.x + gridDim.x, ... (16
 // output rows x all of k each).  n_waves wavefronts; lane (w, q, r) owns blocks
-// (4w+q)*G .. +G-1 of row 16*rg + r.  x is staged (and normalised) once per
-// workgroup; the weights of the next row group are in flight while the current
-// one is multiplied.
+// (4w+q)*G .. +G-1 of row 16*rg + r.  x is staged (normalised, with the input
+// sum of every block beside it) once per workgroup; the weights of the next row
+// group are in flight while the current one is multiplied.
 // The arguments every wavefront needs before its first load come first and
 // one by one: the first 16 dwords of the argument block are preloaded into
 // scalar registers at wavefront launch (see the build flags), which takes one
 // memory round trip off the start of the kernel.
+// k = n_waves * 128 * G, so a thread stages exactly G/2 units of four inputs.
 // UFAST (periodic matrices only): the class length k/32/C when it is known at
 // compile time and divides G, so that a lane's G blocks are G/UFAST whole classes
 // whose constants it reads once per row group; 0 = look the class up per block.
-template <int G, bool ZINT, bool PERIODIC, int UFAST = 0>
+//
+// Dynamic LDS: x in block order (skewed) | block sums, k/32 floats | with the
+// fused norm, x in natural order (k halves).
+template <int G, bool PERIODIC, int UFAST = 0>
 __global__ __launch_bounds__(1024) void gemv_kernel(const u32x4* __restrict__ wq, const half_t* __restrict__ x,
                                                     const half_t* __restrict__ gamma, const half_t* __restrict__ scale,
                                                     const half_t* __restrict__ zp, int32_t k, int32_t nblk,
                                                     int32_t n_waves, int32_t m, int32_t prologue, int32_t C,
                                                     GemvParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  half_t* xs = reinterpret_cast<half_t*>(smem);  // x in block order, k halves
+  half_t* xs = reinterpret_cast<half_t*>(smem);                                  // k halves + skew
+  float* xsum = reinterpret_cast<float*>(smem + (size_t)(k + (nblk / G) * 8) * 2);  // nblk floats
+  half_t* xn = reinterpret_cast<half_t*>(xsum + nblk);                           // k halves (fused norm only)
   __shared__ float red[2][16][16];  // double-buffered: one barrier per row group
-  __shared__ float nbuf[256];
+  __shared__ __attribute__((aligned(16))) float part[256];
   __shared__ GroupConst gtab[2][PERIODIC ? 64 : 1];
-  constexpr int MAXU = 8;  // 8-byte units of x a thread may hold in registers
+  constexpr int MAXU = G / 2;  // units of four inputs a thread stages
+  static_assert(G >= 2, "a thread stages whole units");
 
   const int tid = threadIdx.x;
   const int nthreads = n_waves * 64;
@@ -296,108 +279,126 @@ __global__ __launch_bounds__(1024) void gemv_kernel(const u32x4* __restrict__ wq
   const u32x4* wp = wq + ((int64_t)rg * nblk + blk0) * 16 + r;
   u32x4 w[G], wn[G];
 
-  // ---- x into LDS in block order ------------------------------------------
-  // Unit u of a thread is the 4 consecutive block-order elements 4*(tid + u*nthreads)..+3;
-  // in natural order they are 4 consecutive indices too unless the matrix is
-  // periodic (then they are C apart and are gathered one by one).
-  const int total_units = k >> 2;  // at most MAXU * nthreads (checked by the launcher)
+  // ---- x: unit u of a thread is the 4 consecutive block-order elements
+  // 4*(tid + u*nthreads)..+3; in natural order they are 4 consecutive indices too
+  // unless the matrix is periodic (then they are C apart and are gathered one by one)
   const bool norm = prologue == PRO_RMSNORM;
   uint2 xu[MAXU], gu[MAXU];
 #pragma unroll
   for (int u = 0; u < MAXU; ++u) {
-    if (tid + u * nthreads < total_units) {
-      const int e = 4 * (tid + u * nthreads);
-      if (PERIODIC) {
-        half_t hx[4], hg[4];
+    const int unit = tid + u * nthreads;
+    if (PERIODIC) {
+      half_t hx[4], hg[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int j = (int)awq_block_elem(k, C, (e + i) >> 5, (e + i) & 31);
-          hx[i] = x[j];
-          hg[i] = norm ? gamma[j] : (half_t)0.0f;
-        }
-        xu[u] = __builtin_bit_cast(uint2, *reinterpret_cast<uint64_t*>(hx));
-        gu[u] = __builtin_bit_cast(uint2, *reinterpret_cast<uint64_t*>(hg));
-      } else {
-        xu[u] = reinterpret_cast<const uint2*>(x)[tid + u * nthreads];
-        if (norm) gu[u] = reinterpret_cast<const uint2*>(gamma)[tid + u * nthreads];
+      for (int i = 0; i < 4; ++i) {
+        const int j = (int)awq_block_elem(k, C, (4 * unit + i) >> 5, (4 * unit + i) & 31);
+        hx[i] = x[j];
+        hg[i] = norm ? gamma[j] : (half_t)0.0f;
       }
+      xu[u] = __builtin_bit_cast(uint2, *reinterpret_cast<uint64_t*>(hx));
+      gu[u] = __builtin_bit_cast(uint2, *reinterpret_cast<uint64_t*>(hg));
+    } else {
+      xu[u] = reinterpret_cast<const uint2*>(x)[unit];
+      if (norm) gu[u] = reinterpret_cast<const uint2*>(gamma)[unit];
     }
   }
-  // x first, and almost alone: once every wavefront of the device has its 8 KiB of
-  // weight loads in flight, a small load of x (an L2 hit) waits microseconds in
-  // the same queues.  So only the first weight block is requested along with x
-  // (it brings the stream's first round trip forward: +2.8 % tokens/s over none;
-  // two blocks +2.4 %, four +0.6 %) and the rest starts when x has arrived.
-  w[0] = __builtin_nontemporal_load(wp);
-  asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
+  // Every request for x of this workgroup goes out before any of its requests
+  // for weights: the memory pipeline of a compute unit serves requests in order,
+  // and a small load of x that queues behind kilobytes of weight loads arrives
+  // microseconds late (measured: 7.9 -> 7.45 us per launch at 12288 x 4096).
+  __syncthreads();
 #pragma unroll
-  for (int b = 1; b < G; ++b) w[b] = __builtin_nontemporal_load(wp + b * 16);
+  for (int b = 0; b < G; ++b) w[b] = __builtin_nontemporal_load(wp + b * 16);
   if (norm) {
     // rmsNormKernel, Inference.cu:111-145: 256 strided fma partial sums over the
-    // natural order, the stride-halving tree, then two binary16 multiplies.
-    // The raw values go through LDS in natural order (unskewed, in the same
-    // buffer; it is overwritten afterwards) for the partial sums.
-    half_t* xn = xs;
+    // natural order, the stride-halving tree, then two binary16 multiplies
 #pragma unroll
     for (int u = 0; u < MAXU; ++u) {
-      if (tid + u * nthreads < total_units) {
-        const int e = 4 * (tid + u * nthreads);
-        if (PERIODIC) {
-          half_t hx[4];
-          *reinterpret_cast<uint64_t*>(hx) = __builtin_bit_cast(uint64_t, xu[u]);
+      const int unit = tid + u * nthreads;
+      if (PERIODIC) {
+        half_t hx[4];
+        *reinterpret_cast<uint64_t*>(hx) = __builtin_bit_cast(uint64_t, xu[u]);
 #pragma unroll
-          for (int i = 0; i < 4; ++i) xn[awq_block_elem(k, C, (e + i) >> 5, (e + i) & 31)] = hx[i];
-        } else {
-          reinterpret_cast<uint2*>(xn)[tid + u * nthreads] = xu[u];
-        }
+        for (int i = 0; i < 4; ++i) xn[awq_block_elem(k, C, (4 * unit + i) >> 5, (4 * unit + i) & 31)] = hx[i];
+      } else {
+        reinterpret_cast<uint2*>(xn)[unit] = xu[u];
       }
     }
     __syncthreads();
-    if (tid < 256) {
+    for (int pi = tid; pi < 256; pi += nthreads) {
       float acc = 0.0f;
-      for (int i = tid; i < k; i += 256) {
-        float v = (float)xn[i];
+      for (int i = pi; i < k; i += 256) {
+        const float v = (float)xn[i];
         acc = __builtin_fmaf(v, v, acc);
       }
-      nbuf[tid] = acc;
+      part[pi] = acc;
     }
     __syncthreads();
-    if (tid < 128) nbuf[tid] += nbuf[tid + 128];
-    __syncthreads();
-    if (tid < 64) {
-      float v = nbuf[tid] + nbuf[tid + 64];
+    // the tree of Inference.cu:130-135, by every wavefront for itself: lane t of a
+    // row of 16 takes part[t + 16 j]; strides 128..16 are then additions in its own
+    // registers and strides 8..1 exchanges within the row (a + b == b + a, so
+    // the butterfly leaves in lane 0 what the one-sided tree leaves in part[0])
+    float pv[16];
 #pragma unroll
-      for (int stride = 32; stride > 0; stride >>= 1) v += __shfl_down(v, stride, 64);
-      if (tid == 0) nbuf[0] = v;
+    for (int j = 0; j < 16; ++j) pv[j] = part[r + 16 * j];
+#pragma unroll
+    for (int n = 8; n >= 1; n >>= 1) {
+#pragma unroll
+      for (int j = 0; j < n; ++j) pv[j] += pv[j + n];
     }
-    __syncthreads();
-    const half_t sc = (half_t)awq_rsqrtf(nbuf[0] / (float)k + p.eps);
+    float tot = pv[0];
+    tot += dpp_f<kDppRor8>(tot);
+    tot += dpp_f<kDppRor4>(tot);
+    tot += dpp_f<kDppXor2>(tot);
+    tot += dpp_f<kDppXor1>(tot);
+    tot = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, tot)));
+    const half_t sc = (half_t)awq_rsqrtf(tot / (float)k + p.eps);
     const half2_t sc2 = half2_t{sc, sc};
 #pragma unroll
     for (int u = 0; u < MAXU; ++u) {
-      if (tid + u * nthreads < total_units) {
-        half2_t t0 = as_half2(xu[u].x) * sc2, t1 = as_half2(xu[u].y) * sc2;
-        t0 = t0 * as_half2(gu[u].x);
-        t1 = t1 * as_half2(gu[u].y);
-        xu[u].x = __builtin_bit_cast(uint32_t, t0);
-        xu[u].y = __builtin_bit_cast(uint32_t, t1);
-      }
+      half2_t t0 = as_half2(xu[u].x) * sc2, t1 = as_half2(xu[u].y) * sc2;
+      t0 = t0 * as_half2(gu[u].x);
+      t1 = t1 * as_half2(gu[u].y);
+      xu[u].x = __builtin_bit_cast(uint32_t, t0);
+      xu[u].y = __builtin_bit_cast(uint32_t, t1);
     }
   }
-  if (norm) __syncthreads();  // everyone is done with the natural-order copy
+  // x and the input sum of every block (adjacent-pair tree over its 32 inputs:
+  // four in this thread, then the eight threads that share the block)
 #pragma unroll
-  for (int u = 0; u < MAXU; ++u)
-    if (tid + u * nthreads < total_units)
-      *reinterpret_cast<uint2*>(xs + xs_index<G>(4 * (tid + u * nthreads))) = xu[u];
+  for (int u = 0; u < MAXU; ++u) {
+    const int unit = tid + u * nthreads;
+    *reinterpret_cast<uint2*>(xs + xs_index<G>(4 * unit)) = xu[u];
+    const half2_t t0 = as_half2(xu[u].x), t1 = as_half2(xu[u].y);
+    float sx = ((float)t0.x + (float)t0.y) + ((float)t1.x + (float)t1.y);
+    sx += dpp_f<kDppXor1>(sx);
+    sx += dpp_f<kDppXor2>(sx);
+    sx += dpp_f<kDppHalfMirror>(sx);
+    if ((tid & 7) == 0) xsum[unit >> 3] = sx;
+  }
 
   // Group constants.  When the scale group depends on the input index it is
   // constant within a class of blocks; the (at most 64) classes of a row group
   // go through a table in LDS, filled one row group ahead.
   if (PERIODIC && tid < C && rg < n_rg) {
     int gi = (int)((((int64_t)tid * p.mg + (rg >> 3)) % p.kg) % p.mg);
-    gtab[0][tid] = make_group<ZINT>(scale[gi], zp[gi]);
+    gtab[0][tid] = make_group(scale[gi], zp[gi]);
   }
-  __syncthreads();  // xs and the first table
+  __syncthreads();  // xs, the block sums and the first table
+  float xb[G];
+  if (G >= 4) {
+#pragma unroll
+    for (int b = 0; b < G; b += 4) {
+      const float4 t = *reinterpret_cast<const float4*>(xsum + blk0 + b);
+      xb[b] = t.x;
+      xb[b + 1] = t.y;
+      xb[b + 2] = t.z;
+      xb[b + 3] = t.w;
+    }
+  } else {
+#pragma unroll
+    for (int b = 0; b < G; ++b) xb[b] = xsum[blk0 + b];
+  }
   for (int it = 0; rg < n_rg; rg += gridDim.x, ++it) {
     const int rg_next = rg + gridDim.x;
     if (rg_next < n_rg) {
@@ -415,11 +416,11 @@ __global__ __launch_bounds__(1024) void gemv_kernel(const u32x4* __restrict__ wq
     GroupConst g;
     if (!PERIODIC) {
       int gi = (a % p.kg) % p.mg;
-      g = make_group<ZINT>(scale[gi], zp[gi]);
+      g = make_group(scale[gi], zp[gi]);
     } else if (tid < C && rg_next < n_rg) {
       // the next row group's table; its buffer was last read two barriers ago
       int gi = (int)((((int64_t)tid * p.mg + (rg_next >> 3)) % p.kg) % p.mg);
-      gtab[(it + 1) & 1][tid] = make_group<ZINT>(scale[gi], zp[gi]);
+      gtab[(it + 1) & 1][tid] = make_group(scale[gi], zp[gi]);
     }
     int cls = 0, cls_left = 0;  // class of the next block and blocks left in it
     if (PERIODIC) {
@@ -433,8 +434,10 @@ __global__ __launch_bounds__(1024) void gemv_kernel(const u32x4* __restrict__ wq
 #pragma unroll
       for (int c = 0; c < NC; ++c) gc[c] = gtab[it & 1][blk0 / UFAST + c];
 #pragma unroll
-      for (int b = 0; b < G; ++b)
-        bs[b] = block_dot<ZINT>(w[b], xs + xs_index<G>((blk0 + b) * AWQ_BLOCK_K), gc[UFAST > 0 ? b / UFAST : 0]);
+      for (int b = 0; b < G; ++b) {
+        const GroupConst& gb = gc[UFAST > 0 ? b / UFAST : 0];
+        bs[b] = __builtin_fmaf(gb.zn, xb[b], block_dot(w[b], xs + xs_index<G>((blk0 + b) * AWQ_BLOCK_K))) * gb.s;
+      }
     } else {
 #pragma unroll
       for (int b = 0; b < G; ++b) {
@@ -445,7 +448,7 @@ __global__ __launch_bounds__(1024) void gemv_kernel(const u32x4* __restrict__ wq
             cls_left = U;
           }
         }
-        bs[b] = block_dot<ZINT>(w[b], xs + xs_index<G>((blk0 + b) * AWQ_BLOCK_K), g);
+        bs[b] = __builtin_fmaf(g.zn, xb[b], block_dot(w[b], xs + xs_index<G>((blk0 + b) * AWQ_BLOCK_K))) * g.s;
       }
     }
     // adjacent-pair tree: this lane's G blocks, then the four quarters of the
@@ -497,17 +500,16 @@ struct GemvPlan {
 
 // Lane groups per workgroup = (k/32)/G must be a multiple of 4 and at most 64.
 // Prefer long per-lane runs (G = 8) unless that leaves the device with few
-// wavefronts.
+// wavefronts.  G >= 2: a thread stages whole units of four inputs.
 bool plan_gemv(int64_t m, int64_t k, GemvPlan* out) {
   const int64_t nblk = k / AWQ_BLOCK_K;
   bool found = false;
-  for (int g = 8; g >= 1; g >>= 1) {
+  for (int g = 8; g >= 2; g >>= 1) {
     if (nblk % g) continue;
     int64_t groups = nblk / g;
     if (groups % 4 || groups > 64) continue;
     *out = GemvPlan{g, (int)(groups / 4)};
     found = true;
-    // at least 4 wavefronts: the fused norm sums with 256 threads
     if (groups / 4 >= 4 && (m / 16) * (groups / 4) >= 2048) break;
   }
   return found;
@@ -515,19 +517,13 @@ bool plan_gemv(int64_t m, int64_t k, GemvPlan* out) {
 
 #define GEMV_HOT_ARGS p.wq, p.x, p.gamma, p.scale, p.zp, p.k, p.nblk, p.n_waves, p.m, p.prologue, p.C
 template <int G>
-void launch_g(const GemvParams& p, bool zint, bool periodic, dim3 grid, dim3 block, size_t lds, hipStream_t st) {
+void launch_g(const GemvParams& p, bool periodic, dim3 grid, dim3 block, size_t lds, hipStream_t st) {
   if (G == 8 && periodic && p.nblk / p.C == 4) {  // the unembedding: classes of 4 blocks
-    if (zint) hipLaunchKernelGGL((gemv_kernel<G, true, true, G == 8 ? 4 : 0>), grid, block, lds, st, GEMV_HOT_ARGS, p);
-    else hipLaunchKernelGGL((gemv_kernel<G, false, true, G == 8 ? 4 : 0>), grid, block, lds, st, GEMV_HOT_ARGS, p);
+    hipLaunchKernelGGL((gemv_kernel<G, true, G == 8 ? 4 : 0>), grid, block, lds, st, GEMV_HOT_ARGS, p);
     return;
   }
-  if (zint) {
-    if (periodic) hipLaunchKernelGGL((gemv_kernel<G, true, true>), grid, block, lds, st, GEMV_HOT_ARGS, p);
-    else hipLaunchKernelGGL((gemv_kernel<G, true, false>), grid, block, lds, st, GEMV_HOT_ARGS, p);
-  } else {
-    if (periodic) hipLaunchKernelGGL((gemv_kernel<G, false, true>), grid, block, lds, st, GEMV_HOT_ARGS, p);
-    else hipLaunchKernelGGL((gemv_kernel<G, false, false>), grid, block, lds, st, GEMV_HOT_ARGS, p);
-  }
+  if (periodic) hipLaunchKernelGGL((gemv_kernel<G, true>), grid, block, lds, st, GEMV_HOT_ARGS, p);
+  else hipLaunchKernelGGL((gemv_kernel<G, false>), grid, block, lds, st, GEMV_HOT_ARGS, p);
 }
 
 }  // namespace
@@ -548,7 +544,7 @@ int launch_dequant(const uint8_t* packed, const half_t* scale, const half_t* zp,
 static int check_linear_shape(int64_t m, int64_t k) {
   AWQ_REQUIRE(m > 0 && k > 0 && m % 128 == 0, "m must be a positive multiple of 128");
   AWQ_REQUIRE(k % 512 == 0, "k must be a positive multiple of 512");
-  AWQ_REQUIRE(m < (1ll << 31) && k <= 24576, "shape too large (k is limited to 24576 by the LDS copy of x)");
+  AWQ_REQUIRE(m < (1ll << 31) && k <= 16384, "shape too large (k is limited to 16384: 64 lane groups of 8 blocks per workgroup)");
   int C = awq_group_period(m, k);
   AWQ_REQUIRE((k / AWQ_BLOCK_K) % C == 0, "k/32 must be a multiple of the scale-group period");
   AWQ_REQUIRE(C <= 64, "scale-group period above 64 is not supported");
@@ -614,18 +610,19 @@ int launch_gemv(const LinearArgs& a, hipStream_t st) {
   p.dyn = a.dyn;
   p.best = a.best;
   const bool periodic = p.C > 1;
-  AWQ_REQUIRE(a.k / 4 <= 8 * plan.n_waves * 64, "k too large for this workgroup size");
   // one workgroup per row group while that fits the device a few times over;
   // beyond that a workgroup walks several row groups and stages x once
   int64_t n_rg = a.m / 16, n_wg = n_rg;
   if (n_rg > 1024) n_wg = 1024;
   dim3 grid((unsigned)n_wg), block((unsigned)(plan.n_waves * 64));
-  size_t lds = (size_t)a.k * 2 + (size_t)(a.k / AWQ_BLOCK_K / plan.g) * 16;  // x plus 16 bytes of skew per lane group
+  // x in block order plus 16 bytes of skew per lane group, the block sums, and with the fused norm x in natural order
+  size_t lds = (size_t)a.k * 2 + (size_t)(a.k / AWQ_BLOCK_K / plan.g) * 16 + (size_t)(a.k / AWQ_BLOCK_K) * 4 +
+               (a.prologue == PRO_RMSNORM ? (size_t)a.k * 2 : 0);
+  AWQ_REQUIRE(lds <= 65536, "k too large for the fused norm (x is kept twice in LDS)");
   switch (plan.g) {
-    case 1: launch_g<1>(p, a.zp_integral, periodic, grid, block, lds, st); break;
-    case 2: launch_g<2>(p, a.zp_integral, periodic, grid, block, lds, st); break;
-    case 4: launch_g<4>(p, a.zp_integral, periodic, grid, block, lds, st); break;
-    default: launch_g<8>(p, a.zp_integral, periodic, grid, block, lds, st); break;
+    case 2: launch_g<2>(p, periodic, grid, block, lds, st); break;
+    case 4: launch_g<4>(p, periodic, grid, block, lds, st); break;
+    default: launch_g<8>(p, periodic, grid, block, lds, st); break;
   }
   AWQ_HIP_TRY(hipGetLastError());
   if (a.epilogue == EPI_ARGMAX) {

@@ -11,7 +11,7 @@
  * integer bit manipulation, all of which are correctly rounded on x86-64 and
  * on gfx950 (compile without fast-math and with FP contraction off).
  *
- * Accuracy (measured by tests/test_canon_math.py against libm in double):
+ * Accuracy (measured by tests/test_oracle_ops.py::test_canonical_exp_erf_accuracy against libm in double):
  *   awq_expf   <= 1 ulp on [-104, 88.7]
  *   awq_erff   <= 2 ulp for |x| < 1, absolute error <= 1 ulp(1.0) elsewhere
  *   awq_rsqrtf <= 1 ulp (a correctly rounded sqrt followed by a correctly
@@ -36,7 +36,7 @@
 
 #define AWQ_GROUP_SIZE 128      /* Inference.cu:40 */
 #define AWQ_HEAD_DIM 128        /* Inference.cu:36 */
-#define AWQ_BLOCK_K 32          /* length of one sequential fma chain in a linear layer */
+#define AWQ_BLOCK_K 32          /* inputs per block of a linear layer (two fma chains of 16) */
 
 AWQ_HD float awq_bits_to_f32(uint32_t u) {
   float f;
@@ -155,18 +155,46 @@ AWQ_HD int awq_group_period(int64_t m, int64_t k) {
 }
 
 /*
- * Summation order of a linear layer.  The k inputs of one output are cut into
- * k/32 blocks; block number blk holds, for t = 0..31, input index
+ * Arithmetic of a linear layer, y[i] = sum_j w(i,j) * x[j] with w = (q - z) * s.
+ *
+ * The k inputs of one output are cut into k/32 blocks; block number blk holds,
+ * for t = 0..31, input index
  *     j = c + C*(32*u + t),   C = awq_group_period(m,k), blk = c*(k/(32*C)) + u
- * so that all 32 share one scale group.  A block is accumulated as a
- * sequential fma chain starting from 0; blocks are then combined by
- * awq_tree_sum below.  C must divide k/32.
+ * so that all 32 share one scale group (s, z).  C must divide k/32.  Per block
+ *     T = A + B   A: fma chain from 0 over t with t % 4 < 2, B: over t % 4 >= 2,
+ *                 each in ascending t, multiplier the raw nibble q as a float
+ *     X = the block's 32 inputs added as an adjacent-pair tree (awq_tree_sum)
+ *     v = fma(-z, X, T) * s                      (binary32 throughout)
+ * and the k/32 block values v are combined by awq_tree_sum; the result is
+ * rounded to binary16 once.  The scale and the zero-point are applied to a
+ * block's sum rather than to every weight, so the binary16 rounding of each
+ * dequantised weight (Inference.cu:102-104) does not appear here; it stays in
+ * the standalone dequantisation and in the plain sequential reference that
+ * the tests hold this order to (1e-2 relative).
+ *
+ * Why two chains: on the GPU the masked nibble pairs are read as binary16
+ * subnormals q*2^-24 (nibbles at bits 0-3 of a half) and q*2^-20 (bits 4-7);
+ * the two scalings are powers of two, so each chain equals the unscaled chain
+ * times its power of two exactly, and A*2^-20 + B*2^-20 rounds as A + B does.
  */
 AWQ_HD int64_t awq_block_elem(int64_t k, int C, int64_t blk, int t) {
   int64_t U = k / ((int64_t)AWQ_BLOCK_K * C);
   int64_t c = blk / U, u = blk % U;
   return c + (int64_t)C * (AWQ_BLOCK_K * u + t);
 }
+
+/* T of one block: q[t] in 0..15, x[t] the block's inputs widened to binary32 */
+AWQ_HD float awq_block_qdot(const int* q, const float* x) {
+  float a = 0.0f, b = 0.0f;
+  for (int t = 0; t < AWQ_BLOCK_K; ++t) {
+    if ((t & 2) == 0) a = fmaf((float)q[t], x[t], a);
+    else b = fmaf((float)q[t], x[t], b);
+  }
+  return a + b;
+}
+
+/* v of one block from its T, X and the group's scale and zero-point */
+AWQ_HD float awq_block_value(float T, float X, float s, float z) { return fmaf(-z, X, T) * s; }
 
 /* Combine n partial sums in place: adjacent pairs while the count is even,
  * then left to right.  Returns the total. */
@@ -178,6 +206,13 @@ AWQ_HD float awq_tree_sum(float* v, int64_t n) {
   float s = v[0];
   for (int64_t a = 1; a < n; ++a) s += v[a];
   return s;
+}
+
+/* X of one block: adjacent-pair tree over its 32 inputs */
+AWQ_HD float awq_block_xsum(const float* x) {
+  float t[AWQ_BLOCK_K];
+  for (int i = 0; i < AWQ_BLOCK_K; ++i) t[i] = x[i];
+  return awq_tree_sum(t, AWQ_BLOCK_K);
 }
 
 #endif /* AWQ_CANON_MATH_H */

@@ -148,7 +148,7 @@ int awq_linear_repack(const void* packed_in, void* repacked_out, int64_t m, int6
  * zp_integral: 1 when every zero-point is an integer in [0,1024] (true of AWQ
  * checkpoints) -- a shorter instruction sequence with the same bits; 0 for
  * arbitrary zero-points; -1 to have the call inspect them (synchronises).
- * k <= 24576 (the workgroup keeps x in LDS).
+ * k <= 16384 (the workgroup keeps x in LDS).
  * workspace: awq_gemv_workspace_bytes(m,k) bytes, zero-filled once before its
  * first use (launches leave it zeroed); must not be shared by launches that
  * may overlap. */

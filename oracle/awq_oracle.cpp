@@ -158,11 +158,14 @@ static inline int nibble_at(const uint8_t* packed, int64_t p) {
 //     y[i] = h( sum_j f(w[i + j*m]) * f(x[j]) )        (binary32 accumulation)
 // Batched: row t of x ([M][k]) gives row t of y ([M][m]) (ldb = k, ldc = m).
 //
-// Three summation orders:
-//   awqo_linear_f64   double accumulation, no final rounding (brute-force pin)
-//   awqo_linear_seq   binary32, j ascending, multiply then add
-//   awqo_linear       binary32, the blocked order of awq_canon_math.h that the
-//                     GPU kernels also follow, so results agree bit for bit
+// Three evaluations:
+//   awqo_linear_f64   double accumulation of the dequantised weights h(h(q-z)*s), no final
+//                     rounding (brute-force pin)
+//   awqo_linear_seq   binary32, j ascending, multiply then add, the same dequantised weights:
+//                     the plain FP32-accumulate reference the GPU product is held to (1e-2)
+//   awqo_linear       binary32 in the blocked order of awq_canon_math.h (per block of 32 inputs
+//                     two fma chains over the raw nibbles, the scale and zero-point applied to the
+//                     block's sum), which the GPU kernels also follow: results agree bit for bit
 // ---------------------------------------------------------------------------
 static void build_lut(const half_t* scale, const half_t* zp, int64_t n_groups, std::vector<float>& lut) {
   lut.resize((size_t)n_groups * 16);
@@ -208,8 +211,6 @@ AWQO_API void awqo_linear_seq(const uint8_t* packed, const half_t* scale, const 
 // scalar statement of the blocked order (the definition)
 AWQO_API void awqo_linear_scalar(const uint8_t* packed, const half_t* scale, const half_t* zp, int64_t m, int64_t k,
                                  const half_t* x, half_t* y, int64_t M) {
-  std::vector<float> lut;
-  build_lut(scale, zp, m / AWQ_GROUP_SIZE, lut);
   const int C = awq_group_period(m, k);
   const int64_t nblk = k / AWQ_BLOCK_K;
 #pragma omp parallel for schedule(static)
@@ -217,13 +218,16 @@ AWQO_API void awqo_linear_scalar(const uint8_t* packed, const half_t* scale, con
     std::vector<float> part((size_t)nblk);
     for (int64_t t = 0; t < M; ++t) {
       for (int64_t blk = 0; blk < nblk; ++blk) {
-        float acc = 0.0f;
+        int q[AWQ_BLOCK_K];
+        float xf[AWQ_BLOCK_K];
+        int g = 0;
         for (int e = 0; e < AWQ_BLOCK_K; ++e) {
           int64_t j = awq_block_elem(k, C, blk, e);
-          int g = awq_group_index(m, k, i, j);
-          acc = fmaf(lut[g * 16 + nibble_at(packed, j * m + i)], h2f(x[t * k + j]), acc);
+          g = awq_group_index(m, k, i, j);  // the same for the whole block
+          q[e] = nibble_at(packed, j * m + i);
+          xf[e] = h2f(x[t * k + j]);
         }
-        part[blk] = acc;
+        part[blk] = awq_block_value(awq_block_qdot(q, xf), awq_block_xsum(xf), h2f(scale[g]), h2f(zp[g]));
       }
       y[t * m + i] = f2h(awq_tree_sum(part.data(), nblk));
     }
@@ -231,47 +235,49 @@ AWQO_API void awqo_linear_scalar(const uint8_t* packed, const half_t* scale, con
 }
 
 // AVX2 evaluation of the same order: 8 outputs per vector, each lane its own
-// fma chain, so the bits equal awqo_linear_scalar (tests compare the two).
+// pair of fma chains, so the bits equal awqo_linear_scalar (tests compare the two).
 // Returns the FP32 sums before rounding when y32 != NULL.
-static void linear_blocked(const uint8_t* packed, const float* lut, int64_t m, int64_t k, const half_t* x, half_t* y,
-                           float* y32) {
+static void linear_blocked(const uint8_t* packed, const half_t* scale, const half_t* zp, int64_t m, int64_t k,
+                           const half_t* x, half_t* y, float* y32) {
   const int C = awq_group_period(m, k);
   const int64_t nblk = k / AWQ_BLOCK_K;
   const int64_t RC = 64;  // rows per task
-  std::vector<float> xf((size_t)k);
+  std::vector<float> xf((size_t)k), xsum((size_t)nblk);
   for (int64_t j = 0; j < k; ++j) xf[j] = h2f(x[j]);
+  for (int64_t blk = 0; blk < nblk; ++blk) {
+    float t[AWQ_BLOCK_K];
+    for (int e = 0; e < AWQ_BLOCK_K; ++e) t[e] = xf[awq_block_elem(k, C, blk, e)];
+    xsum[blk] = awq_block_xsum(t);
+  }
   const __m256i shifts = _mm256_setr_epi32(0, 4, 8, 12, 16, 20, 24, 28);
+  const __m256i nib = _mm256_set1_epi32(15);
 #pragma omp parallel
   {
     std::vector<float> part((size_t)nblk * RC);
 #pragma omp for schedule(dynamic, 4)
     for (int64_t i0 = 0; i0 < m; i0 += RC) {
       for (int64_t blk = 0; blk < nblk; ++blk) {
-        __m256 acc[8];
-        for (int v = 0; v < 8; ++v) acc[v] = _mm256_setzero_ps();
-        int g_cached = -1;
-        __m256 lo = _mm256_setzero_ps(), hi = _mm256_setzero_ps();
+        __m256 accA[8], accB[8];
+        for (int v = 0; v < 8; ++v) accA[v] = accB[v] = _mm256_setzero_ps();
+        int g = 0;
         for (int e = 0; e < AWQ_BLOCK_K; ++e) {
           int64_t j = awq_block_elem(k, C, blk, e);
-          int g = awq_group_index(m, k, i0, j);  // 64 rows starting at a multiple of 64 share a group
-          if (g != g_cached) {
-            lo = _mm256_loadu_ps(lut + g * 16);
-            hi = _mm256_loadu_ps(lut + g * 16 + 8);
-            g_cached = g;
-          }
+          g = awq_group_index(m, k, i0, j);  // 64 rows starting at a multiple of 64 share a group, a block too
           const uint8_t* src = packed + ((j * m + i0) >> 1);
           __m256 xv = _mm256_set1_ps(xf[j]);
+          __m256* acc = (e & 2) ? accB : accA;
           for (int v = 0; v < 8; ++v) {
             uint32_t w32;
             memcpy(&w32, src + 4 * v, 4);
-            __m256i idx = _mm256_srlv_epi32(_mm256_set1_epi32((int)w32), shifts);
-            __m256 wl = _mm256_permutevar8x32_ps(lo, idx);
-            __m256 wh = _mm256_permutevar8x32_ps(hi, idx);
-            __m256 w = _mm256_blendv_ps(wl, wh, _mm256_castsi256_ps(_mm256_slli_epi32(idx, 28)));
-            acc[v] = _mm256_fmadd_ps(w, xv, acc[v]);
+            __m256i q = _mm256_and_si256(_mm256_srlv_epi32(_mm256_set1_epi32((int)w32), shifts), nib);
+            acc[v] = _mm256_fmadd_ps(_mm256_cvtepi32_ps(q), xv, acc[v]);
           }
         }
-        for (int v = 0; v < 8; ++v) _mm256_storeu_ps(&part[blk * RC + 8 * v], acc[v]);
+        const __m256 zn = _mm256_set1_ps(-h2f(zp[g])), sc = _mm256_set1_ps(h2f(scale[g])), X = _mm256_set1_ps(xsum[blk]);
+        for (int v = 0; v < 8; ++v) {
+          __m256 T = _mm256_add_ps(accA[v], accB[v]);
+          _mm256_storeu_ps(&part[blk * RC + 8 * v], _mm256_mul_ps(_mm256_fmadd_ps(zn, X, T), sc));
+        }
       }
       // awq_tree_sum over blocks, 64 rows at a time
       int64_t n = nblk;
@@ -298,9 +304,7 @@ static void linear_blocked(const uint8_t* packed, const float* lut, int64_t m, i
 
 AWQO_API void awqo_linear(const uint8_t* packed, const half_t* scale, const half_t* zp, int64_t m, int64_t k,
                           const half_t* x, half_t* y, int64_t M) {
-  std::vector<float> lut;
-  build_lut(scale, zp, m / AWQ_GROUP_SIZE, lut);
-  for (int64_t t = 0; t < M; ++t) linear_blocked(packed, lut.data(), m, k, x + t * k, y + t * m, nullptr);
+  for (int64_t t = 0; t < M; ++t) linear_blocked(packed, scale, zp, m, k, x + t * k, y + t * m, nullptr);
 }
 
 // ---------------------------------------------------------------------------
@@ -496,7 +500,6 @@ struct Tensor {
   std::vector<uint8_t> packed;
   std::vector<half_t> scale, zp;
   int64_t out_dim = 0, in_dim = 0;
-  std::vector<float> lut;
   void alloc(int64_t o, int64_t i) {
     out_dim = o;
     in_dim = i;
@@ -517,7 +520,6 @@ struct awqo_model {
   std::vector<half_t> hidden, normed, qkv, ctx, attn_out, mid, mlp_out, logits;
   std::vector<half_t> last_layer_out;  // hidden state after the last layer of the latest position
   int current_seq_len = 0;
-  bool luts_ready = false;
   // statistics of the last generate call
   std::vector<float> margins;
   double seconds_linear = 0;
@@ -577,7 +579,6 @@ AWQO_API void awqo_model_destroy(awqo_model* m) { delete m; }
 
 // pointer to (and byte size of) one stored array so a caller can fill it
 AWQO_API void* awqo_model_tensor(awqo_model* m, int layer, int kind, int part, int64_t* bytes) {
-  m->luts_ready = false;
   if (kind == T_GAMMA) {
     *bytes = (int64_t)m->gamma[layer].size() * 2;
     return m->gamma[layer].data();
@@ -637,30 +638,17 @@ AWQO_API int awqo_model_load_dir(awqo_model* m, const char* dir) {
     rd("unembed_scale.bin", m->unembed.scale.data(), m->unembed.scale.size() * 2);
     rd("unembed_zp.bin", m->unembed.zp.data(), m->unembed.zp.size() * 2);
   }
-  m->luts_ready = false;
   return rc;
-}
-
-static void ensure_luts(awqo_model* m) {
-  if (m->luts_ready) return;
-  for (int l = 0; l < m->cfg.n_layers; ++l)
-    for (int kind = T_WQKV; kind <= T_W2; ++kind) {
-      Tensor* t = model_tensor(m, l, kind);
-      build_lut(t->scale.data(), t->zp.data(), t->out_dim / AWQ_GROUP_SIZE, t->lut);
-    }
-  build_lut(m->unembed.scale.data(), m->unembed.zp.data(), m->unembed.out_dim / AWQ_GROUP_SIZE, m->unembed.lut);
-  m->luts_ready = true;
 }
 
 static void model_linear(awqo_model* m, Tensor& t, const half_t* x, half_t* y) {
   auto t0 = std::chrono::steady_clock::now();
-  linear_blocked(t.packed.data(), t.lut.data(), t.out_dim, t.in_dim, x, y, nullptr);
+  linear_blocked(t.packed.data(), t.scale.data(), t.zp.data(), t.out_dim, t.in_dim, x, y, nullptr);
   m->seconds_linear += std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
 }
 
 // runOneLayer, I:1029-1230.  L is the attended length current_seq_len_+1 of I:1118.
 AWQO_API void awqo_model_layer(awqo_model* m, int l, int64_t pos, int64_t L) {
-  ensure_luts(m);
   const int H = m->cfg.hidden, I = m->cfg.inter, NH = m->n_heads;
   awqo_rmsnorm(m->hidden.data(), m->gamma[l].data(), m->normed.data(), H, m->cfg.eps);  // I:1040
   model_linear(m, m->wqkv[l], m->normed.data(), m->qkv.data());                          // I:1052
@@ -684,7 +672,6 @@ AWQO_API void awqo_model_layer(awqo_model* m, int l, int64_t pos, int64_t L) {
 
 // sampleNextToken, I:1235-1292
 AWQO_API int awqo_model_sample(awqo_model* m) {
-  ensure_luts(m);
   const int H = m->cfg.hidden;
   awqo_rmsnorm(m->hidden.data(), m->gamma[m->cfg.n_layers - 1].data(), m->normed.data(), H, m->cfg.eps);  // I:1247
   model_linear(m, m->unembed, m->normed.data(), m->logits.data());                                       // I:1260

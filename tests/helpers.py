@@ -89,6 +89,16 @@ def effective_weights_f64(packed, scale, zp, m, k):
     return flat.astype(np.float64).reshape(k, m).T
 
 
+def unrounded_weights_f64(packed, scale, zp, m, k):
+    """W[i, j] = (q - z) * s in float64 for flat element j*m + i: the weights the blocked order of
+    awq_canon_math.h multiplies (scale and zero-point applied to a block's sum, no binary16 rounding
+    of each weight)"""
+    q = nibbles_flat(packed).reshape(m, k).astype(np.float64)
+    g = (np.arange(k) // 128) % (m // 128)
+    flat = ((q - zp.astype(np.float64)[g][None, :]) * scale.astype(np.float64)[g][None, :]).reshape(-1)
+    return flat.reshape(k, m).T
+
+
 def block_elem(k, C, blk, t):
     U = k // (32 * C)
     c, u = divmod(blk, U)

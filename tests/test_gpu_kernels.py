@@ -118,9 +118,14 @@ def test_gemv_bit_exact_and_within_tolerance(awq, lib, oracle, torch_gpu, m, k, 
     print("gemv", m, k, zp_int, flush=True)
     assert np.array_equal(outs[0].view(np.uint16), ref.view(np.uint16))          # same summation order: same bits
     assert np.array_equal(outs[1].view(np.uint16), ref.view(np.uint16))          # and the workspace reset itself
-    # against plain sequential FP32 accumulation: 1e-2 relative (north star tolerance)
-    denom = np.maximum(np.abs(seq.astype(np.float64)), 1e-2 * np.abs(seq.astype(np.float64)).max())
-    assert np.all(np.abs(outs[0].astype(np.float64) - seq.astype(np.float64)) <= 1e-2 * denom)
+    # against plain sequential FP32 accumulation of the binary16-dequantised weights: 1e-2 relative (north
+    # star tolerance); outputs smaller than the root mean square of all outputs are measured against that.
+    # The kernel applies scale and zero-point to block sums, so it differs from this reference by the
+    # binary16 rounding of the weights: 99% of the outputs within 2^-9 of that scale.
+    want = seq.astype(np.float64)
+    denom = np.maximum(np.abs(want), np.sqrt(np.mean(want * want)))
+    err = np.abs(outs[0].astype(np.float64) - want) / denom
+    assert np.all(err <= 1e-2) and np.percentile(err, 99) <= 2.0 ** -9
     if zp_int:
         # the general sequence must give the same bits as the integral-zero-point shortcut
         gen = gemv_gpu(awq, lib, torch, packed, scale, zp, m, k, x, 0)[0]
