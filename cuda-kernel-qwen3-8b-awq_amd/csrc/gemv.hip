@@ -163,9 +163,9 @@ struct GemvParams {
 };
 
 // the 16 finished rows of a workgroup; r = lane = row % 16, lanes 0..15 of wavefront 0
-__device__ __forceinline__ void epilogue(const GemvParams& p, int row, int r, float acc, half_t res) {
+__device__ __forceinline__ void epilogue(const GemvParams& p, int epi, int row, int r, float acc, half_t res) {
   half_t v = (half_t)acc;
-  switch (p.epilogue) {
+  switch (epi) {
     case EPI_RESIDUAL:  // Inference.cu:1149-1155
       p.y[row] = res + v;
       return;
@@ -239,10 +239,11 @@ __device__ __forceinline__ int xs_index(int e) {
 // (4w+q)*G .. +G-1 of row 16*rg + r.  x is staged (normalised, with the input
 // sum of every block beside it) once per workgroup; the weights of the next row
 // group are in flight while the current one is multiplied.
-// The arguments every wavefront needs before its first load come first and
-// one by one: the first 16 dwords of the argument block are preloaded into
-// scalar registers at wavefront launch (see the build flags), which takes one
-// memory round trip off the start of the kernel.
+// The arguments a wavefront needs early (pointers, the norm's and the scale
+// group's scalars, the epilogue selector) come first and one by one: the first
+// 16 dwords of the argument block are preloaded into scalar registers at
+// wavefront launch (see the build flags); the rest of the argument block is a
+// memory round trip away.
 // k = n_waves * 128 * G, so a thread stages exactly G/2 units of four inputs.
 // UFAST (periodic matrices only): the class length k/32/C when it is known at
 // compile time and divides G, so that a lane's G blocks are G/UFAST whole classes
@@ -250,12 +251,19 @@ __device__ __forceinline__ int xs_index(int e) {
 //
 // Dynamic LDS: x in block order (skewed) | block sums, k/32 floats | with the
 // fused norm, x in natural order (k halves).
-template <int G, bool PERIODIC, int UFAST = 0>
-__global__ __launch_bounds__(1024) void gemv_kernel(const u32x4* __restrict__ wq, const half_t* __restrict__ x,
-                                                    const half_t* __restrict__ gamma, const half_t* __restrict__ scale,
-                                                    const half_t* __restrict__ zp, int32_t k, int32_t nblk,
-                                                    int32_t n_waves, int32_t m, int32_t prologue, int32_t C,
-                                                    GemvParams p) {
+// NWC: the number of wavefronts when it is known at compile time (the model's
+// own shapes: k, the staging loops and the reduction are then constants), 0 = take
+// it from the launch.  MULTI: the grid is smaller than the number of row groups
+// and a workgroup walks several of them.
+template <int G, bool PERIODIC, int UFAST = 0, int NWC = 0, bool MULTI = true>
+__global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
+    const u32x4* __restrict__ wq, const half_t* __restrict__ x, const half_t* __restrict__ gamma,
+    const half_t* __restrict__ scale, const half_t* __restrict__ zp, int32_t m, int32_t prologue, int32_t epi,
+    float eps, int32_t mg, int32_t kg, GemvParams p) {
+  const int n_waves = NWC ? NWC : p.n_waves;
+  const int k = NWC ? NWC * 128 * G : p.k;
+  const int nblk = NWC ? NWC * 4 * G : p.nblk;
+  const int C = PERIODIC ? p.C : 1;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   half_t* xs = reinterpret_cast<half_t*>(smem);                                  // k halves + skew
   float* xsum = reinterpret_cast<float*>(smem + (size_t)(k + (nblk / G) * 8) * 2);  // nblk floats
@@ -265,7 +273,6 @@ __global__ __launch_bounds__(1024) void gemv_kernel(const u32x4* __restrict__ wq
   __shared__ GroupConst gtab[2][PERIODIC ? 64 : 1];
   constexpr int MAXU = G / 2;  // units of four inputs a thread stages
   static_assert(G >= 2, "a thread stages whole units");
-
   const int tid = threadIdx.x;
   const int nthreads = n_waves * 64;
   const int lane = tid & 63;
@@ -326,10 +333,18 @@ __global__ __launch_bounds__(1024) void gemv_kernel(const u32x4* __restrict__ wq
     }
     __syncthreads();
     for (int pi = tid; pi < 256; pi += nthreads) {
+      // 16 reads in flight per round: an LDS round trip per term would serialise the chain
       float acc = 0.0f;
-      for (int i = pi; i < k; i += 256) {
-        const float v = (float)xn[i];
-        acc = __builtin_fmaf(v, v, acc);
+      for (int i0 = pi; i0 < k; i0 += 16 * 256) {
+        half_t hv[16];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) hv[j] = i0 + 256 * j < k ? xn[i0 + 256 * j] : (half_t)0.0f;
+#pragma unroll
+        for (int j = 0; j < 16; ++j)
+          if (i0 + 256 * j < k) {
+            const float v = (float)hv[j];
+            acc = __builtin_fmaf(v, v, acc);
+          }
       }
       part[pi] = acc;
     }
@@ -352,7 +367,7 @@ __global__ __launch_bounds__(1024) void gemv_kernel(const u32x4* __restrict__ wq
     tot += dpp_f<kDppXor2>(tot);
     tot += dpp_f<kDppXor1>(tot);
     tot = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, tot)));
-    const half_t sc = (half_t)awq_rsqrtf(tot / (float)k + p.eps);
+    const half_t sc = (half_t)awq_rsqrtf(tot / (float)k + eps);
     const half2_t sc2 = half2_t{sc, sc};
 #pragma unroll
     for (int u = 0; u < MAXU; ++u) {
@@ -381,7 +396,7 @@ __global__ __launch_bounds__(1024) void gemv_kernel(const u32x4* __restrict__ wq
   // constant within a class of blocks; the (at most 64) classes of a row group
   // go through a table in LDS, filled one row group ahead.
   if (PERIODIC && tid < C && rg < n_rg) {
-    int gi = (int)((((int64_t)tid * p.mg + (rg >> 3)) % p.kg) % p.mg);
+    int gi = (int)((((int64_t)tid * mg + (rg >> 3)) % kg) % mg);
     gtab[0][tid] = make_group(scale[gi], zp[gi]);
   }
   __syncthreads();  // xs, the block sums and the first table
@@ -400,8 +415,8 @@ __global__ __launch_bounds__(1024) void gemv_kernel(const u32x4* __restrict__ wq
     for (int b = 0; b < G; ++b) xb[b] = xsum[blk0 + b];
   }
   for (int it = 0; rg < n_rg; rg += gridDim.x, ++it) {
-    const int rg_next = rg + gridDim.x;
-    if (rg_next < n_rg) {
+    const int rg_next = MULTI ? rg + (int)gridDim.x : n_rg;
+    if (MULTI && rg_next < n_rg) {
       const u32x4* wpn = wq + ((int64_t)rg_next * nblk + blk0) * 16 + r;
 #pragma unroll
       for (int b = 0; b < G; ++b) wn[b] = __builtin_nontemporal_load(wpn + b * 16);
@@ -409,17 +424,17 @@ __global__ __launch_bounds__(1024) void gemv_kernel(const u32x4* __restrict__ wq
     // the residual row is requested before the pass multiplies: the end of the
     // launch then does not wait for one more round trip to memory
     half_t res = (half_t)0.0f;
-    if (tid < 16 && p.epilogue == EPI_RESIDUAL) res = p.res[rg * 16 + r];
+    if (tid < 16 && epi == EPI_RESIDUAL) res = p.res[rg * 16 + r];
     // scale group of these 16 rows: row/128, then Inference.cu:90 with the index
     // wrapped to the m/128 stored entries
     const int a = rg >> 3;
     GroupConst g;
     if (!PERIODIC) {
-      int gi = (a % p.kg) % p.mg;
+      int gi = (a % kg) % mg;
       g = make_group(scale[gi], zp[gi]);
-    } else if (tid < C && rg_next < n_rg) {
+    } else if (MULTI && tid < C && rg_next < n_rg) {
       // the next row group's table; its buffer was last read two barriers ago
-      int gi = (int)((((int64_t)tid * p.mg + (rg_next >> 3)) % p.kg) % p.mg);
+      int gi = (int)((((int64_t)tid * mg + (rg_next >> 3)) % kg) % mg);
       gtab[(it + 1) & 1][tid] = make_group(scale[gi], zp[gi]);
     }
     int cls = 0, cls_left = 0;  // class of the next block and blocks left in it
@@ -468,15 +483,26 @@ __global__ __launch_bounds__(1024) void gemv_kernel(const u32x4* __restrict__ wq
     if (q == 0) rd[wave][r] = v;
     __syncthreads();
     if (tid < 16) {
+      // awq_tree_sum over the wavefronts' sums, in registers (all reads in flight at once)
+      float t[16];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) t[i] = i < n_waves ? rd[i][r] : 0.0f;
       int n = n_waves;
-      while (n > 1 && (n & 1) == 0) {
-        n >>= 1;
-        for (int i = 0; i < n; ++i) rd[i][r] = rd[2 * i][r] + rd[2 * i + 1][r];
-      }
-      float tot = rd[0][r];
-      for (int i = 1; i < n; ++i) tot += rd[i][r];
-      epilogue(p, rg * 16 + r, r, tot, res);
+#pragma unroll
+      for (int lvl = 0; lvl < 4; ++lvl)
+        if (n > 1 && (n & 1) == 0) {
+          n >>= 1;
+#pragma unroll
+          for (int i = 0; i < 8; ++i)
+            if (i < n) t[i] = t[2 * i] + t[2 * i + 1];
+        }
+      float tot = t[0];
+#pragma unroll
+      for (int i = 1; i < 16; ++i)
+        if (i < n) tot += t[i];
+      epilogue(p, epi, rg * 16 + r, r, tot, res);
     }
+    if (!MULTI) break;
 #pragma unroll
     for (int b = 0; b < G; ++b) w[b] = wn[b];
   }
@@ -515,14 +541,22 @@ bool plan_gemv(int64_t m, int64_t k, GemvPlan* out) {
   return found;
 }
 
-#define GEMV_HOT_ARGS p.wq, p.x, p.gamma, p.scale, p.zp, p.k, p.nblk, p.n_waves, p.m, p.prologue, p.C
+#define GEMV_HOT_ARGS p.wq, p.x, p.gamma, p.scale, p.zp, p.m, p.prologue, p.epilogue, p.eps, p.mg, p.kg
 template <int G>
-void launch_g(const GemvParams& p, bool periodic, dim3 grid, dim3 block, size_t lds, hipStream_t st) {
+void launch_g(const GemvParams& p, bool periodic, bool multi, dim3 grid, dim3 block, size_t lds, hipStream_t st) {
   if (G == 8 && periodic && p.nblk / p.C == 4) {  // the unembedding: classes of 4 blocks
-    hipLaunchKernelGGL((gemv_kernel<G, true, G == 8 ? 4 : 0>), grid, block, lds, st, GEMV_HOT_ARGS, p);
+    if (p.n_waves == 4) hipLaunchKernelGGL((gemv_kernel<G, true, G == 8 ? 4 : 0, 4, true>), grid, block, lds, st, GEMV_HOT_ARGS, p);
+    else hipLaunchKernelGGL((gemv_kernel<G, true, G == 8 ? 4 : 0>), grid, block, lds, st, GEMV_HOT_ARGS, p);
     return;
   }
-  if (periodic) hipLaunchKernelGGL((gemv_kernel<G, true>), grid, block, lds, st, GEMV_HOT_ARGS, p);
+  if (periodic) {
+    hipLaunchKernelGGL((gemv_kernel<G, true>), grid, block, lds, st, GEMV_HOT_ARGS, p);
+    return;
+  }
+  // the per-layer matrices of the model: 4096 inputs as 4 wavefronts x 8 blocks or 8 x 4, 12288 as 12 x 8
+  if (!multi && G == 8 && p.n_waves == 4) hipLaunchKernelGGL((gemv_kernel<G, false, 0, 4, false>), grid, block, lds, st, GEMV_HOT_ARGS, p);
+  else if (!multi && G == 8 && p.n_waves == 12) hipLaunchKernelGGL((gemv_kernel<G, false, 0, 12, false>), grid, block, lds, st, GEMV_HOT_ARGS, p);
+  else if (!multi && G == 4 && p.n_waves == 8) hipLaunchKernelGGL((gemv_kernel<G, false, 0, 8, false>), grid, block, lds, st, GEMV_HOT_ARGS, p);
   else hipLaunchKernelGGL((gemv_kernel<G, false>), grid, block, lds, st, GEMV_HOT_ARGS, p);
 }
 
@@ -620,9 +654,9 @@ int launch_gemv(const LinearArgs& a, hipStream_t st) {
                (a.prologue == PRO_RMSNORM ? (size_t)a.k * 2 : 0);
   AWQ_REQUIRE(lds <= 65536, "k too large for the fused norm (x is kept twice in LDS)");
   switch (plan.g) {
-    case 2: launch_g<2>(p, periodic, grid, block, lds, st); break;
-    case 4: launch_g<4>(p, periodic, grid, block, lds, st); break;
-    default: launch_g<8>(p, periodic, grid, block, lds, st); break;
+    case 2: launch_g<2>(p, periodic, n_wg < n_rg, grid, block, lds, st); break;
+    case 4: launch_g<4>(p, periodic, n_wg < n_rg, grid, block, lds, st); break;
+    default: launch_g<8>(p, periodic, n_wg < n_rg, grid, block, lds, st); break;
   }
   AWQ_HIP_TRY(hipGetLastError());
   if (a.epilogue == EPI_ARGMAX) {
