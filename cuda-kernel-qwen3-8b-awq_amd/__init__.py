@@ -72,6 +72,8 @@ SIGNATURES = {
     "awq_time_linear": (ctypes.c_int, [_vp, ctypes.c_int, _i32, ctypes.POINTER(_f32), ctypes.POINTER(_i64)]),
     "awq_destroy": (None, [_vp]),
     "awq_write_weight_dir": (ctypes.c_int, [ctypes.c_char_p, _cfgp, _u64]),
+    "awq_write_weight_dir_profile": (ctypes.c_int, [ctypes.c_char_p, _cfgp, _u64, ctypes.c_int]),
+    "awq_last_load_seconds": (ctypes.c_double, []),
     "awq_synth_fill": (ctypes.c_int, [_u64, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp, _i64]),
     "awq_synth_fill_profile": (ctypes.c_int, [ctypes.c_int, _u64, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp, _i64]),
     "awq_synth_normal_f16": (ctypes.c_int, [_u64, _u64, _vp, _i64, _f32, _f32]),

@@ -12,7 +12,11 @@
 #include <sys/stat.h>
 
 #include <algorithm>
+#include <chrono>
+#include <condition_variable>
 #include <memory>
+#include <mutex>
+#include <thread>
 
 static thread_local std::string g_last_error;
 void awq_set_error(const std::string& msg) { g_last_error = msg; }
@@ -124,6 +128,7 @@ struct DevLinear {
   int64_t m = 0, k = 0;
   int zp_integral = 0;
   bool have[3] = {false, false, false};
+  bool reordered = false;  // stream_order already holds the reordered copy (the directory loader does it on the fly)
 };
 
 struct LayerDev {
@@ -347,21 +352,31 @@ int run_step(awq_engine* e, bool gen, StepState s) {
   return enqueue_step_body(e, gen, len_bound);
 }
 
-int read_file(const std::string& path, int64_t bytes, std::vector<uint8_t>& staging) {
+// readBinaryFileToDevice's host half (Inference.cu:297-308): exactly `bytes` bytes of the file
+int read_file(const std::string& path, int64_t bytes, void* dst, std::string* err) {
   FILE* f = fopen(path.c_str(), "rb");
   if (!f) {
-    awq_set_error("could not open " + path);  // Inference.cu:299-302
+    *err = "could not open " + path;  // Inference.cu:299-302
     return AWQ_ERR_IO;
   }
-  staging.resize((size_t)bytes);
-  size_t got = fread(staging.data(), 1, (size_t)bytes, f);
+  size_t got = fread(dst, 1, (size_t)bytes, f);
   fclose(f);
   if ((int64_t)got != bytes) {
-    awq_set_error("read failed for " + path);  // :305-308
+    *err = "read failed for " + path;  // :305-308
     return AWQ_ERR_IO;
   }
   return AWQ_OK;
 }
+
+// Reorders one linear layer on the engine's stream right after its packed bytes were copied.
+int reorder_now(awq_engine* e, DevLinear* t) {
+  if (int rc = dev_alloc(e, &t->stream_order, t->m * (t->k / 2))) return rc;
+  if (int rc = launch_repack(t->packed, t->stream_order, t->m, t->k, e->stream)) return rc;
+  t->reordered = true;
+  return AWQ_OK;
+}
+
+thread_local double g_last_load_seconds = 0.0;
 
 }  // namespace
 
@@ -483,8 +498,11 @@ extern "C" int awq_finalize(awq_engine* e) {
   }
   all.push_back(&e->unembed);
   for (DevLinear* t : all) {
-    if (int rc = dev_alloc(e, &t->stream_order, t->m * (t->k / 2))) return rc;
-    if (int rc = launch_repack(t->packed, t->stream_order, t->m, t->k, st)) return rc;
+    if (!t->reordered) {
+      if (int rc = dev_alloc(e, &t->stream_order, t->m * (t->k / 2))) return rc;
+      if (int rc = launch_repack(t->packed, t->stream_order, t->m, t->k, st)) return rc;
+      t->reordered = true;
+    }
     AWQ_HIP_TRY(hipStreamSynchronize(st));
     if (int rc = dev_free(e, t->packed)) return rc;
     t->packed = nullptr;
@@ -510,6 +528,12 @@ extern "C" int awq_finalize(awq_engine* e) {
   return awq_reset(e);
 }
 
+extern "C" double awq_last_load_seconds(void) { return g_last_load_seconds; }
+
+// Constructor with the loader of Inference.cu:766-903.  Three stages overlap: a reader thread fills
+// two pinned buffers in turn (fread), this thread sends a full buffer to the device (hipMemcpyAsync
+// on the engine's stream) and, for the packed bytes of a linear layer, queues its reordering behind
+// the copy; a buffer goes back to the reader once its copy has completed.
 extern "C" int awq_create(const char* weight_dir, const awq_config* cfg_in, awq_engine** out) {
   AWQ_REQUIRE(weight_dir != nullptr && out != nullptr, "NULL argument");
   *out = nullptr;
@@ -517,16 +541,126 @@ extern "C" int awq_create(const char* weight_dir, const awq_config* cfg_in, awq_
   if (int rc = awq_validate_weight_dir(weight_dir, cfg_in)) return rc;
   awq_engine* e = nullptr;
   if (int rc = awq_create_empty(cfg_in, &e)) return rc;
-  std::vector<uint8_t> staging;
-  for (const WeightFile& wf : awq_weight_files(e->cfg)) {
-    int rc = read_file(std::string(weight_dir) + "/" + wf.name, wf.bytes, staging);
-    if (!rc) rc = awq_upload(e, wf.layer, wf.kind, wf.part, staging.data(), wf.bytes);
-    if (rc) {
-      awq_destroy(e);
-      return rc;
+  const std::vector<WeightFile> files = awq_weight_files(e->cfg);
+  int64_t largest = 0;
+  for (const WeightFile& wf : files) largest = std::max(largest, wf.bytes);
+  const auto t_begin = std::chrono::steady_clock::now();
+
+  struct Slot {
+    void* host = nullptr;      // pinned
+    hipEvent_t copied = nullptr;
+    int file = -1;             // index of the file it holds
+    int state = 0;             // 0 free for the reader, 1 full, 2 copy in flight
+    int rc = AWQ_OK;
+    std::string err;
+  } slot[2];
+  std::mutex mu;
+  std::condition_variable cv;
+  bool stop = false;
+  int rc = AWQ_OK;
+  for (Slot& s : slot) {
+    if (rc == AWQ_OK && hipHostMalloc(&s.host, (size_t)largest, hipHostMallocDefault) != hipSuccess) {
+      awq_set_error("hipHostMalloc of a staging buffer failed");
+      rc = AWQ_ERR_HIP;
+    }
+    if (rc == AWQ_OK && hipEventCreateWithFlags(&s.copied, hipEventDisableTiming) != hipSuccess) {
+      awq_set_error("hipEventCreate failed");
+      rc = AWQ_ERR_HIP;
     }
   }
-  if (int rc = awq_finalize(e)) {
+  std::thread reader;
+  if (rc == AWQ_OK) {
+    reader = std::thread([&]() {
+      for (size_t i = 0; i < files.size(); ++i) {
+        Slot& s = slot[i & 1];
+        {
+          std::unique_lock<std::mutex> lock(mu);
+          cv.wait(lock, [&] { return s.state == 0 || stop; });
+          if (stop) return;
+        }
+        std::string err;
+        int frc = read_file(std::string(weight_dir) + "/" + files[i].name, files[i].bytes, s.host, &err);
+        {
+          std::lock_guard<std::mutex> lock(mu);
+          s.file = (int)i;
+          s.rc = frc;
+          s.err = err;
+          s.state = 1;
+        }
+        cv.notify_all();
+        if (frc) return;
+      }
+    });
+    for (size_t i = 0; i < files.size() && rc == AWQ_OK; ++i) {
+      Slot& s = slot[i & 1];
+      {
+        std::unique_lock<std::mutex> lock(mu);
+        cv.wait(lock, [&] { return s.state == 1; });
+      }
+      if (s.rc) {
+        awq_set_error(s.err);
+        rc = s.rc;
+        break;
+      }
+      const WeightFile& wf = files[i];
+      void* dst = nullptr;
+      DevLinear* t = nullptr;
+      if (wf.kind == AWQ_T_GAMMA) {
+        dst = e->layers[wf.layer].gamma;
+        e->layers[wf.layer].have_gamma = true;
+      } else {
+        t = find_linear(e, wf.layer, wf.kind);
+        dst = wf.part == AWQ_P_PACKED ? (void*)t->packed : wf.part == AWQ_P_SCALE ? (void*)t->scale : (void*)t->zp;
+        if (wf.part == AWQ_P_ZP) t->zp_integral = zp_all_integral((const uint16_t*)s.host, wf.bytes / 2);
+        t->have[wf.part] = true;
+      }
+      if (hipMemcpyAsync(dst, s.host, (size_t)wf.bytes, hipMemcpyHostToDevice, e->stream) != hipSuccess ||
+          hipEventRecord(s.copied, e->stream) != hipSuccess) {
+        awq_set_error("host-to-device copy of " + wf.name + " failed");
+        rc = AWQ_ERR_HIP;
+        break;
+      }
+      // the embedding is only ever gathered from, so it stays in file order
+      if (t && wf.part == AWQ_P_PACKED && wf.kind != AWQ_T_EMBED) rc = reorder_now(e, t);
+      {
+        std::lock_guard<std::mutex> lock(mu);
+        s.state = 2;
+      }
+      // the other buffer's copy was queued one file ago: once it has completed the reader may refill it
+      Slot& o = slot[(i + 1) & 1];
+      if (o.state == 2) {
+        if (hipEventSynchronize(o.copied) != hipSuccess) {
+          awq_set_error("waiting for a host-to-device copy failed");
+          rc = AWQ_ERR_HIP;
+          break;
+        }
+        {
+          std::lock_guard<std::mutex> lock(mu);
+          o.state = 0;
+        }
+        cv.notify_all();
+      }
+    }
+    {
+      std::lock_guard<std::mutex> lock(mu);
+      stop = true;
+    }
+    cv.notify_all();
+    reader.join();
+  }
+  if (rc == AWQ_OK && hipStreamSynchronize(e->stream) != hipSuccess) {
+    awq_set_error("the weight upload did not complete");
+    rc = AWQ_ERR_HIP;
+  } else if (rc != AWQ_OK) {
+    (void)hipStreamSynchronize(e->stream);  // nothing may still read the staging buffers
+  }
+  for (Slot& s : slot) {
+    if (s.copied) (void)hipEventDestroy(s.copied);
+    if (s.host) (void)hipHostFree(s.host);
+  }
+  if (rc == AWQ_OK) g_last_load_seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - t_begin).count();
+  if (rc == AWQ_OK) rc = awq_finalize(e);
+  if (rc) {
     awq_destroy(e);
     return rc;
   }

@@ -104,7 +104,7 @@ static int write_file(const std::string& path, const void* src, size_t bytes) {
   return AWQ_OK;
 }
 
-extern "C" int awq_write_weight_dir(const char* dir, const awq_config* cfg_in, uint64_t seed) {
+extern "C" int awq_write_weight_dir_profile(const char* dir, const awq_config* cfg_in, uint64_t seed, int profile) {
   AWQ_REQUIRE(dir != nullptr, "dir is NULL");
   awq_config cfg;
   if (cfg_in) cfg = *cfg_in;
@@ -114,8 +114,12 @@ extern "C" int awq_write_weight_dir(const char* dir, const awq_config* cfg_in, u
   for (const WeightFile& wf : awq_weight_files(cfg)) {
     buf.resize((size_t)wf.bytes);
     int64_t count = (wf.part == AWQ_P_PACKED && wf.kind != AWQ_T_GAMMA) ? wf.bytes : wf.bytes / 2;
-    if (int rc = awq_synth_fill(seed, wf.layer, wf.kind, wf.part, buf.data(), count)) return rc;
+    if (int rc = awq_synth_fill_profile(profile, seed, wf.layer, wf.kind, wf.part, buf.data(), count)) return rc;
     if (int rc = write_file(std::string(dir) + "/" + wf.name, buf.data(), buf.size())) return rc;
   }
   return AWQ_OK;
+}
+
+extern "C" int awq_write_weight_dir(const char* dir, const awq_config* cfg_in, uint64_t seed) {
+  return awq_write_weight_dir_profile(dir, cfg_in, seed, AWQ_SYNTH_SPEC);
 }

@@ -55,8 +55,18 @@ int awq_validate_weight_dir(const char* dir, const awq_config* cfg);
 
 /* Constructor, Inference.cu:422-470: loads the weight directory onto the
  * current device, repacks, builds rotary tables, zeroes the KV cache.
- * cfg == NULL means the reference constants. */
+ * cfg == NULL means the reference constants.
+ * Loader (readBinaryFileToDevice, Inference.cu:297-311, called from :766-903):
+ * a reader thread fills two pinned staging buffers in turn while the previous
+ * file's host-to-device copy and the previous tensor's reordering run on the
+ * engine's stream, so file reads, copies and reordering overlap.  A missing or
+ * short file fails with AWQ_ERR_IO as the reference does (:299-308); bytes
+ * beyond the expected count are ignored (:304). */
 int awq_create(const char* weight_dir, const awq_config* cfg, awq_engine** out);
+/* Seconds the last successful awq_create on this thread spent between opening
+ * the first file and the last tensor being reordered on the device (0 when
+ * none ran).  No counterpart in the reference. */
+double awq_last_load_seconds(void);
 
 /* Same engine without a directory: allocate, then awq_upload every array, then
  * awq_finalize.  Used with in-memory synthetic weights. */
@@ -112,6 +122,9 @@ void awq_destroy(awq_engine* e);
 /* Writes a weight directory in the layout of Inference.cu:780-899 filled from
  * awq_synth.h under `seed` (the reference ships no producer of its format). */
 int awq_write_weight_dir(const char* dir, const awq_config* cfg, uint64_t seed);
+/* the same with the value distributions chosen: AWQ_SYNTH_SPEC (what awq_write_weight_dir draws) or
+ * AWQ_SYNTH_BALANCED (awq_synth.h) */
+int awq_write_weight_dir_profile(const char* dir, const awq_config* cfg, uint64_t seed, int profile);
 
 /* Host-side synthetic data (awq_synth.h).  `count` is in elements of the
  * array: bytes for AWQ_P_PACKED, halves otherwise. */

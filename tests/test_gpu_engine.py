@@ -155,6 +155,58 @@ def test_weight_directory_round_trip_and_cli(awq, lib, oracle, torch_gpu, tmp_pa
     assert ei.value.code == 2 and "layer_1_w2.bin" in str(ei.value)
 
 
+def test_drop_in_class_and_command_line_on_the_full_size_directory(awq, lib, oracle, torch_gpu, tmp_path):
+    """The reference's own use (Inference.cu:1413-1433): main() builds QWen3AWQInfer(argv[1]) on a directory
+    in the README layout (474 headerless files, 3,642,565,388 bytes), calls generateResponse({151643}, 20) and
+    prints "Generated tokens: " followed by the ids.  Here the built command-line harness runs as a child
+    process on such a directory and its 20 ids must be the CPU oracle's on the same files; the engine that
+    awq_create loads from the directory (pinned double-buffered loader) must then be in the same state, bit
+    for bit, as one filled through awq_upload from memory."""
+    cfg = awq.default_config()
+    d = str(tmp_path / "qwen3_awq_weights")
+    os.makedirs(d)
+    seed = 2025
+    print("writing the 3.64 GB weight directory", flush=True)
+    awq.check(lib.awq_write_weight_dir_profile(d.encode(), ctypes.byref(cfg), seed, awq.SYNTH_BALANCED))
+    total = sum(os.path.getsize(os.path.join(d, f)) for f in os.listdir(d))
+    assert len(os.listdir(d)) == 474 and total == 3642565388          # README sizes, Inference.cu:780-899
+    cli = os.path.join(os.path.dirname(awq.LIB_PATH), "qwen3_awq_infer")
+    print("running", cli, flush=True)
+    res = subprocess.run([cli, d], capture_output=True, text=True, timeout=600)
+    assert res.returncode == 0, res.stderr
+    line = [ln for ln in res.stdout.splitlines() if ln.startswith("Generated tokens: ")]
+    assert len(line) == 1 and res.stdout.endswith(" \n")               # ids separated and followed by a space
+    got = [int(t) for t in line[0][len("Generated tokens: "):].split()]
+    # the oracle on the same files (its cache only needs the 21 positions of this run)
+    ocfg = awq.make_config(max_pos=32)
+    model = make_oracle_model(oracle, ocfg)
+    assert oracle.awqo_model_load_dir(model, d.encode()) == 0
+    ref = oracle_generate(oracle, model, [151643], 20)
+    print("command line:", got, flush=True)
+    assert got == ref
+    assert len(set(got)) > 1                                             # not a collapsed sequence
+    # awq_create(dir) against awq_upload of the same bytes: ids, hidden state and logits
+    eng = awq.QWen3AWQInfer(d, config=ocfg)
+    assert 0.0 < lib.awq_last_load_seconds() < 120.0
+    print("directory loaded in %.2f s" % lib.awq_last_load_seconds(), flush=True)
+    a = eng.generateResponse([151643, 7, 99], 8)
+    ha, la = np.ctypeslib.as_array(eng.read_hidden()).copy(), np.ctypeslib.as_array(eng.read_logits()).copy()
+    eng.close()
+    eng2 = awq.QWen3AWQInfer.empty(ocfg)
+    fill_pair(awq, oracle, ocfg, seed, engine=eng2, model=model, profile=awq.SYNTH_BALANCED)
+    b = eng2.generateResponse([151643, 7, 99], 8)
+    hb, lb = np.ctypeslib.as_array(eng2.read_hidden()).copy(), np.ctypeslib.as_array(eng2.read_logits()).copy()
+    eng2.close()
+    assert a == b and np.array_equal(ha, hb) and np.array_equal(la, lb)
+    assert a == oracle_generate(oracle, model, [151643, 7, 99], 8)
+    oracle.awqo_model_destroy(model)
+    # a file that is too short stops the loader with the reference's message, before anything runs
+    with open(os.path.join(d, "layer_35_w2_zp.bin"), "r+b") as f:
+        f.truncate(10)
+    res = subprocess.run([cli, d], capture_output=True, text=True, timeout=600)
+    assert res.returncode == 1 and "layer_35_w2_zp.bin" in res.stderr
+
+
 @pytest.mark.parametrize("n_layers,prompt_len,n_new", [(2, 3, 6)])
 def test_full_width_model_token_identity(awq, oracle, torch_gpu, n_layers, prompt_len, n_new):
     """reference widths (hidden 4096, intermediate 12288, vocabulary 151936), fewer layers"""
