@@ -9,6 +9,12 @@ seeded weights, 128-token synthetic prompt).  Weights are resident in HBM before
 Prints ONE JSON line: decode tok/s, the HBM roofline of the dominant kernel (the fused int4
 dequant + matrix-vector product, measured live with HIP events on the engine's stream) and the CPU
 oracle timed on this host's cores on a bounded sample of the same workload.
+
+Other modes (plain text output, used for the summaries under profiles/):
+    --mode attention [--one-cache]   decode attention by attended length
+    --mode prefill [--lengths a,b]   batched prompt pass of the 36-layer model by prompt length
+    --mode traffic                   a 1 GiB copy, then the engine's w1 launches (for rocprofv3 --pmc runs)
+    --mode w4a16                     W4A16 products of config 5 (token sweep on the w1 and w2 shapes)
 """
 import argparse
 import ctypes
@@ -29,6 +35,102 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
+def mode_attention(args):
+    """Decode attention (one query per head against the KV cache) at growing attended lengths:
+    microseconds per launch and algorithmic GB/s (keys and values once: 2 x heads x L x 256 bytes).
+    32 heads, caches of 40,960 positions with random binary16 contents, HIP events around the launches.
+    Every launch reads another layer's cache (12 caches, 8 GB), as a decode step does: up to a few
+    thousand positions one cache would stay in the L2 of each die (or the memory-side cache) between
+    launches and flatter the short lengths; --one-cache shows that case."""
+    import torch
+    awq = importlib.import_module("cuda-kernel-qwen3-8b-awq_amd")
+    lib = awq.load_library()
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    H, MP = 32, 40960
+    NL = 1 if args.one_cache else 12
+    kcs = [torch.randn(H, MP, 128, dtype=torch.float16, device="cuda") for _ in range(NL)]
+    vcs = [torch.randn(H, MP, 128, dtype=torch.float16, device="cuda") for _ in range(NL)]
+    q = torch.randn(H * 128, dtype=torch.float16, device="cuda")
+    ctx = torch.empty(H * 128, dtype=torch.float16, device="cuda")
+    ws = torch.zeros(lib.awq_attention_workspace_bytes(H, MP), dtype=torch.uint8, device="cuda")
+    for L in (128, 256, 512, 576, 577, 768, 1024, 1025, 1536, 2048, 2049, 4096, 8192, 16384, 40960):
+        def run(i):
+            awq.check(lib.awq_decode_attention(q.data_ptr(), kcs[i % NL].data_ptr(), vcs[i % NL].data_ptr(),
+                                               ctx.data_ptr(), H, MP, L, ws.data_ptr(), st))
+        for i in range(NL):
+            run(i)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        n = 24
+        e0.record()
+        for i in range(n):
+            run(i)
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1000 / n
+        nbytes = 2 * H * L * 128 * 2
+        print("L=%6d  %9.1f us  %7.1f GB/s" % (L, us, nbytes / us / 1e3), flush=True)
+
+
+def _synthetic_engine(awq, lib, cfg, seed, profile):
+    eng = awq.QWen3AWQInfer.empty(cfg)
+    for layer, kind, part in awq.tensor_list(cfg):
+        count = cfg.part_count(kind, part)
+        nbytes = count if (part == awq.P_PACKED and kind != awq.T_GAMMA) else 2 * count
+        buf = (ctypes.c_uint8 * nbytes)()
+        awq.check(lib.awq_synth_fill_profile(profile, seed, layer, kind, part, buf, count))
+        eng.upload(layer, kind, part, buf, nbytes)
+    eng.finalize()
+    return eng
+
+
+def mode_prefill(args):
+    """Batched prompt pass of the full 36-layer model (awq_prefill_batched): milliseconds and tokens per
+    second by prompt length.  Synthetic balanced weights, cache capacity 40,960 positions, best of two."""
+    awq = importlib.import_module("cuda-kernel-qwen3-8b-awq_amd")
+    lib = awq.load_library()
+    lengths = [int(v) for v in args.lengths.split(",")]
+    eng = _synthetic_engine(awq, lib, awq.make_config(n_layers=36, max_pos=40960), 1, awq.SYNTH_BALANCED)
+    for P in lengths:
+        prompt = [(7 * i + 3) % 1000 for i in range(P)]
+        best = 1e9
+        for rep in range(2):
+            eng.reset()
+            t = time.perf_counter()
+            eng.prefill(prompt, batched=True)   # returns after the device finished
+            best = min(best, time.perf_counter() - t)
+        print("prompt of %6d tokens: %8.1f ms  %7.0f tok/s" % (P, best * 1e3, P / best), flush=True)
+    eng.close()
+
+
+def mode_traffic(args):
+    """Workload for the HBM-traffic counters of the decode GEMV kernel.  Run under
+    `rocprofv3 --pmc FETCH_SIZE` and again under `rocprofv3 --pmc WRITE_SIZE`:
+      1. a plain device-to-device copy of 1 GiB (reads 1 GiB, writes 1 GiB): the calibration of what
+         the counters report per byte;
+      2. the engine's own w1 launches (12288 x 4096 int4, RMSNorm prologue, GeLU epilogue) over the
+         resident weights of a 12-layer model (302 MB of w1 matrices, above the last-level cache), 10 rounds.
+    The per-dispatch counter values of the gemv kernel, scaled by the copy kernel's ratio of known
+    bytes to counted units, give the HBM bytes per launch."""
+    import torch
+    awq = importlib.import_module("cuda-kernel-qwen3-8b-awq_amd")
+    src = torch.full((1 << 28,), 1.0, dtype=torch.float32, device="cuda")  # 1 GiB
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    del src, dst
+    eng = awq.QWen3AWQInfer.from_synthetic(awq.make_config(n_layers=12, max_pos=256), 11)
+    us, nbytes = eng.time_linear(awq.T_W1, 10)
+    print("w1 launch: %.2f us, %d algorithmic bytes" % (us, nbytes))
+    eng.close()
+
+
+def mode_w4a16(args):
+    w4a16 = importlib.import_module("cuda-kernel-qwen3-8b-awq_amd.bench_w4a16")
+    print(json.dumps(w4a16.measure((1, 4, 16, 64, 128, 512, 2048), ("w1", "w2"))), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -41,6 +143,13 @@ def main():
     ap.add_argument("--cpu-prompt", type=int, default=16, help="prompt length of the CPU sample")
     ap.add_argument("--cpu-steps", type=int, default=112, help="generated tokens of the CPU sample (0 = skip)")
     ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--mode", choices=["decode", "attention", "prefill", "traffic", "w4a16"], default="decode")
+    ap.add_argument("--one-cache", action="store_true", help="--mode attention: every launch reads the same cache")
+    ap.add_argument("--lengths", default="32,128,256,576,1024,1280,2040,4096,8192,30000", help="--mode prefill")
+    ap.add_argument("--no-load-test", action="store_true",
+                    help="skip writing the 3.64 GB weight directory and timing the loader on it")
+    ap.add_argument("--no-spec-leg", action="store_true",
+                    help="skip the second decode run on weights drawn from the benchmark definition's distributions")
     ap.add_argument("--profile", choices=["balanced", "spec"], default="balanced",
                     help="value distributions of the synthetic weights (include/awq_synth.h); 'spec' overflows "
                          "binary16 by layer 3 and decodes token 0 forever, so the default keeps activations finite")
@@ -49,6 +158,9 @@ def main():
         print("bench.py: this engine runs the whole model on ONE GPU (the reference's two-GPU layer split is "
               "collapsed onto one MI355X); --gpus %d is not supported, use --gpus 1" % args.gpus, file=sys.stderr)
         sys.exit(2)
+    if args.mode != "decode":
+        return {"attention": mode_attention, "prefill": mode_prefill, "traffic": mode_traffic,
+                "w4a16": mode_w4a16}[args.mode](args)
 
     import numpy as np
     import torch
@@ -75,13 +187,8 @@ def main():
         fill_pair(awq, oracle, cfg, args.seed, engine=eng, model=model, profile=profile)
     else:
         model = None
-        for layer, kind, part in awq.tensor_list(cfg):
-            count = cfg.part_count(kind, part)
-            nbytes = count if (part == awq.P_PACKED and kind != awq.T_GAMMA) else 2 * count
-            buf = (ctypes.c_uint8 * nbytes)()
-            awq.check(lib.awq_synth_fill_profile(profile, args.seed, layer, kind, part, buf, count))
-            eng.upload(layer, kind, part, buf, nbytes)
-        eng.finalize()
+        eng.close()
+        eng = _synthetic_engine(awq, lib, cfg, args.seed, profile)
     eng.set_graph_mode(not args.no_graph)
     log("weights generated, uploaded and reordered in %.1f s" % (time.time() - t0))
 
@@ -132,14 +239,7 @@ def main():
     # the same launches on ONE layer's matrices (25 MB, resident in the last-level cache): the
     # cache-hot figure next to the rotating one above
     hot_cfg = awq.make_config(n_layers=1, max_pos=64)
-    hot = awq.QWen3AWQInfer.empty(hot_cfg)
-    for layer, kind, part in awq.tensor_list(hot_cfg):
-        count = hot_cfg.part_count(kind, part)
-        nbytes = count if (part == awq.P_PACKED and kind != awq.T_GAMMA) else 2 * count
-        buf = (ctypes.c_uint8 * nbytes)()
-        awq.check(lib.awq_synth_fill_profile(profile, args.seed, layer, kind, part, buf, count))
-        hot.upload(layer, kind, part, buf, nbytes)
-    hot.finalize()
+    hot = _synthetic_engine(awq, lib, hot_cfg, args.seed, profile)
     for name, kind in (("w1", awq.T_W1), ("wqkv", awq.T_WQKV), ("w2", awq.T_W2), ("wo", awq.T_WO)):
         us, _ = hot.time_linear(kind, 400)
         kernels[name]["us_cache_hot"] = round(us, 3)
@@ -204,6 +304,56 @@ def main():
                     "frac": g["mfma_frac"], "us_per_launch": g["us"]}
     log("gemm w1 x 2048 tokens: %.1f us, %.0f TFLOP/s (%.1f%% of 2.5 PFLOP/s)" % (g["us"], g["TFLOPs"], 100 * g["mfma_frac"]))
 
+    # ---- the same decode run on weights drawn from the benchmark definition's own distributions (scale
+    #      U[0.002,0.02], zero-point 0..15): activations overflow binary16 within four layers and every id
+    #      is 0, so it proves nothing about the arithmetic, but it shows that the rate does not depend on
+    #      the values -----------------------------------------------------------------------------------
+    spec_leg = None
+    if not args.no_spec_leg and args.profile == "balanced":
+        t6 = time.time()
+        spec = _synthetic_engine(awq, lib, cfg, args.seed, awq.SYNTH_SPEC)
+        spec.set_graph_mode(not args.no_graph)
+        spec.prefill(prompt.tolist())
+        spec.decode(args.warmup)
+        torch.cuda.synchronize()
+        t7 = time.perf_counter()
+        spec_ids = spec.decode(args.steps)
+        torch.cuda.synchronize()
+        spec_elapsed = time.perf_counter() - t7
+        spec.close()
+        spec_leg = {"value": round(args.steps / spec_elapsed, 2), "unit": "tok/s",
+                    "ms_per_step": round(1000.0 * spec_elapsed / args.steps, 4),
+                    "data": "scale U[0.002,0.02], zero-point 0..15 (benchmark definition): activations overflow "
+                            "binary16, distinct ids in the run: %d" % len(set(spec_ids))}
+        log("decode on the benchmark definition's distributions: %.1f tok/s (engine built in %.1f s)" %
+            (spec_leg["value"], time.time() - t6))
+
+    # ---- the loader on a weight directory in the reference's layout (474 files, 3.64 GB), written just
+    #      before, so the files come from the page cache ---------------------------------------------------
+    load = None
+    if not args.no_load_test and args.layers == 36:
+        import shutil
+        import tempfile
+        d = tempfile.mkdtemp(prefix="awq_weights_")
+        try:
+            t8 = time.time()
+            awq.check(lib.awq_write_weight_dir_profile(d.encode(), ctypes.byref(cfg), args.seed, profile))
+            nbytes = sum(os.path.getsize(os.path.join(d, f)) for f in os.listdir(d))
+            log("weight directory written in %.1f s (%d bytes)" % (time.time() - t8, nbytes))
+            t9 = time.perf_counter()
+            loaded = awq.QWen3AWQInfer(d, config=awq.make_config(n_layers=args.layers, max_pos=2176))
+            create_s = time.perf_counter() - t9
+            load = {"load_s": round(lib.awq_last_load_seconds(), 3), "create_s": round(create_s, 3), "bytes": nbytes,
+                    "GBs": round(nbytes / lib.awq_last_load_seconds() / 1e9, 2),
+                    "what": "load_s: first file opened to last tensor reordered on the device (reader thread, two "
+                            "pinned buffers, copies and reordering overlapped); create_s: the whole awq_create with "
+                            "allocation, rotary tables and a zeroed 2176-position cache; page cache warm"}
+            loaded.close()
+            log("loader: %.2f s for %.2f GB (%.1f GB/s), whole constructor %.2f s" %
+                (load["load_s"], nbytes / 1e9, load["GBs"], create_s))
+        finally:
+            shutil.rmtree(d, ignore_errors=True)
+
     # ---- CPU oracle on this host's cores, bounded sample; and token identity on that sample ------
     cpu = None
     tokens_match = None
@@ -229,7 +379,9 @@ def main():
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int4 weights, f16 activations, f32 accumulate",
         "data": "synthetic (seeded random-init; nibbles uniform 0..15; %s)" % (
-            "scale U[0.0025,0.004], zero-point 7 or 8 so that activations stay finite" if args.profile == "balanced"
+            "value: scale U[0.0025,0.004], zero-point 7 or 8 so that activations stay finite; value_spec_profile: the "
+            "benchmark definition's scale U[0.002,0.02], zero-point 0..15, whose activations overflow FP16"
+            if args.profile == "balanced"
             else "scale U[0.002,0.02], zero-point 0..15 as in the benchmark definition: activations overflow FP16"),
         "config": {"workload": "full Qwen3-8B-shaped random-init AWQ model on one GPU: %d layers, hidden 4096, "
                                "intermediate 12288, vocab 151936, int4 g=128; %d-token prompt, batch-1 greedy decode"
@@ -239,6 +391,8 @@ def main():
         "step_algorithmic_bytes": int(step_bytes),
         "step_hbm_frac": round(step_bytes * tok_s / (HBM_PEAK_GBS * 1e9), 4),
         "greedy_tokens_identical_to_cpu": tokens_match,
+        "value_spec_profile": spec_leg,
+        "loader": load,
         "prompt_pass_ms": prefill_ms,
         "layer_512_positions": layer_cfg2,
         "long_context": long_context,

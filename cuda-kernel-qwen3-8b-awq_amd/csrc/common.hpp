@@ -144,7 +144,7 @@ int launch_rope_kv_append(const half_t* qkv, const half_t* cos_t, const half_t* 
                           hipStream_t st);
 // How the decode attention is launched, by an upper bound of the attended length
 // (measured in the decode loop of the 36-layer model, where every layer's cache
-// comes from HBM, and with bench_attention.py):
+// comes from HBM, and with the attention sweep of bench.py):
 //   <= kAttnOneWorkgroupMax  one workgroup per head does everything: a handful of
 //        memory round trips on 32 compute units (6 us at 256, 12.4 us at 704 positions);
 //   <= kAttnTwoLaunchMax     the keys are streamed by all compute units (scores and part
