@@ -143,7 +143,8 @@ def main():
     ap.add_argument("--cpu-prompt", type=int, default=16, help="prompt length of the CPU sample")
     ap.add_argument("--cpu-steps", type=int, default=112, help="generated tokens of the CPU sample (0 = skip)")
     ap.add_argument("--no-graph", action="store_true")
-    ap.add_argument("--mode", choices=["decode", "attention", "prefill", "traffic", "w4a16"], default="decode")
+    ap.add_argument("--mode", choices=["decode", "steps", "attention", "prefill", "traffic", "w4a16"], default="decode",
+                    help="decode: the benchmark line; steps: only the prompt and the timed decode steps (for traces)")
     ap.add_argument("--one-cache", action="store_true", help="--mode attention: every launch reads the same cache")
     ap.add_argument("--lengths", default="32,128,256,576,1024,1280,2040,4096,8192,30000", help="--mode prefill")
     ap.add_argument("--no-load-test", action="store_true",
@@ -158,7 +159,9 @@ def main():
         print("bench.py: this engine runs the whole model on ONE GPU (the reference's two-GPU layer split is "
               "collapsed onto one MI355X); --gpus %d is not supported, use --gpus 1" % args.gpus, file=sys.stderr)
         sys.exit(2)
-    if args.mode != "decode":
+    if args.mode == "steps":
+        args.cpu_steps = 0
+    if args.mode not in ("decode", "steps"):
         return {"attention": mode_attention, "prefill": mode_prefill, "traffic": mode_traffic,
                 "w4a16": mode_w4a16}[args.mode](args)
 
@@ -194,6 +197,18 @@ def main():
 
     prompt = np.zeros(args.prompt_len, dtype=np.int32)
     awq.check(lib.awq_synth_tokens(args.seed, awq.SYNTH_STREAM_INPUT, ptr(prompt), prompt.size, cfg.vocab))
+
+    if args.mode == "steps":
+        eng.prefill(prompt.tolist(), batched=True)
+        eng.decode(args.warmup)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        eng.decode(args.steps)
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t1
+        print(json.dumps({"mode": "steps", "prompt_len": args.prompt_len, "steps": args.steps,
+                          "tok_s": round(args.steps / elapsed, 1), "ms_per_step": round(1e3 * elapsed / args.steps, 4)}))
+        return
 
     # ---- the prompt pass, both ways (not part of `value`): token by token as the reference does,
     #      and all positions through each layer together on the matrix cores ---------------------

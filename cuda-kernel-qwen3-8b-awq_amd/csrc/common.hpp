@@ -114,6 +114,16 @@ struct LinearArgs {
   unsigned long long* best = nullptr;  // EPI_ARGMAX: zero between launches
   int32_t* out_token = nullptr;
   int32_t* out_array = nullptr;
+  // EPI_ARGMAX in the engine's decode step: the small launch that turns the best candidate into the token also
+  // ends the step (keeps a copy of the hidden state, gathers the sampled token's embedding into it for the
+  // next step, advances the step state)
+  half_t* fin_hidden = nullptr;        // [fin_n], null = the launch only samples
+  half_t* fin_hidden_last = nullptr;
+  const uint8_t* fin_emb = nullptr;    // the embedding's token rows (launch_embed_rows), fin_n/2 bytes each
+  const half_t* fin_emb_scale = nullptr;
+  const half_t* fin_emb_zp = nullptr;
+  int32_t fin_n = 0;
+  StepState* fin_state = nullptr;
 };
 
 // Greedy sampling key: an order-preserving integer image of a binary16 logit
@@ -183,6 +193,8 @@ int launch_gelu(half_t* x, int64_t n, hipStream_t st);
 int64_t argmax_workspace_bytes(int64_t n);
 int launch_argmax(const half_t* logits, int64_t n, int32_t* out_token, void* ws, const StepState* dyn,
                   int32_t* out_array, hipStream_t st);
+// token rows of the packed embedding: rows[tok][hidden/2], low nibble = even hidden element
+int launch_embed_rows(const uint8_t* packed, uint8_t* rows, int64_t hidden, int64_t vocab, hipStream_t st);
 int launch_embed(const uint8_t* packed, const half_t* scale, const half_t* zp, int64_t hidden, int64_t vocab,
                  int32_t tok, const StepState* dyn, const int32_t* tok_dev, half_t* out, hipStream_t st);
 int launch_set_state(StepState* dst, StepState v, hipStream_t st);

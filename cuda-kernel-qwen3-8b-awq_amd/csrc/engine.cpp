@@ -151,9 +151,11 @@ struct awq_engine {
   half_t *cos_t = nullptr, *sin_t = nullptr;
   // activations (Inference.cu:334-348)
   half_t *hidden = nullptr, *q = nullptr, *ctx = nullptr, *mid = nullptr, *logits = nullptr;
+  half_t* hidden_last = nullptr;  // the last layer's output of the latest generation step (hidden then holds the next input)
   // workspaces
   void* attn_ws = nullptr;
-  void* sample_ws = nullptr;  // 64-bit best candidate of the sampler
+  void* sample_ws = nullptr;  // best candidate and workgroup counts of the sampling launch
+  uint8_t* embed_rows = nullptr;  // the embedding transposed into token rows, for the sampling launch's gather
   StepState* d_state = nullptr;
   int32_t* d_token = nullptr;
   int32_t* d_out = nullptr;
@@ -301,16 +303,26 @@ int enqueue_sample(awq_engine* e) {
   a.best = (unsigned long long*)e->sample_ws;
   a.out_token = e->d_token;
   a.out_array = e->d_out;
+  // the launch also ends the step: the sampled token's embedding becomes the next input (:1384-1398)
+  a.fin_hidden = e->hidden;
+  a.fin_hidden_last = e->hidden_last;
+  a.fin_emb = e->embed_rows;
+  a.fin_emb_scale = e->embed.scale;
+  a.fin_emb_zp = e->embed.zp;
+  a.fin_n = e->cfg.hidden;
+  a.fin_state = e->d_state;
   return launch_gemv(a, e->stream);
 }
 
 // everything of one position after the step state has been written
 int enqueue_step_body(awq_engine* e, bool gen, int64_t len_bound) {
-  // embedding gather (Inference.cu:1310-1324, 1384-1398), skipped on the device
-  // when the state says to keep the hidden state (:1357)
-  if (int rc = launch_embed(e->embed.packed, e->embed.scale, e->embed.zp, e->cfg.hidden, e->cfg.vocab, 0, e->d_state,
-                            e->d_token, e->hidden, e->stream))
-    return rc;
+  // Prompt positions gather their token's embedding (Inference.cu:1310-1324).  A generation step starts
+  // from the hidden state as it stands: the last layer's output after the prompt (:1357), afterwards the
+  // embedding that the previous step's sampling launch gathered (:1384-1398).
+  if (!gen)
+    if (int rc = launch_embed(e->embed.packed, e->embed.scale, e->embed.zp, e->cfg.hidden, e->cfg.vocab, 0,
+                              e->d_state, e->d_token, e->hidden, e->stream))
+      return rc;
   const int split = gen ? e->cfg.split_idx : 1;
   for (int l = 0; l < e->cfg.n_layers; ++l)
     if (int rc = enqueue_layer(e, l, l >= split, len_bound)) return rc;
@@ -333,8 +345,10 @@ int build_graph(awq_engine* e, bool gen, int64_t len_bound, hipGraphExec_t* out)
   return AWQ_OK;
 }
 
-int run_step(awq_engine* e, bool gen, StepState s) {
-  if (int rc = launch_set_state(e->d_state, s, e->stream)) return rc;
+// `write_state` false: the device already holds `s` (the previous generation step advanced it)
+int run_step(awq_engine* e, bool gen, StepState s, bool write_state = true) {
+  if (write_state)
+    if (int rc = launch_set_state(e->d_state, s, e->stream)) return rc;
   // the attention launches are specialised by an upper bound of the attended
   // length (one workgroup per head, or two to four launches cut along the
   // sequence); one captured graph per bound
@@ -426,11 +440,12 @@ extern "C" int awq_create_empty(const awq_config* cfg_in, awq_engine** out) {
   struct {
     half_t** p;
     int64_t n;
-  } acts[] = {{&e->hidden, H}, {&e->q, H}, {&e->ctx, H}, {&e->mid, I}, {&e->logits, V}};
+  } acts[] = {{&e->hidden, H}, {&e->hidden_last, H}, {&e->q, H}, {&e->ctx, H}, {&e->mid, I}, {&e->logits, V}};
   for (auto& a : acts)
     if (int rc = dev_alloc(ep, (void**)a.p, a.n * 2)) return fail(rc);
   if (int rc = dev_alloc(ep, &e->attn_ws, attention_workspace_bytes(e->n_heads, cfg.max_pos))) return fail(rc);
-  if (int rc = dev_alloc(ep, &e->sample_ws, 64)) return fail(rc);
+  if (int rc = dev_alloc(ep, &e->sample_ws, gemv_workspace_bytes(V, H))) return fail(rc);
+  if (int rc = dev_alloc(ep, (void**)&e->embed_rows, V * (H / 2))) return fail(rc);
   if (int rc = dev_alloc(ep, (void**)&e->d_state, sizeof(StepState))) return fail(rc);
   if (int rc = dev_alloc(ep, (void**)&e->d_token, 4)) return fail(rc);
   if (int rc = dev_alloc(ep, (void**)&e->d_out, (int64_t)cfg.max_pos * 4)) return fail(rc);
@@ -520,7 +535,8 @@ extern "C" int awq_finalize(awq_engine* e) {
     if (int rc = launch_fill_zero(L.kcache, kv_bytes, st)) return rc;
     if (int rc = launch_fill_zero(L.vcache, kv_bytes, st)) return rc;
   }
-  if (int rc = launch_fill_zero(e->sample_ws, 64, st)) return rc;
+  if (int rc = launch_fill_zero(e->sample_ws, gemv_workspace_bytes(e->cfg.vocab, e->cfg.hidden), st)) return rc;
+  if (int rc = launch_embed_rows((const uint8_t*)e->embed.packed, e->embed_rows, e->cfg.hidden, e->cfg.vocab, st)) return rc;
   if (int rc = launch_fill_zero(e->d_token, 4, st)) return rc;
   if (int rc = launch_fill_zero(e->hidden, (int64_t)e->cfg.hidden * 2, st)) return rc;
   AWQ_HIP_TRY(hipStreamSynchronize(st));
@@ -860,12 +876,11 @@ extern "C" int awq_decode(awq_engine* e, int32_t n_steps, int32_t* out_ids) {
     s.pos = pos;
     s.len_lo = e->current_seq_len + 1;  // layers below split_idx run before :1364
     s.len_hi = pos + 1;                 // the others after it
-    // first step: the hidden state left by the last layer is the input (:1357);
-    // afterwards: the embedding of the token sampled by the previous step (:1392)
-    s.token = (e->n_generated == 0) ? -1 : -2;
+    s.token = -1;
     s.out_index = e->n_generated;
     s.sample = 1;
-    if (int rc = run_step(e, true, s)) return rc;
+    // the state is written for the first step of the call; every step leaves the next one's on the device
+    if (int rc = run_step(e, true, s, i == 0)) return rc;
     e->current_seq_len = pos;
     e->n_positions = pos + 1;
     e->n_generated += 1;
@@ -890,7 +905,8 @@ extern "C" int awq_generate(awq_engine* e, const int32_t* prompt_ids, int32_t n_
 extern "C" int awq_read_hidden(awq_engine* e, uint16_t* host_dst) {
   AWQ_REQUIRE(e && host_dst, "NULL argument");
   AWQ_HIP_TRY(hipStreamSynchronize(e->stream));
-  AWQ_HIP_TRY(hipMemcpy(host_dst, e->hidden, (size_t)e->cfg.hidden * 2, hipMemcpyDeviceToHost));
+  const half_t* src = e->n_generated > 0 ? e->hidden_last : e->hidden;
+  AWQ_HIP_TRY(hipMemcpy(host_dst, src, (size_t)e->cfg.hidden * 2, hipMemcpyDeviceToHost));
   return AWQ_OK;
 }
 

@@ -162,6 +162,21 @@ struct GemvParams {
   unsigned long long* best;
 };
 
+// arguments of the sampling step's last launch
+struct SampleFinish {
+  unsigned long long* best;
+  int32_t* out_token;
+  int32_t* out_array;
+  const StepState* dyn;
+  half_t* hidden;  // null = only the token id is produced
+  half_t* hidden_last;
+  const uint8_t* emb_rows;
+  const half_t* emb_scale;
+  const half_t* emb_zp;
+  int32_t n;
+  StepState* state;
+};
+
 // the 16 finished rows of a workgroup; r = lane = row % 16, lanes 0..15 of wavefront 0
 __device__ __forceinline__ void epilogue(const GemvParams& p, int epi, int row, int r, float acc, half_t res) {
   half_t v = (half_t)acc;
@@ -223,6 +238,52 @@ __device__ __forceinline__ void epilogue(const GemvParams& p, int epi, int row, 
     }
     default:
       p.y[row] = v;
+  }
+}
+
+// Last launch of the sampling step (Inference.cu:1282-1290, then :1384-1398): turns the best candidate into
+// the token id and, in the engine's decode step, prepares the next step: a copy of the hidden state for
+// readers, the sampled token's embedding (gather lambda, Inference.cu:1310-1324) as the new hidden state,
+// and the step state advanced by one position.  One workgroup; the embedding comes from the table's
+// token rows, fin_n/2 contiguous bytes.  (Counting the GEMV's workgroups so that its last one does this
+// work was measured: the agent-scope release every workgroup then needs costs far more than this launch.)
+__global__ __launch_bounds__(256) void sample_finish_kernel(SampleFinish f) {
+  const int tid = threadIdx.x;
+  const unsigned long long b = *f.best;
+  const int32_t tok = (int32_t)(0xffffffffu - (uint32_t)(b & 0xffffffffull));
+  if (f.hidden) {
+    const int g = (tok / AWQ_GROUP_SIZE) % (f.n / AWQ_GROUP_SIZE);
+    const half_t es = f.emb_scale[g], ez = f.emb_zp[g];
+    const uint8_t* row = f.emb_rows + (int64_t)tok * (f.n >> 1);
+    for (int i = tid; i < f.n / 8; i += 256) {  // 8 hidden elements = one dword of the row
+      const uint32_t w = *reinterpret_cast<const uint32_t*>(row + 4 * i);
+      const u32x4 keep = *reinterpret_cast<const u32x4*>(f.hidden + 8 * i);
+      union {
+        u32x4 v;
+        half_t h[8];
+      } o;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const half_t d = (half_t)(float)((w >> (4 * e)) & 15u) - ez;
+        o.h[e] = d * es;
+      }
+      *reinterpret_cast<u32x4*>(f.hidden_last + 8 * i) = keep;
+      *reinterpret_cast<u32x4*>(f.hidden + 8 * i) = o.v;
+    }
+  }
+  if (tid == 0) {
+    *f.out_token = tok;
+    if (f.out_array && f.dyn) f.out_array[f.dyn->out_index] = tok;
+    if (f.state) {
+      StepState s = *f.state;
+      s.pos += 1;
+      s.len_lo = s.pos;  // layers below the split still see the previous length (Inference.cu:1118, 1364)
+      s.len_hi = s.pos + 1;
+      s.token = -1;
+      s.out_index += 1;
+      *f.state = s;
+    }
+    *f.best = 0ull;
   }
 }
 
@@ -508,17 +569,6 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
   }
 }
 
-// Inference.cu:1282-1290, last step: turn the best candidate into the token id
-__global__ void sample_finish_kernel(unsigned long long* best, int32_t* out_token, const StepState* dyn,
-                                     int32_t* out_array) {
-  if (threadIdx.x != 0) return;
-  unsigned long long b = *best;
-  int32_t tok = (int32_t)(0xffffffffu - (uint32_t)(b & 0xffffffffull));
-  *out_token = tok;
-  if (out_array && dyn) out_array[dyn->out_index] = tok;
-  *best = 0;
-}
-
 struct GemvPlan {
   int g;        // blocks per lane: 1, 2, 4 or 8
   int n_waves;  // wavefronts per workgroup
@@ -660,7 +710,9 @@ int launch_gemv(const LinearArgs& a, hipStream_t st) {
   }
   AWQ_HIP_TRY(hipGetLastError());
   if (a.epilogue == EPI_ARGMAX) {
-    hipLaunchKernelGGL(sample_finish_kernel, dim3(1), dim3(64), 0, st, a.best, a.out_token, a.dyn, a.out_array);
+    SampleFinish f{a.best,      a.out_token, a.out_array,     a.dyn,        a.fin_hidden, a.fin_hidden_last,
+                   a.fin_emb,   a.fin_emb_scale, a.fin_emb_zp, a.fin_n,      a.fin_state};
+    hipLaunchKernelGGL(sample_finish_kernel, dim3(1), dim3(256), 0, st, f);
     AWQ_HIP_TRY(hipGetLastError());
   }
   return AWQ_OK;

@@ -91,6 +91,38 @@ __global__ __launch_bounds__(256) void embed_kernel(const uint8_t* __restrict__ 
   out[idx] = d * scale[g];
 }
 
+// One-time transposition of the packed [hidden][vocab] embedding into token rows: byte j of row tok holds
+// the weights of hidden elements 2j (low nibble) and 2j+1 (high nibble) of token tok, so that the gather
+// lambda's column (Inference.cu:1310-1324) is hidden/2 contiguous bytes.  A workgroup turns a tile of 128
+// hidden elements by 128 tokens through LDS; both sides move 64-byte runs.
+__global__ __launch_bounds__(256) void embed_rows_kernel(const uint8_t* __restrict__ packed, uint8_t* __restrict__ rows,
+                                                         int hidden, int64_t vocab) {
+  __shared__ uint32_t tile[128][17];  // [hidden element][16 words = 128 tokens], one word of skew
+  const int tid = threadIdx.x;
+  const int64_t tok0 = (int64_t)blockIdx.x * 128;
+  const int idx0 = blockIdx.y * 128;
+  const int c = tid & 15, r0 = tid >> 4;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int r = r0 + 16 * i;
+    tile[r][c] = *reinterpret_cast<const uint32_t*>(packed + (int64_t)(idx0 + r) * (vocab >> 1) + (tok0 >> 1) + 4 * c);
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int t = r0 + 16 * i;  // token of the tile; this thread writes bytes 4c..4c+3 of its row
+    uint32_t out = 0;
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const int e = 8 * c + 2 * b;
+      const uint32_t lo = (tile[e][t >> 3] >> (4 * (t & 7))) & 15u;
+      const uint32_t hi = (tile[e + 1][t >> 3] >> (4 * (t & 7))) & 15u;
+      out |= (lo | (hi << 4)) << (8 * b);
+    }
+    *reinterpret_cast<uint32_t*>(rows + (tok0 + t) * (hidden >> 1) + (idx0 >> 1) + 4 * c) = out;
+  }
+}
+
 // Greedy sampling (Inference.cu:1278-1290) without leaving the device.
 __global__ __launch_bounds__(256) void argmax_kernel(const uint16_t* __restrict__ logits, int64_t n,
                                                      unsigned long long* cand, int32_t* counter, int32_t* out_token,
@@ -202,6 +234,14 @@ int launch_embed(const uint8_t* packed, const half_t* scale, const half_t* zp, i
   AWQ_REQUIRE(dyn || (tok >= 0 && tok < vocab), "token id out of range");
   hipLaunchKernelGGL(embed_kernel, dim3((unsigned)((hidden + 255) / 256)), dim3(256), 0, st, packed, scale, zp,
                      (int)hidden, vocab, tok, dyn, tok_dev, out);
+  AWQ_HIP_TRY(hipGetLastError());
+  return AWQ_OK;
+}
+
+int launch_embed_rows(const uint8_t* packed, uint8_t* rows, int64_t hidden, int64_t vocab, hipStream_t st) {
+  AWQ_REQUIRE(hidden > 0 && hidden % 128 == 0 && vocab > 0 && vocab % 128 == 0, "bad embedding shape");
+  hipLaunchKernelGGL(embed_rows_kernel, dim3((unsigned)(vocab / 128), (unsigned)(hidden / 128)), dim3(256), 0, st,
+                     packed, rows, (int)hidden, vocab);
   AWQ_HIP_TRY(hipGetLastError());
   return AWQ_OK;
 }

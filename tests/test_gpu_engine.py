@@ -279,7 +279,7 @@ def test_config2_one_decoder_layer_at_position_512(awq, lib, oracle, torch_gpu):
     d_q = torch.zeros(H, dtype=torch.float16, device="cuda")
     d_ctx = torch.zeros(H, dtype=torch.float16, device="cuda")
     d_mid = torch.zeros(I, dtype=torch.float16, device="cuda")
-    ws = torch.zeros(4096, dtype=torch.uint8, device="cuda")
+    ws = torch.zeros(lib.awq_gemv_workspace_bytes(H, H), dtype=torch.uint8, device="cuda")
     att_ws = torch.zeros(lib.awq_attention_workspace_bytes(nh, mp), dtype=torch.uint8, device="cuda")
 
     def linear(kind, x, y, **kw):

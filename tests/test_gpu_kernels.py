@@ -504,7 +504,7 @@ def test_gemv_fused_norm_unembed_argmax(awq, lib, oracle, torch_gpu, m, k):
         torch.cuda.synchronize()
         assert np.array_equal(d_y.cpu().numpy().view(np.uint16), logits.view(np.uint16))
         assert int(tok.item()) == oracle.awqo_argmax(ptr(logits), m)
-    assert int(keep["ws"][:64].to(torch.int32).abs().sum().item()) == 0  # sampler workspace left zeroed
+    assert int(keep["ws"].to(torch.int32).abs().sum().item()) == 0  # sampler workspace left zeroed
 
 
 # ----------------------------------------------------------------------------- W4A16 GEMM on the matrix cores
