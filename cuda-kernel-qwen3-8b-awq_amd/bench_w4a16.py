@@ -68,10 +68,16 @@ def measure(tokens, shapes=("w1", "w2")):
                 else:
                     awq.check(lib.awq_gemm(w.data_ptr(), d_s.data_ptr(), d_z.data_ptr(), m, k, x.data_ptr(),
                                            y.data_ptr(), M, 1, gws.data_ptr(), st))
-            iters = 24 if M >= 512 else 120
-            for i in range(n_mat):
-                launch(i)
-            torch.cuda.synchronize()
+            iters = 48 if M >= 512 else 120
+            # warm-up by time, not by count: after an idle stretch (the host generating matrices) the
+            # device needs some tens of milliseconds of work before its clocks are back up; a timing
+            # taken right after 12 launches reads up to 20 % slow
+            import time
+            t_warm = time.perf_counter()
+            while time.perf_counter() - t_warm < 0.06:
+                for i in range(n_mat):
+                    launch(i)
+                torch.cuda.synchronize()
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
             for i in range(iters):

@@ -929,7 +929,20 @@ extern "C" int awq_time_linear(awq_engine* e, int kind, int32_t n_rounds, float*
   }
   AWQ_REQUIRE(kind == AWQ_T_WQKV || kind == AWQ_T_WO || kind == AWQ_T_W1 || kind == AWQ_T_W2 || kind == AWQ_T_UNEMBED,
               "kind must be a linear layer");
-  hipEvent_t ev0, ev1;
+  // events and the graph are released on every way out
+  struct Held {
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    ~Held() {
+      if (exec) (void)hipGraphExecDestroy(exec);
+      if (graph) (void)hipGraphDestroy(graph);
+      if (ev0) (void)hipEventDestroy(ev0);
+      if (ev1) (void)hipEventDestroy(ev1);
+    }
+  } held;
+  hipEvent_t& ev0 = held.ev0;
+  hipEvent_t& ev1 = held.ev1;
   AWQ_HIP_TRY(hipEventCreate(&ev0));
   AWQ_HIP_TRY(hipEventCreate(&ev1));
   const int n_mats = kind == AWQ_T_UNEMBED ? 1 : e->cfg.n_layers;
@@ -984,8 +997,8 @@ extern "C" int awq_time_linear(awq_engine* e, int kind, int32_t n_rounds, float*
   if (int rc = one_round()) return rc;  // warm-up
   // A round is replayed as a captured graph, which is how the decode step issues
   // these launches: the host's launch rate stays out of the figure.
-  hipGraph_t graph = nullptr;
-  hipGraphExec_t exec = nullptr;
+  hipGraph_t& graph = held.graph;
+  hipGraphExec_t& exec = held.exec;
   // (with few matrices several rounds go into one graph, so that a replay is long
   // against the cost of starting one)
   const int per_graph = std::min<int>(n_rounds, std::max(1, 32 / n_mats));
@@ -994,13 +1007,9 @@ extern "C" int awq_time_linear(awq_engine* e, int kind, int32_t n_rounds, float*
   int crc = AWQ_OK;
   for (int r = 0; r < per_graph && crc == AWQ_OK; ++r) crc = one_round();
   hipError_t cerr = hipStreamEndCapture(e->stream, &graph);
-  if (crc || cerr != hipSuccess) {
-    if (graph) (void)hipGraphDestroy(graph);
-    if (crc) return crc;
-    AWQ_HIP_TRY(cerr);
-  }
+  if (crc) return crc;
+  AWQ_HIP_TRY(cerr);
   AWQ_HIP_TRY(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0));
-  AWQ_HIP_TRY(hipGraphDestroy(graph));
   AWQ_HIP_TRY(hipGraphLaunch(exec, e->stream));  // warm-up of the graph itself
   AWQ_HIP_TRY(hipEventRecord(ev0, e->stream));
   for (int r = 0; r < replays; ++r) AWQ_HIP_TRY(hipGraphLaunch(exec, e->stream));
@@ -1008,15 +1017,12 @@ extern "C" int awq_time_linear(awq_engine* e, int kind, int32_t n_rounds, float*
   AWQ_HIP_TRY(hipEventSynchronize(ev1));
   float ms = 0.0f;
   AWQ_HIP_TRY(hipEventElapsedTime(&ms, ev0, ev1));
-  (void)hipGraphExecDestroy(exec);
   *avg_us_per_launch = ms * 1000.0f / (float)((int64_t)replays * per_graph * n_mats);
   if (bytes_per_launch) {
     const DevLinear& t = *find_linear(e, 0, kind);
     // packed weights + scales + zero-points + input vector + output vector
     *bytes_per_launch = t.m * (t.k / 2) + 2 * (t.m / 128) * 2 + t.k * 2 + t.m * 2;
   }
-  (void)hipEventDestroy(ev0);
-  (void)hipEventDestroy(ev1);
   return awq_reset(e);
 }
 

@@ -582,11 +582,13 @@ __global__ __launch_bounds__(256, (MODE == WIDE_K && TT == 4) ? 1 : ((MODE == WI
               __hip_atomic_store(mine + ((a * TT + t) * 8 + i) * 256 + tl, __builtin_bit_cast(u64, v), __ATOMIC_RELAXED,
                                  __HIP_MEMORY_SCOPE_AGENT);
             }
+        // every wavefront's sums have reached the device-coherent level before the barrier; the count is a
+        // release at agent scope, paired with the acquire after the owner's wait below
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         if (tid == 0) {
           const int owner = sk_wg_of((int64_t)(tile + 1) * S2 - 1, W2, gridDim.x);
-          __hip_atomic_fetch_add(p.sk_head + 16 + owner, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_fetch_add(p.sk_head + 16 + owner, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
         }
         continue;
       }
@@ -602,6 +604,7 @@ __global__ __launch_bounds__(256, (MODE == WIDE_K && TT == 4) ? 1 : ((MODE == WI
               break;
             }
           }
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");  // the counted workgroups' sums are visible from here
           __hip_atomic_store(p.sk_head + 16 + b, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
         }
         __syncthreads();

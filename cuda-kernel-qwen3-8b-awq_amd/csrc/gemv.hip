@@ -588,12 +588,19 @@ bool plan_gemv(int64_t m, int64_t k, GemvPlan* out) {
     found = true;
     if (groups / 4 >= 4 && (m / 16) * (groups / 4) >= 2048) break;
   }
+  // many row groups per workgroup (the unembedding): eight wavefronts of four blocks per lane keep more
+  // loads in flight per SIMD than four wavefronts of eight
+  if (found && m / 16 > 1024 && out->g == 8 && out->n_waves == 4) *out = GemvPlan{4, 8};
   return found;
 }
 
 #define GEMV_HOT_ARGS p.wq, p.x, p.gamma, p.scale, p.zp, p.m, p.prologue, p.epilogue, p.eps, p.mg, p.kg
 template <int G>
 void launch_g(const GemvParams& p, bool periodic, bool multi, dim3 grid, dim3 block, size_t lds, hipStream_t st) {
+  if (G == 4 && periodic && p.nblk / p.C == 4 && p.n_waves == 8) {  // the unembedding: one class of 4 blocks per lane
+    hipLaunchKernelGGL((gemv_kernel<G, true, G == 4 ? 4 : 0, 8, true>), grid, block, lds, st, GEMV_HOT_ARGS, p);
+    return;
+  }
   if (G == 8 && periodic && p.nblk / p.C == 4) {  // the unembedding: classes of 4 blocks
     if (p.n_waves == 4) hipLaunchKernelGGL((gemv_kernel<G, true, G == 8 ? 4 : 0, 4, true>), grid, block, lds, st, GEMV_HOT_ARGS, p);
     else hipLaunchKernelGGL((gemv_kernel<G, true, G == 8 ? 4 : 0>), grid, block, lds, st, GEMV_HOT_ARGS, p);
@@ -697,7 +704,8 @@ int launch_gemv(const LinearArgs& a, hipStream_t st) {
   // one workgroup per row group while that fits the device a few times over;
   // beyond that a workgroup walks several row groups and stages x once
   int64_t n_rg = a.m / 16, n_wg = n_rg;
-  if (n_rg > 1024) n_wg = 1024;
+  if (n_rg > 1024) n_wg = 4096 / plan.n_waves;  // four wavefronts per SIMD (measured: 151936 x 4096 as 512 workgroups of
+                                                // 8 wavefronts 59 us, as 1024 of 4 wavefronts 63 us, 576 of 8: 80 us)
   dim3 grid((unsigned)n_wg), block((unsigned)(plan.n_waves * 64));
   // x in block order plus 16 bytes of skew per lane group, the block sums, and with the fused norm x in natural order
   size_t lds = (size_t)a.k * 2 + (size_t)(a.k / AWQ_BLOCK_K / plan.g) * 16 + (size_t)(a.k / AWQ_BLOCK_K) * 4 +
