@@ -1049,14 +1049,7 @@ extern "C" int awq_gemv_fused(const awq_linear_args* u, void* stream) {
   AWQ_REQUIRE(u->m > 0 && u->m % 128 == 0, "m must be a positive multiple of 128");
   AWQ_REQUIRE(u->prologue == AWQ_PRO_NONE || u->prologue == AWQ_PRO_RMSNORM, "bad prologue");
   AWQ_REQUIRE(u->epilogue >= AWQ_EPI_STORE && u->epilogue <= AWQ_EPI_ARGMAX, "bad epilogue");
-  int zp_integral = u->zp_integral;
-  if (zp_integral < 0) {
-    // look at the zero-points on the device (synchronises the stream)
-    std::vector<uint16_t> zph((size_t)(u->m / 128));
-    AWQ_HIP_TRY(hipMemcpyAsync(zph.data(), u->zp, zph.size() * 2, hipMemcpyDeviceToHost, (hipStream_t)stream));
-    AWQ_HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
-    zp_integral = zp_all_integral(zph.data(), (int64_t)zph.size());
-  }
+  // zp_integral is not looked at: the block-sum arithmetic has no special case for integral zero-points
   LinearArgs a;
   a.wq = u->repacked;
   a.scale = (const half_t*)u->scale;
@@ -1067,7 +1060,7 @@ extern "C" int awq_gemv_fused(const awq_linear_args* u, void* stream) {
   a.best = (unsigned long long*)u->workspace;  // the sampler's best candidate
   a.m = u->m;
   a.k = u->k;
-  a.zp_integral = zp_integral != 0;
+  a.zp_integral = false;
   a.prologue = u->prologue;
   a.epilogue = u->epilogue;
   a.gamma = (const half_t*)u->gamma;

@@ -155,12 +155,15 @@ int awq_linear_repack(const void* packed_in, void* repacked_out, int64_t m, int6
 
 /* cublasGemmEx with n = 1, Inference.cu:1052-1065, 1128-1141, 1176-1189,
  * 1201-1214, 1260-1273, fused with the dequantisation:
- *     y[i] = h( sum_j w(i,j) * x[j] ),  FP32 accumulation in the blocked order
- *     of awq_canon_math.h.
+ *     y[i] = h( sum over blocks of 32 inputs of s * (sum q*x - z * sum x) ),
+ *     FP32 in the blocked order of awq_canon_math.h (q the raw nibble; scale
+ *     and zero-point are applied to a block's sums, not to every weight).
  * repacked from awq_linear_repack; scale/zp [m/128]; x [k], y [m] FP16.
- * zp_integral: 1 when every zero-point is an integer in [0,1024] (true of AWQ
- * checkpoints) -- a shorter instruction sequence with the same bits; 0 for
- * arbitrary zero-points; -1 to have the call inspect them (synchronises).
+ * zp_integral: kept for the matrix-core product (awq_gemm), where 1 selects a
+ * shorter conversion for zero-points that are integers in [0,1024] (true of
+ * AWQ checkpoints), 0 takes arbitrary zero-points and -1 has the call inspect
+ * them (synchronises); awq_gemv and awq_gemv_fused accept and ignore it: their
+ * arithmetic has no special case.
  * k <= 16384 (the workgroup keeps x in LDS).
  * workspace: awq_gemv_workspace_bytes(m,k) bytes, zero-filled once before its
  * first use (launches leave it zeroed); must not be shared by launches that

@@ -12,8 +12,11 @@
 //   function            follows            pinned by
 //   awqo_dequant        I:76-106           exhaustive nibble x (scale,zp) grid vs an
 //                                          integer-only soft-float; byte 0xA3 known answer
-//   awqo_linear*        I:1052-1065 (+4)   FP64 brute force, one-hot weight probe of the
-//                                          column-major reading, M>1 == M single products
+//   awqo_linear*        I:1052-1065 (+4)   FP64 brute force over the unrounded weights, a second
+//                                          (numpy) statement of the block order, one-hot weight
+//                                          probe of the column-major reading, 1e-2 against the
+//                                          sequential FP32 sum over the reference's rounded
+//                                          weights, M>1 == M single products
 //   awqo_rmsnorm        I:111-145          constant-vector closed form, FP64 comparison
 //   awqo_rope_tables    I:443-454          pos 0 == (1,0), FP64 comparison
 //   awqo_rotary         I:150-177          pos 0 identity, pair structure, norm preservation
@@ -23,6 +26,13 @@
 //   awqo_argmax         I:1282-1290        ties -> lowest index, NaN rule
 //   awqo_embed          I:1310-1324        equals dequant of the [H][V] matrix, column tok
 //   awqo_generate       I:1297-1408        position/length schedule table, L bookkeeping
+//   awqo_kv_append      I:1094-1103        numpy [head][pos][128] indexing
+//   awqo_model_layer    I:1029-1230        one decoder layer composed in Python from the
+//                                          primitives above in the order of I:1035-1228, bit
+//                                          for bit (which gamma, what is rotated, where the
+//                                          cache rows go, which buffer the residual takes)
+//   awqo_model_sample   I:1235-1292        RMSNorm with the last layer's gamma + linear +
+//                                          argmax composed in Python, bit for bit
 //
 // Parity unpinned (no executable reference exists for them, see the notes in
 // each function): the accumulation order inside cuBLAS (I:1052), the bits of

@@ -110,6 +110,37 @@ def test_small_model_tokens_and_state_identical(awq, oracle, torch_gpu, graph):
     oracle.awqo_model_destroy(model)
 
 
+@pytest.mark.parametrize("graph", [False, True])
+def test_decode_in_pieces_equals_one_call(awq, oracle, torch_gpu, graph):
+    """awq_decode leaves the next step's state and input on the device (the sampled token's embedding in the
+    hidden buffer, the advanced position and lengths), and the host writes the state once per call: a
+    generation cut into calls of 1, 2, 0, 5 and 16 steps, with the hidden state and the logits read in
+    between, gives the tokens and the state of one call.  Also without a prompt, where the first step
+    starts from the zero hidden state."""
+    cfg = awq.make_config(**SMALL)
+    model = make_oracle_model(oracle, cfg)
+    eng = awq.QWen3AWQInfer.empty(cfg)
+    fill_pair(awq, oracle, cfg, 4321, engine=eng, model=model)
+    eng.set_graph_mode(graph)
+    for prompt in ([3, 1000, 77, 512, 9], []):
+        pieces = (1, 2, 0, 5, 16)
+        print("piecewise decode graph=", graph, "prompt", prompt, flush=True)
+        eng.reset()
+        eng.prefill(prompt)
+        got = []
+        for n in pieces:
+            got += eng.decode(n)
+            ref = oracle_generate(oracle, model, prompt, len(got))
+            assert got == ref
+            if got:
+                compare_state(awq, oracle, eng, model, cfg)   # reading does not disturb the sequence
+        assert len(set(got)) > 1
+    with pytest.raises(awq.AwqError):
+        eng.prefill([1])            # prompt tokens cannot follow generated ones
+    eng.close()
+    oracle.awqo_model_destroy(model)
+
+
 def test_unembed_period_model(awq, oracle, torch_gpu):
     """vocab/128 coprime to hidden/128 gives the unembedding the j-dependent scale groups of the
     real 151936 x 4096 matrix"""
