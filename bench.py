@@ -128,7 +128,8 @@ def mode_traffic(args):
 
 def mode_w4a16(args):
     w4a16 = importlib.import_module("cuda-kernel-qwen3-8b-awq_amd.bench_w4a16")
-    print(json.dumps(w4a16.measure((1, 4, 16, 64, 128, 512, 2048), ("w1", "w2"))), flush=True)
+    tokens = tuple(int(v) for v in args.tokens.split(","))
+    print(json.dumps(w4a16.measure(tokens, tuple(args.shapes.split(",")))), flush=True)
 
 
 def main():
@@ -147,6 +148,8 @@ def main():
                     help="decode: the benchmark line; steps: only the prompt and the timed decode steps (for traces)")
     ap.add_argument("--one-cache", action="store_true", help="--mode attention: every launch reads the same cache")
     ap.add_argument("--lengths", default="32,128,256,576,1024,1280,2040,4096,8192,30000", help="--mode prefill")
+    ap.add_argument("--tokens", default="1,4,16,64,128,512,2048", help="--mode w4a16: token counts")
+    ap.add_argument("--shapes", default="w1,w2", help="--mode w4a16: of w1 (12288x4096), w2 (4096x12288), wo (4096x4096)")
     ap.add_argument("--no-load-test", action="store_true",
                     help="skip writing the 3.64 GB weight directory and timing the loader on it")
     ap.add_argument("--no-spec-leg", action="store_true",

@@ -11,7 +11,7 @@ An optional argument lists the token counts to run, e.g. 128,2048; a second one 
 wo is the 4096 x 4096 attention output matrix).
 
 Weights rotate over several distinct matrices so that they come from HBM, not from cache.
-Prints one JSON object.  Run on the GPU box: python cuda-kernel-qwen3-8b-awq_amd/bench_w4a16.py
+Prints one JSON object.  Run on the GPU box: python bench.py --mode w4a16 [--tokens 128,2048] [--shapes w1,w2,wo]
 """
 import ctypes
 import importlib

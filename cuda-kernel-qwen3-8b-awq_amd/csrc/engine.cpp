@@ -294,7 +294,7 @@ int enqueue_layer(awq_engine* e, int l, int use_len_hi, int64_t len_bound) {
 
 // sampleNextToken, Inference.cu:1235-1292: final RMSNorm (gamma of the last
 // layer), unembedding and greedy argmax in one launch
-int enqueue_sample(awq_engine* e) {
+LinearArgs sample_args(awq_engine* e) {
   const int NL = e->cfg.n_layers;
   LinearArgs a = linear_args(e, e->unembed, e->hidden, e->logits);
   a.prologue = PRO_RMSNORM;
@@ -311,8 +311,10 @@ int enqueue_sample(awq_engine* e) {
   a.fin_emb_zp = e->embed.zp;
   a.fin_n = e->cfg.hidden;
   a.fin_state = e->d_state;
-  return launch_gemv(a, e->stream);
+  return a;
 }
+
+int enqueue_sample(awq_engine* e) { return launch_gemv(sample_args(e), e->stream); }
 
 // everything of one position after the step state has been written
 int enqueue_step_body(awq_engine* e, bool gen, int64_t len_bound) {
@@ -982,9 +984,11 @@ extern "C" int awq_time_linear(awq_engine* e, int kind, int32_t n_rounds, float*
           a.res = e->hidden;
           break;
         default:
-          a = linear_args(e, t, e->hidden, e->logits);
-          a.prologue = PRO_RMSNORM;
-          a.gamma = e->layers[e->cfg.n_layers - 1].gamma;
+          // the sampling launch as the decode step issues it (norm, logits, argmax, then the small
+          // launch that ends the step); both launches count as one in the average
+          a = sample_args(e);
+          a.out_array = nullptr;  // nothing is appended to the output and the step state stays as set below
+          a.fin_state = nullptr;
           break;
       }
       rc = launch_gemv(a, e->stream);

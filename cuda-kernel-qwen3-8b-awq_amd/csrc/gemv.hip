@@ -178,7 +178,8 @@ struct SampleFinish {
 };
 
 // the 16 finished rows of a workgroup; r = lane = row % 16, lanes 0..15 of wavefront 0
-__device__ __forceinline__ void epilogue(const GemvParams& p, int epi, int row, int r, float acc, half_t res) {
+__device__ __forceinline__ void epilogue(const GemvParams& p, int epi, int row, int r, float acc, half_t res,
+                                         unsigned long long& best_here) {
   half_t v = (half_t)acc;
   switch (epi) {
     case EPI_RESIDUAL:  // Inference.cu:1149-1155
@@ -218,22 +219,15 @@ __device__ __forceinline__ void epilogue(const GemvParams& p, int epi, int row, 
       return;
     }
     case EPI_ARGMAX: {
-      // Inference.cu:1278-1290 on the device: the best (value, lowest index)
-      // pair of the vocabulary is kept with a 64-bit atomic max, which does
-      // not depend on arrival order.  Most workgroups find a better candidate
-      // already there and skip the atomic.
+      // Inference.cu:1278-1290 on the device: the best (value, lowest index) pair is a maximum over
+      // 64-bit candidates, which does not depend on the order; each lane keeps the best of its rows
+      // and the workgroup publishes one candidate when it has walked all its row groups
       p.y[row] = v;
       const unsigned short bits = __builtin_bit_cast(unsigned short, v);
       int32_t key = awq_logit_key(bits);
       if (row == 0 && (bits & 0x7fffu) > 0x7c00u) key = INT32_MAX;  // a NaN at index 0 is never displaced
-      unsigned long long cand = awq_pack_candidate(key, (uint32_t)row);
-#pragma unroll
-      for (int mask = 1; mask < 16; mask <<= 1) {
-        unsigned long long o = __shfl_xor(cand, mask, 64);
-        cand = o > cand ? o : cand;
-      }
-      if (r == 0 && cand > __hip_atomic_load(p.best, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
-        __hip_atomic_fetch_max(p.best, cand, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const unsigned long long cand = awq_pack_candidate(key, (uint32_t)row);
+      best_here = cand > best_here ? cand : best_here;
       return;
     }
     default:
@@ -475,6 +469,7 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
 #pragma unroll
     for (int b = 0; b < G; ++b) xb[b] = xsum[blk0 + b];
   }
+  unsigned long long best_here = 0;  // EPI_ARGMAX: best candidate among this lane's rows
   for (int it = 0; rg < n_rg; rg += gridDim.x, ++it) {
     const int rg_next = MULTI ? rg + (int)gridDim.x : n_rg;
     if (MULTI && rg_next < n_rg) {
@@ -561,11 +556,22 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
 #pragma unroll
       for (int i = 1; i < 16; ++i)
         if (i < n) tot += t[i];
-      epilogue(p, epi, rg * 16 + r, r, tot, res);
+      epilogue(p, epi, rg * 16 + r, r, tot, res, best_here);
     }
     if (!MULTI) break;
 #pragma unroll
     for (int b = 0; b < G; ++b) w[b] = wn[b];
+  }
+  if (epi == EPI_ARGMAX && tid < 16) {
+    // one 64-bit atomic max per workgroup at most: a workgroup that finds a better candidate already
+    // there skips it (additions to one address are served one after the other)
+#pragma unroll
+    for (int mask = 1; mask < 16; mask <<= 1) {
+      const unsigned long long o = __shfl_xor(best_here, mask, 64);
+      best_here = o > best_here ? o : best_here;
+    }
+    if (r == 0 && best_here > __hip_atomic_load(p.best, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
+      __hip_atomic_fetch_max(p.best, best_here, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 }
 
@@ -704,8 +710,8 @@ int launch_gemv(const LinearArgs& a, hipStream_t st) {
   // one workgroup per row group while that fits the device a few times over;
   // beyond that a workgroup walks several row groups and stages x once
   int64_t n_rg = a.m / 16, n_wg = n_rg;
-  if (n_rg > 1024) n_wg = 4096 / plan.n_waves;  // four wavefronts per SIMD (measured: 151936 x 4096 as 512 workgroups of
-                                                // 8 wavefronts 59 us, as 1024 of 4 wavefronts 63 us, 576 of 8: 80 us)
+  if (n_rg > 1024) n_wg = 4096 / plan.n_waves;  // four wavefronts per SIMD (measured: 151936 x 4096 with argmax as 512
+                                                // workgroups of 8 wavefronts 60 us, as 1024 of 4 wavefronts 64 us, 576 of 8: 80 us)
   dim3 grid((unsigned)n_wg), block((unsigned)(plan.n_waves * 64));
   // x in block order plus 16 bytes of skew per lane group, the block sums, and with the fused norm x in natural order
   size_t lds = (size_t)a.k * 2 + (size_t)(a.k / AWQ_BLOCK_K / plan.g) * 16 + (size_t)(a.k / AWQ_BLOCK_K) * 4 +

@@ -113,7 +113,9 @@ int awq_set_graph_mode(awq_engine* e, int enabled);
  * engine's stream (a round is captured once and replayed as a graph, the way
  * the decode step issues these launches).  Returns the mean launch duration and the algorithmic bytes
  * of one launch (packed weights + scales + zero-points + input + output).
- * Resets the sequence. */
+ * AWQ_T_UNEMBED is timed as the decode step issues it: final norm, logits,
+ * argmax and the small launch that ends the step, counted as one launch.
+ * Overwrites the activations and resets the sequence. */
 int awq_time_linear(awq_engine* e, int kind, int32_t n_rounds, float* avg_us_per_launch, int64_t* bytes_per_launch);
 
 /* Destructor, Inference.cu:475-558 */
