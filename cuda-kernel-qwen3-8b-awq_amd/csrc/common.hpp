@@ -71,7 +71,7 @@ struct StepState {
   int32_t pos;        // position written to the KV cache this step
   int32_t len_lo;     // attended length for layers <  split
   int32_t len_hi;     // attended length for layers >= split
-  int32_t token;      // token to embed at the start of the step, -1 = keep the hidden state
+  int32_t token;      // prompt token to embed at the start of the step, -1 = keep the hidden state
   int32_t out_index;  // where the sampled token goes in the output array
   int32_t sample;     // 1 = run the sampler at the end of the step
 };
@@ -196,7 +196,7 @@ int launch_argmax(const half_t* logits, int64_t n, int32_t* out_token, void* ws,
 // token rows of the packed embedding: rows[tok][hidden/2], low nibble = even hidden element
 int launch_embed_rows(const uint8_t* packed, uint8_t* rows, int64_t hidden, int64_t vocab, hipStream_t st);
 int launch_embed(const uint8_t* packed, const half_t* scale, const half_t* zp, int64_t hidden, int64_t vocab,
-                 int32_t tok, const StepState* dyn, const int32_t* tok_dev, half_t* out, hipStream_t st);
+                 int32_t tok, const StepState* dyn, half_t* out, hipStream_t st);
 int launch_set_state(StepState* dst, StepState v, hipStream_t st);
 int launch_fill_zero(void* p, int64_t bytes, hipStream_t st);
 int launch_copy(const void* src, void* dst, int64_t bytes, hipStream_t st);

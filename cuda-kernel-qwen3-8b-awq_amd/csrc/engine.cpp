@@ -323,7 +323,7 @@ int enqueue_step_body(awq_engine* e, bool gen, int64_t len_bound) {
   // embedding that the previous step's sampling launch gathered (:1384-1398).
   if (!gen)
     if (int rc = launch_embed(e->embed.packed, e->embed.scale, e->embed.zp, e->cfg.hidden, e->cfg.vocab, 0,
-                              e->d_state, e->d_token, e->hidden, e->stream))
+                              e->d_state, e->hidden, e->stream))
       return rc;
   const int split = gen ? e->cfg.split_idx : 1;
   for (int l = 0; l < e->cfg.n_layers; ++l)
@@ -1178,5 +1178,5 @@ extern "C" int awq_embed_gather(const void* packed, const void* scale, const voi
                                 int32_t tok, void* out, void* stream) {
   AWQ_REQUIRE(packed && scale && zp && out, "NULL pointer");
   return launch_embed((const uint8_t*)packed, (const half_t*)scale, (const half_t*)zp, hidden, vocab, tok, nullptr,
-                      nullptr, (half_t*)out, (hipStream_t)stream);
+                      (half_t*)out, (hipStream_t)stream);
 }

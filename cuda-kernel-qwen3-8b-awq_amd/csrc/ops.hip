@@ -75,12 +75,11 @@ __global__ __launch_bounds__(256) void gelu_kernel(half_t* x, int64_t n) {
 __global__ __launch_bounds__(256) void embed_kernel(const uint8_t* __restrict__ packed,
                                                     const half_t* __restrict__ scale, const half_t* __restrict__ zp,
                                                     int hidden, int64_t vocab, int tok_arg, const StepState* dyn,
-                                                    const int32_t* tok_dev, half_t* __restrict__ out) {
+                                                    half_t* __restrict__ out) {
   int tok = tok_arg;
   if (dyn) {
     tok = dyn->token;
-    if (tok == -2) tok = *tok_dev;  // the token sampled by the previous step
-    if (tok < 0) return;            // keep the hidden state (Inference.cu:1357)
+    if (tok < 0) return;  // keep the hidden state (Inference.cu:1357)
   }
   int idx = blockIdx.x * 256 + threadIdx.x;
   if (idx >= hidden) return;
@@ -229,11 +228,11 @@ int launch_gelu(half_t* x, int64_t n, hipStream_t st) {
 }
 
 int launch_embed(const uint8_t* packed, const half_t* scale, const half_t* zp, int64_t hidden, int64_t vocab,
-                 int32_t tok, const StepState* dyn, const int32_t* tok_dev, half_t* out, hipStream_t st) {
+                 int32_t tok, const StepState* dyn, half_t* out, hipStream_t st) {
   AWQ_REQUIRE(hidden > 0 && hidden % 128 == 0 && vocab > 0 && vocab % 2 == 0, "bad embedding shape");
   AWQ_REQUIRE(dyn || (tok >= 0 && tok < vocab), "token id out of range");
   hipLaunchKernelGGL(embed_kernel, dim3((unsigned)((hidden + 255) / 256)), dim3(256), 0, st, packed, scale, zp,
-                     (int)hidden, vocab, tok, dyn, tok_dev, out);
+                     (int)hidden, vocab, tok, dyn, out);
   AWQ_HIP_TRY(hipGetLastError());
   return AWQ_OK;
 }
