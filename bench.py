@@ -250,7 +250,7 @@ def main():
     kernels = {}
     for name, kind in (("w1", awq.T_W1), ("wqkv", awq.T_WQKV), ("w2", awq.T_W2), ("wo", awq.T_WO),
                        ("unembed", awq.T_UNEMBED)):
-        us, nbytes = eng.time_linear(kind, 20 if kind != awq.T_UNEMBED else 200)
+        us, nbytes = eng.time_linear(kind, 60 if kind != awq.T_UNEMBED else 200)
         kernels[name] = {"us": round(us, 3), "bytes": nbytes, "GBs": round(nbytes / us / 1e3, 1)}
         log("gemv %-8s %8.2f us/launch  %7.1f GB/s  (%.1f%% of peak)" % (name, us, nbytes / us / 1e3,
                                                                         nbytes / us / 1e3 / HBM_PEAK_GBS * 100))

@@ -581,9 +581,11 @@ struct GemvPlan {
 };
 
 // Lane groups per workgroup = (k/32)/G must be a multiple of 4 and at most 64.
-// Prefer long per-lane runs (G = 8) unless that leaves the device with few
-// wavefronts.  G >= 2: a thread stages whole units of four inputs.
+// The longest per-lane run (G = 8, 4, 2) that still gives a workgroup eight wavefronts: with k = 4096
+// eight wavefronts of four blocks per lane beat four wavefronts of eight (12288 x 4096: 7.8 against
+// 8.2 us; sixteen wavefronts of two: 8.1 us).  G >= 2: a thread stages whole units of four inputs.
 bool plan_gemv(int64_t m, int64_t k, GemvPlan* out) {
+  (void)m;
   const int64_t nblk = k / AWQ_BLOCK_K;
   bool found = false;
   for (int g = 8; g >= 2; g >>= 1) {
@@ -592,11 +594,8 @@ bool plan_gemv(int64_t m, int64_t k, GemvPlan* out) {
     if (groups % 4 || groups > 64) continue;
     *out = GemvPlan{g, (int)(groups / 4)};
     found = true;
-    if (groups / 4 >= 4 && (m / 16) * (groups / 4) >= 2048) break;
+    if (groups / 4 >= 8) break;
   }
-  // many row groups per workgroup (the unembedding): eight wavefronts of four blocks per lane keep more
-  // loads in flight per SIMD than four wavefronts of eight
-  if (found && m / 16 > 1024 && out->g == 8 && out->n_waves == 4) *out = GemvPlan{4, 8};
   return found;
 }
 
@@ -607,9 +606,8 @@ void launch_g(const GemvParams& p, bool periodic, bool multi, dim3 grid, dim3 bl
     hipLaunchKernelGGL((gemv_kernel<G, true, G == 4 ? 4 : 0, 8, true>), grid, block, lds, st, GEMV_HOT_ARGS, p);
     return;
   }
-  if (G == 8 && periodic && p.nblk / p.C == 4) {  // the unembedding: classes of 4 blocks
-    if (p.n_waves == 4) hipLaunchKernelGGL((gemv_kernel<G, true, G == 8 ? 4 : 0, 4, true>), grid, block, lds, st, GEMV_HOT_ARGS, p);
-    else hipLaunchKernelGGL((gemv_kernel<G, true, G == 8 ? 4 : 0>), grid, block, lds, st, GEMV_HOT_ARGS, p);
+  if (G == 8 && periodic && p.nblk / p.C == 4) {  // classes of 4 blocks, long k
+    hipLaunchKernelGGL((gemv_kernel<G, true, G == 8 ? 4 : 0>), grid, block, lds, st, GEMV_HOT_ARGS, p);
     return;
   }
   if (periodic) {
@@ -617,8 +615,7 @@ void launch_g(const GemvParams& p, bool periodic, bool multi, dim3 grid, dim3 bl
     return;
   }
   // the per-layer matrices of the model: 4096 inputs as 4 wavefronts x 8 blocks or 8 x 4, 12288 as 12 x 8
-  if (!multi && G == 8 && p.n_waves == 4) hipLaunchKernelGGL((gemv_kernel<G, false, 0, 4, false>), grid, block, lds, st, GEMV_HOT_ARGS, p);
-  else if (!multi && G == 8 && p.n_waves == 12) hipLaunchKernelGGL((gemv_kernel<G, false, 0, 12, false>), grid, block, lds, st, GEMV_HOT_ARGS, p);
+  if (!multi && G == 8 && p.n_waves == 12) hipLaunchKernelGGL((gemv_kernel<G, false, 0, 12, false>), grid, block, lds, st, GEMV_HOT_ARGS, p);
   else if (!multi && G == 4 && p.n_waves == 8) hipLaunchKernelGGL((gemv_kernel<G, false, 0, 8, false>), grid, block, lds, st, GEMV_HOT_ARGS, p);
   else hipLaunchKernelGGL((gemv_kernel<G, false>), grid, block, lds, st, GEMV_HOT_ARGS, p);
 }
