@@ -310,14 +310,20 @@ __device__ __forceinline__ int xs_index(int e) {
 // own shapes: k, the staging loops and the reduction are then constants), 0 = take
 // it from the launch.  MULTI: the grid is smaller than the number of row groups
 // and a workgroup walks several of them.
-template <int G, bool PERIODIC, int UFAST = 0, int NWC = 0, bool MULTI = true>
+// RH: output rows per workgroup, 16 or 8.  With 8 a wavefront's lanes are (eighth q = lane/8, r = lane%8): a
+// workgroup takes half a 16-row group (its wavefront loads are eight 128-byte pieces) and covers the same
+// number of blocks per wavefront with half the blocks per lane, so a matrix with few rows and long k
+// (4096 x 12288: 256 row groups, 12 wavefronts each) runs as twice the workgroups -- two per compute unit.
+template <int G, bool PERIODIC, int UFAST = 0, int NWC = 0, bool MULTI = true, int RH = 16>
 __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
     const u32x4* __restrict__ wq, const half_t* __restrict__ x, const half_t* __restrict__ gamma,
     const half_t* __restrict__ scale, const half_t* __restrict__ zp, int32_t m, int32_t prologue, int32_t epi,
     float eps, int32_t mg, int32_t kg, GemvParams p) {
   const int n_waves = NWC ? NWC : p.n_waves;
-  const int k = NWC ? NWC * 128 * G : p.k;
-  const int nblk = NWC ? NWC * 4 * G : p.nblk;
+  constexpr int Q = 64 / RH;  // lanes that share a row = consecutive block ranges of a wavefront
+  static_assert(RH == 16 || (RH == 8 && !PERIODIC), "half row groups are for one scale group per 16 rows");
+  const int k = NWC ? NWC * Q * 32 * G : p.k;
+  const int nblk = NWC ? NWC * Q * G : p.nblk;
   const int C = PERIODIC ? p.C : 1;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   half_t* xs = reinterpret_cast<half_t*>(smem);                                  // k halves + skew
@@ -326,19 +332,20 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
   __shared__ float red[2][16][16];  // double-buffered: one barrier per row group
   __shared__ __attribute__((aligned(16))) float part[256];
   __shared__ GroupConst gtab[2][PERIODIC ? 64 : 1];
-  constexpr int MAXU = G / 2;  // units of four inputs a thread stages
-  static_assert(G >= 2, "a thread stages whole units");
+  constexpr int MAXU = G * Q / 8;  // units of four inputs a thread stages
+  static_assert(G * Q >= 8, "a thread stages whole units");
   const int tid = threadIdx.x;
   const int nthreads = n_waves * 64;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int q = lane >> 4, r = lane & 15;
-  const int n_rg = m >> 4;
-  const int blk0 = (4 * wave + q) * G;
+  const int q = lane / RH, r = lane % RH;
+  const int n_rg = m / RH;
+  const int blk0 = (Q * wave + q) * G;
   const int U = nblk / C;  // blocks per class (PERIODIC)
 
   int rg = blockIdx.x;
-  const u32x4* wp = wq + ((int64_t)rg * nblk + blk0) * 16 + r;
+  // row group of 16 in the weight stream and the row inside it
+  const u32x4* wp = wq + ((int64_t)(rg * RH >> 4) * nblk + blk0) * 16 + ((rg * RH) & 15) + r;
   u32x4 w[G], wn[G];
 
   // ---- x: unit u of a thread is the 4 consecutive block-order elements
@@ -410,7 +417,7 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
     // the butterfly leaves in lane 0 what the one-sided tree leaves in part[0])
     float pv[16];
 #pragma unroll
-    for (int j = 0; j < 16; ++j) pv[j] = part[r + 16 * j];
+    for (int j = 0; j < 16; ++j) pv[j] = part[(lane & 15) + 16 * j];
 #pragma unroll
     for (int n = 8; n >= 1; n >>= 1) {
 #pragma unroll
@@ -473,17 +480,17 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
   for (int it = 0; rg < n_rg; rg += gridDim.x, ++it) {
     const int rg_next = MULTI ? rg + (int)gridDim.x : n_rg;
     if (MULTI && rg_next < n_rg) {
-      const u32x4* wpn = wq + ((int64_t)rg_next * nblk + blk0) * 16 + r;
+      const u32x4* wpn = wq + ((int64_t)(rg_next * RH >> 4) * nblk + blk0) * 16 + ((rg_next * RH) & 15) + r;
 #pragma unroll
       for (int b = 0; b < G; ++b) wn[b] = __builtin_nontemporal_load(wpn + b * 16);
     }
     // the residual row is requested before the pass multiplies: the end of the
     // launch then does not wait for one more round trip to memory
     half_t res = (half_t)0.0f;
-    if (tid < 16 && epi == EPI_RESIDUAL) res = p.res[rg * 16 + r];
+    if (tid < RH && epi == EPI_RESIDUAL) res = p.res[rg * RH + r];
     // scale group of these 16 rows: row/128, then Inference.cu:90 with the index
     // wrapped to the m/128 stored entries
-    const int a = rg >> 3;
+    const int a = rg * RH >> 7;
     GroupConst g;
     if (!PERIODIC) {
       int gi = (a % kg) % mg;
@@ -530,15 +537,15 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
       for (int i = 0; i < n / 2; ++i) bs[i] = bs[2 * i] + bs[2 * i + 1];
     }
     float v = bs[0];
-    v += __shfl_xor(v, 16, 64);
-    v += __shfl_xor(v, 32, 64);
+#pragma unroll
+    for (int mask = RH; mask < 64; mask <<= 1) v += __shfl_xor(v, mask, 64);
     // The only barrier of the pass.  The 16 finishing lanes read this pass's
     // buffer while the other wavefronts already multiply the next row group; the
     // buffer is written again two passes on, after a barrier those lanes are part of.
     float(*rd)[16] = red[it & 1];
     if (q == 0) rd[wave][r] = v;
     __syncthreads();
-    if (tid < 16) {
+    if (tid < RH) {
       // awq_tree_sum over the wavefronts' sums, in registers (all reads in flight at once)
       float t[16];
 #pragma unroll
@@ -556,17 +563,17 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
 #pragma unroll
       for (int i = 1; i < 16; ++i)
         if (i < n) tot += t[i];
-      epilogue(p, epi, rg * 16 + r, r, tot, res, best_here);
+      epilogue(p, epi, rg * RH + r, r, tot, res, best_here);
     }
     if (!MULTI) break;
 #pragma unroll
     for (int b = 0; b < G; ++b) w[b] = wn[b];
   }
-  if (epi == EPI_ARGMAX && tid < 16) {
+  if (epi == EPI_ARGMAX && tid < RH) {
     // one 64-bit atomic max per workgroup at most: a workgroup that finds a better candidate already
     // there skips it (additions to one address are served one after the other)
 #pragma unroll
-    for (int mask = 1; mask < 16; mask <<= 1) {
+    for (int mask = 1; mask < RH; mask <<= 1) {
       const unsigned long long o = __shfl_xor(best_here, mask, 64);
       best_here = o > best_here ? o : best_here;
     }
@@ -578,6 +585,7 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
 struct GemvPlan {
   int g;        // blocks per lane: 1, 2, 4 or 8
   int n_waves;  // wavefronts per workgroup
+  int rh;       // output rows per workgroup: 16, or 8 (half a row group)
 };
 
 // Lane groups per workgroup = (k/32)/G must be a multiple of 4 and at most 64.
@@ -585,23 +593,34 @@ struct GemvPlan {
 // eight wavefronts of four blocks per lane beat four wavefronts of eight (12288 x 4096: 7.8 against
 // 8.2 us; sixteen wavefronts of two: 8.1 us).  G >= 2: a thread stages whole units of four inputs.
 bool plan_gemv(int64_t m, int64_t k, GemvPlan* out) {
-  (void)m;
   const int64_t nblk = k / AWQ_BLOCK_K;
   bool found = false;
   for (int g = 8; g >= 2; g >>= 1) {
     if (nblk % g) continue;
     int64_t groups = nblk / g;
     if (groups % 4 || groups > 64) continue;
-    *out = GemvPlan{g, (int)(groups / 4)};
+    *out = GemvPlan{g, (int)(groups / 4), 16};
     found = true;
     if (groups / 4 >= 8) break;
+  }
+  // few rows and long k (4096 x 12288: one 16-row workgroup of 12 wavefronts per compute unit): half the rows
+  // and half the blocks per lane, twice the workgroups (8.2 -> 7.55 us; 4096 x 4096 the same way: 4.3 -> 4.4 us,
+  // so only where a lane has eight blocks)
+  if (found && m / 16 <= 256 && out->g == 8 && out->n_waves >= 8) {
+    out->g = 4;
+    out->rh = 8;
   }
   return found;
 }
 
 #define GEMV_HOT_ARGS p.wq, p.x, p.gamma, p.scale, p.zp, p.m, p.prologue, p.epilogue, p.eps, p.mg, p.kg
 template <int G>
-void launch_g(const GemvParams& p, bool periodic, bool multi, dim3 grid, dim3 block, size_t lds, hipStream_t st) {
+void launch_g(const GemvParams& p, bool periodic, bool multi, int rh, dim3 grid, dim3 block, size_t lds, hipStream_t st) {
+  if (rh == 8) {  // plan_gemv: four blocks per lane, not periodic, one row group per workgroup
+    if (p.n_waves == 12) hipLaunchKernelGGL((gemv_kernel<4, false, 0, 12, false, 8>), grid, block, lds, st, GEMV_HOT_ARGS, p);
+    else hipLaunchKernelGGL((gemv_kernel<4, false, 0, 0, true, 8>), grid, block, lds, st, GEMV_HOT_ARGS, p);
+    return;
+  }
   if (G == 4 && periodic && p.nblk / p.C == 4 && p.n_waves == 8) {  // the unembedding: one class of 4 blocks per lane
     hipLaunchKernelGGL((gemv_kernel<G, true, G == 4 ? 4 : 0, 8, true>), grid, block, lds, st, GEMV_HOT_ARGS, p);
     return;
@@ -704,9 +723,13 @@ int launch_gemv(const LinearArgs& a, hipStream_t st) {
   p.dyn = a.dyn;
   p.best = a.best;
   const bool periodic = p.C > 1;
+  if (periodic && plan.rh == 8) {  // half row groups only with one scale group per 16 rows
+    plan.g *= 2;
+    plan.rh = 16;
+  }
   // one workgroup per row group while that fits the device a few times over;
   // beyond that a workgroup walks several row groups and stages x once
-  int64_t n_rg = a.m / 16, n_wg = n_rg;
+  int64_t n_rg = a.m / plan.rh, n_wg = n_rg;
   if (n_rg > 1024) n_wg = 4096 / plan.n_waves;  // four wavefronts per SIMD (measured: 151936 x 4096 with argmax as 512
                                                 // workgroups of 8 wavefronts 60 us, as 1024 of 4 wavefronts 64 us, 576 of 8: 80 us)
   dim3 grid((unsigned)n_wg), block((unsigned)(plan.n_waves * 64));
@@ -715,9 +738,9 @@ int launch_gemv(const LinearArgs& a, hipStream_t st) {
                (a.prologue == PRO_RMSNORM ? (size_t)a.k * 2 : 0);
   AWQ_REQUIRE(lds <= 65536, "k too large for the fused norm (x is kept twice in LDS)");
   switch (plan.g) {
-    case 2: launch_g<2>(p, periodic, n_wg < n_rg, grid, block, lds, st); break;
-    case 4: launch_g<4>(p, periodic, n_wg < n_rg, grid, block, lds, st); break;
-    default: launch_g<8>(p, periodic, n_wg < n_rg, grid, block, lds, st); break;
+    case 2: launch_g<2>(p, periodic, n_wg < n_rg, plan.rh, grid, block, lds, st); break;
+    case 4: launch_g<4>(p, periodic, n_wg < n_rg, plan.rh, grid, block, lds, st); break;
+    default: launch_g<8>(p, periodic, n_wg < n_rg, plan.rh, grid, block, lds, st); break;
   }
   AWQ_HIP_TRY(hipGetLastError());
   if (a.epilogue == EPI_ARGMAX) {

@@ -99,8 +99,9 @@ def gemv_gpu(awq, lib, torch, packed, scale, zp, m, k, x, zp_integral, repeat=1)
     return outs
 
 
+# the last two: few rows and long k, where a workgroup takes half a row group (general and 16-wavefront forms)
 GEMV_SHAPES = [(128, 512), (256, 1024), (384, 512), (128, 1536), (640, 2048), (4096, 4096), (12288, 4096),
-               (4096, 12288)]
+               (4096, 12288), (512, 8192), (1024, 16384)]
 
 
 @pytest.mark.parametrize("m,k", GEMV_SHAPES)
