@@ -9,7 +9,7 @@
 // Cache layout [head][max_pos][128] FP16 (Inference.cu:1097): a position is one
 // 256-byte row, so a wavefront load of 16 bytes per lane covers 4 positions.
 //
-// One workgroup of NW wavefronts per head (16 for decode).  Scores: the
+// Workgroups of NW wavefronts (16 for decode), kHeadParts per head.  Scores: the
 // positions go round the wavefronts in groups of 4, so all wavefronts stream
 // keys even for short sequences.  Context: one wavefront per chunk.
 #include "common.hpp"
@@ -23,6 +23,8 @@ constexpr int kLdsChunks = 32;      // chunk vectors kept in LDS up to this many
 constexpr int kWaves = 16;   // wavefronts per workgroup of the decode variants
 constexpr int kThreads = kWaves * 64;
 constexpr int kSplit = 32;   // parts per head when the sequence is cut over several workgroups
+constexpr int kHeadParts = 4;  // workgroups per head in attention_kernel, a quarter of the head's dimensions each
+                               // (decode at 448..576 positions: 683 tok/s with one, 706 with two, 716 with four)
 
 // v + (value of lane ^ mask) inside a row of 16 lanes.  After the xor-1 and
 // xor-2 steps all four lanes of a quad hold the same sum, so mirroring inside
@@ -62,7 +64,11 @@ __device__ __forceinline__ float wave_tree_sum(float v) {
 // FROM_SCORES: the scores and the maxima of their kSplit parts were left in memory
 // by attn_scores_kernel (all compute units stream the keys); this launch does the
 // rest of the head.
-template <int NW, int SCAP, int CCAP, bool FROM_SCORES = false>
+// DS: workgroups per head (blockIdx.y).  Every one of them computes the head's scores, exponentials and
+// sums (the same instructions on the same data: the same bits) and then the context of its 128/DS of the
+// head's dimensions, i.e. it reads all keys but only 1/DS of every value row.  One compute unit keeps only
+// about 37 KB of requests in flight, so the bytes a unit has to pull set the time beyond about 128 positions.
+template <int NW, int SCAP, int CCAP, bool FROM_SCORES = false, int DS = 1>
 __global__ __launch_bounds__(NW * 64) void attention_kernel(const half_t* __restrict__ q,
                                                              const half_t* __restrict__ kc,
                                                              const half_t* __restrict__ vc, half_t* __restrict__ ctx,
@@ -73,9 +79,13 @@ __global__ __launch_bounds__(NW * 64) void attention_kernel(const half_t* __rest
   __shared__ float cs[CCAP];
   __shared__ float wmax[NW];
   __shared__ float s[SCAP];
-  __shared__ float cv[CCAP * AWQ_HEAD_DIM];
+  constexpr int DP = AWQ_HEAD_DIM / DS;  // dimensions of this workgroup
+  constexpr int DL = 8 / DS;             // dimensions per lane in the context phase
+  typedef _Float16 vrow_t __attribute__((ext_vector_type(DL)));
+  __shared__ float cv[CCAP * DP];
   const int L = dyn ? (use_len_hi ? dyn->len_hi : dyn->len_lo) : L_arg;
   const int head = blockIdx.x;
+  const int d0 = blockIdx.y * DP;  // first dimension of this workgroup
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int tq = lane >> 4, dl = lane & 15;
   const half_t* kh = kc;
@@ -83,7 +93,7 @@ __global__ __launch_bounds__(NW * 64) void attention_kernel(const half_t* __rest
   const int nchunks = (L + 63) >> 6;
   const float scale = 1.0f / sqrtf((float)AWQ_HEAD_DIM);  // Inference.cu:218
 
-  half8_t vv[16];
+  vrow_t vv[16];
   float mx;
   if constexpr (FROM_SCORES) {
     // the values of this wavefront's first chunk travel while the scores arrive
@@ -91,7 +101,7 @@ __global__ __launch_bounds__(NW * 64) void attention_kernel(const half_t* __rest
 #pragma unroll
       for (int nl = 0; nl < 16; ++nl) {
         const int t = (wave << 6) + 4 * nl + tq;
-        if (t < L) vv[nl] = *reinterpret_cast<const half8_t*>(vh + kv_row(lay, head, t) + 8 * dl);
+        if (t < L) vv[nl] = *reinterpret_cast<const vrow_t*>(vh + kv_row(lay, head, t) + d0 + DL * dl);
       }
     }
     for (int t = tid; t < L; t += NW * 64) s[t] = scores_g[(int64_t)head * max_pos + t];
@@ -124,7 +134,7 @@ __global__ __launch_bounds__(NW * 64) void attention_kernel(const half_t* __rest
 #pragma unroll
       for (int nl = 0; nl < 16; ++nl) {
         const int t = (wave << 6) + 4 * nl + tq;
-        if (t < L) vv[nl] = *reinterpret_cast<const half8_t*>(vh + kv_row(lay, head, t) + 8 * dl);
+        if (t < L) vv[nl] = *reinterpret_cast<const vrow_t*>(vh + kv_row(lay, head, t) + d0 + DL * dl);
       }
     }
 #pragma unroll
@@ -175,39 +185,39 @@ __global__ __launch_bounds__(NW * 64) void attention_kernel(const half_t* __rest
 #pragma unroll
       for (int nl = 0; nl < 16; ++nl) {
         const int t = base + 4 * nl + tq;
-        if (t < L) vv[nl] = *reinterpret_cast<const half8_t*>(vh + kv_row(lay, head, t) + 8 * dl);
+        if (t < L) vv[nl] = *reinterpret_cast<const vrow_t*>(vh + kv_row(lay, head, t) + d0 + DL * dl);
       }
     }
     // one division per position (lane = position in the chunk), handed to the 16 lanes that
     // multiply that position's values
     const float p_lane = base + lane < L ? s[base + lane] / Z : 0.0f;
-    float acc[8];
+    float acc[DL];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
+    for (int i = 0; i < DL; ++i) acc[i] = 0.0f;
 #pragma unroll
     for (int nl = 0; nl < 16; ++nl) {
       const int t = base + 4 * nl + tq;
       const float p = __shfl(p_lane, 4 * nl + tq, 64);
       if (t < L) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) acc[i] = __builtin_fmaf(p, (float)vv[nl][i], acc[i]);
+        for (int i = 0; i < DL; ++i) acc[i] = __builtin_fmaf(p, (float)vv[nl][i], acc[i]);
       }
     }
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < DL; ++i) {
       acc[i] = xor_add(acc[i], 16);
       acc[i] = xor_add(acc[i], 32);
     }
     if (tq == 0) {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) cv[chunk * AWQ_HEAD_DIM + 8 * dl + i] = acc[i];
+      for (int i = 0; i < DL; ++i) cv[chunk * DP + DL * dl + i] = acc[i];
     }
   }
   __syncthreads();
-  if (tid < AWQ_HEAD_DIM) {
+  if (tid < DP) {
     float out = cv[tid];
-    for (int c = 1; c < nchunks; ++c) out += cv[c * AWQ_HEAD_DIM + tid];
-    ctx[head * AWQ_HEAD_DIM + tid] = (half_t)out;
+    for (int c = 1; c < nchunks; ++c) out += cv[c * DP + tid];
+    ctx[head * AWQ_HEAD_DIM + d0 + tid] = (half_t)out;
   }
 }
 
@@ -588,8 +598,9 @@ static int launch_attention_ws(const half_t* q, const half_t* kc, const half_t* 
     hipLaunchKernelGGL(attn_scores_kernel, grid, block, 0, st, a);
     if (bound <= kAttnTwoLaunchMax) {
       // the rest of the head in one workgroup: at most one chunk per wavefront
-      hipLaunchKernelGGL((attention_kernel<kWaves, kLdsChunks * 64, kLdsChunks, true>), dim3(n_heads), dim3(kThreads), 0,
-                         st, q, kc, vc, ctx, kv, (int)L, dyn, use_len_hi, max_pos, a.scores, a.pmax);
+      hipLaunchKernelGGL((attention_kernel<kWaves, kLdsChunks * 64, kLdsChunks, true, kHeadParts>),
+                         dim3(n_heads, kHeadParts), dim3(kThreads), 0, st, q, kc, vc, ctx, kv, (int)L, dyn, use_len_hi,
+                         max_pos, a.scores, a.pmax);
       AWQ_HIP_TRY(hipGetLastError());
       return AWQ_OK;
     }
@@ -603,8 +614,9 @@ static int launch_attention_ws(const half_t* q, const half_t* kc, const half_t* 
     AWQ_HIP_TRY(hipGetLastError());
     return AWQ_OK;
   }
-  hipLaunchKernelGGL((attention_kernel<kWaves, kLdsChunks * 64, kLdsChunks>), dim3(n_heads), dim3(kThreads), 0,
-                     st, q, kc, vc, ctx, kv, (int)L, dyn, use_len_hi, max_pos, (const float*)nullptr, (const float*)nullptr);
+  hipLaunchKernelGGL((attention_kernel<kWaves, kLdsChunks * 64, kLdsChunks, false, kHeadParts>),
+                     dim3(n_heads, kHeadParts), dim3(kThreads), 0, st, q, kc, vc, ctx, kv, (int)L, dyn, use_len_hi,
+                     max_pos, (const float*)nullptr, (const float*)nullptr);
   AWQ_HIP_TRY(hipGetLastError());
   return AWQ_OK;
 }

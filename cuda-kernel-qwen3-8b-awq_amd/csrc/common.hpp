@@ -155,22 +155,21 @@ int launch_rope_kv_append(const half_t* qkv, const half_t* cos_t, const half_t* 
 // How the decode attention is launched, by an upper bound of the attended length
 // (measured in the decode loop of the 36-layer model, where every layer's cache
 // comes from HBM, and with the attention sweep of bench.py):
-//   <= kAttnOneWorkgroupMax  one workgroup per head does everything: a handful of
-//        memory round trips on 32 compute units (6 us at 256, 12.4 us at 704 positions);
+//   <= kAttnOneWorkgroupMax  four workgroups per head, each with all of the head's keys and a
+//        quarter of every value row, do everything: a handful of memory round trips on 128
+//        compute units;
 //   <= kAttnTwoLaunchMax     the keys are streamed by all compute units (scores and part
-//        maxima to memory), a second launch with one workgroup per head does the rest,
-//        one 64-position chunk per wavefront (11 us at 705, 12.8 us at 1024 positions;
-//        with two chunks per wavefront 24 us at 1536);
+//        maxima to memory), a second launch with four workgroups per head does the rest,
+//        one 64-position chunk per wavefront;
 //   <= kAttnMergedMax        three launches: scores; exponentials, chunk sums and chunk
 //        vectors per part (the exponentials are recomputed by every workgroup of a
 //        head); ordered sum (17.7 us at 1536, 20.1 us at 2048 positions);
 //   beyond                   four launches (26.5 us at 4096; three would take 29.1 us).
-// Tokens per second over 264 decode steps, one workgroup per head against the cut
-// path: 582 / 567 at 258..522 positions, 556 / 557 at 408..672, 539 / 523 at 708..972
-// (before the two-launch form: 513), 458 / 510 at 908..1172, 378 / 480 at 1708..1972.
-// With the cache in blocks of 64 positions: 590 / 566 at 258..522, 569 / 561 at 358..622,
-// 547 / 555 at 458..722 -- the two forms meet near 540 positions.
-constexpr int64_t kAttnOneWorkgroupMax = 576;
+// Tokens per second over 128 decode steps, one launch against two: 691 / 685 at 568..696
+// positions, 668 / 673 at 708..836 with the switch at 768 -- the two forms meet near 700.
+// (With one workgroup per head they met near 576: 716 against 683 tok/s at 448..576 positions
+// and 669 against 649 at 708..836 is what the four workgroups per head brought.)
+constexpr int64_t kAttnOneWorkgroupMax = 704;
 constexpr int64_t kAttnTwoLaunchMax = 1024;
 constexpr int64_t kAttnMergedMax = 2048;
 int64_t attention_workspace_bytes(int n_heads, int64_t max_pos);

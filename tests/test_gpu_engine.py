@@ -34,15 +34,15 @@ SMALL = dict(n_layers=4, hidden=512, inter=1536, vocab=1024, max_pos=128)
 
 
 def test_small_model_sequence_crossing_the_attention_switch(awq, oracle, torch_gpu):
-    """a 560-token prompt and 24 new tokens: the attended length passes 576, where the engine
+    """a 690-token prompt and 24 new tokens: the attended length passes 704, where the engine
     changes attention launches (and captured graph); tokens and state stay the oracle's"""
-    cfg = awq.make_config(n_layers=2, hidden=512, inter=512, vocab=1024, max_pos=640)
+    cfg = awq.make_config(n_layers=2, hidden=512, inter=512, vocab=1024, max_pos=768)
     model = make_oracle_model(oracle, cfg)
     eng = awq.QWen3AWQInfer.empty(cfg)
     fill_pair(awq, oracle, cfg, 99, engine=eng, model=model, profile=awq.SYNTH_BALANCED)
     rng = np.random.default_rng(3)
-    prompt = rng.integers(0, cfg.vocab, 560).tolist()
-    print("small model, sequence crossing 576 positions", flush=True)
+    prompt = rng.integers(0, cfg.vocab, 690).tolist()
+    print("small model, sequence crossing 704 positions", flush=True)
     got = eng.generateResponse(prompt, 24)
     ref = oracle_generate(oracle, model, prompt, 24)
     assert got == ref

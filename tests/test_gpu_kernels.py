@@ -232,7 +232,7 @@ def test_rope_kv_append_bit_exact(awq, lib, oracle, torch_gpu):
                                   d_v.data_ptr(), nh, mp, mp, stream(torch)) != 0  # pos out of range
 
 
-@pytest.mark.parametrize("L", [1, 2, 63, 64, 65, 129, 513, 576, 577, 1500])
+@pytest.mark.parametrize("L", [1, 2, 63, 64, 65, 129, 513, 576, 577, 704, 705, 1500])
 def test_decode_attention_bit_exact(awq, lib, oracle, torch_gpu, L):
     torch = torch_gpu
     nh, mp = 32, 2048
@@ -261,9 +261,9 @@ def test_decode_attention_bit_exact(awq, lib, oracle, torch_gpu, L):
                                     ws.data_ptr(), stream(torch)) != 0
 
 
-@pytest.mark.parametrize("L", [577, 1000, 1024, 1025, 2048, 2049, 4097, 9001, 20000])
+@pytest.mark.parametrize("L", [577, 704, 705, 1000, 1024, 1025, 2048, 2049, 4097, 9001, 20000])
 def test_decode_attention_long_sequences_bit_exact(awq, lib, oracle, torch_gpu, L):
-    """beyond 576 positions the launches are cut along the sequence (32 parts per head, some of them
+    """beyond 704 positions the launches are cut along the sequence (32 parts per head, some of them
     empty while the sequence has fewer than 32 chunks; two launches up to 1024 positions, three up to 2048,
     four beyond);
     the summation orders are those of the short

@@ -185,7 +185,7 @@ def test_long_prompt_takes_the_rows_split_products(awq, oracle, torch_gpu):
 def test_maximum_sequence_length_one_layer(awq, oracle, torch_gpu):
     """The reference's MAX_POSITION_EMBEDDINGS (40960, Inference.cu:39) on one full-width layer: a
     40,950-token prompt through the batched pass and, token by token, through the bit-exact decode
-    kernels (attention cut along the sequence beyond 576 positions), then generation up to the
+    kernels (attention cut along the sequence beyond 704 positions), then generation up to the
     last position; one more token is an error, not a cache overrun."""
     cfg = awq.make_config(n_layers=1, vocab=2048, max_pos=40960)
     model = make_oracle_model(oracle, cfg)   # only as the host buffer of the weights here
