@@ -256,7 +256,8 @@ int awq_rope_kv_append(const void* qkv, const void* cos_t, const void* sin_t, vo
                        void* v_cache, int32_t n_heads, int64_t max_pos, int64_t pos, void* stream);
 
 /* attentionKernel, Inference.cu:182-266, for one query over L cached
- * positions.  Up to 576 positions one workgroup per head; beyond, the sequence
+ * positions.  Up to 704 positions one launch, four workgroups per head (each
+ * with all keys and a quarter of the head's dimensions); beyond, the sequence
  * is cut into 32 parts per head over two to four launches with the same summation
  * orders (bit-identical results).  workspace:
  * awq_attention_workspace_bytes(n_heads, max_pos), contents irrelevant. */
