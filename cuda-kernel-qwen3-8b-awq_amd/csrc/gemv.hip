@@ -7,15 +7,15 @@
 // the order of awq_block_elem (awq_canon_math.h).  One 16-byte load hands a
 // lane one whole block of its row:
 //     byte offset = ((rg * (k/32) + blk) * 16 + r) * 16,   rg = row/16, r = row%16
-// A workgroup owns one row group and all of k, so no partial sums ever leave
-// the workgroup: lane (wavefront w, quarter q = lane/16, r = lane%16) takes the
-// G consecutive blocks starting at (4w+q)*G of row 16*rg + r; a wavefront load
-// is four contiguous 256-byte pieces, and the G loads of a lane walk 256*G
-// contiguous bytes per quarter.  Inside the 16 bytes, dword c holds elements
-// 8c..8c+7 with nibble positions {0,16,4,20,8,24,12,28}[t & 7]: masking with
-// 0x000f000f / 0x00f000f0 (and the same after one shift by 8) yields two
-// weights as the low mantissa bits of a packed pair of binary16 numbers 1024+q
-// or 1024+16q.
+// A workgroup owns one row group (or half of one) and all of k, so no partial
+// sums ever leave the workgroup: lane (wavefront w, quarter q = lane/16,
+// r = lane%16) takes the G consecutive blocks starting at (4w+q)*G of row
+// 16*rg + r; a wavefront load is four contiguous 256-byte pieces, and the G
+// loads of a lane walk 256*G contiguous bytes per quarter.  Inside the 16
+// bytes, dword c holds elements 8c..8c+7 with nibble positions
+// {0,16,4,20,8,24,12,28}[t & 7]: masking with 0x000f000f / 0x00f000f0 (and the
+// same after one shift by 8) yields two weights as a packed pair of binary16
+// subnormals q * 2^-24 or q * 2^-20.
 #include "common.hpp"
 #include <stdlib.h>
 
