@@ -646,7 +646,12 @@ extern "C" int awq_create(const char* weight_dir, const awq_config* cfg_in, awq_
       }
       // the other buffer's copy was queued one file ago: once it has completed the reader may refill it
       Slot& o = slot[(i + 1) & 1];
-      if (o.state == 2) {
+      bool in_flight;
+      {
+        std::lock_guard<std::mutex> lock(mu);
+        in_flight = o.state == 2;
+      }
+      if (in_flight) {
         if (hipEventSynchronize(o.copied) != hipSuccess) {
           awq_set_error("waiting for a host-to-device copy failed");
           rc = AWQ_ERR_HIP;
