@@ -334,6 +334,10 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
   __shared__ GroupConst gtab[2][PERIODIC ? 64 : 1];
   constexpr int MAXU = G * Q / 8;  // units of four inputs a thread stages
   static_assert(G * Q >= 8, "a thread stages whole units");
+  // WIDE: a thread's units come in adjacent pairs (8 consecutive inputs, one 16-byte request for x and one
+  // for gamma instead of two 8-byte ones: -0.05 to -0.18 us per launch); unit u of thread tid is then
+  // 2 * (tid + (u/2) * nthreads) + u%2 instead of tid + u * nthreads
+  constexpr bool WIDE = !PERIODIC && MAXU % 2 == 0;
   const int tid = threadIdx.x;
   const int nthreads = n_waves * 64;
   const int lane = tid & 63;
@@ -355,7 +359,7 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
   uint2 xu[MAXU], gu[MAXU];
 #pragma unroll
   for (int u = 0; u < MAXU; ++u) {
-    const int unit = tid + u * nthreads;
+    const int unit = WIDE ? 2 * (tid + (u >> 1) * nthreads) + (u & 1) : tid + u * nthreads;
     if (PERIODIC) {
       half_t hx[4], hg[4];
 #pragma unroll
@@ -366,6 +370,17 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
       }
       xu[u] = __builtin_bit_cast(uint2, *reinterpret_cast<uint64_t*>(hx));
       gu[u] = __builtin_bit_cast(uint2, *reinterpret_cast<uint64_t*>(hg));
+    } else if (WIDE) {
+      if ((u & 1) == 0) {
+        const uint4 t = reinterpret_cast<const uint4*>(x)[unit >> 1];
+        xu[u] = uint2{t.x, t.y};
+        xu[u + (MAXU > 1 ? 1 : 0)] = uint2{t.z, t.w};
+        if (norm) {
+          const uint4 g4 = reinterpret_cast<const uint4*>(gamma)[unit >> 1];
+          gu[u] = uint2{g4.x, g4.y};
+          gu[u + (MAXU > 1 ? 1 : 0)] = uint2{g4.z, g4.w};
+        }
+      }
     } else {
       xu[u] = reinterpret_cast<const uint2*>(x)[unit];
       if (norm) gu[u] = reinterpret_cast<const uint2*>(gamma)[unit];
@@ -383,7 +398,7 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
     // natural order, the stride-halving tree, then two binary16 multiplies
 #pragma unroll
     for (int u = 0; u < MAXU; ++u) {
-      const int unit = tid + u * nthreads;
+      const int unit = WIDE ? 2 * (tid + (u >> 1) * nthreads) + (u & 1) : tid + u * nthreads;
       if (PERIODIC) {
         half_t hx[4];
         *reinterpret_cast<uint64_t*>(hx) = __builtin_bit_cast(uint64_t, xu[u]);
@@ -442,16 +457,29 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
   }
   // x and the input sum of every block (adjacent-pair tree over its 32 inputs:
   // four in this thread, then the eight threads that share the block)
+  float sx_prev = 0.0f;
 #pragma unroll
   for (int u = 0; u < MAXU; ++u) {
-    const int unit = tid + u * nthreads;
+    const int unit = WIDE ? 2 * (tid + (u >> 1) * nthreads) + (u & 1) : tid + u * nthreads;
     *reinterpret_cast<uint2*>(xs + xs_index<G>(4 * unit)) = xu[u];
     const half2_t t0 = as_half2(xu[u].x), t1 = as_half2(xu[u].y);
     float sx = ((float)t0.x + (float)t0.y) + ((float)t1.x + (float)t1.y);
-    sx += dpp_f<kDppXor1>(sx);
-    sx += dpp_f<kDppXor2>(sx);
-    sx += dpp_f<kDppHalfMirror>(sx);
-    if ((tid & 7) == 0) xsum[unit >> 3] = sx;
+    if (WIDE) {
+      // the pair of units of this thread first, then the four threads that share the block
+      if ((u & 1) == 0) {
+        sx_prev = sx;
+      } else {
+        sx = sx_prev + sx;
+        sx += dpp_f<kDppXor1>(sx);
+        sx += dpp_f<kDppXor2>(sx);
+        if ((tid & 3) == 0) xsum[unit >> 3] = sx;
+      }
+    } else {
+      sx += dpp_f<kDppXor1>(sx);
+      sx += dpp_f<kDppXor2>(sx);
+      sx += dpp_f<kDppHalfMirror>(sx);
+      if ((tid & 7) == 0) xsum[unit >> 3] = sx;
+    }
   }
 
   // Group constants.  When the scale group depends on the input index it is
