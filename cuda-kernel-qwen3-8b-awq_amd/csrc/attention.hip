@@ -68,7 +68,7 @@ __device__ __forceinline__ float wave_tree_sum(float v) {
 // sums (the same instructions on the same data: the same bits) and then the context of its 128/DS of the
 // head's dimensions, i.e. it reads all keys but only 1/DS of every value row.  One compute unit keeps only
 // about 37 KB of requests in flight, so the bytes a unit has to pull set the time beyond about 128 positions.
-template <int NW, int SCAP, int CCAP, bool FROM_SCORES = false, int DS = 1>
+template <int NW, int SCAP, int CCAP, bool FROM_SCORES = false, int DS = 1, int EAGER = 0>
 __global__ __launch_bounds__(NW * 64) void attention_kernel(const half_t* __restrict__ q,
                                                              const half_t* __restrict__ kc,
                                                              const half_t* __restrict__ vc, half_t* __restrict__ ctx,
@@ -120,17 +120,37 @@ __global__ __launch_bounds__(NW * 64) void attention_kernel(const half_t* __rest
   // scores (Inference.cu:202-226) and their maximum (:229-233): groups of four
   // positions go round the wavefronts, six groups' loads in flight.  The values
   // of this wavefront's first chunk are requested right behind the first keys,
-  // so that both arrive in one memory round trip.
+  // so that both arrive in one memory round trip.  The keys and values of the
+  // first EAGER positions are requested before the attended length is known
+  // (it sits in memory, a round trip of its own); rows past the length are valid
+  // cache memory and are never used.
+  constexpr int kEagerGroups = EAGER / (4 * NW);
+  static_assert(kEagerGroups <= 6 && EAGER % 64 == 0 && EAGER % (4 * NW) == 0, "eager part of the first trip");
+  const int last_row = (int)max_pos - 1;
+  half8_t kv[6];
+#pragma unroll
+  for (int u = 0; u < kEagerGroups; ++u) {
+    const int t = min(4 * (wave + u * NW) + tq, last_row);
+    kv[u] = *reinterpret_cast<const half8_t*>(kh + kv_row(lay, head, t) + 8 * dl);
+  }
+  if (wave < EAGER / 64) {
+#pragma unroll
+    for (int nl = 0; nl < 16; ++nl) {
+      const int t = min((wave << 6) + 4 * nl + tq, last_row);
+      vv[nl] = *reinterpret_cast<const vrow_t*>(vh + kv_row(lay, head, t) + d0 + DL * dl);
+    }
+  }
   float lmax = -1e9f;
   const int nquads = (L + 3) >> 2;
   for (int q0 = wave; q0 < nquads; q0 += 6 * NW) {
-    half8_t kv[6];
+    const bool first = q0 == wave;
 #pragma unroll
     for (int u = 0; u < 6; ++u) {
       const int t = 4 * (q0 + u * NW) + tq;
-      if (t < L) kv[u] = *reinterpret_cast<const half8_t*>(kh + kv_row(lay, head, t) + 8 * dl);
+      if (t < L && !(first && u < kEagerGroups))
+        kv[u] = *reinterpret_cast<const half8_t*>(kh + kv_row(lay, head, t) + 8 * dl);
     }
-    if (q0 == wave && wave < nchunks) {
+    if (first && wave >= EAGER / 64 && wave < nchunks) {
 #pragma unroll
       for (int nl = 0; nl < 16; ++nl) {
         const int t = (wave << 6) + 4 * nl + tq;
@@ -614,9 +634,16 @@ static int launch_attention_ws(const half_t* q, const half_t* kc, const half_t* 
     AWQ_HIP_TRY(hipGetLastError());
     return AWQ_OK;
   }
-  hipLaunchKernelGGL((attention_kernel<kWaves, kLdsChunks * 64, kLdsChunks, false, kHeadParts>),
-                     dim3(n_heads, kHeadParts), dim3(kThreads), 0, st, q, kc, vc, ctx, kv, (int)L, dyn, use_len_hi,
-                     max_pos, (const float*)nullptr, (const float*)nullptr);
+  // A length that sits in device memory and is known to exceed kAttnShortMax: the first rows are
+  // requested before it arrives.
+  if (dyn && bound > kAttnShortMax && max_pos >= kAttnShortMax)
+    hipLaunchKernelGGL((attention_kernel<kWaves, kLdsChunks * 64, kLdsChunks, false, kHeadParts, (int)kAttnShortMax>),
+                       dim3(n_heads, kHeadParts), dim3(kThreads), 0, st, q, kc, vc, ctx, kv, (int)L, dyn, use_len_hi,
+                       max_pos, (const float*)nullptr, (const float*)nullptr);
+  else
+    hipLaunchKernelGGL((attention_kernel<kWaves, kLdsChunks * 64, kLdsChunks, false, kHeadParts>),
+                       dim3(n_heads, kHeadParts), dim3(kThreads), 0, st, q, kc, vc, ctx, kv, (int)L, dyn, use_len_hi,
+                       max_pos, (const float*)nullptr, (const float*)nullptr);
   AWQ_HIP_TRY(hipGetLastError());
   return AWQ_OK;
 }

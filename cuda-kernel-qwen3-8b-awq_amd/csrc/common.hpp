@@ -155,9 +155,13 @@ int launch_rope_kv_append(const half_t* qkv, const half_t* cos_t, const half_t* 
 // How the decode attention is launched, by an upper bound of the attended length
 // (measured in the decode loop of the 36-layer model, where every layer's cache
 // comes from HBM, and with the attention sweep of bench.py):
+//   <= kAttnShortMax         as the next form;
 //   <= kAttnOneWorkgroupMax  four workgroups per head, each with all of the head's keys and a
 //        quarter of every value row, do everything: a handful of memory round trips on 128
-//        compute units;
+//        compute units.  Above kAttnShortMax with the length in device memory the keys and values
+//        of the first kAttnShortMax positions are requested before the length has arrived (one
+//        memory round trip less: -0.15 us per launch, 794.3 -> 797.6 tok/s); a shorter sequence
+//        would pay for rows it does not use, hence the bound of its own;
 //   <= kAttnTwoLaunchMax     the keys are streamed by all compute units (scores and part
 //        maxima to memory), a second launch with four workgroups per head does the rest,
 //        one 64-position chunk per wavefront;
@@ -169,6 +173,7 @@ int launch_rope_kv_append(const half_t* qkv, const half_t* cos_t, const half_t* 
 // positions, 668 / 673 at 708..836 with the switch at 768 -- the two forms meet near 700.
 // (With one workgroup per head they met near 576: 716 against 683 tok/s at 448..576 positions
 // and 669 against 649 at 708..836 is what the four workgroups per head brought.)
+constexpr int64_t kAttnShortMax = 128;
 constexpr int64_t kAttnOneWorkgroupMax = 704;
 constexpr int64_t kAttnTwoLaunchMax = 1024;
 constexpr int64_t kAttnMergedMax = 2048;

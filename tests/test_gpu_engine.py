@@ -34,8 +34,9 @@ SMALL = dict(n_layers=4, hidden=512, inter=1536, vocab=1024, max_pos=128)
 
 
 def test_small_model_sequence_crossing_the_attention_switch(awq, oracle, torch_gpu):
-    """a 690-token prompt and 24 new tokens: the attended length passes 704, where the engine
-    changes attention launches (and captured graph); tokens and state stay the oracle's"""
+    """a 690-token prompt and 24 new tokens: the attended length passes 128 and 704, where the engine
+    changes attention launches (and captured graph); tokens and state stay the oracle's.  Then a second,
+    shorter sequence on the same engine, whose cache still holds the first one's rows past its own length."""
     cfg = awq.make_config(n_layers=2, hidden=512, inter=512, vocab=1024, max_pos=768)
     model = make_oracle_model(oracle, cfg)
     eng = awq.QWen3AWQInfer.empty(cfg)
@@ -45,6 +46,12 @@ def test_small_model_sequence_crossing_the_attention_switch(awq, oracle, torch_g
     print("small model, sequence crossing 704 positions", flush=True)
     got = eng.generateResponse(prompt, 24)
     ref = oracle_generate(oracle, model, prompt, 24)
+    assert got == ref
+    compare_state(awq, oracle, eng, model, cfg)
+    prompt = rng.integers(0, cfg.vocab, 126).tolist()
+    print("second sequence, 126 + 12 positions over the stale cache", flush=True)
+    got = eng.generateResponse(prompt, 12)
+    ref = oracle_generate(oracle, model, prompt, 12)
     assert got == ref
     compare_state(awq, oracle, eng, model, cfg)
     eng.close()

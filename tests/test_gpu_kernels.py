@@ -197,6 +197,32 @@ def test_rmsnorm_bit_exact(awq, lib, oracle, torch_gpu, n):
         assert np.array_equal(d_o.cpu().numpy().view(np.uint16), ref.view(np.uint16))
 
 
+@pytest.mark.parametrize("n,eps", [(256, 1e-6), (256, 0.0), (768, 1e-6)])
+def test_rmsnorm_scale_sweep(awq, lib, oracle, torch_gpu, n, eps):
+    """The scale 1/sqrt(mean + eps) over 4000 magnitudes from 1e-4 to 250, an all-zero and a huge vector (the scale is
+    then subnormal in binary16), with and without eps and for a length that is no power of two: every output bit
+    for bit the oracle's, which pins the divide / square root / divide sequence on the device."""
+    torch = torch_gpu
+    rng = np.random.default_rng(n + int(eps * 1e7))
+    rows = 4000
+    mag = np.exp(rng.uniform(np.log(1e-4), np.log(250.0), rows))
+    x = (rng.standard_normal((rows + 2, n)) * np.append(mag, [0.0, 1.0])[:, None]).astype(np.float16)
+    x[rows + 1] = np.float16(60000.0)
+    if eps == 0.0:
+        x[rows] = np.float16(1.0)  # 0 * inf: the NaN's sign differs between x86 and the device
+    gamma = (1 + 0.02 * rng.standard_normal(n)).astype(np.float16)
+    ref = np.zeros_like(x)
+    for i in range(rows + 2):
+        oracle.awqo_rmsnorm(ptr(x[i]), ptr(gamma), ptr(ref[i]), n, eps)
+    d_x, d_g = dev(torch, x), dev(torch, gamma)
+    d_o = torch.zeros((rows + 2, n), dtype=torch.float16, device="cuda")
+    for i in range(rows + 2):
+        awq.check(lib.awq_rmsnorm(d_x.data_ptr() + 2 * n * i, d_g.data_ptr(), d_o.data_ptr() + 2 * n * i, n, eps,
+                                  stream(torch)))
+    torch.cuda.synchronize()
+    assert np.array_equal(d_o.cpu().numpy().view(np.uint16), ref.view(np.uint16))
+
+
 def test_rope_kv_append_bit_exact(awq, lib, oracle, torch_gpu):
     torch = torch_gpu
     nh, mp = 32, 640
