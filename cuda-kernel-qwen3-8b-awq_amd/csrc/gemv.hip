@@ -79,48 +79,41 @@ __global__ __launch_bounds__(256) void repack_kernel(const uint8_t* __restrict__
 // ---------------------------------------------------------------------------
 // fused dequant + matrix-vector product
 //
-// Arithmetic (awq_canon_math.h): per block of 32 inputs T = A + B, two fma
-// chains over the raw nibbles, then (T - z X) s with X the block's input sum.
-// A masked dword (v & 0x000f000f) is a pair of binary16 subnormals q * 2^-24,
-// (v & 0x00f000f0) a pair q * 2^-20; v_fma_mix_f32 widens them exactly, so a
-// weight costs one multiply-add and an eighth of (one shift + four ANDs): 13
-// instructions per 8 weights.  The powers of two are carried by the group
-// constants: chain A runs at 2^-24, chain B at 2^-20, T' = fma(A, 16, B) is
-// T * 2^-20 (exactly the rounding of A + B), and
-//     fma(-z * 2^-20, X, T') * (s * 2^20)  ==  fma(-z, X, T) * s   bit for bit
-// (every intermediate is a multiple of 2^-68 and far from the binary32
-// exponent limits, so the scalings commute with the roundings).
+// Arithmetic (awq_canon_math.h): the 32 inputs of a block are put into block
+// fixed point once per workgroup, x[t] = I[t] * c with c a power of two taken
+// from the block's largest exponent and I[t] a 16-bit integer (round to nearest
+// even), and a row's block value is
+//     fma(-z, S, D) * (s * c),   D = sum q[t] * I[t],  S = sum I[t]
+// with D and S exact integers below 2^24.  The integers are kept in LDS as
+// U = I + 32768 cut into four planes of nibbles laid out like the weight
+// nibbles of a dword, so that v_dot8_u32_u4 multiplies eight weights by eight
+// input nibbles at once with nothing to unpack: per 8 weights four dot products
+// (one per plane) and a fifth against 0x11111111 that yields sum q for the
+// offset, D = sum_p 16^p dot_p - 32768 sum q: 5 instructions per 8 weights
+// (13 with binary32 multiply-adds on masked nibble pairs).
 // ---------------------------------------------------------------------------
 struct GroupConst {
-  float s;   // scale * 2^20
-  float zn;  // -zero_point * 2^-20
+  float s;   // scale
+  float zn;  // -zero_point
 };
 
-__device__ __forceinline__ GroupConst make_group(half_t s, half_t z) {
-  return GroupConst{(float)s * 1048576.0f, -(float)z * (1.0f / 1048576.0f)};
-}
+__device__ __forceinline__ GroupConst make_group(half_t s, half_t z) { return GroupConst{(float)s, -(float)z}; }
 
-// T * 2^-20 of one block: 32 weights of this lane's row against 32 inputs in LDS
-__device__ __forceinline__ float block_dot(const u32x4& w, const half_t* xs) {
+// D of one block as a float (exact): 32 weights of this lane's row against the block's 16 plane dwords in LDS
+__device__ __forceinline__ float block_dot(const u32x4& w, const unsigned char* xs) {
   const uint32_t d[4] = {w.x, w.y, w.z, w.w};
-  float acc_a = 0.0f, acc_b = 0.0f;
+  uint32_t a0 = 0, a1 = 0, a2 = 0, a3 = 0, aq = 0;
 #pragma unroll
   for (int c = 0; c < 4; ++c) {
-    const uint4 xv = *reinterpret_cast<const uint4*>(xs + 8 * c);
-    const half2_t x0 = as_half2(xv.x), x1 = as_half2(xv.y), x2 = as_half2(xv.z), x3 = as_half2(xv.w);
-    const uint32_t v = d[c], v8 = v >> 8;
-    const half2_t wa = as_half2(v & 0x000f000fu), wb = as_half2(v & 0x00f000f0u);
-    const half2_t wc = as_half2(v8 & 0x000f000fu), wd = as_half2(v8 & 0x00f000f0u);
-    acc_a = __builtin_fmaf((float)wa.x, (float)x0.x, acc_a);
-    acc_a = __builtin_fmaf((float)wa.y, (float)x0.y, acc_a);
-    acc_b = __builtin_fmaf((float)wb.x, (float)x1.x, acc_b);
-    acc_b = __builtin_fmaf((float)wb.y, (float)x1.y, acc_b);
-    acc_a = __builtin_fmaf((float)wc.x, (float)x2.x, acc_a);
-    acc_a = __builtin_fmaf((float)wc.y, (float)x2.y, acc_a);
-    acc_b = __builtin_fmaf((float)wd.x, (float)x3.x, acc_b);
-    acc_b = __builtin_fmaf((float)wd.y, (float)x3.y, acc_b);
+    const uint4 xv = *reinterpret_cast<const uint4*>(xs + 16 * c);
+    a0 = __builtin_amdgcn_udot8(d[c], xv.x, a0, false);
+    a1 = __builtin_amdgcn_udot8(d[c], xv.y, a1, false);
+    a2 = __builtin_amdgcn_udot8(d[c], xv.z, a2, false);
+    a3 = __builtin_amdgcn_udot8(d[c], xv.w, a3, false);
+    aq = __builtin_amdgcn_udot8(d[c], 0x11111111u, aq, false);
   }
-  return __builtin_fmaf(acc_a, 16.0f, acc_b);
+  const uint32_t D = ((((a3 << 4) + a2) << 4) + a1 << 4) + a0 - (aq << 15);
+  return (float)(int32_t)D;
 }
 
 // value of another lane of the same row of 16 (DPP: no LDS round trip)
@@ -132,6 +125,74 @@ constexpr int kDppXor1 = 0xB1;        // quad_perm:[1,0,3,2]
 constexpr int kDppXor2 = 0x4E;        // quad_perm:[2,3,0,1]
 constexpr int kDppHalfMirror = 0x141; // lane i <-> 7 - i within 8
 constexpr int kDppRor4 = 0x124, kDppRor8 = 0x128;
+
+// v(lane) + v(lane ^ 16), then that + the same of lane ^ 32: the four rows of 16 lanes added as
+// (row0 + row1) + (row2 + row3) in every lane.  gfx950's lane-swap instructions exchange rows between
+// two registers without the LDS round trip of a general shuffle (the waits around them are the data
+// hazard slots the compiler would insert if it saw the instruction): after the first swap a holds rows
+// (0,0,2,2) and b rows (1,1,3,3) of v, after the second a holds the low and b the high half of s.
+__device__ __forceinline__ float sum_rows_of_16(float v) {
+  float a = v, b = v;
+  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+  float s = a + b;
+  a = s, b = s;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+  return a + b;
+}
+
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_u(uint32_t v) {
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xf, 0xf, true);
+}
+
+typedef unsigned short ushort2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
+  return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(ushort2_t, a), __builtin_bit_cast(ushort2_t, b)));
+}
+
+// Block fixed point of 8 consecutive block-order inputs h[0..3] (binary16 pairs, one weight dword's worth);
+// the four threads tid & ~3 .. + 3 hold the 32 inputs of one block (awq_block_fixed in awq_canon_math.h).
+// planes: dword p holds nibble p of U = I + 32768 of element t at the bit position of weight nibble t
+// ({0,16,4,20,8,24,12,28}[t]); c: the block's power of two (NaN when the block holds an infinity or a
+// NaN); S: the sum of the block's 32 integers.
+__device__ __forceinline__ void stage_unit8(const uint32_t h[4], u32x4& planes, float& c, float& S) {
+  // the largest magnitude: binary16 magnitudes order like their bit patterns
+  uint32_t mm = pk_max_u16(pk_max_u16(h[0] & 0x7fff7fffu, h[1] & 0x7fff7fffu),
+                           pk_max_u16(h[2] & 0x7fff7fffu, h[3] & 0x7fff7fffu));
+  mm = max(mm & 0xffffu, mm >> 16);
+  mm = max(mm, dpp_u<kDppXor1>(mm));
+  mm = max(mm, dpp_u<kDppXor2>(mm));
+  const uint32_t e = mm >> 10;                       // largest exponent field, 0..31
+  const uint32_t cbits = (max(e, 1u) + 98u) << 23;   // c = 2^(max(e,1) - 29)
+  c = __builtin_bit_cast(float, e == 31u ? 0x7fc00000u : cbits);
+  const float inv = __builtin_bit_cast(float, 0x7f000000u - cbits);  // 1/c
+  // x/c + (1.5 * 2^23 + 32768) rounds to an integer (nearest even) whose low 16 bits are U
+  const float magic = 12615680.0f;
+  uint32_t P[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const half2_t x2 = as_half2(h[i]);
+    const uint32_t lo = __builtin_bit_cast(uint32_t, __builtin_fmaf((float)x2.x, inv, magic));
+    const uint32_t hi = __builtin_bit_cast(uint32_t, __builtin_fmaf((float)x2.y, inv, magic));
+    P[i] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);  // U of element 2i | U of element 2i+1 << 16
+  }
+  uint32_t su = 0;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    su = __builtin_amdgcn_udot2(__builtin_bit_cast(ushort2_t, P[i]), ushort2_t{1, 1}, su, false);
+  su += dpp_u<kDppXor1>(su);
+  su += dpp_u<kDppXor2>(su);
+  S = (float)((int32_t)su - (32 << 15));
+  // nibble planes: bytes of A hold (element 2, element 0) of plane 0 | plane 2, of the low and the high half
+  const uint32_t A0 = (P[0] & 0x0f0f0f0fu) | ((P[1] << 4) & 0xf0f0f0f0u);
+  const uint32_t A1 = (P[2] & 0x0f0f0f0fu) | ((P[3] << 4) & 0xf0f0f0f0u);
+  const uint32_t B0 = ((P[0] >> 4) & 0x0f0f0f0fu) | (P[1] & 0xf0f0f0f0u);
+  const uint32_t B1 = ((P[2] >> 4) & 0x0f0f0f0fu) | (P[3] & 0xf0f0f0f0u);
+  planes.x = __builtin_amdgcn_perm(A1, A0, 0x06020400u);
+  planes.y = __builtin_amdgcn_perm(B1, B0, 0x06020400u);
+  planes.z = __builtin_amdgcn_perm(A1, A0, 0x07030501u);
+  planes.w = __builtin_amdgcn_perm(B1, B0, 0x07030501u);
+}
 
 struct GemvParams {
   const u32x4* wq;
@@ -281,14 +342,6 @@ __global__ __launch_bounds__(256) void sample_finish_kernel(SampleFinish f) {
   }
 }
 
-// LDS position (in halves) of block-order element e of x.  The four quarters of
-// a wavefront read four different lane groups at the same time; 16 bytes of
-// skew per lane group keep those reads in different banks.
-template <int G>
-__device__ __forceinline__ int xs_index(int e) {
-  return e + (e / (G * AWQ_BLOCK_K)) * 8;
-}
-
 // A workgroup takes row groups blockIdx.x, blockIdx.x + gridDim.x, ... (16
 // output rows x all of k each).  n_waves wavefronts; lane (w, q, r) owns blocks
 // (4w+q)*G .. +G-1 of row 16*rg + r.  x is staged (normalised, with the input
@@ -317,8 +370,8 @@ __device__ __forceinline__ int xs_index(int e) {
 template <int G, bool PERIODIC, int UFAST = 0, int NWC = 0, bool MULTI = true, int RH = 16>
 __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
     const u32x4* __restrict__ wq, const half_t* __restrict__ x, const half_t* __restrict__ gamma,
-    const half_t* __restrict__ scale, const half_t* __restrict__ zp, int32_t m, int32_t prologue, int32_t epi,
-    float eps, int32_t mg, int32_t kg, GemvParams p) {
+    const half_t* __restrict__ scale, const half_t* __restrict__ zp, int32_t mg, int32_t kg, int32_t prologue,
+    int32_t epi, int32_t m, float eps, GemvParams p) {
   const int n_waves = NWC ? NWC : p.n_waves;
   constexpr int Q = 64 / RH;  // lanes that share a row = consecutive block ranges of a wavefront
   static_assert(RH == 16 || (RH == 8 && !PERIODIC), "half row groups are for one scale group per 16 rows");
@@ -326,20 +379,20 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
   const int nblk = NWC ? NWC * Q * G : p.nblk;
   const int C = PERIODIC ? p.C : 1;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  half_t* xs = reinterpret_cast<half_t*>(smem);                                  // k halves + skew
-  float* xsum = reinterpret_cast<float*>(smem + (size_t)(k + (nblk / G) * 8) * 2);  // nblk floats
-  half_t* xn = reinterpret_cast<half_t*>(xsum + nblk);                           // k halves (fused norm only)
+  unsigned char* xs = smem;                                                      // 2k bytes of nibble planes + skew
+  float* xc = reinterpret_cast<float*>(smem + (size_t)(k + (nblk / G) * 8) * 2);  // nblk powers of two
+  float* xS = xc + nblk;                                                         // nblk integer sums
+  half_t* xn = reinterpret_cast<half_t*>(xS + nblk);                             // k halves (fused norm only)
   __shared__ float red[2][16][16];  // double-buffered: one barrier per row group
   __shared__ __attribute__((aligned(16))) float part[256];
   __shared__ GroupConst gtab[2][PERIODIC ? 64 : 1];
-  constexpr int MAXU = G * Q / 8;  // units of four inputs a thread stages
+  // A thread stages units of 8 consecutive block-order inputs (the inputs of one weight dword): k/8 units over
+  // n_waves * 64 = k/(G*Q/2) threads, i.e. G*Q/16 units per thread, or one unit in every second thread
+  constexpr int MAXU = G * Q >= 16 ? G * Q / 16 : 1;
   static_assert(G * Q >= 8, "a thread stages whole units");
-  // WIDE: a thread's units come in adjacent pairs (8 consecutive inputs, one 16-byte request for x and one
-  // for gamma instead of two 8-byte ones: -0.05 to -0.18 us per launch); unit u of thread tid is then
-  // 2 * (tid + (u/2) * nthreads) + u%2 instead of tid + u * nthreads
-  constexpr bool WIDE = !PERIODIC && MAXU % 2 == 0;
   const int tid = threadIdx.x;
   const int nthreads = n_waves * 64;
+  const bool stager = G * Q >= 16 || tid < nthreads / 2;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int q = lane / RH, r = lane % RH;
@@ -352,39 +405,38 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
   const u32x4* wp = wq + ((int64_t)(rg * RH >> 4) * nblk + blk0) * 16 + ((rg * RH) & 15) + r;
   u32x4 w[G], wn[G];
 
-  // ---- x: unit u of a thread is the 4 consecutive block-order elements
-  // 4*(tid + u*nthreads)..+3; in natural order they are 4 consecutive indices too
-  // unless the matrix is periodic (then they are C apart and are gathered one by one)
+  // ---- x: unit u of a thread is the 8 consecutive block-order elements 8*(tid + u*nthreads)..+7; in natural
+  // order they are 8 consecutive indices too unless the matrix is periodic (then they are C apart and are
+  // gathered one by one)
   const bool norm = prologue == PRO_RMSNORM;
-  uint2 xu[MAXU], gu[MAXU];
+  uint4 xu[MAXU], gu[MAXU];
 #pragma unroll
   for (int u = 0; u < MAXU; ++u) {
-    const int unit = WIDE ? 2 * (tid + (u >> 1) * nthreads) + (u & 1) : tid + u * nthreads;
-    if (PERIODIC) {
-      half_t hx[4], hg[4];
+    const int unit = tid + u * nthreads;
+    if (!stager) {
+      xu[u] = gu[u] = uint4{0, 0, 0, 0};
+    } else if (PERIODIC) {
+      half_t hx[8], hg[8];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int j = (int)awq_block_elem(k, C, (4 * unit + i) >> 5, (4 * unit + i) & 31);
+      for (int i = 0; i < 8; ++i) {
+        const int j = (int)awq_block_elem(k, C, unit >> 2, (8 * unit + i) & 31);
         hx[i] = x[j];
         hg[i] = norm ? gamma[j] : (half_t)0.0f;
       }
-      xu[u] = __builtin_bit_cast(uint2, *reinterpret_cast<uint64_t*>(hx));
-      gu[u] = __builtin_bit_cast(uint2, *reinterpret_cast<uint64_t*>(hg));
-    } else if (WIDE) {
-      if ((u & 1) == 0) {
-        const uint4 t = reinterpret_cast<const uint4*>(x)[unit >> 1];
-        xu[u] = uint2{t.x, t.y};
-        xu[u + (MAXU > 1 ? 1 : 0)] = uint2{t.z, t.w};
-        if (norm) {
-          const uint4 g4 = reinterpret_cast<const uint4*>(gamma)[unit >> 1];
-          gu[u] = uint2{g4.x, g4.y};
-          gu[u + (MAXU > 1 ? 1 : 0)] = uint2{g4.z, g4.w};
-        }
-      }
+      xu[u] = *reinterpret_cast<uint4*>(hx);
+      gu[u] = *reinterpret_cast<uint4*>(hg);
     } else {
-      xu[u] = reinterpret_cast<const uint2*>(x)[unit];
-      if (norm) gu[u] = reinterpret_cast<const uint2*>(gamma)[unit];
+      xu[u] = reinterpret_cast<const uint4*>(x)[unit];
+      if (norm) gu[u] = reinterpret_cast<const uint4*>(gamma)[unit];
     }
+  }
+  // scale and zero-point of the first row group (row/128, then Inference.cu:90 with the index wrapped to
+  // the m/128 stored entries): requested with x, so that they are there when the first block is done
+  half_t gs = (half_t)0.0f, gz = (half_t)0.0f;
+  if (!PERIODIC) {
+    const unsigned gi = ((unsigned)(rg * RH >> 7) % (unsigned)kg) % (unsigned)mg;
+    gs = scale[gi];
+    gz = zp[gi];
   }
   // Every request for x of this workgroup goes out before any of its requests
   // for weights: the memory pipeline of a compute unit serves requests in order,
@@ -398,14 +450,15 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
     // natural order, the stride-halving tree, then two binary16 multiplies
 #pragma unroll
     for (int u = 0; u < MAXU; ++u) {
-      const int unit = WIDE ? 2 * (tid + (u >> 1) * nthreads) + (u & 1) : tid + u * nthreads;
+      const int unit = tid + u * nthreads;
+      if (!stager) continue;
       if (PERIODIC) {
-        half_t hx[4];
-        *reinterpret_cast<uint64_t*>(hx) = __builtin_bit_cast(uint64_t, xu[u]);
+        half_t hx[8];
+        *reinterpret_cast<uint4*>(hx) = xu[u];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) xn[awq_block_elem(k, C, (4 * unit + i) >> 5, (4 * unit + i) & 31)] = hx[i];
+        for (int i = 0; i < 8; ++i) xn[awq_block_elem(k, C, unit >> 2, (8 * unit + i) & 31)] = hx[i];
       } else {
-        reinterpret_cast<uint2*>(xn)[unit] = xu[u];
+        reinterpret_cast<uint4*>(xn)[unit] = xu[u];
       }
     }
     __syncthreads();
@@ -448,37 +501,30 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
     const half2_t sc2 = half2_t{sc, sc};
 #pragma unroll
     for (int u = 0; u < MAXU; ++u) {
-      half2_t t0 = as_half2(xu[u].x) * sc2, t1 = as_half2(xu[u].y) * sc2;
-      t0 = t0 * as_half2(gu[u].x);
-      t1 = t1 * as_half2(gu[u].y);
-      xu[u].x = __builtin_bit_cast(uint32_t, t0);
-      xu[u].y = __builtin_bit_cast(uint32_t, t1);
+      uint32_t* d = reinterpret_cast<uint32_t*>(&xu[u]);
+      const uint32_t* g = reinterpret_cast<const uint32_t*>(&gu[u]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        half2_t t = as_half2(d[i]) * sc2;
+        t = t * as_half2(g[i]);
+        d[i] = __builtin_bit_cast(uint32_t, t);
+      }
     }
   }
-  // x and the input sum of every block (adjacent-pair tree over its 32 inputs:
-  // four in this thread, then the eight threads that share the block)
-  float sx_prev = 0.0f;
+  // x in block fixed point: nibble planes, the power of two and the integer sum of every block
+  // (four threads share a block)
 #pragma unroll
   for (int u = 0; u < MAXU; ++u) {
-    const int unit = WIDE ? 2 * (tid + (u >> 1) * nthreads) + (u & 1) : tid + u * nthreads;
-    *reinterpret_cast<uint2*>(xs + xs_index<G>(4 * unit)) = xu[u];
-    const half2_t t0 = as_half2(xu[u].x), t1 = as_half2(xu[u].y);
-    float sx = ((float)t0.x + (float)t0.y) + ((float)t1.x + (float)t1.y);
-    if (WIDE) {
-      // the pair of units of this thread first, then the four threads that share the block
-      if ((u & 1) == 0) {
-        sx_prev = sx;
-      } else {
-        sx = sx_prev + sx;
-        sx += dpp_f<kDppXor1>(sx);
-        sx += dpp_f<kDppXor2>(sx);
-        if ((tid & 3) == 0) xsum[unit >> 3] = sx;
-      }
-    } else {
-      sx += dpp_f<kDppXor1>(sx);
-      sx += dpp_f<kDppXor2>(sx);
-      sx += dpp_f<kDppHalfMirror>(sx);
-      if ((tid & 7) == 0) xsum[unit >> 3] = sx;
+    const int unit = tid + u * nthreads;
+    if (!stager) continue;
+    const uint32_t h[4] = {xu[u].x, xu[u].y, xu[u].z, xu[u].w};
+    u32x4 planes;
+    float c, S;
+    stage_unit8(h, planes, c, S);
+    *reinterpret_cast<u32x4*>(xs + (size_t)(unit + (unit / (4 * G))) * 16) = planes;
+    if ((tid & 3) == 0) {
+      xc[unit >> 2] = c;
+      xS[unit >> 2] = S;
     }
   }
 
@@ -490,20 +536,21 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
     gtab[0][tid] = make_group(scale[gi], zp[gi]);
   }
   __syncthreads();  // xs, the block sums and the first table
-  float xb[G];
+  float xcb[G], xSb[G];
   if (G >= 4) {
 #pragma unroll
     for (int b = 0; b < G; b += 4) {
-      const float4 t = *reinterpret_cast<const float4*>(xsum + blk0 + b);
-      xb[b] = t.x;
-      xb[b + 1] = t.y;
-      xb[b + 2] = t.z;
-      xb[b + 3] = t.w;
+      const float4 t = *reinterpret_cast<const float4*>(xc + blk0 + b);
+      const float4 v = *reinterpret_cast<const float4*>(xS + blk0 + b);
+      xcb[b] = t.x, xcb[b + 1] = t.y, xcb[b + 2] = t.z, xcb[b + 3] = t.w;
+      xSb[b] = v.x, xSb[b + 1] = v.y, xSb[b + 2] = v.z, xSb[b + 3] = v.w;
     }
   } else {
 #pragma unroll
-    for (int b = 0; b < G; ++b) xb[b] = xsum[blk0 + b];
+    for (int b = 0; b < G; ++b) xcb[b] = xc[blk0 + b], xSb[b] = xS[blk0 + b];
   }
+  // the G blocks of this lane in LDS: 64 bytes each, the lane group's skew included
+  const unsigned char* xl = xs + (size_t)(blk0 * 4 + blk0 / G) * 16;
   unsigned long long best_here = 0;  // EPI_ARGMAX: best candidate among this lane's rows
   for (int it = 0; rg < n_rg; rg += gridDim.x, ++it) {
     const int rg_next = MULTI ? rg + (int)gridDim.x : n_rg;
@@ -516,13 +563,14 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
     // launch then does not wait for one more round trip to memory
     half_t res = (half_t)0.0f;
     if (tid < RH && epi == EPI_RESIDUAL) res = p.res[rg * RH + r];
-    // scale group of these 16 rows: row/128, then Inference.cu:90 with the index
-    // wrapped to the m/128 stored entries
-    const int a = rg * RH >> 7;
     GroupConst g;
     if (!PERIODIC) {
-      int gi = (a % kg) % mg;
-      g = make_group(scale[gi], zp[gi]);
+      g = make_group(gs, gz);
+      if (MULTI && rg_next < n_rg) {  // the next row group's
+        const unsigned gi = ((unsigned)(rg_next * RH >> 7) % (unsigned)kg) % (unsigned)mg;
+        gs = scale[gi];
+        gz = zp[gi];
+      }
     } else if (MULTI && tid < C && rg_next < n_rg) {
       // the next row group's table; its buffer was last read two barriers ago
       int gi = (int)((((int64_t)tid * mg + (rg_next >> 3)) % kg) % mg);
@@ -542,7 +590,7 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
 #pragma unroll
       for (int b = 0; b < G; ++b) {
         const GroupConst& gb = gc[UFAST > 0 ? b / UFAST : 0];
-        bs[b] = __builtin_fmaf(gb.zn, xb[b], block_dot(w[b], xs + xs_index<G>((blk0 + b) * AWQ_BLOCK_K))) * gb.s;
+        bs[b] = __builtin_fmaf(gb.zn, xSb[b], block_dot(w[b], xl + 64 * b)) * (gb.s * xcb[b]);
       }
     } else {
 #pragma unroll
@@ -554,7 +602,7 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
             cls_left = U;
           }
         }
-        bs[b] = __builtin_fmaf(g.zn, xb[b], block_dot(w[b], xs + xs_index<G>((blk0 + b) * AWQ_BLOCK_K))) * g.s;
+        bs[b] = __builtin_fmaf(g.zn, xSb[b], block_dot(w[b], xl + 64 * b)) * (g.s * xcb[b]);
       }
     }
     // adjacent-pair tree: this lane's G blocks, then the four quarters of the
@@ -565,8 +613,8 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
       for (int i = 0; i < n / 2; ++i) bs[i] = bs[2 * i] + bs[2 * i + 1];
     }
     float v = bs[0];
-#pragma unroll
-    for (int mask = RH; mask < 64; mask <<= 1) v += __shfl_xor(v, mask, 64);
+    if (RH == 8) v += dpp_f<kDppRor8>(v);  // lane i + lane i ^ 8
+    v = sum_rows_of_16(v);
     // The only barrier of the pass.  The 16 finishing lanes read this pass's
     // buffer while the other wavefronts already multiply the next row group; the
     // buffer is written again two passes on, after a barrier those lanes are part of.
@@ -641,7 +689,7 @@ bool plan_gemv(int64_t m, int64_t k, GemvPlan* out) {
   return found;
 }
 
-#define GEMV_HOT_ARGS p.wq, p.x, p.gamma, p.scale, p.zp, p.m, p.prologue, p.epilogue, p.eps, p.mg, p.kg
+#define GEMV_HOT_ARGS p.wq, p.x, p.gamma, p.scale, p.zp, p.mg, p.kg, p.prologue, p.epilogue, p.m, p.eps
 template <int G>
 void launch_g(const GemvParams& p, bool periodic, bool multi, int rh, dim3 grid, dim3 block, size_t lds, hipStream_t st) {
   if (rh == 8) {  // plan_gemv: four blocks per lane, not periodic, one row group per workgroup
@@ -762,7 +810,7 @@ int launch_gemv(const LinearArgs& a, hipStream_t st) {
                                                 // workgroups of 8 wavefronts 60 us, as 1024 of 4 wavefronts 64 us, 576 of 8: 80 us)
   dim3 grid((unsigned)n_wg), block((unsigned)(plan.n_waves * 64));
   // x in block order plus 16 bytes of skew per lane group, the block sums, and with the fused norm x in natural order
-  size_t lds = (size_t)a.k * 2 + (size_t)(a.k / AWQ_BLOCK_K / plan.g) * 16 + (size_t)(a.k / AWQ_BLOCK_K) * 4 +
+  size_t lds = (size_t)a.k * 2 + (size_t)(a.k / AWQ_BLOCK_K / plan.g) * 16 + (size_t)(a.k / AWQ_BLOCK_K) * 8 +
                (a.prologue == PRO_RMSNORM ? (size_t)a.k * 2 : 0);
   AWQ_REQUIRE(lds <= 65536, "k too large for the fused norm (x is kept twice in LDS)");
   switch (plan.g) {

@@ -36,7 +36,7 @@
 
 #define AWQ_GROUP_SIZE 128      /* Inference.cu:40 */
 #define AWQ_HEAD_DIM 128        /* Inference.cu:36 */
-#define AWQ_BLOCK_K 32          /* inputs per block of a linear layer (two fma chains of 16) */
+#define AWQ_BLOCK_K 32          /* inputs per block of a linear layer (one power of two per block) */
 
 AWQ_HD float awq_bits_to_f32(uint32_t u) {
   float f;
@@ -160,22 +160,29 @@ AWQ_HD int awq_group_period(int64_t m, int64_t k) {
  * The k inputs of one output are cut into k/32 blocks; block number blk holds,
  * for t = 0..31, input index
  *     j = c + C*(32*u + t),   C = awq_group_period(m,k), blk = c*(k/(32*C)) + u
- * so that all 32 share one scale group (s, z).  C must divide k/32.  Per block
- *     T = A + B   A: fma chain from 0 over t with t % 4 < 2, B: over t % 4 >= 2,
- *                 each in ascending t, multiplier the raw nibble q as a float
- *     X = the block's 32 inputs added as an adjacent-pair tree (awq_tree_sum)
- *     v = fma(-z, X, T) * s                      (binary32 throughout)
- * and the k/32 block values v are combined by awq_tree_sum; the result is
- * rounded to binary16 once.  The scale and the zero-point are applied to a
- * block's sum rather than to every weight, so the binary16 rounding of each
- * dequantised weight (Inference.cu:102-104) does not appear here; it stays in
- * the standalone dequantisation and in the plain sequential reference that
- * the tests hold this order to (1e-2 relative).
+ * so that all 32 share one scale group (s, z).  C must divide k/32.
  *
- * Why two chains: on the GPU the masked nibble pairs are read as binary16
- * subnormals q*2^-24 (nibbles at bits 0-3 of a half) and q*2^-20 (bits 4-7);
- * the two scalings are powers of two, so each chain equals the unscaled chain
- * times its power of two exactly, and A*2^-20 + B*2^-20 rounds as A + B does.
+ * The inputs of a block are first put into block fixed point (once per input
+ * vector, the same for every output row):
+ *     e    = the largest binary16 exponent field among the 32 inputs (0..31)
+ *     c    = 2^(max(e,1) - 29)                  (a NaN when e == 31: the block holds an infinity or a NaN)
+ *     I[t] = x[t] / c rounded to the nearest integer, ties to even;  |I[t]| <= 32752
+ *     S    = sum I[t]
+ * i.e. a 16-bit integer per input under the block's common power of two: the block's largest inputs keep
+ * all 11 significand bits, an input 2^-n below the largest exponent loses its last n - 5 bits.  Per row
+ *     D = sum q[t] * I[t]                       exact in integers, |D| < 2^24, q the raw nibble
+ *     v = fma(-z, S, D) * (s * c)               binary32; S and D convert exactly, s * c is exact
+ * and the k/32 block values v are combined by awq_tree_sum; the result is rounded to binary16 once.
+ * The scale and the zero-point are applied to a block's sums rather than to every weight, so the binary16
+ * rounding of each dequantised weight (Inference.cu:102-104) does not appear here; it stays in the
+ * standalone dequantisation and in the plain sequential FP32 reference that the tests hold this arithmetic
+ * to (1e-2 relative).  Against the exact product of the unrounded weights the only errors are the
+ * rounding of I (at most c/2 per input, 2^-16 of the block's largest magnitude), one rounding per block
+ * value and the tree.
+ *
+ * Why integers: on the GPU v_dot8_u32_u4 multiplies eight weight nibbles by eight 4-bit digits of the
+ * inputs and adds them up exactly in one instruction, straight from the packed weight dword; a CPU adds
+ * the same integers.  Nothing depends on an order of summation inside a block.
  */
 AWQ_HD int64_t awq_block_elem(int64_t k, int C, int64_t blk, int t) {
   int64_t U = k / ((int64_t)AWQ_BLOCK_K * C);
@@ -183,18 +190,39 @@ AWQ_HD int64_t awq_block_elem(int64_t k, int C, int64_t blk, int t) {
   return c + (int64_t)C * (AWQ_BLOCK_K * u + t);
 }
 
-/* T of one block: q[t] in 0..15, x[t] the block's inputs widened to binary32 */
-AWQ_HD float awq_block_qdot(const int* q, const float* x) {
-  float a = 0.0f, b = 0.0f;
+/* Block fixed point of one block: x[t] the block's 32 inputs widened to binary32 (binary16 values).
+ * Writes I[0..31] and *S, returns c. */
+AWQ_HD float awq_block_fixed(const float* x, int32_t* I, int32_t* S) {
+  uint32_t emax = 0;
   for (int t = 0; t < AWQ_BLOCK_K; ++t) {
-    if ((t & 2) == 0) a = fmaf((float)q[t], x[t], a);
-    else b = fmaf((float)q[t], x[t], b);
+    uint32_t e = (awq_f32_to_bits(x[t]) & 0x7fffffffu) >> 23; /* binary16 field + 112 for a normal half */
+    if (e > emax) emax = e;
   }
-  return a + b;
+  const uint32_t e16 = emax == 255u ? 31u : (emax > 113u ? emax - 112u : 1u); /* max(e,1), 31 = not finite */
+  const uint32_t cbits = (e16 + 98u) << 23;
+  const float inv = awq_bits_to_f32(0x7f000000u - cbits); /* 1/c */
+  int32_t sum = 0;
+  for (int t = 0; t < AWQ_BLOCK_K; ++t) {
+    /* adding 1.5 * 2^23 + 32768 rounds x/c to an integer; its low 16 bits are I + 32768 */
+    const uint32_t u = awq_f32_to_bits(fmaf(x[t], inv, 12615680.0f)) & 0xffffu;
+    I[t] = (int32_t)u - 32768;
+    sum += I[t];
+  }
+  *S = sum;
+  return awq_bits_to_f32(e16 == 31u ? 0x7fc00000u : cbits);
 }
 
-/* v of one block from its T, X and the group's scale and zero-point */
-AWQ_HD float awq_block_value(float T, float X, float s, float z) { return fmaf(-z, X, T) * s; }
+/* D of one block: q[t] in 0..15 */
+AWQ_HD int32_t awq_block_idot(const int* q, const int32_t* I) {
+  int32_t d = 0;
+  for (int t = 0; t < AWQ_BLOCK_K; ++t) d += q[t] * I[t];
+  return d;
+}
+
+/* v of one block from its D, the block's S and c, and the group's scale and zero-point */
+AWQ_HD float awq_block_value(int32_t D, int32_t S, float c, float s, float z) {
+  return fmaf(-z, (float)S, (float)D) * (s * c);
+}
 
 /* Combine n partial sums in place: adjacent pairs while the count is even,
  * then left to right.  Returns the total. */
@@ -206,13 +234,6 @@ AWQ_HD float awq_tree_sum(float* v, int64_t n) {
   float s = v[0];
   for (int64_t a = 1; a < n; ++a) s += v[a];
   return s;
-}
-
-/* X of one block: adjacent-pair tree over its 32 inputs */
-AWQ_HD float awq_block_xsum(const float* x) {
-  float t[AWQ_BLOCK_K];
-  for (int i = 0; i < AWQ_BLOCK_K; ++i) t[i] = x[i];
-  return awq_tree_sum(t, AWQ_BLOCK_K);
 }
 
 #endif /* AWQ_CANON_MATH_H */

@@ -173,9 +173,10 @@ static inline int nibble_at(const uint8_t* packed, int64_t p) {
 //                     rounding (brute-force pin)
 //   awqo_linear_seq   binary32, j ascending, multiply then add, the same dequantised weights:
 //                     the plain FP32-accumulate reference the GPU product is held to (1e-2)
-//   awqo_linear       binary32 in the blocked order of awq_canon_math.h (per block of 32 inputs
-//                     two fma chains over the raw nibbles, the scale and zero-point applied to the
-//                     block's sum), which the GPU kernels also follow: results agree bit for bit
+//   awqo_linear       the blocked arithmetic of awq_canon_math.h (per block of 32 inputs: the inputs in
+//                     block fixed point, exact integer sums over the raw nibbles, the scale and
+//                     zero-point applied to the block's sums in binary32), which the GPU kernels also
+//                     follow: results agree bit for bit
 // ---------------------------------------------------------------------------
 static void build_lut(const half_t* scale, const half_t* zp, int64_t n_groups, std::vector<float>& lut) {
   lut.resize((size_t)n_groups * 16);
@@ -218,7 +219,7 @@ AWQO_API void awqo_linear_seq(const uint8_t* packed, const half_t* scale, const 
   }
 }
 
-// scalar statement of the blocked order (the definition)
+// scalar statement of the blocked arithmetic (the definition)
 AWQO_API void awqo_linear_scalar(const uint8_t* packed, const half_t* scale, const half_t* zp, int64_t m, int64_t k,
                                  const half_t* x, half_t* y, int64_t M) {
   const int C = awq_group_period(m, k);
@@ -230,6 +231,7 @@ AWQO_API void awqo_linear_scalar(const uint8_t* packed, const half_t* scale, con
       for (int64_t blk = 0; blk < nblk; ++blk) {
         int q[AWQ_BLOCK_K];
         float xf[AWQ_BLOCK_K];
+        int32_t I[AWQ_BLOCK_K], S;
         int g = 0;
         for (int e = 0; e < AWQ_BLOCK_K; ++e) {
           int64_t j = awq_block_elem(k, C, blk, e);
@@ -237,27 +239,29 @@ AWQO_API void awqo_linear_scalar(const uint8_t* packed, const half_t* scale, con
           q[e] = nibble_at(packed, j * m + i);
           xf[e] = h2f(x[t * k + j]);
         }
-        part[blk] = awq_block_value(awq_block_qdot(q, xf), awq_block_xsum(xf), h2f(scale[g]), h2f(zp[g]));
+        const float c = awq_block_fixed(xf, I, &S);
+        part[blk] = awq_block_value(awq_block_idot(q, I), S, c, h2f(scale[g]), h2f(zp[g]));
       }
       y[t * m + i] = f2h(awq_tree_sum(part.data(), nblk));
     }
   }
 }
 
-// AVX2 evaluation of the same order: 8 outputs per vector, each lane its own
-// pair of fma chains, so the bits equal awqo_linear_scalar (tests compare the two).
+// AVX2 evaluation of the same arithmetic: 8 outputs per vector, integer sums per lane (exact, so the
+// bits equal awqo_linear_scalar; tests compare the two).
 // Returns the FP32 sums before rounding when y32 != NULL.
 static void linear_blocked(const uint8_t* packed, const half_t* scale, const half_t* zp, int64_t m, int64_t k,
                            const half_t* x, half_t* y, float* y32) {
   const int C = awq_group_period(m, k);
   const int64_t nblk = k / AWQ_BLOCK_K;
   const int64_t RC = 64;  // rows per task
-  std::vector<float> xf((size_t)k), xsum((size_t)nblk);
-  for (int64_t j = 0; j < k; ++j) xf[j] = h2f(x[j]);
+  // block fixed point of x, once per input vector
+  std::vector<int32_t> xi((size_t)k), xS((size_t)nblk);
+  std::vector<float> xc((size_t)nblk);
   for (int64_t blk = 0; blk < nblk; ++blk) {
     float t[AWQ_BLOCK_K];
-    for (int e = 0; e < AWQ_BLOCK_K; ++e) t[e] = xf[awq_block_elem(k, C, blk, e)];
-    xsum[blk] = awq_block_xsum(t);
+    for (int e = 0; e < AWQ_BLOCK_K; ++e) t[e] = h2f(x[awq_block_elem(k, C, blk, e)]);
+    xc[blk] = awq_block_fixed(t, &xi[blk * AWQ_BLOCK_K], &xS[blk]);
   }
   const __m256i shifts = _mm256_setr_epi32(0, 4, 8, 12, 16, 20, 24, 28);
   const __m256i nib = _mm256_set1_epi32(15);
@@ -267,27 +271,26 @@ static void linear_blocked(const uint8_t* packed, const half_t* scale, const hal
 #pragma omp for schedule(dynamic, 4)
     for (int64_t i0 = 0; i0 < m; i0 += RC) {
       for (int64_t blk = 0; blk < nblk; ++blk) {
-        __m256 accA[8], accB[8];
-        for (int v = 0; v < 8; ++v) accA[v] = accB[v] = _mm256_setzero_ps();
+        __m256i acc[8];
+        for (int v = 0; v < 8; ++v) acc[v] = _mm256_setzero_si256();
         int g = 0;
         for (int e = 0; e < AWQ_BLOCK_K; ++e) {
           int64_t j = awq_block_elem(k, C, blk, e);
           g = awq_group_index(m, k, i0, j);  // 64 rows starting at a multiple of 64 share a group, a block too
           const uint8_t* src = packed + ((j * m + i0) >> 1);
-          __m256 xv = _mm256_set1_ps(xf[j]);
-          __m256* acc = (e & 2) ? accB : accA;
+          // q (0..15) times I (16 bits) as one 16-bit multiply-add per 32-bit lane: the upper halves are zero
+          const __m256i iv = _mm256_set1_epi32(xi[blk * AWQ_BLOCK_K + e] & 0xffff);
           for (int v = 0; v < 8; ++v) {
             uint32_t w32;
             memcpy(&w32, src + 4 * v, 4);
             __m256i q = _mm256_and_si256(_mm256_srlv_epi32(_mm256_set1_epi32((int)w32), shifts), nib);
-            acc[v] = _mm256_fmadd_ps(_mm256_cvtepi32_ps(q), xv, acc[v]);
+            acc[v] = _mm256_add_epi32(acc[v], _mm256_madd_epi16(q, iv));
           }
         }
-        const __m256 zn = _mm256_set1_ps(-h2f(zp[g])), sc = _mm256_set1_ps(h2f(scale[g])), X = _mm256_set1_ps(xsum[blk]);
-        for (int v = 0; v < 8; ++v) {
-          __m256 T = _mm256_add_ps(accA[v], accB[v]);
-          _mm256_storeu_ps(&part[blk * RC + 8 * v], _mm256_mul_ps(_mm256_fmadd_ps(zn, X, T), sc));
-        }
+        const __m256 zn = _mm256_set1_ps(-h2f(zp[g])), sc = _mm256_set1_ps(h2f(scale[g]) * xc[blk]),
+                     S = _mm256_set1_ps((float)xS[blk]);
+        for (int v = 0; v < 8; ++v)
+          _mm256_storeu_ps(&part[blk * RC + 8 * v], _mm256_mul_ps(_mm256_fmadd_ps(zn, S, _mm256_cvtepi32_ps(acc[v])), sc));
       }
       // awq_tree_sum over blocks, 64 rows at a time
       int64_t n = nblk;

@@ -135,6 +135,39 @@ def test_gemv_bit_exact_and_within_tolerance(awq, lib, oracle, torch_gpu, m, k, 
         assert np.array_equal(auto.view(np.uint16), ref.view(np.uint16))
 
 
+@pytest.mark.parametrize("m,k", [(256, 1024), (384, 512), (4096, 4096), (128 * 37, 512)])
+def test_gemv_input_dynamic_range(awq, lib, oracle, torch_gpu, m, k):
+    """the inputs' block fixed point at its corners: subnormal and zero blocks, inputs far below their
+    block's largest, the largest binary16 values, and blocks that hold an infinity or a NaN"""
+    torch = torch_gpu
+    rng = np.random.default_rng(m + 7 * k)
+    packed, scale, zp = rand_awq(rng, m, k, zp_int=False)
+    x = rng.standard_normal(k).astype(np.float16)
+    x[0:32] = 0                                                     # a block of zeros (one of them negative)
+    x[5] = np.float16(-0.0)
+    x[32:64] = (rng.integers(-1023, 1024, 32).astype(np.float64) * 2.0 ** -24).astype(np.float16)   # subnormals only
+    x[64:96] *= np.float16(2.0 ** -12)                              # small normals and subnormals mixed
+    x[96:128] = np.clip(rng.standard_normal(32) * 20000, -65504, 65504).astype(np.float16)  # up to the top of the range
+    x[100] = np.float16(65504)
+    x[130] = np.float16(3000)                                       # one large input among ordinary ones
+    x[200] = np.float16(6e-8)                                       # the smallest subnormal among ordinary ones
+    for case in ("finite", "inf", "nan"):
+        if case == "inf":
+            x[300] = np.inf
+            x[40] = -np.inf
+        if case == "nan":
+            x[450] = np.nan
+        ref = np.zeros(m, dtype=np.float16)
+        oracle.awqo_linear(ptr(packed), ptr(scale), ptr(zp), m, k, ptr(x), ptr(ref), 1)
+        got = gemv_gpu(awq, lib, torch, packed, scale, zp, m, k, x, 0)[0]
+        print("gemv range", m, k, case, flush=True)
+        assert np.array_equal(got.view(np.uint16), ref.view(np.uint16))
+        if case == "finite":
+            assert not np.any(np.isnan(ref))                        # a large sum may round to an infinity
+        else:
+            assert np.all(ref.view(np.uint16) == 0x7e00)            # every row sums every block
+
+
 def test_gemv_unembed_shape_and_argmax(awq, lib, oracle, torch_gpu):
     """config 3: 151936 x 4096 unembedding (scale-group period 32) followed by greedy argmax"""
     torch = torch_gpu

@@ -221,14 +221,17 @@ def test_linear_orders_agree(oracle, m, k):
 
 
 def test_linear_blocked_order_definition(oracle):
-    # independent numpy statement of the blocked order: per block of 32 inputs two fma chains over the
-    # raw nibbles (t % 4 < 2 and t % 4 >= 2), their sum, minus zero-point times the block's input sum
-    # (adjacent-pair tree), times the scale; blocks combined by the adjacent-pair tree
+    # independent numpy statement of the blocked arithmetic: per block of 32 inputs the inputs in block fixed
+    # point (16-bit integers under the power of two of the block's largest exponent, round to nearest even),
+    # the exact integer sums D = sum q*I and S = sum I, v = fma(-z, S, D) * (s*c) in binary32; blocks
+    # combined by the adjacent-pair tree
     m, k = 384, 512  # period 4
     C = oracle.awqo_group_period(m, k)
     assert C == 4
     packed, scale, zp = rand_awq(m, k)
     x = RNG.standard_normal(k).astype(np.float16)
+    x[7] = np.float16(6e-6)      # a subnormal among normals
+    x[64:96] *= np.float16(1e-4)  # blocks of small inputs, some of them subnormal
     nib = nibbles_flat(packed)
     y = run_linear(oracle, "awqo_linear", packed, scale, zp, m, k, x[None, :].copy(), 1, np.float16)[0]
     nblk = k // 32
@@ -248,26 +251,49 @@ def test_linear_blocked_order_definition(oracle):
     for i in [0, 1, 127, 128, 383]:
         parts = []
         for blk in range(nblk):
-            a = b = f32(0)
-            xs = []
-            g = None
-            for t in range(32):
-                j = block_elem(k, C, blk, t)
-                gj = oracle.awqo_group_index(m, k, i, j)
-                assert g is None or g == gj      # a block never straddles scale groups
-                g = gj
-                q = float(nib[j * m + i])
-                # fma in binary32: q * x is exact in float64, one rounding of the sum
-                if t % 4 < 2:
-                    a = f32(np.float64(q) * np.float64(x[j]) + np.float64(a))
-                else:
-                    b = f32(np.float64(q) * np.float64(x[j]) + np.float64(b))
-                xs.append(f32(x[j]))
-            T = f32(a + b)
-            X = tree(xs)
-            v = f32(np.float64(-f32(zp[g])) * np.float64(X) + np.float64(T))      # fma(-z, X, T)
-            parts.append(f32(v * f32(scale[g])))
+            js = [block_elem(k, C, blk, t) for t in range(32)]
+            gs = {oracle.awqo_group_index(m, k, i, j) for j in js}
+            assert len(gs) == 1                  # a block never straddles scale groups
+            g = gs.pop()
+            xb = x[js]
+            e = int((xb.view(np.uint16) & 0x7fff).max()) >> 10
+            c = 2.0 ** (max(e, 1) - 29)
+            I = np.rint(xb.astype(np.float64) / c).astype(np.int64)   # rint: ties to even
+            assert np.abs(I).max() <= 32752
+            D = int(sum(int(nib[j * m + i]) * int(v) for j, v in zip(js, I)))
+            S = int(I.sum())
+            assert abs(D) < 2 ** 24
+            v = f32(-np.float64(zp[g]) * S + D)                       # one rounding: the fma
+            parts.append(f32(np.float64(v) * np.float64(f32(np.float64(scale[g]) * c))))
         assert np.float16(tree(parts)) == y[i], i
+
+
+def test_linear_block_fixed_point_is_exact_for_narrow_blocks(oracle):
+    # inputs whose exponents lie within 5 of the block's largest are represented exactly, so with scale 1 and
+    # zero-point 0 the product is the exact integer-weighted sum rounded once per block and once at the end;
+    # small integers make every step exact
+    m, k = 128, 512
+    scale = np.ones(1, dtype=np.float16)
+    zp = np.full(1, 3, dtype=np.float16)
+    packed = RNG.integers(0, 256, m * k // 2, dtype=np.uint8)
+    x = RNG.integers(-12, 13, k).astype(np.float16)
+    y = run_linear(oracle, "awqo_linear", packed, scale, zp, m, k, x[None, :].copy(), 1, np.float16)[0]
+    W = nibbles_flat(packed).reshape(k, m).T.astype(np.int64) - 3
+    ref = W @ x.astype(np.int64)
+    assert np.abs(ref).max() < 2 ** 24
+    assert np.array_equal(y.astype(np.float64), ref.astype(np.float16).astype(np.float64))
+
+
+def test_linear_infinity_or_nan_in_a_block_gives_nan(oracle):
+    # a block that holds a value that is not finite has no power of two: its value is a NaN for every row
+    m, k = 128, 512
+    packed, scale, zp = rand_awq(m, k)
+    for bad in (np.inf, -np.inf, np.nan):
+        x = RNG.standard_normal(k).astype(np.float16)
+        x[100] = bad
+        for fn in ("awqo_linear", "awqo_linear_scalar"):
+            y = run_linear(oracle, fn, packed, scale, zp, m, k, x[None, :].copy(), 1, np.float16)[0]
+            assert np.all(y.view(np.uint16) == 0x7e00), (fn, bad)
 
 
 # ----------------------------------------------------------------------------- RMSNorm (Inference.cu:111-145)
