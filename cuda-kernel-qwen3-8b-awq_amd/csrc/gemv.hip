@@ -112,7 +112,7 @@ __device__ __forceinline__ float block_dot(const u32x4& w, const unsigned char* 
     a3 = __builtin_amdgcn_udot8(d[c], xv.w, a3, false);
     aq = __builtin_amdgcn_udot8(d[c], 0x11111111u, aq, false);
   }
-  const uint32_t D = ((((a3 << 4) + a2) << 4) + a1 << 4) + a0 - (aq << 15);
+  const uint32_t D = a0 + (a1 << 4) + (a2 << 8) + (a3 << 12) - (aq << 15);
   return (float)(int32_t)D;
 }
 
@@ -125,6 +125,20 @@ constexpr int kDppXor1 = 0xB1;        // quad_perm:[1,0,3,2]
 constexpr int kDppXor2 = 0x4E;        // quad_perm:[2,3,0,1]
 constexpr int kDppHalfMirror = 0x141; // lane i <-> 7 - i within 8
 constexpr int kDppRor4 = 0x124, kDppRor8 = 0x128;
+
+// (half)awq_rsqrtf(v), i.e. the binary16 rounding of a correctly rounded 1/sqrt (Inference.cu:137-138), in a
+// handful of instructions for almost every argument.  The hardware's reciprocal square root e is within one
+// unit in the last place of 1/sqrt(v), and so is the canonical value (a correctly rounded square root, then
+// a correctly rounded reciprocal); both lie between e (1 - 2^-20) and e (1 + 2^-20).  When those two bounds
+// round to the same binary16 number, everything between them does, so that number is the result; otherwise
+// (one argument in a few hundred, and NaNs) the canonical sequence of some forty instructions decides.  The
+// argument is the same in every lane, so the branch does not diverge.
+__device__ __forceinline__ half_t rsqrt_half(float v) {
+  const float e = __builtin_amdgcn_rsqf(v);
+  const half_t lo = (half_t)(e * 0.99999905f), hi = (half_t)(e * 1.00000095f);
+  if (__builtin_bit_cast(unsigned short, lo) == __builtin_bit_cast(unsigned short, hi) && lo == lo) return lo;
+  return (half_t)awq_rsqrtf(v);
+}
 
 // v(lane) + v(lane ^ 16), then that + the same of lane ^ 32: the four rows of 16 lanes added as
 // (row0 + row1) + (row2 + row3) in every lane.  gfx950's lane-swap instructions exchange rows between
@@ -497,7 +511,7 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
     tot += dpp_f<kDppXor2>(tot);
     tot += dpp_f<kDppXor1>(tot);
     tot = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, tot)));
-    const half_t sc = (half_t)awq_rsqrtf(tot / (float)k + eps);
+    const half_t sc = rsqrt_half(tot / (float)k + eps);
     const half2_t sc2 = half2_t{sc, sc};
 #pragma unroll
     for (int u = 0; u < MAXU; ++u) {
