@@ -19,6 +19,8 @@
 #include "common.hpp"
 #include <stdlib.h>
 
+#include <algorithm>
+
 namespace {
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -396,10 +398,13 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
   unsigned char* xs = smem;                                                      // 2k bytes of nibble planes + skew
   float* xc = reinterpret_cast<float*>(smem + (size_t)(k + (nblk / G) * 8) * 2);  // nblk powers of two
   float* xS = xc + nblk;                                                         // nblk integer sums
-  half_t* xn = reinterpret_cast<half_t*>(xS + nblk);                             // k halves (fused norm only)
+  // PERIODIC: the group constants of every (pass, class) of this workgroup, filled once
+  GroupConst* gt = reinterpret_cast<GroupConst*>(xS + nblk);
+  const int n_pass = MULTI ? (m / RH + (int)gridDim.x - 1) / (int)gridDim.x : 1;  // passes of the longest-running workgroup
+  float* ysum = reinterpret_cast<float*>(gt + (PERIODIC ? (n_pass * C + 1 & ~1) : 0));  // MULTI: a pass's finished sums, RH per pass
+  half_t* xn = reinterpret_cast<half_t*>(ysum + (MULTI ? n_pass * RH : 0));      // k halves (fused norm only)
   __shared__ float red[2][16][16];  // double-buffered: one barrier per row group
   __shared__ __attribute__((aligned(16))) float part[256];
-  __shared__ GroupConst gtab[2][PERIODIC ? 64 : 1];
   // A thread stages units of 8 consecutive block-order inputs (the inputs of one weight dword): k/8 units over
   // n_waves * 64 = k/(G*Q/2) threads, i.e. G*Q/16 units per thread, or one unit in every second thread
   constexpr int MAXU = G * Q >= 16 ? G * Q / 16 : 1;
@@ -545,11 +550,23 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
   // Group constants.  When the scale group depends on the input index it is
   // constant within a class of blocks; the (at most 64) classes of a row group
   // go through a table in LDS, filled one row group ahead.
-  if (PERIODIC && tid < C && rg < n_rg) {
-    int gi = (int)((((int64_t)tid * mg + (rg >> 3)) % kg) % mg);
-    gtab[0][tid] = make_group(scale[gi], zp[gi]);
+  // Group constants.  When the scale group depends on the input index it is constant within a class of
+  // blocks; the (at most 64) classes of every row group this workgroup will walk go into a table in LDS
+  // here, so that the loop issues no loads but the weights'.  (A value requested and used inside the loop
+  // makes its wavefront wait for every load issued before it, the weights just requested for the next pass
+  // among them, and the whole workgroup with it at the pass's barrier.)
+  if (PERIODIC) {
+    for (int e = tid; e < n_pass * C; e += nthreads) {
+      const int pass = e / C, cls = e - pass * C;
+      const int row_group = blockIdx.x + pass * (int)gridDim.x;
+      if (row_group < n_rg) {
+        // 32-bit arithmetic: class * m/128 stays far below 2^31
+        const unsigned gi = (((unsigned)cls * (unsigned)mg + (unsigned)(row_group >> 3)) % (unsigned)kg) % (unsigned)mg;
+        gt[e] = make_group(scale[gi], zp[gi]);
+      }
+    }
   }
-  __syncthreads();  // xs, the block sums and the first table
+  __syncthreads();  // xs, the block sums and the table
   float xcb[G], xSb[G];
   if (G >= 4) {
 #pragma unroll
@@ -566,30 +583,30 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
   // the G blocks of this lane in LDS: 64 bytes each, the lane group's skew included
   const unsigned char* xl = xs + (size_t)(blk0 * 4 + blk0 / G) * 16;
   unsigned long long best_here = 0;  // EPI_ARGMAX: best candidate among this lane's rows
-  for (int it = 0; rg < n_rg; rg += gridDim.x, ++it) {
-    const int rg_next = MULTI ? rg + (int)gridDim.x : n_rg;
-    if (MULTI && rg_next < n_rg) {
-      const u32x4* wpn = wq + ((int64_t)(rg_next * RH >> 4) * nblk + blk0) * 16 + ((rg_next * RH) & 15) + r;
+
+  // the weights of one row group, and (one scale group per 16 rows) its scale and zero-point
+  auto request = [&](u32x4(&dst)[G], half_t& s_out, half_t& z_out, int row_group) {
+    const u32x4* src = wq + ((int64_t)(row_group * RH >> 4) * nblk + blk0) * 16 + ((row_group * RH) & 15) + r;
 #pragma unroll
-      for (int b = 0; b < G; ++b) wn[b] = __builtin_nontemporal_load(wpn + b * 16);
+    for (int b = 0; b < G; ++b) dst[b] = __builtin_nontemporal_load(src + b * 16);
+    if (!PERIODIC) {
+      const unsigned gi = ((unsigned)(row_group * RH >> 7) % (unsigned)kg) % (unsigned)mg;
+      s_out = scale[gi];
+      z_out = zp[gi];
     }
+  };
+
+  // One pass: row group row_group from the weights in wc.  With MULTI the finished sums stay in LDS until
+  // the workgroup has walked all its row groups: a store inside the loop would share the counter of
+  // outstanding memory operations with the loads requested for the next pass, and since loads and stores
+  // complete in no fixed order relative to each other every wait for weights would have to wait for
+  // everything outstanding -- the next pass's weights included (151936 x 4096: 59 -> 5x us).
+  auto pass = [&](const u32x4(&wc)[G], half_t s_cur, half_t z_cur, int row_group, int it) {
     // the residual row is requested before the pass multiplies: the end of the
     // launch then does not wait for one more round trip to memory
     half_t res = (half_t)0.0f;
-    if (tid < RH && epi == EPI_RESIDUAL) res = p.res[rg * RH + r];
-    GroupConst g;
-    if (!PERIODIC) {
-      g = make_group(gs, gz);
-      if (MULTI && rg_next < n_rg) {  // the next row group's
-        const unsigned gi = ((unsigned)(rg_next * RH >> 7) % (unsigned)kg) % (unsigned)mg;
-        gs = scale[gi];
-        gz = zp[gi];
-      }
-    } else if (MULTI && tid < C && rg_next < n_rg) {
-      // the next row group's table; its buffer was last read two barriers ago
-      int gi = (int)((((int64_t)tid * mg + (rg_next >> 3)) % kg) % mg);
-      gtab[(it + 1) & 1][tid] = make_group(scale[gi], zp[gi]);
-    }
+    if (!MULTI && tid < RH && epi == EPI_RESIDUAL) res = p.res[row_group * RH + r];
+    GroupConst g = make_group(s_cur, z_cur);
     int cls = 0, cls_left = 0;  // class of the next block and blocks left in it
     if (PERIODIC) {
       cls = blk0 / U;
@@ -600,23 +617,23 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
       constexpr int NC = UFAST > 0 ? G / UFAST : 1;
       GroupConst gc[NC];
 #pragma unroll
-      for (int c = 0; c < NC; ++c) gc[c] = gtab[it & 1][blk0 / UFAST + c];
+      for (int c = 0; c < NC; ++c) gc[c] = gt[it * C + blk0 / UFAST + c];
 #pragma unroll
       for (int b = 0; b < G; ++b) {
         const GroupConst& gb = gc[UFAST > 0 ? b / UFAST : 0];
-        bs[b] = __builtin_fmaf(gb.zn, xSb[b], block_dot(w[b], xl + 64 * b)) * (gb.s * xcb[b]);
+        bs[b] = __builtin_fmaf(gb.zn, xSb[b], block_dot(wc[b], xl + 64 * b)) * (gb.s * xcb[b]);
       }
     } else {
 #pragma unroll
       for (int b = 0; b < G; ++b) {
         if (PERIODIC) {
-          g = gtab[it & 1][cls];
+          g = gt[it * C + cls];
           if (--cls_left == 0) {
             ++cls;
             cls_left = U;
           }
         }
-        bs[b] = __builtin_fmaf(g.zn, xSb[b], block_dot(w[b], xl + 64 * b)) * (g.s * xcb[b]);
+        bs[b] = __builtin_fmaf(g.zn, xSb[b], block_dot(wc[b], xl + 64 * b)) * (g.s * xcb[b]);
       }
     }
     // adjacent-pair tree: this lane's G blocks, then the four quarters of the
@@ -653,11 +670,47 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
 #pragma unroll
       for (int i = 1; i < 16; ++i)
         if (i < n) tot += t[i];
-      epilogue(p, epi, rg * RH + r, r, tot, res, best_here);
+      if (MULTI) ysum[it * RH + r] = tot;
+      else epilogue(p, epi, row_group * RH + r, r, tot, res, best_here);
     }
-    if (!MULTI) break;
-#pragma unroll
-    for (int b = 0; b < G; ++b) w[b] = wn[b];
+  };
+
+  if (!MULTI) {
+    pass(w, gs, gz, rg, 0);
+  } else if (rg < n_rg) {
+    // Two register sets take turns, so that no pass copies weights, and the last pass is written out
+    // on its own, so that every request inside the loop is unconditional: the compiler then knows how
+    // many younger loads are outstanding when it waits for a pass's weights and lets them stay in flight.
+    // (Requesting two passes ahead with three register sets measured the same, 151936 x 4096 in 57 us
+    // either way: a compute unit keeps about 37 KB of requests in flight whatever its wavefronts have
+    // asked for, which at the memory's latency under load is about 6 TB/s for the device.)
+    const int step = (int)gridDim.x;
+    half_t gsn = (half_t)0.0f, gzn = (half_t)0.0f;
+    int it = 0;
+    while (true) {
+      if (rg + step >= n_rg) {
+        pass(w, gs, gz, rg, it);
+        break;
+      }
+      request(wn, gsn, gzn, rg + step);
+      pass(w, gs, gz, rg, it);
+      rg += step, ++it;
+      if (rg + step >= n_rg) {
+        pass(wn, gsn, gzn, rg, it);
+        break;
+      }
+      request(w, gs, gz, rg + step);
+      pass(wn, gsn, gzn, rg, it);
+      rg += step, ++it;
+    }
+    // the epilogues of all passes: each finishing lane reads back what it wrote
+    if (tid < RH) {
+      int row_group = blockIdx.x;
+      for (int i = 0; row_group < n_rg; row_group += step, ++i) {
+        const half_t res = epi == EPI_RESIDUAL ? p.res[row_group * RH + r] : (half_t)0.0f;
+        epilogue(p, epi, row_group * RH + r, r, ysum[i * RH + r], res, best_here);
+      }
+    }
   }
   if (epi == EPI_ARGMAX && tid < RH) {
     // one 64-bit atomic max per workgroup at most: a workgroup that finds a better candidate already
@@ -820,11 +873,15 @@ int launch_gemv(const LinearArgs& a, hipStream_t st) {
   // one workgroup per row group while that fits the device a few times over;
   // beyond that a workgroup walks several row groups and stages x once
   int64_t n_rg = a.m / plan.rh, n_wg = n_rg;
-  if (n_rg > 1024) n_wg = 4096 / plan.n_waves;  // four wavefronts per SIMD (measured: 151936 x 4096 with argmax as 512
+  if (n_rg > 1024) n_wg = std::max<int64_t>(4096 / plan.n_waves, (n_rg + 31) / 32);  // at most 32 passes: the table of
+                                                                                      // group constants is per pass  // four wavefronts per SIMD (measured: 151936 x 4096 with argmax as 512
                                                 // workgroups of 8 wavefronts 60 us, as 1024 of 4 wavefronts 64 us, 576 of 8: 80 us)
   dim3 grid((unsigned)n_wg), block((unsigned)(plan.n_waves * 64));
-  // x in block order plus 16 bytes of skew per lane group, the block sums, and with the fused norm x in natural order
+  // x as nibble planes plus 16 bytes of skew per lane group, two floats per block, the table of group
+  // constants of a periodic matrix (passes x classes), and with the fused norm x in natural order
+  const int64_t n_pass = (n_rg + n_wg - 1) / n_wg;
   size_t lds = (size_t)a.k * 2 + (size_t)(a.k / AWQ_BLOCK_K / plan.g) * 16 + (size_t)(a.k / AWQ_BLOCK_K) * 8 +
+               (periodic ? (size_t)(n_pass * p.C + 1 & ~1) * sizeof(GroupConst) : 0) + (size_t)n_pass * plan.rh * 4 +
                (a.prologue == PRO_RMSNORM ? (size_t)a.k * 2 : 0);
   AWQ_REQUIRE(lds <= 65536, "k too large for the fused norm (x is kept twice in LDS)");
   switch (plan.g) {
