@@ -255,6 +255,9 @@ struct SampleFinish {
 };
 
 // the 16 finished rows of a workgroup; r = lane = row % 16, lanes 0..15 of wavefront 0
+// (Requesting the position, cosine and sine of the rotary epilogue at the start of the launch instead of after
+// the reduction was tried in three forms -- position before the weight requests, after them, as a vector load
+// with x -- and made the launch 0.4 to 1.0 us slower each time.)
 __device__ __forceinline__ void epilogue(const GemvParams& p, int epi, int row, int r, float acc, half_t res,
                                          unsigned long long& best_here) {
   half_t v = (half_t)acc;
@@ -383,11 +386,15 @@ __global__ __launch_bounds__(256) void sample_finish_kernel(SampleFinish f) {
 // workgroup takes half a 16-row group (its wavefront loads are eight 128-byte pieces) and covers the same
 // number of blocks per wavefront with half the blocks per lane, so a matrix with few rows and long k
 // (4096 x 12288: 256 row groups, 12 wavefronts each) runs as twice the workgroups -- two per compute unit.
-template <int G, bool PERIODIC, int UFAST = 0, int NWC = 0, bool MULTI = true, int RH = 16>
+// PRO, EPI: the prologue and the epilogue when they are known at compile time (the model's own launches), -1 =
+// taken from the arguments.
+template <int G, bool PERIODIC, int UFAST = 0, int NWC = 0, bool MULTI = true, int RH = 16, int PRO = -1, int EPI = -1>
 __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
     const u32x4* __restrict__ wq, const half_t* __restrict__ x, const half_t* __restrict__ gamma,
-    const half_t* __restrict__ scale, const half_t* __restrict__ zp, int32_t mg, int32_t kg, int32_t prologue,
-    int32_t epi, int32_t m, float eps, GemvParams p) {
+    const half_t* __restrict__ scale, const half_t* __restrict__ zp, int32_t mg, int32_t kg, int32_t prologue_arg,
+    int32_t epi_arg, int32_t m, float eps, GemvParams p) {
+  const int prologue = PRO >= 0 ? PRO : prologue_arg;
+  const int epi = EPI >= 0 ? EPI : epi_arg;
   const int n_waves = NWC ? NWC : p.n_waves;
   constexpr int Q = 64 / RH;  // lanes that share a row = consecutive block ranges of a wavefront
   static_assert(RH == 16 || (RH == 8 && !PERIODIC), "half row groups are for one scale group per 16 rows");
@@ -760,7 +767,9 @@ bool plan_gemv(int64_t m, int64_t k, GemvPlan* out) {
 template <int G>
 void launch_g(const GemvParams& p, bool periodic, bool multi, int rh, dim3 grid, dim3 block, size_t lds, hipStream_t st) {
   if (rh == 8) {  // plan_gemv: four blocks per lane, not periodic, one row group per workgroup
-    if (p.n_waves == 12) hipLaunchKernelGGL((gemv_kernel<4, false, 0, 12, false, 8>), grid, block, lds, st, GEMV_HOT_ARGS, p);
+    if (p.n_waves == 12 && p.prologue == PRO_NONE && p.epilogue == EPI_RESIDUAL)
+      hipLaunchKernelGGL((gemv_kernel<4, false, 0, 12, false, 8, PRO_NONE, EPI_RESIDUAL>), grid, block, lds, st, GEMV_HOT_ARGS, p);
+    else if (p.n_waves == 12) hipLaunchKernelGGL((gemv_kernel<4, false, 0, 12, false, 8>), grid, block, lds, st, GEMV_HOT_ARGS, p);
     else hipLaunchKernelGGL((gemv_kernel<4, false, 0, 0, true, 8>), grid, block, lds, st, GEMV_HOT_ARGS, p);
     return;
   }
@@ -778,8 +787,17 @@ void launch_g(const GemvParams& p, bool periodic, bool multi, int rh, dim3 grid,
   }
   // the per-layer matrices of the model: 4096 inputs as 4 wavefronts x 8 blocks or 8 x 4, 12288 as 12 x 8
   if (!multi && G == 8 && p.n_waves == 12) hipLaunchKernelGGL((gemv_kernel<G, false, 0, 12, false>), grid, block, lds, st, GEMV_HOT_ARGS, p);
-  else if (!multi && G == 4 && p.n_waves == 8) hipLaunchKernelGGL((gemv_kernel<G, false, 0, 8, false>), grid, block, lds, st, GEMV_HOT_ARGS, p);
-  else hipLaunchKernelGGL((gemv_kernel<G, false>), grid, block, lds, st, GEMV_HOT_ARGS, p);
+  else if (!multi && G == 4 && p.n_waves == 8) {
+    // the model's own launches with 4096 inputs: prologue and epilogue are compile-time constants too
+    if (p.prologue == PRO_RMSNORM && p.epilogue == EPI_QKV_ROPE)
+      hipLaunchKernelGGL((gemv_kernel<G, false, 0, 8, false, 16, PRO_RMSNORM, EPI_QKV_ROPE>), grid, block, lds, st, GEMV_HOT_ARGS, p);
+    else if (p.prologue == PRO_RMSNORM && p.epilogue == EPI_GELU)
+      hipLaunchKernelGGL((gemv_kernel<G, false, 0, 8, false, 16, PRO_RMSNORM, EPI_GELU>), grid, block, lds, st, GEMV_HOT_ARGS, p);
+    else if (p.prologue == PRO_NONE && p.epilogue == EPI_RESIDUAL)
+      hipLaunchKernelGGL((gemv_kernel<G, false, 0, 8, false, 16, PRO_NONE, EPI_RESIDUAL>), grid, block, lds, st, GEMV_HOT_ARGS, p);
+    else
+      hipLaunchKernelGGL((gemv_kernel<G, false, 0, 8, false>), grid, block, lds, st, GEMV_HOT_ARGS, p);
+  } else hipLaunchKernelGGL((gemv_kernel<G, false>), grid, block, lds, st, GEMV_HOT_ARGS, p);
 }
 
 }  // namespace
