@@ -1019,7 +1019,9 @@ extern "C" int awq_time_linear(awq_engine* e, int kind, int32_t n_rounds, float*
   if (crc) return crc;
   AWQ_HIP_TRY(cerr);
   AWQ_HIP_TRY(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0));
-  AWQ_HIP_TRY(hipGraphLaunch(exec, e->stream));  // warm-up of the graph itself
+  // warm-up: as many replays as are timed (at most 16): the first rounds after other work (another
+  // shape's launches, an idle stretch) read up to 5 % long
+  for (int r = 0; r < std::min(replays, 16); ++r) AWQ_HIP_TRY(hipGraphLaunch(exec, e->stream));
   AWQ_HIP_TRY(hipEventRecord(ev0, e->stream));
   for (int r = 0; r < replays; ++r) AWQ_HIP_TRY(hipGraphLaunch(exec, e->stream));
   AWQ_HIP_TRY(hipEventRecord(ev1, e->stream));

@@ -13,9 +13,11 @@
 // 16*rg + r; a wavefront load is four contiguous 256-byte pieces, and the G
 // loads of a lane walk 256*G contiguous bytes per quarter.  Inside the 16
 // bytes, dword c holds elements 8c..8c+7 with nibble positions
-// {0,16,4,20,8,24,12,28}[t & 7]: masking with 0x000f000f / 0x00f000f0 (and the
-// same after one shift by 8) yields two weights as a packed pair of binary16
-// subnormals q * 2^-24 or q * 2^-20.
+// {0,16,4,20,8,24,12,28}[t & 7].  The decode kernel multiplies a dword as it
+// is (eight 4-bit weights against eight 4-bit digits of the inputs, laid out the
+// same way, in one v_dot8_u32_u4); the matrix-core kernels mask with 0x000f000f /
+// 0x00f000f0 (and the same after one shift by 8) to get two weights at a time as
+// a packed pair of binary16 values.
 #include "common.hpp"
 #include <stdlib.h>
 
@@ -371,13 +373,16 @@ __global__ __launch_bounds__(256) void sample_finish_kernel(SampleFinish f) {
 // 16 dwords of the argument block are preloaded into scalar registers at
 // wavefront launch (see the build flags); the rest of the argument block is a
 // memory round trip away.
-// k = n_waves * 128 * G, so a thread stages exactly G/2 units of four inputs.
+// k = n_waves * 64/RH * 32 * G, so a thread stages G * (64/RH) / 16 units of eight inputs
+// (with G * 64/RH = 8 every second thread stages one).
 // UFAST (periodic matrices only): the class length k/32/C when it is known at
 // compile time and divides G, so that a lane's G blocks are G/UFAST whole classes
 // whose constants it reads once per row group; 0 = look the class up per block.
 //
-// Dynamic LDS: x in block order (skewed) | block sums, k/32 floats | with the
-// fused norm, x in natural order (k halves).
+// Dynamic LDS: x in block order as nibble planes, 2 bytes per input (skewed 16 bytes per lane group) | the
+// blocks' powers of two, k/32 floats | the blocks' integer sums, k/32 floats | periodic matrices: group
+// constants per (pass, class) | several row groups per workgroup: the finished sums, RH floats per pass |
+// with the fused norm, x in natural order (k halves).
 // NWC: the number of wavefronts when it is known at compile time (the model's
 // own shapes: k, the staging loops and the reduction are then constants), 0 = take
 // it from the launch.  MULTI: the grid is smaller than the number of row groups
@@ -573,7 +578,7 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
       }
     }
   }
-  __syncthreads();  // xs, the block sums and the table
+  __syncthreads();  // the planes, the blocks' constants and the table
   float xcb[G], xSb[G];
   if (G >= 4) {
 #pragma unroll
@@ -740,8 +745,8 @@ struct GemvPlan {
 
 // Lane groups per workgroup = (k/32)/G must be a multiple of 4 and at most 64.
 // The longest per-lane run (G = 8, 4, 2) that still gives a workgroup eight wavefronts: with k = 4096
-// eight wavefronts of four blocks per lane beat four wavefronts of eight (12288 x 4096: 7.8 against
-// 8.2 us; sixteen wavefronts of two: 8.1 us).  G >= 2: a thread stages whole units of four inputs.
+// eight wavefronts of four blocks per lane beat four wavefronts of eight (12288 x 4096: 6.85 against
+// 7.15 us).  G >= 2: the staging works in units of eight inputs.
 bool plan_gemv(int64_t m, int64_t k, GemvPlan* out) {
   const int64_t nblk = k / AWQ_BLOCK_K;
   bool found = false;
@@ -754,8 +759,8 @@ bool plan_gemv(int64_t m, int64_t k, GemvPlan* out) {
     if (groups / 4 >= 8) break;
   }
   // few rows and long k (4096 x 12288: one 16-row workgroup of 12 wavefronts per compute unit): half the rows
-  // and half the blocks per lane, twice the workgroups (8.2 -> 7.55 us; 4096 x 4096 the same way: 4.3 -> 4.4 us,
-  // so only where a lane has eight blocks)
+  // and half the blocks per lane, twice the workgroups (8.2 -> 7.55 us with the first arithmetic; 4096 x 4096
+  // the same way measured no different, 3.94 against 3.95 us, so only where a lane has eight blocks)
   if (found && m / 16 <= 256 && out->g == 8 && out->n_waves >= 8) {
     out->g = 4;
     out->rh = 8;

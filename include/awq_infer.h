@@ -157,9 +157,14 @@ int awq_linear_repack(const void* packed_in, void* repacked_out, int64_t m, int6
 
 /* cublasGemmEx with n = 1, Inference.cu:1052-1065, 1128-1141, 1176-1189,
  * 1201-1214, 1260-1273, fused with the dequantisation:
- *     y[i] = h( sum over blocks of 32 inputs of s * (sum q*x - z * sum x) ),
- *     FP32 in the blocked order of awq_canon_math.h (q the raw nibble; scale
- *     and zero-point are applied to a block's sums, not to every weight).
+ *     y[i] = h( sum over blocks of 32 inputs of s * c * (sum q*I - z * sum I) ),
+ *     the blocked arithmetic of awq_canon_math.h: the inputs of a block as 16-bit
+ *     integers I under the block's power of two c (x = I*c up to a rounding of
+ *     2^-16 of the block's largest input), exact integer sums over the raw
+ *     nibbles q, scale and zero-point applied to a block's sums in FP32, block
+ *     values added in a fixed tree; a block that holds an infinity or a NaN
+ *     makes every output a NaN.  Within 1e-2 (in practice a few 1e-4) of the
+ *     FP32-accumulated product of the FP16-dequantised weights.
  * repacked from awq_linear_repack; scale/zp [m/128]; x [k], y [m] FP16.
  * zp_integral: kept for the matrix-core product (awq_gemm), where 1 selects a
  * shorter conversion for zero-points that are integers in [0,1024] (true of
