@@ -99,9 +99,10 @@ def gemv_gpu(awq, lib, torch, packed, scale, zp, m, k, x, zp_integral, repeat=1)
     return outs
 
 
-# the last two: few rows and long k, where a workgroup takes half a row group (general and 16-wavefront forms)
+# (512, 8192), (1024, 16384): few rows and long k, where a workgroup takes half a row group (general and
+# 16-wavefront forms); the last two: more than 1024 row groups, several per workgroup
 GEMV_SHAPES = [(128, 512), (256, 1024), (384, 512), (128, 1536), (640, 2048), (4096, 4096), (12288, 4096),
-               (4096, 12288), (512, 8192), (1024, 16384)]
+               (4096, 12288), (512, 8192), (1024, 16384), (20480, 1024), (40960, 512)]
 
 
 @pytest.mark.parametrize("m,k", GEMV_SHAPES)
@@ -465,7 +466,9 @@ def fused_setup(awq, lib, torch, rng, m, k, zp_int=True):
     return packed, scale, zp, a, keep
 
 
-@pytest.mark.parametrize("m,k", [(256, 512), (12288, 4096), (4096, 12288)])
+# the last two: more than 1024 row groups, so a workgroup walks several of them and runs the epilogues of all its
+# passes at the end (one scale group per 16 rows, and a scale group that depends on the input index)
+@pytest.mark.parametrize("m,k", [(256, 512), (12288, 4096), (4096, 12288), (20480, 1024), (128 * 147, 512)])
 def test_gemv_fused_norm_gelu_residual(awq, lib, oracle, torch_gpu, m, k):
     torch = torch_gpu
     rng = np.random.default_rng(m + 3 * k)
