@@ -41,7 +41,40 @@ __device__ __forceinline__ float dpp_add_half_mirror(float v) {
 __device__ __forceinline__ float dpp_add_mirror(float v) {
   return v + __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x140, 0xf, 0xf, true));
 }
-__device__ __forceinline__ float xor_add(float v, int mask) { return v + __shfl_xor(v, mask, 64); }
+// v + (value of lane ^ 16), v + (value of lane ^ 32): gfx950's lane-swap instructions exchange rows of 16 lanes
+// (halves of the wavefront) between two registers, a register operation where a general shuffle is an LDS
+// round trip.  After the swap a holds rows (0,0,2,2) and b rows (1,1,3,3) of v (resp. the low and the high
+// half), so a + b is the sum in every lane; a + b and b + a are the same number.  The waits around the
+// instruction are the data-hazard slots the compiler would insert if it saw it.
+__device__ __forceinline__ void swap16(float& a, float& b) {
+  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ void swap32(float& a, float& b) {
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ float add_xor16(float v) {
+  float a = v, b = v;
+  swap16(a, b);
+  return a + b;
+}
+__device__ __forceinline__ float add_xor32(float v) {
+  float a = v, b = v;
+  swap32(a, b);
+  return a + b;
+}
+// maximum over the 64 lanes of a wavefront, in every lane (the maximum does not depend on the order)
+__device__ __forceinline__ float wave_max(float v) {
+  v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, true)));
+  v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, true)));
+  v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x141, 0xf, 0xf, true)));
+  v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x140, 0xf, 0xf, true)));
+  float a = v, b = v;
+  swap16(a, b);
+  v = fmaxf(a, b);
+  a = v, b = v;
+  swap32(a, b);
+  return fmaxf(a, b);
+}
 
 // sum over the 16 lanes of a row, adjacent pairs first
 __device__ __forceinline__ float row16_tree_sum(float v) {
@@ -54,8 +87,8 @@ __device__ __forceinline__ float row16_tree_sum(float v) {
 // sum over the 64 lanes of a wavefront, adjacent pairs first
 __device__ __forceinline__ float wave_tree_sum(float v) {
   v = row16_tree_sum(v);
-  v = xor_add(v, 16);
-  v = xor_add(v, 32);
+  v = add_xor16(v);
+  v = add_xor32(v);
   return v;
 }
 
@@ -90,6 +123,19 @@ __global__ __launch_bounds__(NW * 64) void attention_kernel(const half_t* __rest
   const int tq = lane >> 4, dl = lane & 15;
   const half_t* kh = kc;
   const half_t* vh = vc;
+  // Row addresses.  Rows 64 positions apart are a constant apart in both cache arrangements (whole blocks of 64
+  // positions, or one run per head), and with 16 wavefronts the groups of a round are 64 positions apart, so a
+  // wavefront's requests are one row address plus multiples of a constant instead of a 64-bit row computation
+  // per request (18 of them before the first request left: 0.3 us of the launch).
+  static_assert(4 * NW == 64, "groups of a round are one block of 64 positions apart");
+  const int64_t step64 = kv_row(lay, 0, 64) - kv_row(lay, 0, 0);
+  const int64_t head0 = kv_row(lay, head, 0);
+  auto key_row = [&](int t) -> const half_t* {  // this lane's 8 elements of row t
+    return kh + head0 + (int64_t)(t >> 6) * step64 + (t & 63) * AWQ_HEAD_DIM + 8 * dl;
+  };
+  auto value_row = [&](int chunk) -> const half_t* {  // this lane's elements of row 64 chunk + tq
+    return vh + head0 + (int64_t)chunk * step64 + tq * AWQ_HEAD_DIM + d0 + DL * dl;
+  };
   const int nchunks = (L + 63) >> 6;
   const float scale = 1.0f / sqrtf((float)AWQ_HEAD_DIM);  // Inference.cu:218
 
@@ -101,7 +147,7 @@ __global__ __launch_bounds__(NW * 64) void attention_kernel(const half_t* __rest
 #pragma unroll
       for (int nl = 0; nl < 16; ++nl) {
         const int t = (wave << 6) + 4 * nl + tq;
-        if (t < L) vv[nl] = *reinterpret_cast<const vrow_t*>(vh + kv_row(lay, head, t) + d0 + DL * dl);
+        if (t < L) vv[nl] = *reinterpret_cast<const vrow_t*>(value_row(wave) + nl * (4 * AWQ_HEAD_DIM));
       }
     }
     for (int t = tid; t < L; t += NW * 64) s[t] = scores_g[(int64_t)head * max_pos + t];
@@ -126,35 +172,32 @@ __global__ __launch_bounds__(NW * 64) void attention_kernel(const half_t* __rest
   // cache memory and are never used.
   constexpr int kEagerGroups = EAGER / (4 * NW);
   static_assert(kEagerGroups <= 6 && EAGER % 64 == 0 && EAGER % (4 * NW) == 0, "eager part of the first trip");
-  const int last_row = (int)max_pos - 1;
+  // (an eager launch is only made for caches of at least EAGER positions, so its rows need no clamp)
   half8_t kv[6];
+  const half_t* const k_wave = key_row(4 * wave + tq);
 #pragma unroll
-  for (int u = 0; u < kEagerGroups; ++u) {
-    const int t = min(4 * (wave + u * NW) + tq, last_row);
-    kv[u] = *reinterpret_cast<const half8_t*>(kh + kv_row(lay, head, t) + 8 * dl);
-  }
+  for (int u = 0; u < kEagerGroups; ++u) kv[u] = *reinterpret_cast<const half8_t*>(k_wave + u * step64);
   if (wave < EAGER / 64) {
+    const half_t* const v_wave = value_row(wave);
 #pragma unroll
-    for (int nl = 0; nl < 16; ++nl) {
-      const int t = min((wave << 6) + 4 * nl + tq, last_row);
-      vv[nl] = *reinterpret_cast<const vrow_t*>(vh + kv_row(lay, head, t) + d0 + DL * dl);
-    }
+    for (int nl = 0; nl < 16; ++nl) vv[nl] = *reinterpret_cast<const vrow_t*>(v_wave + nl * (4 * AWQ_HEAD_DIM));
   }
   float lmax = -1e9f;
   const int nquads = (L + 3) >> 2;
   for (int q0 = wave; q0 < nquads; q0 += 6 * NW) {
     const bool first = q0 == wave;
+    const half_t* const k_round = key_row(4 * q0 + tq);
 #pragma unroll
     for (int u = 0; u < 6; ++u) {
       const int t = 4 * (q0 + u * NW) + tq;
-      if (t < L && !(first && u < kEagerGroups))
-        kv[u] = *reinterpret_cast<const half8_t*>(kh + kv_row(lay, head, t) + 8 * dl);
+      if (t < L && !(first && u < kEagerGroups)) kv[u] = *reinterpret_cast<const half8_t*>(k_round + u * step64);
     }
     if (first && wave >= EAGER / 64 && wave < nchunks) {
+      const half_t* const v_wave = value_row(wave);
 #pragma unroll
       for (int nl = 0; nl < 16; ++nl) {
         const int t = (wave << 6) + 4 * nl + tq;
-        if (t < L) vv[nl] = *reinterpret_cast<const vrow_t*>(vh + kv_row(lay, head, t) + d0 + DL * dl);
+        if (t < L) vv[nl] = *reinterpret_cast<const vrow_t*>(v_wave + nl * (4 * AWQ_HEAD_DIM));
       }
     }
 #pragma unroll
@@ -173,8 +216,7 @@ __global__ __launch_bounds__(NW * 64) void attention_kernel(const half_t* __rest
       }
     }
   }
-#pragma unroll
-  for (int mask = 1; mask < 64; mask <<= 1) lmax = fmaxf(lmax, __shfl_xor(lmax, mask, 64));
+  lmax = wave_max(lmax);
   if (lane == 0) wmax[wave] = lmax;
   __syncthreads();
   mx = wmax[0];
@@ -194,8 +236,20 @@ __global__ __launch_bounds__(NW * 64) void attention_kernel(const half_t* __rest
     if (lane == 0) cs[chunk] = e;
   }
   __syncthreads();
-  float Z = cs[0];
-  for (int c = 1; c < nchunks; ++c) Z += cs[c];
+  // the chunk sums, added in chunk order; the first 16 reads are issued together (a read per term is an LDS
+  // round trip per chunk, serialised by the additions)
+  constexpr int kBatch = CCAP < 16 ? CCAP : 16;
+  float Z;
+  {
+    float zc[kBatch];
+#pragma unroll
+    for (int c = 0; c < kBatch; ++c) zc[c] = cs[c];  // entries past nchunks are never added
+    Z = zc[0];
+#pragma unroll
+    for (int c = 1; c < kBatch; ++c)
+      if (c < nchunks) Z += zc[c];
+    for (int c = kBatch; c < nchunks; ++c) Z += cs[c];
+  }
 
   // weighted sum of V (Inference.cu:251-265), one wavefront per chunk; the 16
   // loads of a chunk are issued together
@@ -205,7 +259,7 @@ __global__ __launch_bounds__(NW * 64) void attention_kernel(const half_t* __rest
 #pragma unroll
       for (int nl = 0; nl < 16; ++nl) {
         const int t = base + 4 * nl + tq;
-        if (t < L) vv[nl] = *reinterpret_cast<const vrow_t*>(vh + kv_row(lay, head, t) + d0 + DL * dl);
+        if (t < L) vv[nl] = *reinterpret_cast<const vrow_t*>(value_row(chunk) + nl * (4 * AWQ_HEAD_DIM));
       }
     }
     // one division per position (lane = position in the chunk), handed to the 16 lanes that
@@ -214,19 +268,25 @@ __global__ __launch_bounds__(NW * 64) void attention_kernel(const half_t* __rest
     float acc[DL];
 #pragma unroll
     for (int i = 0; i < DL; ++i) acc[i] = 0.0f;
+    // all 16 exchanges are issued before the first product, and a position past the length keeps the sum
+    // by a select, not a branch: with a branch per position the compiler waits for every exchange (an LDS
+    // round trip) before it issues the next, 16 round trips in a row
+    float pp[16];
+#pragma unroll
+    for (int nl = 0; nl < 16; ++nl) pp[nl] = __shfl(p_lane, 4 * nl + tq, 64);
 #pragma unroll
     for (int nl = 0; nl < 16; ++nl) {
-      const int t = base + 4 * nl + tq;
-      const float p = __shfl(p_lane, 4 * nl + tq, 64);
-      if (t < L) {
+      const bool in = base + 4 * nl + tq < L;
 #pragma unroll
-        for (int i = 0; i < DL; ++i) acc[i] = __builtin_fmaf(p, (float)vv[nl][i], acc[i]);
+      for (int i = 0; i < DL; ++i) {
+        const float r = __builtin_fmaf(pp[nl], (float)vv[nl][i], acc[i]);
+        acc[i] = in ? r : acc[i];
       }
     }
 #pragma unroll
     for (int i = 0; i < DL; ++i) {
-      acc[i] = xor_add(acc[i], 16);
-      acc[i] = xor_add(acc[i], 32);
+      acc[i] = add_xor16(acc[i]);
+      acc[i] = add_xor32(acc[i]);
     }
     if (tq == 0) {
 #pragma unroll
@@ -235,8 +295,14 @@ __global__ __launch_bounds__(NW * 64) void attention_kernel(const half_t* __rest
   }
   __syncthreads();
   if (tid < DP) {
-    float out = cv[tid];
-    for (int c = 1; c < nchunks; ++c) out += cv[c * DP + tid];
+    float oc[kBatch];
+#pragma unroll
+    for (int c = 0; c < kBatch; ++c) oc[c] = cv[c * DP + tid];
+    float out = oc[0];
+#pragma unroll
+    for (int c = 1; c < kBatch; ++c)
+      if (c < nchunks) out += oc[c];
+    for (int c = kBatch; c < nchunks; ++c) out += cv[c * DP + tid];
     ctx[head * AWQ_HEAD_DIM + d0 + tid] = (half_t)out;
   }
 }
@@ -334,8 +400,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void attn_scores_kernel(SplitArgs
       }
     }
   }
-#pragma unroll
-  for (int mask = 1; mask < 64; mask <<= 1) lmax = fmaxf(lmax, __shfl_xor(lmax, mask, 64));
+  lmax = wave_max(lmax);
   if (lane == 0) wmax[wave] = lmax;
   __syncthreads();
   if (tid == 0) {
@@ -417,30 +482,35 @@ __global__ __launch_bounds__(kSplitWaves * 64) void attn_pv_kernel(SplitArgs a) 
     float acc[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
+    // the 16 exchanges go out together and a position past the length keeps the sum by a select (a branch
+    // per position makes the compiler wait for each exchange, an LDS round trip, before it issues the next)
+    float pp[16];
+#pragma unroll
+    for (int nl = 0; nl < 16; ++nl) pp[nl] = __shfl(p_lane, 4 * nl + tq, 64);
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
-      const int t = base + 4 * u + tq;
-      const float pr = __shfl(p_lane, 4 * u + tq, 64);
-      if (t < L) {
+      const bool in = base + 4 * u + tq < L;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) acc[i] = __builtin_fmaf(pr, (float)va[u][i], acc[i]);
+      for (int i = 0; i < 8; ++i) {
+        const float r = __builtin_fmaf(pp[u], (float)va[u][i], acc[i]);
+        acc[i] = in ? r : acc[i];
       }
     }
     load_half(nxt, 0, va);
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
-      const int t = base + 4 * (8 + u) + tq;
-      const float pr = __shfl(p_lane, 4 * (8 + u) + tq, 64);
-      if (t < L) {
+      const bool in = base + 4 * (8 + u) + tq < L;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) acc[i] = __builtin_fmaf(pr, (float)vb[u][i], acc[i]);
+      for (int i = 0; i < 8; ++i) {
+        const float r = __builtin_fmaf(pp[8 + u], (float)vb[u][i], acc[i]);
+        acc[i] = in ? r : acc[i];
       }
     }
     load_half(nxt, 1, vb);
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      acc[i] = xor_add(acc[i], 16);
-      acc[i] = xor_add(acc[i], 32);
+      acc[i] = add_xor16(acc[i]);
+      acc[i] = add_xor32(acc[i]);
     }
     if (tq == 0) {
 #pragma unroll
@@ -503,19 +573,22 @@ __global__ __launch_bounds__(kSplitWaves * 64) void attn_exp_pv_kernel(SplitArgs
   float acc[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
+  float pp[16];  // all exchanges before the first product; selects, not branches (see attn_pv_kernel)
+#pragma unroll
+  for (int nl = 0; nl < 16; ++nl) pp[nl] = __shfl(p_lane, 4 * nl + tq, 64);
 #pragma unroll
   for (int nl = 0; nl < 16; ++nl) {
-    const int t = base + 4 * nl + tq;
-    const float pr = __shfl(p_lane, 4 * nl + tq, 64);
-    if (t < L) {
+    const bool in = base + 4 * nl + tq < L;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) acc[i] = __builtin_fmaf(pr, (float)vv[nl][i], acc[i]);
+    for (int i = 0; i < 8; ++i) {
+      const float r = __builtin_fmaf(pp[nl], (float)vv[nl][i], acc[i]);
+      acc[i] = in ? r : acc[i];
     }
   }
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    acc[i] = xor_add(acc[i], 16);
-    acc[i] = xor_add(acc[i], 32);
+    acc[i] = add_xor16(acc[i]);
+    acc[i] = add_xor32(acc[i]);
   }
   if (tq == 0) {
 #pragma unroll
@@ -587,6 +660,7 @@ static int launch_attention_ws(const half_t* q, const half_t* kc, const half_t* 
   AWQ_REQUIRE(n_heads > 0 && max_pos > 0 && max_pos <= (int64_t)kMaxChunks * 64, "max_pos must be in 1..65536");
   AWQ_REQUIRE(dyn || (L >= 1 && L <= max_pos && L <= cache_pos), "attended length out of range");
   AWQ_REQUIRE(ws != nullptr, "workspace required");
+  AWQ_REQUIRE(kv.shift == 6 || kv.block_stride == 0, "cache rows 64 positions apart must be a constant apart");
   float* scores = (float*)ws;
   float* cv = scores + (int64_t)n_heads * max_pos;
   // With a device-side length the caller states an upper bound for it (it
