@@ -235,19 +235,25 @@ __global__ __launch_bounds__(NW * 64) void attention_kernel(const half_t* __rest
     e = wave_tree_sum(e);
     if (lane == 0) cs[chunk] = e;
   }
+  // A wavefront without a chunk among the first NW leaves zeros in its places: the sums below then add the
+  // first NW entries unconditionally (x + 0 is x for the non-negative sums and for the chunk vectors, which
+  // are never -0: every chain starts at +0)
+  constexpr int kBatch = CCAP < NW ? CCAP : NW;
+  if (wave >= nchunks && wave < kBatch) {
+    if (lane == 0) cs[wave] = 0.0f;
+    if (lane < DP) cv[wave * DP + lane] = 0.0f;
+  }
   __syncthreads();
-  // the chunk sums, added in chunk order; the first 16 reads are issued together (a read per term is an LDS
+  // the chunk sums, added in chunk order; the first reads are issued together (a read per term is an LDS
   // round trip per chunk, serialised by the additions)
-  constexpr int kBatch = CCAP < 16 ? CCAP : 16;
   float Z;
   {
     float zc[kBatch];
 #pragma unroll
-    for (int c = 0; c < kBatch; ++c) zc[c] = cs[c];  // entries past nchunks are never added
+    for (int c = 0; c < kBatch; ++c) zc[c] = cs[c];
     Z = zc[0];
 #pragma unroll
-    for (int c = 1; c < kBatch; ++c)
-      if (c < nchunks) Z += zc[c];
+    for (int c = 1; c < kBatch; ++c) Z += zc[c];
     for (int c = kBatch; c < nchunks; ++c) Z += cs[c];
   }
 
@@ -300,8 +306,7 @@ __global__ __launch_bounds__(NW * 64) void attention_kernel(const half_t* __rest
     for (int c = 0; c < kBatch; ++c) oc[c] = cv[c * DP + tid];
     float out = oc[0];
 #pragma unroll
-    for (int c = 1; c < kBatch; ++c)
-      if (c < nchunks) out += oc[c];
+    for (int c = 1; c < kBatch; ++c) out += oc[c];
     for (int c = kBatch; c < nchunks; ++c) out += cv[c * DP + tid];
     ctx[head * AWQ_HEAD_DIM + d0 + tid] = (half_t)out;
   }
@@ -482,28 +487,25 @@ __global__ __launch_bounds__(kSplitWaves * 64) void attn_pv_kernel(SplitArgs a) 
     float acc[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
-    // the 16 exchanges go out together and a position past the length keeps the sum by a select (a branch
-    // per position makes the compiler wait for each exchange, an LDS round trip, before it issues the next)
-    float pp[16];
-#pragma unroll
-    for (int nl = 0; nl < 16; ++nl) pp[nl] = __shfl(p_lane, 4 * nl + tq, 64);
+    // (this loop streams: exchange and product per position under a branch measured 7 % faster here than all
+    // exchanges first with selects, the form of the one-workgroup kernel, which holds 16 more registers)
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
-      const bool in = base + 4 * u + tq < L;
+      const int t = base + 4 * u + tq;
+      const float pr = __shfl(p_lane, 4 * u + tq, 64);
+      if (t < L) {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const float r = __builtin_fmaf(pp[u], (float)va[u][i], acc[i]);
-        acc[i] = in ? r : acc[i];
+        for (int i = 0; i < 8; ++i) acc[i] = __builtin_fmaf(pr, (float)va[u][i], acc[i]);
       }
     }
     load_half(nxt, 0, va);
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
-      const bool in = base + 4 * (8 + u) + tq < L;
+      const int t = base + 4 * (8 + u) + tq;
+      const float pr = __shfl(p_lane, 4 * (8 + u) + tq, 64);
+      if (t < L) {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const float r = __builtin_fmaf(pp[8 + u], (float)vb[u][i], acc[i]);
-        acc[i] = in ? r : acc[i];
+        for (int i = 0; i < 8; ++i) acc[i] = __builtin_fmaf(pr, (float)vb[u][i], acc[i]);
       }
     }
     load_half(nxt, 1, vb);
@@ -573,7 +575,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void attn_exp_pv_kernel(SplitArgs
   float acc[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
-  float pp[16];  // all exchanges before the first product; selects, not branches (see attn_pv_kernel)
+  float pp[16];  // all exchanges before the first product; selects, not branches (see attention_kernel)
 #pragma unroll
   for (int nl = 0; nl < 16; ++nl) pp[nl] = __shfl(p_lane, 4 * nl + tq, 64);
 #pragma unroll
