@@ -126,9 +126,13 @@ __device__ __forceinline__ half8_t dequant8(uint32_t v, half_t s, half_t z) {
 // dword c the four quarters' blocks form one 32-wide contraction: lane (q, r)
 // supplies dword c of block (4w+q)*G+b, lane (q, n) of the token operand
 // supplies X[token n][that block, elements 8c..8c+7].
-template <int G, int TT, bool ZINT>
+template <int G, int TT, bool ZINT, int XR>
 __global__ __launch_bounds__(1024) void gemm_small_kernel(GemmParams p, int n_waves) {
   __shared__ float red[16][TT][64][4];
+  // the tokens of this workgroup, [token][k] with 16 bytes of skew per lane group of G blocks (the four
+  // quarters of a wavefront read four lane groups at once) and 16 bytes between token rows
+  extern __shared__ __attribute__((aligned(16))) unsigned char small_lds[];
+  half_t* xs = reinterpret_cast<half_t*>(small_lds);
   typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -136,28 +140,65 @@ __global__ __launch_bounds__(1024) void gemm_small_kernel(GemmParams p, int n_wa
   const int rg = blockIdx.x;
   const int t0 = blockIdx.y * (16 * TT);
   const int blk0 = (4 * wave + q) * G;
+  // Loads return in the order of their requests. Scale and zero-point go first (small, needed by the first
+  // product), then XR 16-byte pieces of the tokens per thread (the host picks the smallest
+  // of 2, 4 and 8 that covers them: every request costs its slot in the memory pipeline, needed or not), then the weights: the tokens come out of
+  // L2 and are in LDS while the weights are still arriving, so that the products start with the first weights
+  // instead of after the last. Pieces beyond XR per thread (more tokens) follow the weights.
   const int gi = ((rg >> 3) % p.kg) % p.mg;
   const half_t sc = p.scale[gi], zz = p.zp[gi];
+  // piece e8 of token row j lies at j * stride + e8 * 8 + (e8 / (4 G)) * 8 halves
+  const int n_tok = min(16 * TT, p.M - t0);
+  const int k8 = p.k >> 3;
+  const int stride = p.k + (p.nblk / G) * 8 + 8;
+  const int n_pc = n_tok * k8, n_thr = n_waves * 64;
+  u32x4 xv[XR];
+  int xo[XR];
+#pragma unroll
+  for (int i = 0; i < XR; ++i) {
+    const int pc = min(tid + i * n_thr, n_pc - 1);
+    const int j = pc / k8, e8 = pc - j * k8;
+    xv[i] = *reinterpret_cast<const u32x4*>(p.x + (int64_t)(t0 + j) * p.k + e8 * 8);
+    xo[i] = j * stride + e8 * 8 + (e8 / (4 * G)) * 8;
+  }
   const u32x4* wp = reinterpret_cast<const u32x4*>(p.wq) + ((int64_t)rg * p.nblk + blk0) * 16 + r;
   u32x4 w[G];
 #pragma unroll
   for (int b = 0; b < G; ++b) w[b] = __builtin_nontemporal_load(wp + b * 16);
+#pragma unroll
+  for (int i = 0; i < XR; ++i)
+    if (tid + i * n_thr < n_pc) *reinterpret_cast<u32x4*>(xs + xo[i]) = xv[i];
+  for (int pc = tid + XR * n_thr; pc < n_pc; pc += n_thr) {
+    const int j = pc / k8, e8 = pc - j * k8;
+    const u32x4 v = *reinterpret_cast<const u32x4*>(p.x + (int64_t)(t0 + j) * p.k + e8 * 8);
+    *reinterpret_cast<u32x4*>(xs + j * stride + e8 * 8 + (e8 / (4 * G)) * 8) = v;
+  }
+  __syncthreads();
   float4_t acc[TT];
 #pragma unroll
   for (int t = 0; t < TT; ++t) acc[t] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+  // this lane's token row (r) and lane group in LDS; lanes beyond the last token read the last token's row
+  // (their accumulator columns are never stored)
+  const half_t* xl = xs + (blk0 * 32) + (blk0 / G) * 8;
+  // The token operands are read from LDS in batches of up to 16, each batch ahead of its products: a read per
+  // product would put an LDS round trip between every two matrix instructions.
+  constexpr int NB = G * 4 < 16 ? G * 4 : 16;
+  const half_t* row[TT];
 #pragma unroll
-  for (int b = 0; b < G; ++b) {
-    const uint32_t d[4] = {w[b].x, w[b].y, w[b].z, w[b].w};
+  for (int t = 0; t < TT; ++t) row[t] = xl + min(t * 16 + r, n_tok - 1) * stride;
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      const half8_t wop = dequant8<ZINT>(d[c], sc, zz);
+  for (int b0 = 0; b0 < G * 4; b0 += NB) {
+    half8_t xr[TT][NB];
 #pragma unroll
-      for (int t = 0; t < TT; ++t) {
-        const int tok = t0 + t * 16 + r;
-        half8_t xop = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
-        if (tok < p.M) xop = *reinterpret_cast<const half8_t*>(p.x + (int64_t)tok * p.k + (blk0 + b) * 32 + c * 8);
-        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xop, wop, acc[t], 0, 0, 0);
-      }
+    for (int t = 0; t < TT; ++t)
+#pragma unroll
+      for (int i = 0; i < NB; ++i) xr[t][i] = *reinterpret_cast<const half8_t*>(row[t] + (b0 + i) * 8);
+#pragma unroll
+    for (int i = 0; i < NB; ++i) {
+      const int bc = b0 + i;
+      const half8_t wop = dequant8<ZINT>(w[bc >> 2][bc & 3], sc, zz);
+#pragma unroll
+      for (int t = 0; t < TT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xr[t][i], wop, acc[t], 0, 0, 0);
     }
   }
 #pragma unroll
@@ -169,10 +210,18 @@ __global__ __launch_bounds__(1024) void gemm_small_kernel(GemmParams p, int n_wa
   with_epilogue(p, [&](auto E) {
 #pragma unroll
     for (int t = 0; t < TT; ++t) {
+      // the wavefronts' sums in wavefront order; all 16-byte reads are issued together (a read per term is an
+      // LDS round trip each, serialised by the additions)
+      float4_t part[16];
+#pragma unroll
+      for (int wv = 0; wv < 16; ++wv)
+        if (wv < n_waves) part[wv] = *reinterpret_cast<const float4_t*>(&red[wv][t][lane][0]);
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        float v = red[0][t][lane][i];
-        for (int wv = 1; wv < n_waves; ++wv) v += red[wv][t][lane][i];
+        float v = part[0][i];
+#pragma unroll
+        for (int wv = 1; wv < 16; ++wv)
+          if (wv < n_waves) v += part[wv][i];
         const int tok = t0 + t * 16 + q * 4 + i;  // D[token 4*(lane/16)+i][row lane%16]
         if (tok < p.M) store_out<decltype(E)::value>(p, tok, rg * 16 + r, v);
       }
@@ -745,9 +794,20 @@ int launch_wide(const GemmParams& p, bool zint, int n_wgs, hipStream_t st) {
 }
 
 template <int G, int TT>
-void launch_small(const GemmParams& p, bool zint, int n_waves, dim3 grid, hipStream_t st) {
-  if (zint) hipLaunchKernelGGL((gemm_small_kernel<G, TT, true>), grid, dim3(n_waves * 64), 0, st, p, n_waves);
-  else hipLaunchKernelGGL((gemm_small_kernel<G, TT, false>), grid, dim3(n_waves * 64), 0, st, p, n_waves);
+int launch_small(const GemmParams& p, bool zint, int n_waves, dim3 grid, hipStream_t st) {
+  // the tokens of a workgroup in LDS: rows of k halves plus the skew and 16 bytes between rows
+  const size_t lds = (size_t)std::min<int64_t>(16 * TT, p.M) * (p.k + (p.nblk / G) * 8 + 8) * 2;
+  // token pieces per thread that are requested ahead of the weights
+  const int64_t pieces = (std::min<int64_t>(16 * TT, p.M) * (p.k / 8) + n_waves * 64 - 1) / (n_waves * 64);
+  auto kern = pieces <= 2 ? (zint ? gemm_small_kernel<G, TT, true, 2> : gemm_small_kernel<G, TT, false, 2>)
+            : pieces <= 4 ? (zint ? gemm_small_kernel<G, TT, true, 4> : gemm_small_kernel<G, TT, false, 4>)
+                          : (zint ? gemm_small_kernel<G, TT, true, 8> : gemm_small_kernel<G, TT, false, 8>);
+  if (lds > 65536 - sizeof(float) * 16 * TT * 64 * 4) {
+    // more LDS than a launch gets by default: raise this kernel's limit (cheap, so done per call)
+    AWQ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  }
+  hipLaunchKernelGGL(kern, grid, dim3(n_waves * 64), lds, st, p, n_waves);
+  return AWQ_OK;
 }
 
 }  // namespace
@@ -840,21 +900,24 @@ int launch_gemm(const void* wq, const half_t* scale, const half_t* zp, int64_t m
   if (M <= 4) {
     // lane groups of G blocks: (k/32)/G of them, a multiple of 4 and at most 64
     const int64_t nblk = k / AWQ_BLOCK_K;
+    // the longest run per lane that still gives the workgroup eight wavefronts (as in the decode kernel)
     for (int c : {8, 4, 2, 1})
       if (nblk % c == 0 && (nblk / c) % 4 == 0 && nblk / c <= 64) {
         g = c;
-        break;
+        if (nblk / c / 4 >= 8) break;
       }
   }
   if (g) {
     const int n_waves = (int)(k / AWQ_BLOCK_K / g / 4);
     dim3 grid((unsigned)(m / 16), 1);
+    int rc;
     switch (g) {
-      case 8: launch_small<8, 1>(p, zp_integral, n_waves, grid, st); break;
-      case 4: launch_small<4, 1>(p, zp_integral, n_waves, grid, st); break;
-      case 2: launch_small<2, 1>(p, zp_integral, n_waves, grid, st); break;
-      default: launch_small<1, 1>(p, zp_integral, n_waves, grid, st); break;
+      case 8: rc = launch_small<8, 1>(p, zp_integral, n_waves, grid, st); break;
+      case 4: rc = launch_small<4, 1>(p, zp_integral, n_waves, grid, st); break;
+      case 2: rc = launch_small<2, 1>(p, zp_integral, n_waves, grid, st); break;
+      default: rc = launch_small<1, 1>(p, zp_integral, n_waves, grid, st); break;
     }
+    if (rc) return rc;
   } else {
     const int64_t nr = (m + 255) / 256;
     const int64_t tiles = nr * ((M + kWideTokens - 1) / kWideTokens);
