@@ -229,6 +229,100 @@ __global__ __launch_bounds__(1024) void gemm_small_kernel(GemmParams p, int n_wa
   });
 }
 
+// Two to sixteen tokens, k a multiple of 4096: still a weight stream, but every workgroup of the kernel above
+// needs all tokens' inputs (2 k bytes each) for its 8 k bytes of weights.  Here a workgroup of 16 wavefronts
+// takes RG row groups and all of k: wavefront w, quarter q holds blocks (4w+q)G.. of each of its rows -- the
+// operand shapes of the kernel above -- so per pair of blocks (a "slice": b = 2h, 2h+1) the wavefront needs
+// four 128-byte pieces of every token, once for the RG row groups.  It reads them 16 bytes per lane, two
+// tokens per instruction (a lane reading its own operand straight from memory touches 64 cache lines per
+// instruction, and the compute unit looks up one line per clock: 14 us at 16 tokens), and turns them into
+// operand order through a piece of LDS of its own -- no workgroup barrier: the LDS instructions of one
+// wavefront execute in order.  Requests go out in the order of need: scales, the first two slices of tokens,
+// all RG G blocks of weights per lane (96 KB per workgroup for the model's shapes, as in the decode kernel);
+// a further slice of tokens is requested as soon as a register set is free, long before the weights ahead
+// of it have arrived.  The 16 wavefronts' sums meet in LDS, in the place of the token pieces.
+constexpr int kMidRow = 4 * 144 + 16;  // bytes per token in a wavefront's piece: quarters 144 bytes apart (conflict-free operand reads)
+template <int G, int RG, bool ZINT>
+__global__ __launch_bounds__(1024) void gemm_mid_kernel(GemmParams p, int n_rg) {
+  constexpr int NW = 16, NS = G / 2, S = NS < 2 ? NS : 2;
+  static_assert(G % 2 == 0 && RG * G <= 8, "slices of two blocks; register budget of 1024 threads");
+  extern __shared__ __attribute__((aligned(16))) unsigned char mid_lds[];
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int q = lane >> 4, r = lane & 15;
+  const int rg0 = blockIdx.x * RG;
+  const int blk0 = (4 * wave + q) * G;
+  half_t sc[RG], zz[RG];
+#pragma unroll
+  for (int i = 0; i < RG; ++i) {
+    const int rg = min(rg0 + i, n_rg - 1);  // a workgroup past the last row group repeats it and stores nothing
+    const int gi = ((rg >> 3) % p.kg) % p.mg;
+    sc[i] = p.scale[gi];
+    zz[i] = p.zp[gi];
+  }
+  // instruction i of a slice brings tokens 2i and 2i+1: lane = (token parity, quarter, 16-byte piece); tokens
+  // beyond the last repeat the last (their accumulator columns are never stored)
+  const int n_tok = min(16, p.M);
+  const int tpar = lane >> 5, tq = (lane >> 3) & 3, tp = lane & 7;
+  const half_t* xg = p.x + ((4 * wave + tq) * G) * 32 + tp * 8;
+  u32x4 xs[S][8];
+  auto request = [&](int h, u32x4* dst) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      dst[i] = *reinterpret_cast<const u32x4*>(xg + (int64_t)min(2 * i + tpar, n_tok - 1) * p.k + h * 64);
+  };
+#pragma unroll
+  for (int h = 0; h < S; ++h) request(h, xs[h]);
+  u32x4 w[RG][G];
+#pragma unroll
+  for (int i = 0; i < RG; ++i) {
+    const int rg = min(rg0 + i, n_rg - 1);
+    const u32x4* wp = reinterpret_cast<const u32x4*>(p.wq) + ((int64_t)rg * p.nblk + blk0) * 16 + r;
+#pragma unroll
+    for (int b = 0; b < G; ++b) w[i][b] = __builtin_nontemporal_load(wp + b * 16);
+  }
+  unsigned char* mine = mid_lds + wave * (16 * kMidRow);
+  unsigned char* put = mine + tpar * kMidRow + tq * 144 + tp * 16;
+  const unsigned char* get = mine + r * kMidRow + q * 144;
+  float4_t acc[RG];
+#pragma unroll
+  for (int i = 0; i < RG; ++i) acc[i] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+  for (int h = 0; h < NS; ++h) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4*>(put + 2 * i * kMidRow) = xs[h % S][i];
+    if (h + S < NS) request(h + S, xs[h % S]);
+    half8_t xr[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) xr[i] = *reinterpret_cast<const half8_t*>(get + i * 16);
+#pragma unroll
+    for (int i = 0; i < RG; ++i)
+#pragma unroll
+      for (int bc = 0; bc < 8; ++bc) {
+        const half8_t wop = dequant8<ZINT>(w[i][2 * h + (bc >> 2)][bc & 3], sc[i], zz[i]);
+        acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xr[bc], wop, acc[i], 0, 0, 0);
+      }
+  }
+  __syncthreads();  // every wavefront has read its operands: the token pieces make room for the sums
+  float* red = reinterpret_cast<float*>(mid_lds);  // [NW][RG][64][4]
+#pragma unroll
+  for (int i = 0; i < RG; ++i) *reinterpret_cast<float4_t*>(red + ((wave * RG + i) * 64 + lane) * 4) = acc[i];
+  __syncthreads();
+  // D[token 4 (lane / 16) + e][row lane % 16] sits in element e of the lane: thread (i, token, row), rows fastest
+  if (tid >= RG * 256) return;
+  const int i = tid >> 8, tok = (tid >> 4) & 15, row = tid & 15;
+  if (tok >= p.M || rg0 + i >= n_rg) return;
+  const float* first = red + (i * 64 + (tok >> 2) * 16 + row) * 4 + (tok & 3);
+  float part[NW];
+#pragma unroll
+  for (int wv = 0; wv < NW; ++wv) part[wv] = first[wv * (RG * 256)];
+  float v = part[0];
+#pragma unroll
+  for (int wv = 1; wv < NW; ++wv) v += part[wv];
+  with_epilogue(p, [&](auto E) { store_out<decltype(E)::value>(p, tok, (rg0 + i) * 16 + row, v); });
+}
+
 // Many tokens: a wavefront owns 64 weight rows x 128 tokens as 2 x 4 accumulator
 // tiles of v_mfma_f32_32x32x16_f16 (twice the rate of the 16x16x32 shape on this
 // device).  Every token operand read from LDS feeds two products and every
@@ -812,6 +906,29 @@ int launch_small(const GemmParams& p, bool zint, int n_waves, dim3 grid, hipStre
 
 }  // namespace
 
+constexpr int kMidLdsBytes = 16 * 16 * kMidRow;  // 16 wavefronts x 16 tokens (the sums need less)
+template <int G, int RG>
+int launch_mid(const GemmParams& p, bool zint, int n_rg, hipStream_t st) {
+  auto kern = zint ? gemm_mid_kernel<G, RG, true> : gemm_mid_kernel<G, RG, false>;
+  // more LDS than a launch gets by default: raise this kernel's limit (cheap, so done per call)
+  AWQ_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kMidLdsBytes));
+  hipLaunchKernelGGL(kern, dim3((unsigned)((n_rg + RG - 1) / RG)), dim3(1024), kMidLdsBytes, st, p, n_rg);
+  return AWQ_OK;
+}
+// 2..16 tokens and k of 128, 256, 384 or 512 blocks: the row groups per workgroup (0: this kernel does not
+// take the product).  As many as the registers hold (at most three) while at least 256 workgroups remain.
+#ifndef AWQ_MID_MIN_TOKENS
+#define AWQ_MID_MIN_TOKENS 2
+#endif
+int mid_row_groups(int64_t m, int64_t k, int64_t M) {
+  if (M < AWQ_MID_MIN_TOKENS || M > 16 || k % 4096 != 0 || k > 16384 || m % 16 != 0) return 0;
+  int rg = (int)(4 / (k / 4096));
+  if (rg > 3) rg = 3;
+  if (rg < 1) rg = 1;
+  while (rg > 1 && (m / 16 + rg - 1) / rg < 256) --rg;
+  return rg;
+}
+
 // Which workgroup shape a many-token product takes (measured on the three matrix shapes of the
 // model, 128 to 4096 tokens):
 //   fewer than 80 tiles of 256 rows x 128 tokens          k split
@@ -843,8 +960,10 @@ static WidePlan plan_wide(int64_t m, int64_t k, int64_t M, bool has_workspace) {
 
 // room for a header and the partial sums of a product whose work is cut over workgroups (0: never cut)
 // the shape awq_gemm takes for a product (diagnostics and tests): 0 few tokens, 1 k split, 2 rows split
-// with a tile per workgroup, 3 rows split with 64 tokens per workgroup, 4 rows split with the work cut evenly
+// with a tile per workgroup, 3 rows split with 64 tokens per workgroup, 4 rows split with the work cut evenly,
+// 5 up to 16 tokens with several row groups per workgroup
 int gemm_plan(int64_t m, int64_t k, int64_t M, int has_workspace) {
+  if (M >= 2 && mid_row_groups(m, k, M)) return 5;
   if (M <= 4) return 0;
   switch (plan_wide(m, k, M, has_workspace != 0)) {
     case PLAN_K: return 1;
@@ -855,7 +974,7 @@ int gemm_plan(int64_t m, int64_t k, int64_t M, int has_workspace) {
 }
 
 int64_t gemm_workspace_bytes(int64_t m, int64_t k, int64_t M) {
-  if (M <= 4) return 0;
+  if (M <= 4 || mid_row_groups(m, k, M)) return 0;
   switch (plan_wide(m, k, M, true)) {
     case PLAN_ROWS_CUT: return kSkHeaderBytes + (int64_t)kSkWgs * kSkTileFloats * 4;
     case PLAN_K: {
@@ -895,6 +1014,22 @@ int launch_gemm(const void* wq, const half_t* scale, const half_t* zp, int64_t m
   p.nr = p.n_tiles = 0;
   p.sk_head = nullptr;
   p.sk_part = nullptr;
+  if (const int rgs = mid_row_groups(m, k, M)) {
+    const int n_rg = (int)(m / 16);
+    int rc;
+    switch ((int)(k / 4096) * 4 + rgs) {
+      case 1 * 4 + 3: rc = launch_mid<2, 3>(p, zp_integral, n_rg, st); break;
+      case 1 * 4 + 2: rc = launch_mid<2, 2>(p, zp_integral, n_rg, st); break;
+      case 1 * 4 + 1: rc = launch_mid<2, 1>(p, zp_integral, n_rg, st); break;
+      case 2 * 4 + 2: rc = launch_mid<4, 2>(p, zp_integral, n_rg, st); break;
+      case 2 * 4 + 1: rc = launch_mid<4, 1>(p, zp_integral, n_rg, st); break;
+      case 3 * 4 + 1: rc = launch_mid<6, 1>(p, zp_integral, n_rg, st); break;
+      default: rc = launch_mid<8, 1>(p, zp_integral, n_rg, st); break;
+    }
+    if (rc) return rc;
+    AWQ_HIP_TRY(hipGetLastError());
+    return AWQ_OK;
+  }
   // up to 4 tokens: the decode kernel's decomposition (one 16-token operand tile, mostly padding)
   int g = 0;
   if (M <= 4) {

@@ -173,8 +173,9 @@ def test_gemm_plan_for_the_model_matrices(lib):
     K_SPLIT, ROWS, ROWS_64, ROWS_CUT = 1, 2, 3, 4
     w1, w2, wo = (12288, 4096), (4096, 12288), (4096, 4096)
     plan = lambda shape, M, ws=1: lib.awq_gemm_plan(shape[0], shape[1], M, ws)
-    assert plan(w1, 1) == 0 and plan(w1, 4) == 0
-    assert [plan(w1, M) for M in (5, 64, 128)] == [K_SPLIT] * 3
+    assert plan(w1, 1) == 0 and plan((256, 512), 4) == 0 and plan((256, 512), 5) == K_SPLIT
+    assert [plan(s, M) for s in (w1, w2, wo) for M in (2, 4, 16)] == [5] * 9   # k a multiple of 4096
+    assert [plan(w1, M) for M in (17, 64, 128)] == [K_SPLIT] * 3
     assert [plan(w1, M) for M in (256, 384)] == [ROWS_64] * 2           # 96..144 tiles: units would idle
     assert [plan(w1, M) for M in (512, 640)] == [ROWS] * 2              # 192..240 tiles, one per unit
     assert [plan(w1, M) for M in (704, 1024)] == [ROWS_64] * 2          # 288..384 tiles: three per unit in one round

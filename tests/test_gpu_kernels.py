@@ -581,7 +581,12 @@ def test_gemv_fused_norm_unembed_argmax(awq, lib, oracle, torch_gpu, m, k):
                                           (12288, 4096, 2048, True), (4096, 12288, 2048, True),
                                           (12288, 4096, 1, True), (4096, 12288, 1, True),
                                           (12288, 4096, 4, True), (4096, 12288, 4, True),
-                                          (4096, 12288, 16, True), (12288, 4096, 64, True)])
+                                          (4096, 12288, 16, True), (12288, 4096, 64, True),
+                                          # 5..16 tokens: several row groups per workgroup (three, with a last
+                                          # workgroup of two; two; one), k of 128, 256 and 384 blocks
+                                          (12288, 4096, 5, False), (16384, 4096, 11, True), (4096, 8192, 9, False),
+                                          (8192, 8192, 13, True), (4096, 12288, 7, True), (4096, 4096, 16, False),
+                                          (2048, 16384, 10, True), (4096, 4096, 2, True), (1024, 4096, 3, False)])
 def test_gemm_matches_fp32_accumulate_reference(awq, lib, oracle, torch_gpu, m, k, M, zp_int):
     """config 5: dequant-on-load MFMA product; 1e-2 relative against the sequential FP32-accumulate
     reference, and the weights it multiplies are the bit-exact dequantised ones (one-hot check below).
@@ -638,9 +643,11 @@ def test_gemm_matches_fp32_accumulate_reference(awq, lib, oracle, torch_gpu, m, 
     assert np.all(np.isfinite(got2)) and np.all(np.abs(got2 - want) <= 1e-2 * denom)
     # much tighter in practice (FP32 accumulation either way; the many-token kernel applies the scale
     # to the sum instead of to every weight, one binary16 rounding fewer per weight than the oracle):
-    # 99% of the outputs within two binary16 roundings
-    assert np.percentile(np.abs(got - want) / denom, 99) <= 2.0 ** -10
-    assert np.percentile(np.abs(got2 - want) / denom, 99) <= 2.0 ** -10
+    # 99% of the outputs within two binary16 roundings; four for the kernels of up to 16 tokens, which round
+    # every weight twice as Inference.cu:102-104 does, where the oracle's integer sums round none
+    p99 = 2.0 ** -10 if M > 16 else 2.0 ** -9
+    assert np.percentile(np.abs(got - want) / denom, 99) <= p99
+    assert np.percentile(np.abs(got2 - want) / denom, 99) <= p99
 
 
 def _random_gemm_shapes(n, seed):

@@ -43,9 +43,16 @@ def oracle_run(oracle, model, prompt, n_new):
     return out[:n_new].tolist(), margins
 
 
-@pytest.mark.parametrize("n_prompt", [1, 2, 5, 37, 100])
-def test_small_model_batched_prompt_matches_sequential(awq, oracle, torch_gpu, n_prompt):
-    cfg = awq.make_config(**SMALL)
+# hidden 4096 and an intermediate size of 8192: the products of a prompt of 2..16 tokens go to the kernel for
+# up to 16 tokens (k a multiple of 4096) with its residual and GeLU endings, one and two slices of k
+WIDE = dict(n_layers=2, hidden=4096, inter=8192, vocab=1024, max_pos=64)
+
+
+@pytest.mark.parametrize("shape,n_prompt", [(SMALL, 1), (SMALL, 2), (SMALL, 5), (SMALL, 37), (SMALL, 100),
+                                            (WIDE, 3), (WIDE, 12), (WIDE, 16)],
+                         ids=lambda v: ("hidden%d" % v["hidden"]) if isinstance(v, dict) else str(v))
+def test_small_model_batched_prompt_matches_sequential(awq, oracle, torch_gpu, shape, n_prompt):
+    cfg = awq.make_config(**shape)
     model = make_oracle_model(oracle, cfg)
     eng = awq.QWen3AWQInfer.empty(cfg)
     fill_pair(awq, oracle, cfg, 77, engine=eng, model=model, profile=awq.SYNTH_BALANCED)
