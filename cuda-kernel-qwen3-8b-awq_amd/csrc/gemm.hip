@@ -11,10 +11,12 @@
 // rounding fewer per weight than the reference).
 //
 // Same weight stream as the decode kernel: [16-row group][32-wide block][row][16 B],
-// dword c of a row holding elements 8c..8c+7 of the block.  Two kernels:
-//   up to 4 tokens  the decode kernel's decomposition, products on v_mfma_f32_16x16x32_f16
-//   more tokens     64 rows x 32..128 tokens per wavefront on v_mfma_f32_32x32x16_f16,
-//                   tokens staged through LDS
+// dword c of a row holding elements 8c..8c+7 of the block.  Three kernels:
+//   up to 4 tokens   the decode kernel's decomposition, products on v_mfma_f32_16x16x32_f16
+//   up to 16 tokens, k a multiple of 4096 (taken first)
+//                    the same operand shapes, 16 wavefronts sharing up to three row groups
+//   more tokens      64 rows x 32..128 tokens per wavefront on v_mfma_f32_32x32x16_f16,
+//                    tokens staged through LDS
 #include "common.hpp"
 
 #include <atomic>
