@@ -316,7 +316,13 @@ def main():
 
     # ---- the prompt pass's product on the matrix cores: w1 shape, 2048 tokens (config 5) ---------
     w4a16 = importlib.import_module("cuda-kernel-qwen3-8b-awq_amd.bench_w4a16")
-    g = w4a16.measure((2048,), ("w1",))["shapes"]["w1"]["M=2048"]
+    sweep = w4a16.measure((4, 16, 64, 2048), ("w1",))["shapes"]["w1"]
+    g = sweep["M=2048"]
+    # config 5's decode-batch points on the same matrix: a weight stream, priced against the HBM peak
+    batch_gemm = {"workload": "W4A16 product 12288 x 4096 (int4 g=128) x 4 / 16 / 64 tokens, 12 rotating matrices",
+                  "bound": "hbm", "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                  "tokens": {str(M): {"us_per_launch": sweep["M=%d" % M]["us"], "achieved": sweep["M=%d" % M]["GBs"],
+                                      "frac": sweep["M=%d" % M]["hbm_frac"]} for M in (4, 16, 64)}}
     prefill_gemm = {"workload": "W4A16 product 12288 x 4096 (int4 g=128) x 2048 tokens, 12 rotating matrices",
                     "bound": "mfma", "achieved": g["TFLOPs"], "peak": 2500.0, "unit": "TFLOP/s",
                     "frac": g["mfma_frac"], "us_per_launch": g["us"]}
@@ -434,6 +440,7 @@ def main():
         "layer_512_positions": layer_cfg2,
         "long_context": long_context,
         "prefill_gemm": prefill_gemm,
+        "batch_gemm": batch_gemm,
         "roofline": roofline,
         "cpu_baseline": cpu,
     }
