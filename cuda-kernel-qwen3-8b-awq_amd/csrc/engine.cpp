@@ -175,6 +175,10 @@ struct awq_engine {
   } pb;
   bool batched_prefill = false;
   std::vector<void*> allocations;
+  // the reordered weight streams of all layers and the unembedding share one allocation, in the order the
+  // decode step reads them
+  char* stream_slab = nullptr;
+  int64_t slab_used = 0, slab_size = 0;
 };
 
 namespace {
@@ -182,6 +186,22 @@ namespace {
 int dev_alloc(awq_engine* e, void** p, int64_t bytes) {
   AWQ_HIP_TRY(hipMalloc(p, (size_t)(bytes > 0 ? bytes : 4)));
   e->allocations.push_back(*p);
+  return AWQ_OK;
+}
+
+// Room for one reordered weight stream.  One allocation for all of them (3.3 GB for the reference model) instead
+// of one per matrix: measured 0.5 % on the decode rate (fewer, larger pages for the address translation to hold).
+int stream_alloc(awq_engine* e, void** p, int64_t bytes) {
+  const auto pad = [](int64_t b) { return (b + 4095) & ~4095ll; };
+  if (!e->stream_slab) {
+    const int64_t H = e->cfg.hidden, I = e->cfg.inter, V = e->cfg.vocab;
+    const int64_t total = e->cfg.n_layers * (pad(3 * H * H / 2) + pad(H * H / 2) + 2 * pad(I * H / 2)) + pad(V * H / 2);
+    if (int rc = dev_alloc(e, (void**)&e->stream_slab, total)) return rc;
+    e->slab_size = total;
+  }
+  if (e->slab_used + pad(bytes) > e->slab_size) return dev_alloc(e, p, bytes);  // not one of the model's own matrices
+  *p = e->stream_slab + e->slab_used;
+  e->slab_used += pad(bytes);
   return AWQ_OK;
 }
 
@@ -386,7 +406,7 @@ int read_file(const std::string& path, int64_t bytes, void* dst, std::string* er
 
 // Reorders one linear layer on the engine's stream right after its packed bytes were copied.
 int reorder_now(awq_engine* e, DevLinear* t) {
-  if (int rc = dev_alloc(e, &t->stream_order, t->m * (t->k / 2))) return rc;
+  if (int rc = stream_alloc(e, &t->stream_order, t->m * (t->k / 2))) return rc;
   if (int rc = launch_repack(t->packed, t->stream_order, t->m, t->k, e->stream)) return rc;
   t->reordered = true;
   return AWQ_OK;
@@ -516,7 +536,7 @@ extern "C" int awq_finalize(awq_engine* e) {
   all.push_back(&e->unembed);
   for (DevLinear* t : all) {
     if (!t->reordered) {
-      if (int rc = dev_alloc(e, &t->stream_order, t->m * (t->k / 2))) return rc;
+      if (int rc = stream_alloc(e, &t->stream_order, t->m * (t->k / 2))) return rc;
       if (int rc = launch_repack(t->packed, t->stream_order, t->m, t->k, st)) return rc;
       t->reordered = true;
     }
