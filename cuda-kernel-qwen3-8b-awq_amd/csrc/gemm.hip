@@ -919,11 +919,8 @@ int launch_mid(const GemmParams& p, bool zint, int n_rg, hipStream_t st) {
 }
 // 2..16 tokens and k of 128, 256, 384 or 512 blocks: the row groups per workgroup (0: this kernel does not
 // take the product).  As many as the registers hold (at most three) while at least 256 workgroups remain.
-#ifndef AWQ_MID_MIN_TOKENS
-#define AWQ_MID_MIN_TOKENS 2
-#endif
 int mid_row_groups(int64_t m, int64_t k, int64_t M) {
-  if (M < AWQ_MID_MIN_TOKENS || M > 16 || k % 4096 != 0 || k > 16384 || m % 16 != 0) return 0;
+  if (M < 2 || M > 16 || k % 4096 != 0 || k > 16384 || m % 16 != 0) return 0;
   int rg = (int)(4 / (k / 4096));
   if (rg > 3) rg = 3;
   if (rg < 1) rg = 1;
