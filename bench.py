@@ -264,10 +264,18 @@ def main():
     hot.close()
     log("cache-hot (one layer's matrices): " + ", ".join("%s %.2f us" % (n, kernels[n]["us_cache_hot"])
                                                          for n in ("w1", "wqkv", "w2", "wo")))
+    # HBM bytes per launch from the counter runs summarised under profiles/: only while the kernel's source is
+    # the one they were measured on (the summary carries its SHA-256), null otherwise
     traffic = None
     tpath = os.path.join(ROOT, "profiles", "gemv_w1_traffic.json")
     if os.path.exists(tpath):
-        traffic = json.load(open(tpath)).get("hbm_bytes_per_launch")
+        import hashlib
+        rec = json.load(open(tpath))
+        src = os.path.join(ROOT, awq.__name__, "csrc", "gemv.hip")
+        if os.path.exists(src) and hashlib.sha256(open(src, "rb").read()).hexdigest() == rec.get("gemv_hip_sha256"):
+            traffic = rec.get("hbm_bytes_per_launch")
+        else:
+            log("profiles/gemv_w1_traffic.json was measured on another version of csrc/gemv.hip: traffic = null")
     w1 = kernels["w1"]
     roofline = {"bound": "hbm", "kernel": "gemv_kernel (int4 dequant + GEMV, m=12288 k=4096, GeLU epilogue)",
                 "achieved": w1["GBs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
@@ -420,7 +428,8 @@ def main():
         "metric": "decode tok/s @bs1, 8B-shape AWQ; int4 GEMV achieved HBM GB/s vs peak",
         "value": round(tok_s, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "int4 weights, f16 activations, f32 accumulate",
+        "dtype": "int4 weights; f16 activations held as 16-bit block fixed point per 32 inputs; exact integer dot "
+                 "products; f32 per-block scaling and accumulation; f16 outputs",
         "data": "synthetic (seeded random-init; nibbles uniform 0..15; %s)" % (
             "value: scale U[0.0025,0.004], zero-point 7 or 8 so that activations stay finite; value_spec_profile: the "
             "benchmark definition's scale U[0.002,0.02], zero-point 0..15, whose activations overflow FP16"

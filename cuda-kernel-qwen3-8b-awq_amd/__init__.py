@@ -66,6 +66,7 @@ SIGNATURES = {
     "awq_decode": (ctypes.c_int, [_vp, _i32, _vp]),
     "awq_prefill_batched": (ctypes.c_int, [_vp, _vp, _i32]),
     "awq_set_prefill_mode": (ctypes.c_int, [_vp, ctypes.c_int]),
+    "awq_debug_force_handover_giveup": (ctypes.c_int, [_vp, ctypes.c_int]),
     "awq_read_hidden": (ctypes.c_int, [_vp, _vp]),
     "awq_read_logits": (ctypes.c_int, [_vp, _vp]),
     "awq_set_graph_mode": (ctypes.c_int, [_vp, ctypes.c_int]),
@@ -82,7 +83,7 @@ SIGNATURES = {
     "awq_dequant": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "awq_linear_repack": (ctypes.c_int, [_vp, _vp, _i64, _i64, _vp]),
     "awq_gemv_workspace_bytes": (_i64, [_i64, _i64]),
-    "awq_gemv": (ctypes.c_int, [_vp, _vp, _vp, _i64, _i64, _vp, _vp, _i32, _vp, _vp]),
+    "awq_gemv": (ctypes.c_int, [_vp, _vp, _vp, _i64, _i64, _vp, _vp, _vp, _vp]),
     "awq_gemm_workspace_bytes": (_i64, [_i64, _i64, _i64]),
     "awq_gemm_plan": (_i32, [_i64, _i64, _i64, _i32]),
     "awq_gemm": (ctypes.c_int, [_vp, _vp, _vp, _i64, _i64, _vp, _vp, _i64, _i32, _vp, _vp]),
@@ -105,7 +106,7 @@ class AwqLinearArgs(ctypes.Structure):
     """struct awq_linear_args"""
     _fields_ = [
         ("repacked", _vp), ("scale", _vp), ("zp", _vp), ("m", _i64), ("k", _i64), ("x", _vp), ("y", _vp),
-        ("zp_integral", _i32), ("prologue", _i32), ("epilogue", _i32), ("eps", _f32), ("gamma", _vp),
+        ("reserved0", _i32), ("prologue", _i32), ("epilogue", _i32), ("eps", _f32), ("gamma", _vp),
         ("residual", _vp), ("cos_t", _vp), ("sin_t", _vp), ("k_cache", _vp), ("v_cache", _vp), ("hidden", _i32),
         ("reserved", _i32), ("max_pos", _i64), ("pos", _i64), ("out_token", _vp), ("workspace", _vp),
     ]

@@ -64,7 +64,7 @@ def measure(tokens, shapes=("w1", "w2")):
                 w = mats[i % n_mat]
                 if M == 1:
                     awq.check(lib.awq_gemv(w.data_ptr(), d_s.data_ptr(), d_z.data_ptr(), m, k, x.data_ptr(),
-                                           y.data_ptr(), 1, ws.data_ptr(), st))
+                                           y.data_ptr(), ws.data_ptr(), st))
                 else:
                     awq.check(lib.awq_gemm(w.data_ptr(), d_s.data_ptr(), d_z.data_ptr(), m, k, x.data_ptr(),
                                            y.data_ptr(), M, 1, gws.data_ptr(), st))

@@ -97,7 +97,6 @@ struct LinearArgs {
   half_t* y = nullptr;            // [m] ([hidden] rotated Q for EPI_QKV_ROPE)
   const half_t* res = nullptr;    // EPI_RESIDUAL: [m], may alias y
   int64_t m = 0, k = 0;
-  int zp_integral = 0;            // all zero-points are integers in [0,1024]: take the 2-op dequant
   int prologue = PRO_NONE;
   int epilogue = EPI_STORE;
   const half_t* gamma = nullptr;  // PRO_RMSNORM: [k]

@@ -258,7 +258,6 @@ LinearArgs linear_args(awq_engine* e, const DevLinear& t, const half_t* x, half_
   a.y = y;
   a.m = t.m;
   a.k = t.k;
-  a.zp_integral = t.zp_integral;
   a.eps = e->cfg.eps;
   a.dyn = e->d_state;
   return a;
@@ -911,6 +910,15 @@ extern "C" int awq_prefill_batched(awq_engine* e, const int32_t* prompt_ids, int
   return AWQ_OK;
 }
 
+extern "C" int awq_debug_force_handover_giveup(awq_engine* e, int on) {
+  AWQ_REQUIRE(e != nullptr, "engine is NULL");
+  if (int rc = ensure_prefill_buffers(e)) return rc;
+  const int32_t word = on ? 1 : 0;
+  AWQ_HIP_TRY(hipStreamSynchronize(e->stream));
+  AWQ_HIP_TRY(hipMemcpy((int32_t*)e->pb.gemm_ws + 1, &word, 4, hipMemcpyHostToDevice));
+  return AWQ_OK;
+}
+
 extern "C" int awq_set_prefill_mode(awq_engine* e, int batched) {
   AWQ_REQUIRE(e != nullptr, "engine is NULL");
   e->batched_prefill = batched != 0;
@@ -1109,7 +1117,6 @@ extern "C" int awq_gemv_fused(const awq_linear_args* u, void* stream) {
   AWQ_REQUIRE(u->m > 0 && u->m % 128 == 0, "m must be a positive multiple of 128");
   AWQ_REQUIRE(u->prologue == AWQ_PRO_NONE || u->prologue == AWQ_PRO_RMSNORM, "bad prologue");
   AWQ_REQUIRE(u->epilogue >= AWQ_EPI_STORE && u->epilogue <= AWQ_EPI_ARGMAX, "bad epilogue");
-  // zp_integral is not looked at: the block-sum arithmetic has no special case for integral zero-points
   LinearArgs a;
   a.wq = u->repacked;
   a.scale = (const half_t*)u->scale;
@@ -1120,7 +1127,6 @@ extern "C" int awq_gemv_fused(const awq_linear_args* u, void* stream) {
   a.best = (unsigned long long*)u->workspace;  // the sampler's best candidate
   a.m = u->m;
   a.k = u->k;
-  a.zp_integral = false;
   a.prologue = u->prologue;
   a.epilogue = u->epilogue;
   a.gamma = (const half_t*)u->gamma;
@@ -1138,7 +1144,7 @@ extern "C" int awq_gemv_fused(const awq_linear_args* u, void* stream) {
 }
 
 extern "C" int awq_gemv(const void* repacked, const void* scale, const void* zp, int64_t m, int64_t k, const void* x,
-                        void* y, int32_t zp_integral, void* workspace, void* stream) {
+                        void* y, void* workspace, void* stream) {
   awq_linear_args u;
   memset(&u, 0, sizeof(u));
   u.repacked = repacked;
@@ -1148,7 +1154,6 @@ extern "C" int awq_gemv(const void* repacked, const void* scale, const void* zp,
   u.k = k;
   u.x = x;
   u.y = y;
-  u.zp_integral = zp_integral;
   u.workspace = workspace;
   return awq_gemv_fused(&u, stream);
 }

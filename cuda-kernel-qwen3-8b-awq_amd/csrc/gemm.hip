@@ -42,7 +42,7 @@ struct GemmParams {
   int32_t kz;           // k is cut into kz chunks over blockIdx.z (k-split workgroups only)
   float* part;          // kz > 1: FP32 partial sums [kz][M][m], finished by reduce_parts_kernel
   int32_t nr, n_tiles;  // rows split: 256-row blocks, tiles = row blocks x 128-token blocks (row block fastest)
-  int32_t* sk_head;     // rows split with handed-over sums: status word at [0], counters at [16 + workgroup]
+  int32_t* sk_head;     // rows split with handed-over sums: status word at [0], "give up now" at [1], counters at [16 + workgroup]
   float* sk_part;       // and one tile of FP32 sums per workgroup
 };
 
@@ -740,19 +740,30 @@ __global__ __launch_bounds__(256, (MODE == WIDE_K && TT == 4) ? 1 : ((MODE == WI
       if (CUT && s_lo != 0) {
         // the tile's first steps were taken by workgroups first .. b - 1, one slot each
         const int first = sk_wg_of((int64_t)tile * S2, W2, gridDim.x);
+        // A wait that gives up (too many polls, or the host's "give up now" word at [1], looked at before the
+        // first poll: the tests set it so that this path runs without any wait ever timing out) reports
+        // through the status word, and the workgroup leaves its tile unwritten rather than storing sums
+        // it does not have.
+        __shared__ int gave_up;
         if (tid == 0) {
           int spins = 0;
-          while (__hip_atomic_load(p.sk_head + 16 + b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < b - first) {
-            __builtin_amdgcn_s_sleep(4);
-            if (++spins > kSkSpinLimit) {
-              __hip_atomic_store(p.sk_head, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-              break;
-            }
+          int lost = __hip_atomic_load(p.sk_head + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0;
+          while (!lost && __hip_atomic_load(p.sk_head + 16 + b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < b - first) {
+            if (++spins > kSkSpinLimit) lost = 1;
+            else __builtin_amdgcn_s_sleep(4);
           }
+          if (lost) __hip_atomic_store(p.sk_head, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");  // the counted workgroups' sums are visible from here
-          __hip_atomic_store(p.sk_head + 16 + b, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
+          // for the next launch.  (After giving up, the counted workgroups may still add to it: the host
+          // clears the whole header when it sees the status word.)
+          __hip_atomic_store(p.sk_head + 16 + b, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          gave_up = lost;
         }
         __syncthreads();
+        if (gave_up) {
+          __syncthreads();  // every thread has read the flag before the next tile's wait may write it
+          continue;
+        }
         for (int c = first; c < b; ++c) {
           const u64* theirs = reinterpret_cast<const u64*>(p.sk_part) + (int64_t)c * (kSkTileFloats / 2);
 #pragma unroll

@@ -559,9 +559,6 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
     }
   }
 
-  // Group constants.  When the scale group depends on the input index it is
-  // constant within a class of blocks; the (at most 64) classes of a row group
-  // go through a table in LDS, filled one row group ahead.
   // Group constants.  When the scale group depends on the input index it is constant within a class of
   // blocks; the (at most 64) classes of every row group this workgroup will walk go into a table in LDS
   // here, so that the loop issues no loads but the weights'.  (A value requested and used inside the loop
@@ -896,9 +893,9 @@ int launch_gemv(const LinearArgs& a, hipStream_t st) {
   // one workgroup per row group while that fits the device a few times over;
   // beyond that a workgroup walks several row groups and stages x once
   int64_t n_rg = a.m / plan.rh, n_wg = n_rg;
-  if (n_rg > 1024) n_wg = std::max<int64_t>(4096 / plan.n_waves, (n_rg + 31) / 32);  // at most 32 passes: the table of
-                                                                                      // group constants is per pass  // four wavefronts per SIMD (measured: 151936 x 4096 with argmax as 512
-                                                // workgroups of 8 wavefronts 60 us, as 1024 of 4 wavefronts 64 us, 576 of 8: 80 us)
+  // Four wavefronts per SIMD (measured: 151936 x 4096 with argmax as 512 workgroups of 8 wavefronts 60 us, as
+  // 1024 of 4 wavefronts 64 us, 576 of 8: 80 us), and at most 32 passes: the table of group constants is per pass.
+  if (n_rg > 1024) n_wg = std::max<int64_t>(4096 / plan.n_waves, (n_rg + 31) / 32);
   dim3 grid((unsigned)n_wg), block((unsigned)(plan.n_waves * 64));
   // x as nibble planes plus 16 bytes of skew per lane group, two floats per block, the table of group
   // constants of a periodic matrix (passes x classes), and with the fused norm x in natural order
@@ -906,7 +903,9 @@ int launch_gemv(const LinearArgs& a, hipStream_t st) {
   size_t lds = (size_t)a.k * 2 + (size_t)(a.k / AWQ_BLOCK_K / plan.g) * 16 + (size_t)(a.k / AWQ_BLOCK_K) * 8 +
                (periodic ? (size_t)(n_pass * p.C + 1 & ~1) * sizeof(GroupConst) : 0) + (size_t)n_pass * plan.rh * 4 +
                (a.prologue == PRO_RMSNORM ? (size_t)a.k * 2 : 0);
-  AWQ_REQUIRE(lds <= 65536, "k too large for the fused norm (x is kept twice in LDS)");
+  // the kernel's static arrays (the wavefronts' sums, double-buffered, and the norm's partial sums) come on top
+  constexpr size_t kStaticLds = 2 * 16 * 16 * sizeof(float) + 256 * sizeof(float);
+  AWQ_REQUIRE(lds + kStaticLds <= 65536, "k too large for the fused norm (x is kept twice in LDS)");
   switch (plan.g) {
     case 2: launch_g<2>(p, periodic, n_wg < n_rg, plan.rh, grid, block, lds, st); break;
     case 4: launch_g<4>(p, periodic, n_wg < n_rg, plan.rh, grid, block, lds, st); break;

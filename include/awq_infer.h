@@ -99,6 +99,13 @@ int awq_decode(awq_engine* e, int32_t n_steps, int32_t* out_ids);
  * token-by-token loop. */
 int awq_prefill_batched(awq_engine* e, const int32_t* prompt_ids, int32_t n_prompt);
 int awq_set_prefill_mode(awq_engine* e, int batched);
+/* Test hook, no counterpart in the reference: some of the batched pass's
+ * products hand partial sums from workgroup to workgroup through a bounded
+ * wait (see awq_gemm).  With `on` non-zero every such wait of the next
+ * awq_prefill_batched call gives up before its first poll: all kernels end
+ * normally, the call returns AWQ_ERR_HIP, and the engine is usable again
+ * after awq_reset. */
+int awq_debug_force_handover_giveup(awq_engine* e, int on);
 
 /* Copies of internal state for tests: hidden state [hidden] and the logits of
  * the last sampled position [vocab], both FP16, to host memory. */
@@ -166,18 +173,13 @@ int awq_linear_repack(const void* packed_in, void* repacked_out, int64_t m, int6
  *     makes every output a NaN.  Within 1e-2 (in practice a few 1e-4) of the
  *     FP32-accumulated product of the FP16-dequantised weights.
  * repacked from awq_linear_repack; scale/zp [m/128]; x [k], y [m] FP16.
- * zp_integral: kept for the matrix-core product (awq_gemm), where 1 selects a
- * shorter conversion for zero-points that are integers in [0,1024] (true of
- * AWQ checkpoints), 0 takes arbitrary zero-points and -1 has the call inspect
- * them (synchronises); awq_gemv and awq_gemv_fused accept and ignore it: their
- * arithmetic has no special case.
  * k <= 16384 (the workgroup keeps x in LDS).
  * workspace: awq_gemv_workspace_bytes(m,k) bytes, zero-filled once before its
  * first use (launches leave it zeroed); must not be shared by launches that
  * may overlap. */
 int64_t awq_gemv_workspace_bytes(int64_t m, int64_t k);
 int awq_gemv(const void* repacked, const void* scale, const void* zp, int64_t m, int64_t k, const void* x, void* y,
-             int32_t zp_integral, void* workspace, void* stream);
+             void* workspace, void* stream);
 
 /* The same kernel with the neighbouring operators of runOneLayer /
  * sampleNextToken fused in, as the engine launches it:
@@ -204,7 +206,7 @@ typedef struct awq_linear_args {
   int64_t m, k;
   const void* x;
   void* y;
-  int32_t zp_integral;
+  int32_t reserved0;     /* 0 */
   int32_t prologue;
   int32_t epilogue;
   float eps;
@@ -238,9 +240,14 @@ int awq_gemv_fused(const awq_linear_args* args, void* stream);
  * waits for the others; they have lower indices and never wait themselves, so
  * the wait ends while the device dispatches workgroups in index order.  It is
  * bounded all the same: should it expire, the first int32 of the workspace
- * becomes 1 (read it after synchronising; the outputs are then wrong and the
- * header must be zeroed again).  Calls that share a workspace must not
- * overlap. */
+ * becomes 1 (read it after synchronising; the workgroup that gave up leaves
+ * its tile of y unwritten, and the header must be zeroed again).  The second
+ * int32 is a "give up now" word: non-zero makes every such wait give up
+ * before its first poll, so that a test can drive this path with every kernel
+ * ending normally.  Calls that share a workspace must not overlap.
+ * zp_integral: 1 selects a shorter conversion for zero-points that are
+ * integers in [0,1024] (true of AWQ checkpoints), 0 takes arbitrary
+ * zero-points and -1 has the call inspect them (synchronises). */
 int64_t awq_gemm_workspace_bytes(int64_t m, int64_t k, int64_t M);
 /* Which workgroup shape awq_gemm takes for a product (host arithmetic only; no counterpart in the
  * reference, for diagnostics and tests): 0 the few-token kernel (M <= 4), 1 k split over the

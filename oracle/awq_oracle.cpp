@@ -205,16 +205,29 @@ AWQO_API void awqo_linear_seq(const uint8_t* packed, const half_t* scale, const 
                               const half_t* x, half_t* y, int64_t M) {
   std::vector<float> lut;
   build_lut(scale, zp, m / AWQ_GROUP_SIZE, lut);
+  // Every row keeps its own accumulator and sees j = 0, 1, 2, ... in that order (multiply, then add, both
+  // rounded to binary32), so the loops may run with j outside and the rows of a 128-row block inside: the
+  // nibbles of consecutive rows are consecutive in memory, and a block of 128 aligned rows shares one scale
+  // group for a given j (j*m and k are multiples of 128).
+  std::vector<float> xf((size_t)k);
+  for (int64_t t = 0; t < M; ++t) {
+    for (int64_t j = 0; j < k; ++j) xf[j] = h2f(x[t * k + j]);
 #pragma omp parallel for schedule(static)
-  for (int64_t i = 0; i < m; ++i) {
-    for (int64_t t = 0; t < M; ++t) {
-      float acc = 0.0f;
+    for (int64_t i0 = 0; i0 < m; i0 += AWQ_GROUP_SIZE) {
+      float acc[AWQ_GROUP_SIZE];
+      for (int r = 0; r < AWQ_GROUP_SIZE; ++r) acc[r] = 0.0f;
       for (int64_t j = 0; j < k; ++j) {
-        int g = awq_group_index(m, k, i, j);
-        float prod = lut[g * 16 + nibble_at(packed, j * m + i)] * h2f(x[t * k + j]);
-        acc = acc + prod;
+        const float* lg = &lut[(size_t)awq_group_index(m, k, i0, j) * 16];
+        const uint8_t* src = packed + ((j * m + i0) >> 1);  // j*m + i0 is even
+        const float xj = xf[j];
+        for (int r = 0; r < AWQ_GROUP_SIZE; r += 2) {
+          const uint8_t b = src[r >> 1];
+          const float p0 = lg[b & 15] * xj, p1 = lg[b >> 4] * xj;
+          acc[r] = acc[r] + p0;
+          acc[r + 1] = acc[r + 1] + p1;
+        }
       }
-      y[t * m + i] = f2h(acc);
+      for (int r = 0; r < AWQ_GROUP_SIZE; ++r) y[t * m + i0 + r] = f2h(acc[r]);
     }
   }
 }
@@ -536,6 +549,10 @@ struct awqo_model {
   // statistics of the last generate call
   std::vector<float> margins;
   double seconds_linear = 0;
+  // 0: the blocked arithmetic the GPU kernels follow (awqo_linear); 1: the reference's own -- weights rounded to
+  // binary16 as dequantAwqKernel leaves them (I:102-104), binary32 accumulation in input order (awqo_linear_seq).
+  // Mode 1 exists so that the distance between the two can be measured on a whole model.
+  int linear_mode = 0;
 };
 
 static Tensor* model_tensor(awqo_model* m, int layer, int kind) {
@@ -656,7 +673,8 @@ AWQO_API int awqo_model_load_dir(awqo_model* m, const char* dir) {
 
 static void model_linear(awqo_model* m, Tensor& t, const half_t* x, half_t* y) {
   auto t0 = std::chrono::steady_clock::now();
-  linear_blocked(t.packed.data(), t.scale.data(), t.zp.data(), t.out_dim, t.in_dim, x, y, nullptr);
+  if (m->linear_mode == 1) awqo_linear_seq(t.packed.data(), t.scale.data(), t.zp.data(), t.out_dim, t.in_dim, x, y, 1);
+  else linear_blocked(t.packed.data(), t.scale.data(), t.zp.data(), t.out_dim, t.in_dim, x, y, nullptr);
   m->seconds_linear += std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
 }
 
@@ -763,3 +781,4 @@ AWQO_API int awqo_model_margins(awqo_model* m, float* out, int cap) {
   return n;
 }
 AWQO_API double awqo_model_seconds_linear(awqo_model* m) { return m->seconds_linear; }
+AWQO_API void awqo_model_set_linear_mode(awqo_model* m, int mode) { m->linear_mode = mode; }

@@ -147,3 +147,22 @@ def fill_pair(awq, oracle, cfg, seed, engine=None, model=None, profile=0, mutate
             engine.upload(layer, kind, part, p, nbytes)
     if engine is not None:
         engine.finalize()
+
+
+# ---- activation shapes that stress the block fixed point of the linear layers ------------------
+def heavy_tailed_inputs(rng, k):
+    """name -> binary16 input vector of length k.  The linear layers round each input to 2^-16 of the largest
+    magnitude in its block of 32, so what matters is how the magnitudes inside a block are spread."""
+    out = {}
+    x = rng.standard_normal(k)
+    idx = 32 * np.arange(k // 32) + rng.integers(0, 32, size=k // 32)
+    x[idx] = 1024.0 * np.where(rng.random(k // 32) < 0.5, -1.0, 1.0)
+    out["one 2^10 outlier per block over N(0,1)"] = x.astype(np.float16)
+    x = 1e-3 * rng.standard_normal(k)
+    x[rng.choice(k, size=3, replace=False)] = np.array([3000.0, -2500.0, 1800.0])
+    out["three massive channels over 1e-3 noise"] = x.astype(np.float16)
+    out["Student-t, 2 degrees of freedom"] = np.clip(rng.standard_t(2, size=k), -60000, 60000).astype(np.float16)
+    from math import erf
+    g = rng.standard_normal(k)
+    out["GeLU of N(0,1)"] = np.array([0.5 * v * (1.0 + erf(v * 0.70710678)) for v in g]).astype(np.float16)
+    return out

@@ -55,6 +55,7 @@ SIG = {
     "awqo_model_vcache": (vp, [vp, ctypes.c_int]),
     "awqo_model_margins": (ctypes.c_int, [vp, vp, ctypes.c_int]),
     "awqo_model_seconds_linear": (f64, [vp]),
+    "awqo_model_set_linear_mode": (None, [vp, ctypes.c_int]),
 }
 
 _lib = None

@@ -325,7 +325,7 @@ def test_config2_one_decoder_layer_at_position_512(awq, lib, oracle, torch_gpu):
         w, s, z = dev_w[kind]
         a.repacked, a.scale, a.zp = w.data_ptr(), s.data_ptr(), z.data_ptr()
         a.m, a.k = dims[kind]
-        a.x, a.y, a.zp_integral, a.workspace, a.eps = x.data_ptr(), y.data_ptr(), 1, ws.data_ptr(), 1e-6
+        a.x, a.y, a.workspace, a.eps = x.data_ptr(), y.data_ptr(), ws.data_ptr(), 1e-6
         for key, val in kw.items():
             setattr(a, key, val)
         awq.check(lib.awq_gemv_fused(C.byref(a), st))
@@ -366,6 +366,34 @@ def test_full_model_32_greedy_tokens_identical(awq, oracle, torch_gpu):
     print("top-1/top-2 logit margins: min %.4f median %.4f" % (margins[:n].min(), np.median(margins[:n])), flush=True)
     assert got == ref
     assert len(set(got)) > 1 and np.isfinite(margins[:n]).all() and margins[:n].min() < 0.5
+    compare_state(awq, oracle, eng, model, cfg)
+    eng.close()
+    oracle.awqo_model_destroy(model)
+
+
+def test_config4_at_its_stated_length(awq, oracle, torch_gpu):
+    """config 4 as the benchmark definition states it: all 36 layers at the reference widths, a prompt of
+    128 token ids uniform in [0, 151936), 256 new tokens greedily at batch 1 -- 384 forward passes of
+    generateResponse (Inference.cu:1297-1408) on both paths; all 256 ids, the last layer's output and the
+    last logits must be the CPU path's bit for bit"""
+    cfg = awq.make_config(max_pos=384)
+    assert (cfg.n_layers, cfg.hidden, cfg.inter, cfg.vocab, cfg.split_idx) == (36, 4096, 12288, 151936, 18)
+    model = make_oracle_model(oracle, cfg)
+    eng = awq.QWen3AWQInfer.empty(cfg)
+    fill_pair(awq, oracle, cfg, 31, engine=eng, model=model, profile=awq.SYNTH_BALANCED)
+    prompt = np.zeros(128, dtype=np.int32)
+    awq.check(awq.load_library().awq_synth_tokens(31, awq.SYNTH_STREAM_INPUT, ptr(prompt), prompt.size, cfg.vocab))
+    assert prompt.min() >= 0 and prompt.max() < cfg.vocab and len(set(prompt.tolist())) > 100
+    print("36-layer model: 128-token prompt, 256 greedy tokens on the GPU", flush=True)
+    got = eng.generateResponse(prompt.tolist(), 256)
+    print("the same on the CPU oracle (384 forward passes)", flush=True)
+    ref = oracle_generate(oracle, model, prompt.tolist(), 256)
+    margins = np.zeros(256, dtype=np.float32)
+    n = oracle.awqo_model_margins(model, ptr(margins), 256)
+    print("distinct ids %d, top-1/top-2 logit margins: min %.4f median %.4f" %
+          (len(set(ref)), margins[:n].min(), np.median(margins[:n])), flush=True)
+    assert len(got) == 256 and got == ref
+    assert len(set(got)) > 1 and np.isfinite(margins[:n]).all()
     compare_state(awq, oracle, eng, model, cfg)
     eng.close()
     oracle.awqo_model_destroy(model)

@@ -82,7 +82,7 @@ def test_repack_matches_numpy_layout(awq, lib, oracle, torch_gpu, m, k):
     assert np.array_equal(d_out.cpu().numpy().view(np.uint32), ref)
 
 
-def gemv_gpu(awq, lib, torch, packed, scale, zp, m, k, x, zp_integral, repeat=1):
+def gemv_gpu(awq, lib, torch, packed, scale, zp, m, k, x, repeat=1):
     d_in = dev(torch, packed)
     d_w = torch.zeros(m * k // 2, dtype=torch.uint8, device="cuda")
     awq.check(lib.awq_linear_repack(d_in.data_ptr(), d_w.data_ptr(), m, k, stream(torch)))
@@ -92,7 +92,7 @@ def gemv_gpu(awq, lib, torch, packed, scale, zp, m, k, x, zp_integral, repeat=1)
     for _ in range(repeat):
         d_y = torch.full((m,), float("nan"), dtype=torch.float16, device="cuda")
         awq.check(lib.awq_gemv(d_w.data_ptr(), d_s.data_ptr(), d_z.data_ptr(), m, k, d_x.data_ptr(), d_y.data_ptr(),
-                               zp_integral, ws.data_ptr(), stream(torch)))
+                               ws.data_ptr(), stream(torch)))
         torch.cuda.synchronize()
         outs.append(d_y.cpu().numpy())
     assert int(ws.to(torch.int32).abs().sum().item()) == 0  # the workspace is left zeroed
@@ -116,7 +116,7 @@ def test_gemv_bit_exact_and_within_tolerance(awq, lib, oracle, torch_gpu, m, k, 
     oracle.awqo_linear(ptr(packed), ptr(scale), ptr(zp), m, k, ptr(x), ptr(ref), 1)
     seq = np.zeros(m, dtype=np.float16)
     oracle.awqo_linear_seq(ptr(packed), ptr(scale), ptr(zp), m, k, ptr(x), ptr(seq), 1)
-    outs = gemv_gpu(awq, lib, torch, packed, scale, zp, m, k, x, 1 if zp_int else 0, repeat=2)
+    outs = gemv_gpu(awq, lib, torch, packed, scale, zp, m, k, x, repeat=2)
     print("gemv", m, k, zp_int, flush=True)
     assert np.array_equal(outs[0].view(np.uint16), ref.view(np.uint16))          # same summation order: same bits
     assert np.array_equal(outs[1].view(np.uint16), ref.view(np.uint16))          # and the workspace reset itself
@@ -128,12 +128,34 @@ def test_gemv_bit_exact_and_within_tolerance(awq, lib, oracle, torch_gpu, m, k, 
     denom = np.maximum(np.abs(want), np.sqrt(np.mean(want * want)))
     err = np.abs(outs[0].astype(np.float64) - want) / denom
     assert np.all(err <= 1e-2) and np.percentile(err, 99) <= 2.0 ** -9
-    if zp_int:
-        # the general sequence must give the same bits as the integral-zero-point shortcut
-        gen = gemv_gpu(awq, lib, torch, packed, scale, zp, m, k, x, 0)[0]
-        assert np.array_equal(gen.view(np.uint16), ref.view(np.uint16))
-        auto = gemv_gpu(awq, lib, torch, packed, scale, zp, m, k, x, -1)[0]
-        assert np.array_equal(auto.view(np.uint16), ref.view(np.uint16))
+
+
+@pytest.mark.parametrize("m,k", [(4096, 4096), (12288, 4096), (4096, 12288)])
+def test_gemv_heavy_tailed_inputs_stay_within_tolerance(awq, lib, oracle, torch_gpu, m, k):
+    """outliers, massive channels, heavy tails and post-GeLU inputs at the model's own matrix shapes: the fused
+    product must still give the oracle's bits, and stay within 1e-2 of max(|y|, rms y) of the plain
+    FP32-accumulate product over the reference's binary16-rounded weights (awqo_linear_seq); the block fixed
+    point rounds each input to 2^-16 of its block's largest magnitude, so the distance depends on the shape
+    of x"""
+    from helpers import heavy_tailed_inputs
+    torch = torch_gpu
+    rng = np.random.default_rng(m + 3 * k)
+    packed, scale, zp = rand_awq(rng, m, k)
+    for name, x in heavy_tailed_inputs(rng, k).items():
+        ref = np.zeros(m, dtype=np.float16)
+        oracle.awqo_linear(ptr(packed), ptr(scale), ptr(zp), m, k, ptr(x), ptr(ref), 1)
+        seq = np.zeros(m, dtype=np.float16)
+        oracle.awqo_linear_seq(ptr(packed), ptr(scale), ptr(zp), m, k, ptr(x), ptr(seq), 1)
+        got = gemv_gpu(awq, lib, torch, packed, scale, zp, m, k, x)[0]
+        print("gemv", m, k, name, flush=True)
+        assert np.array_equal(got.view(np.uint16), ref.view(np.uint16)), name
+        want = seq.astype(np.float64)
+        if not np.isfinite(want).all():
+            assert np.array_equal(np.isfinite(want), np.isfinite(got.astype(np.float64))), name
+            continue
+        denom = np.maximum(np.abs(want), np.sqrt(np.mean(want * want)))
+        err = np.abs(got.astype(np.float64) - want) / denom
+        assert err.max() <= 1e-2, (name, err.max())
 
 
 @pytest.mark.parametrize("m,k", [(256, 1024), (384, 512), (4096, 4096), (128 * 37, 512)])
@@ -160,7 +182,7 @@ def test_gemv_input_dynamic_range(awq, lib, oracle, torch_gpu, m, k):
             x[450] = np.nan
         ref = np.zeros(m, dtype=np.float16)
         oracle.awqo_linear(ptr(packed), ptr(scale), ptr(zp), m, k, ptr(x), ptr(ref), 1)
-        got = gemv_gpu(awq, lib, torch, packed, scale, zp, m, k, x, 0)[0]
+        got = gemv_gpu(awq, lib, torch, packed, scale, zp, m, k, x)[0]
         print("gemv range", m, k, case, flush=True)
         assert np.array_equal(got.view(np.uint16), ref.view(np.uint16))
         if case == "finite":
@@ -178,7 +200,7 @@ def test_gemv_unembed_shape_and_argmax(awq, lib, oracle, torch_gpu):
     x = rng.standard_normal(k).astype(np.float16)
     ref = np.zeros(m, dtype=np.float16)
     oracle.awqo_linear(ptr(packed), ptr(scale), ptr(zp), m, k, ptr(x), ptr(ref), 1)
-    got = gemv_gpu(awq, lib, torch, packed, scale, zp, m, k, x, 1)[0]
+    got = gemv_gpu(awq, lib, torch, packed, scale, zp, m, k, x)[0]
     assert np.array_equal(got.view(np.uint16), ref.view(np.uint16))
     d_l = dev(torch, got)
     ws = torch.zeros(lib.awq_argmax_workspace_bytes(m), dtype=torch.uint8, device="cuda")
@@ -197,7 +219,7 @@ def test_gemv_one_hot_column_major(awq, lib, torch_gpu):
     for p, q in [(0, 5), (1, 9), (m - 1, 3), (m, 7), (3 * m + 17, 15), (k * m - 1, 1)]:
         packed = np.zeros(m * k // 2, dtype=np.uint8)
         packed[p >> 1] = q << (4 * (p & 1))
-        y = gemv_gpu(awq, lib, torch, packed, scale, zp, m, k, x, 1)[0].astype(np.float64)
+        y = gemv_gpu(awq, lib, torch, packed, scale, zp, m, k, x)[0].astype(np.float64)
         expect = np.zeros(m)
         expect[p % m] = q * float(x[p // m])
         assert np.array_equal(y, expect), p
@@ -207,9 +229,9 @@ def test_gemv_rejects_bad_shapes(awq, lib, torch_gpu):
     torch = torch_gpu
     buf = torch.zeros(1 << 20, dtype=torch.uint8, device="cuda")
     p = buf.data_ptr()
-    assert lib.awq_gemv(p, p, p, 100, 512, p, p, 1, p, None) != 0
+    assert lib.awq_gemv(p, p, p, 100, 512, p, p, p, None) != 0
     assert b"multiple of 128" in lib.awq_last_error()
-    assert lib.awq_gemv(p, p, p, 128, 384, p, p, 1, p, None) != 0
+    assert lib.awq_gemv(p, p, p, 128, 384, p, p, p, None) != 0
     assert lib.awq_linear_repack(p, p, 128, 512, None) != 0
     assert lib.awq_dequant(p, p, p, p, 4, 7, 1, None) != 0
 
@@ -462,7 +484,7 @@ def fused_setup(awq, lib, torch, rng, m, k, zp_int=True):
                 ws=torch.zeros(lib.awq_gemv_workspace_bytes(m, k), dtype=torch.uint8, device="cuda"))
     a = awq.AwqLinearArgs()
     a.repacked, a.scale, a.zp = keep["d_w"].data_ptr(), keep["d_s"].data_ptr(), keep["d_z"].data_ptr()
-    a.m, a.k, a.zp_integral, a.workspace = m, k, 1 if zp_int else 0, keep["ws"].data_ptr()
+    a.m, a.k, a.workspace = m, k, keep["ws"].data_ptr()
     return packed, scale, zp, a, keep
 
 
@@ -602,7 +624,8 @@ def test_gemm_matches_fp32_accumulate_reference(awq, lib, oracle, torch_gpu, m, 
     sel = np.sort(rng.choice(M, size=Mo, replace=False))
     ref = np.zeros((Mo, m), dtype=np.float16)
     xs = np.ascontiguousarray(x[sel])
-    oracle.awqo_linear(ptr(packed), ptr(scale), ptr(zp), m, k, ptr(xs), ptr(ref), Mo)
+    # the reference arithmetic: binary16-dequantised weights (Inference.cu:102-104), binary32 accumulation
+    oracle.awqo_linear_seq(ptr(packed), ptr(scale), ptr(zp), m, k, ptr(xs), ptr(ref), Mo)
     d_in = dev(torch, packed)
     d_w = torch.zeros(m * k // 2, dtype=torch.uint8, device="cuda")
     awq.check(lib.awq_linear_repack(d_in.data_ptr(), d_w.data_ptr(), m, k, stream(torch)))
@@ -641,13 +664,13 @@ def test_gemm_matches_fp32_accumulate_reference(awq, lib, oracle, torch_gpu, m, 
     assert np.all(np.isfinite(got))
     assert np.all(np.abs(got - want) <= 1e-2 * denom)
     assert np.all(np.isfinite(got2)) and np.all(np.abs(got2 - want) <= 1e-2 * denom)
-    # much tighter in practice (FP32 accumulation either way; the many-token kernel applies the scale
-    # to the sum instead of to every weight, one binary16 rounding fewer per weight than the oracle):
-    # 99% of the outputs within two binary16 roundings; four for the kernels of up to 16 tokens, which round
-    # every weight twice as Inference.cu:102-104 does, where the oracle's integer sums round none
-    p99 = 2.0 ** -10 if M > 16 else 2.0 ** -9
-    assert np.percentile(np.abs(got - want) / denom, 99) <= p99
-    assert np.percentile(np.abs(got2 - want) / denom, 99) <= p99
+    # much tighter in practice: both sides accumulate in FP32.  The kernels of up to 16 tokens round every
+    # weight twice as Inference.cu:102-104 does and differ from the reference only in the order of the sum;
+    # the many-token kernel applies the scale to the sum instead of to every weight (one binary16 rounding
+    # fewer per weight).  99% of the outputs within two binary16 roundings.
+    p99a, p99b = np.percentile(np.abs(got - want) / denom, 99), np.percentile(np.abs(got2 - want) / denom, 99)
+    print("99th percentile of the relative error: %.3g %.3g (2^-10 = %.3g)" % (p99a, p99b, 2.0 ** -10), flush=True)
+    assert p99a <= 2.0 ** -10 and p99b <= 2.0 ** -10
 
 
 def _random_gemm_shapes(n, seed):

@@ -57,3 +57,54 @@ def test_static_scratch_attention_matches_the_workspace_entry_point(awq, lib, or
     assert lib.awq_decode_attention_static(d_q.data_ptr(), d_k.data_ptr(), d_v.data_ptr(), got.data_ptr(), 33, mp, 10,
                                            st) != 0
     assert b"32 heads" in lib.awq_last_error()
+
+
+def test_static_scratch_attention_allocates_nothing_and_can_be_captured(awq, lib, oracle, torch_gpu):
+    """What the entry point is for: no device memory is allocated by any call after the first (which looks up
+    the array's address), and a call issued under stream capture replays to the same bits."""
+    torch = torch_gpu
+    nh, mp = 32, 4096
+    rng = np.random.default_rng(78)
+    d_k = torch.from_numpy((0.3 * rng.standard_normal((nh, mp, 128))).astype(np.float16)).cuda()
+    d_v = torch.from_numpy(rng.standard_normal((nh, mp, 128)).astype(np.float16)).cuda()
+    d_q = torch.from_numpy(rng.standard_normal(nh * 128).astype(np.float16)).cuda()
+    ws = torch.zeros(lib.awq_attention_workspace_bytes(nh, mp), dtype=torch.uint8, device="cuda")
+    outs = {L: torch.zeros(nh * 128, dtype=torch.float16, device="cuda") for L in (3000, 1500, 900, 300)}
+    wants = {L: torch.zeros(nh * 128, dtype=torch.float16, device="cuda") for L in outs}
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for L in outs:
+        awq.check(lib.awq_decode_attention(d_q.data_ptr(), d_k.data_ptr(), d_v.data_ptr(), wants[L].data_ptr(), nh, mp,
+                                           L, ws.data_ptr(), st))
+    # the first call on this device looks the array's address up
+    awq.check(lib.awq_decode_attention_static(d_q.data_ptr(), d_k.data_ptr(), d_v.data_ptr(), outs[300].data_ptr(), nh,
+                                              mp, 300, st))
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    for _ in range(3):
+        for L in outs:
+            awq.check(lib.awq_decode_attention_static(d_q.data_ptr(), d_k.data_ptr(), d_v.data_ptr(), outs[L].data_ptr(),
+                                                      nh, mp, L, st))
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before, (free_before, free_after)
+    for L in outs:
+        assert torch.equal(outs[L].view(torch.int16), wants[L].view(torch.int16)), L
+    # under stream capture: every launch form, replayed three times with eager work in between
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    cap = {L: torch.zeros(nh * 128, dtype=torch.float16, device="cuda") for L in outs}
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.graph(graph, stream=side):
+        cst = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        for L in outs:
+            awq.check(lib.awq_decode_attention_static(d_q.data_ptr(), d_k.data_ptr(), d_v.data_ptr(), cap[L].data_ptr(),
+                                                      nh, mp, L, cst))
+    for replay in range(3):
+        for L in outs:
+            cap[L].fill_(float("nan"))
+        torch.cuda.synchronize()
+        print("replay", replay, flush=True)
+        graph.replay()
+        torch.cuda.synchronize()
+        for L in outs:
+            assert torch.equal(cap[L].view(torch.int16), wants[L].view(torch.int16)), (replay, L)
