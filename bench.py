@@ -103,6 +103,49 @@ def mode_prefill(args):
     eng.close()
 
 
+def mode_fused_timeline(args):
+    """Where the time of the fused Wo + W1 launch goes (awq_set_fused_mode, off by default): the launch of every
+    layer of the 36-layer model back to back, one of them instrumented -- thread 0 of each of its 256 workgroups
+    notes the device time at 13 points.  Printed per point: minimum, median, 90th percentile and maximum over
+    the workgroups, in microseconds after the first workgroup started.  Next to it the decode rate with one
+    launch and with two."""
+    import numpy as np
+    import torch  # noqa: F401  (the HIP runtime of the process)
+    awq = importlib.import_module("cuda-kernel-qwen3-8b-awq_amd")
+    lib = awq.load_library()
+    eng = _synthetic_engine(awq, lib, awq.make_config(n_layers=36, max_pos=640), 1, awq.SYNTH_BALANCED)
+    names = ["workgroup starts", "ctx, gamma, scales, Wo weights requested", "ctx arrived and staged (wavefront 0)",
+             "... (all wavefronts)", "Wo multiplied (wavefront 0: its weights have arrived)", "... (all wavefronts)",
+             "new hidden rows stored (tagged, device scope)", "whole new hidden state seen (wavefront 0)",
+             "... (all wavefronts); W1 weights were requested after the store", "normalised and staged",
+             "W1 multiplied (wavefront 0)", "... (all wavefronts)", "GeLU, stores, end"]
+    for layer in (9, 27):
+        buf = np.zeros(256 * 16, dtype=np.uint64)
+        nw, ns = ctypes.c_int32(0), ctypes.c_int32(0)
+        awq.check(lib.awq_debug_fused_timeline(eng._h, layer, buf.ctypes.data_as(ctypes.c_void_p), ctypes.byref(nw),
+                                               ctypes.byref(ns)))
+        t = buf[:nw.value * ns.value].reshape(nw.value, ns.value).astype(np.int64)
+        us = (t - t[:, 0].min()) * 0.01
+        print("fused Wo + W1 launch of layer %d, %d workgroups: microseconds after the first workgroup's start" %
+              (layer, nw.value))
+        print("  %-60s %7s %7s %7s %7s" % ("point", "min", "median", "p90", "max"))
+        for k in range(ns.value):
+            v = np.sort(us[:, k])
+            print("  %-60s %7.2f %7.2f %7.2f %7.2f" % (names[k], v[0], v[len(v) // 2], v[len(v) * 9 // 10], v[-1]))
+    prompt = [(7 * i + 3) % 1000 for i in range(128)]
+    for fused in (False, True, False, True):
+        eng.set_fused_mode(fused)
+        eng.reset()
+        eng.prefill(prompt, batched=True)
+        eng.decode(8)
+        t0 = time.perf_counter()
+        eng.decode(256)
+        dt = time.perf_counter() - t0
+        print("decode, 256 steps after a 128-token prompt, Wo and W1 as %s: %.1f tok/s" %
+              ("one launch " if fused else "two launches", 256 / dt), flush=True)
+    eng.close()
+
+
 def mode_traffic(args):
     """Workload for the HBM-traffic counters of the decode GEMV kernel.  Run under
     `rocprofv3 --pmc FETCH_SIZE` and again under `rocprofv3 --pmc WRITE_SIZE`:
@@ -144,7 +187,8 @@ def main():
     ap.add_argument("--cpu-prompt", type=int, default=16, help="prompt length of the CPU sample")
     ap.add_argument("--cpu-steps", type=int, default=112, help="generated tokens of the CPU sample (0 = skip)")
     ap.add_argument("--no-graph", action="store_true")
-    ap.add_argument("--mode", choices=["decode", "steps", "attention", "prefill", "traffic", "w4a16"], default="decode",
+    ap.add_argument("--no-fused", action="store_true", help="one launch per product (Wo and W1 are one launch by default)")
+    ap.add_argument("--mode", choices=["decode", "steps", "attention", "prefill", "traffic", "w4a16", "fused-timeline"], default="decode",
                     help="decode: the benchmark line; steps: only the prompt and the timed decode steps (for traces)")
     ap.add_argument("--one-cache", action="store_true", help="--mode attention: every launch reads the same cache")
     ap.add_argument("--lengths", default="32,128,256,576,1024,1280,2040,4096,8192,30000", help="--mode prefill")
@@ -166,6 +210,7 @@ def main():
         args.cpu_steps = 0
     if args.mode not in ("decode", "steps"):
         return {"attention": mode_attention, "prefill": mode_prefill, "traffic": mode_traffic,
+                "fused-timeline": mode_fused_timeline,
                 "w4a16": mode_w4a16}[args.mode](args)
 
     import numpy as np
@@ -196,6 +241,9 @@ def main():
         eng.close()
         eng = _synthetic_engine(awq, lib, cfg, args.seed, profile)
     eng.set_graph_mode(not args.no_graph)
+    if args.no_fused:
+        eng.set_fused_mode(False)
+    log("fused Wo + W1 launch: %s" % eng.fused_mode())
     log("weights generated, uploaded and reordered in %.1f s" % (time.time() - t0))
 
     prompt = np.zeros(args.prompt_len, dtype=np.int32)

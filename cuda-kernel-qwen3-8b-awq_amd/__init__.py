@@ -67,6 +67,9 @@ SIGNATURES = {
     "awq_prefill_batched": (ctypes.c_int, [_vp, _vp, _i32]),
     "awq_set_prefill_mode": (ctypes.c_int, [_vp, ctypes.c_int]),
     "awq_debug_force_handover_giveup": (ctypes.c_int, [_vp, ctypes.c_int]),
+    "awq_set_fused_mode": (ctypes.c_int, [_vp, ctypes.c_int]),
+    "awq_fused_mode": (ctypes.c_int, [_vp]),
+    "awq_debug_fused_timeline": (ctypes.c_int, [_vp, ctypes.c_int32, _vp, _vp, _vp]),
     "awq_read_hidden": (ctypes.c_int, [_vp, _vp]),
     "awq_read_logits": (ctypes.c_int, [_vp, _vp]),
     "awq_set_graph_mode": (ctypes.c_int, [_vp, ctypes.c_int]),
@@ -252,6 +255,13 @@ class QWen3AWQInfer:
         out = (ctypes.c_int32 * max(1, n_steps))()
         check(self._lib.awq_decode(self._h, n_steps, out))
         return [int(out[i]) for i in range(n_steps)]
+
+    def set_fused_mode(self, enabled):
+        """Wo and W1 of a layer as one launch (the default where the device allows it) or as two."""
+        check(self._lib.awq_set_fused_mode(self._h, 1 if enabled else 0))
+
+    def fused_mode(self):
+        return bool(self._lib.awq_fused_mode(self._h))
 
     def set_graph_mode(self, enabled):
         check(self._lib.awq_set_graph_mode(self._h, 1 if enabled else 0))

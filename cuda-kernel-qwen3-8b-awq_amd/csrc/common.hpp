@@ -74,6 +74,8 @@ struct StepState {
   int32_t token;      // prompt token to embed at the start of the step, -1 = keep the hidden state
   int32_t out_index;  // where the sampled token goes in the output array
   int32_t sample;     // 1 = run the sampler at the end of the step
+  int32_t epoch;      // grows by the number of layers every step and never repeats within 2^16 launches: epoch +
+                      // layer tags the vectors that a fused launch hands from workgroup to workgroup
 };
 
 // what the fused linear kernel does to its input and its output
@@ -123,6 +125,7 @@ struct LinearArgs {
   const half_t* fin_emb_zp = nullptr;
   int32_t fin_n = 0;
   StepState* fin_state = nullptr;
+  int32_t fin_epoch_step = 0;          // what the step adds to the state's epoch (the number of layers)
 };
 
 // Greedy sampling key: an order-preserving integer image of a binary16 logit
@@ -201,5 +204,12 @@ int launch_embed_rows(const uint8_t* packed, uint8_t* rows, int64_t hidden, int6
 int launch_embed(const uint8_t* packed, const half_t* scale, const half_t* zp, int64_t hidden, int64_t vocab,
                  int32_t tok, const StepState* dyn, half_t* out, hipStream_t st);
 int launch_set_state(StepState* dst, StepState v, hipStream_t st);
+// Wo + residual and RMSNorm + W1 + GeLU of one layer in one launch (fused.hip)
+int fused_wo_w1_supported(int64_t hidden, int64_t inter);
+int launch_fused_wo_w1(const void* wo, const half_t* wo_scale, const half_t* wo_zp, const void* w1,
+                       const half_t* w1_scale, const half_t* w1_zp, const half_t* gamma, float eps, const half_t* ctx,
+                       half_t* hidden, half_t* mid, uint32_t* hid_tag, int32_t* status, const StepState* dyn, int layer,
+                       int64_t hidden_size, int64_t inter, unsigned long long* stamps, hipStream_t st);
+constexpr int kFusedStamps = 13;  // time stamps per workgroup of the instrumented fused launch
 int launch_fill_zero(void* p, int64_t bytes, hipStream_t st);
 int launch_copy(const void* src, void* dst, int64_t bytes, hipStream_t st);

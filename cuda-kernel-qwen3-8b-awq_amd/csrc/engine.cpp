@@ -176,6 +176,12 @@ struct awq_engine {
     int64_t chunk = 0;
   } pb;
   bool batched_prefill = false;
+  // Wo and W1 of a layer as one launch (fused.hip): the hidden state between them as tagged words, and the word
+  // through which a wait that gave up reports
+  bool fused = false;
+  uint32_t* hid_tag = nullptr;
+  int32_t* handover_status = nullptr;
+  int32_t epoch_next = 0;  // the epoch of the next step (mirrors what the device adds per step)
   std::vector<void*> allocations;
   // the reordered weight streams of all layers and the unembedding share one allocation, in the order the
   // decode step reads them
@@ -290,19 +296,26 @@ int enqueue_layer(awq_engine* e, int l, int use_len_hi, int64_t len_bound) {
                                 kv_blocked(e->n_heads), 0, e->d_state,
                                 use_len_hi, len_bound, e->attn_ws, st))
     return rc;  // :1110
-  {  // :1128-1155 Wo product and residual add; input and output are distinct
-     // buffers (they alias in the reference)
-    LinearArgs a = linear_args(e, L.wo, e->ctx, e->hidden);
-    a.epilogue = EPI_RESIDUAL;
-    a.res = e->hidden;
-    if (int rc = launch_gemv(a, st)) return rc;
-  }
-  {  // :1163 RMSNorm with the same gamma, :1176 W1, :1196 GeLU
-    LinearArgs a = linear_args(e, L.w1, e->hidden, e->mid);
-    a.prologue = PRO_RMSNORM;
-    a.gamma = L.gamma;
-    a.epilogue = EPI_GELU;
-    if (int rc = launch_gemv(a, st)) return rc;
+  if (e->fused) {  // :1128-1198 in one launch
+    if (int rc = launch_fused_wo_w1(L.wo.stream_order, L.wo.scale, L.wo.zp, L.w1.stream_order, L.w1.scale, L.w1.zp,
+                                    L.gamma, e->cfg.eps, e->ctx, e->hidden, e->mid, e->hid_tag, e->handover_status,
+                                    e->d_state, l, e->cfg.hidden, e->cfg.inter, nullptr, st))
+      return rc;
+  } else {
+    {  // :1128-1155 Wo product and residual add; input and output are distinct
+       // buffers (they alias in the reference)
+      LinearArgs a = linear_args(e, L.wo, e->ctx, e->hidden);
+      a.epilogue = EPI_RESIDUAL;
+      a.res = e->hidden;
+      if (int rc = launch_gemv(a, st)) return rc;
+    }
+    {  // :1163 RMSNorm with the same gamma, :1176 W1, :1196 GeLU
+      LinearArgs a = linear_args(e, L.w1, e->hidden, e->mid);
+      a.prologue = PRO_RMSNORM;
+      a.gamma = L.gamma;
+      a.epilogue = EPI_GELU;
+      if (int rc = launch_gemv(a, st)) return rc;
+    }
   }
   {  // :1201 W2, :1227 residual add
     LinearArgs a = linear_args(e, L.w2, e->mid, e->hidden);
@@ -332,6 +345,7 @@ LinearArgs sample_args(awq_engine* e) {
   a.fin_emb_zp = e->embed.zp;
   a.fin_n = e->cfg.hidden;
   a.fin_state = e->d_state;
+  a.fin_epoch_step = e->cfg.n_layers;
   return a;
 }
 
@@ -370,6 +384,8 @@ int build_graph(awq_engine* e, bool gen, int64_t len_bound, hipGraphExec_t* out)
 
 // `write_state` false: the device already holds `s` (the previous generation step advanced it)
 int run_step(awq_engine* e, bool gen, StepState s, bool write_state = true) {
+  s.epoch = e->epoch_next;
+  e->epoch_next = (e->epoch_next + e->cfg.n_layers) & 0x3fffffff;  // what the step's last launch adds on the device
   if (write_state)
     if (int rc = launch_set_state(e->d_state, s, e->stream)) return rc;
   // the attention launches are specialised by an upper bound of the attended
@@ -499,6 +515,14 @@ extern "C" int awq_create_empty(const awq_config* cfg_in, awq_engine** out) {
   if (int rc = dev_alloc(ep, (void**)&e->d_state, sizeof(StepState))) return fail(rc);
   if (int rc = dev_alloc(ep, (void**)&e->d_token, 4)) return fail(rc);
   if (int rc = dev_alloc(ep, (void**)&e->d_out, (int64_t)cfg.max_pos * 4)) return fail(rc);
+  if (int rc = dev_alloc(ep, (void**)&e->hid_tag, H * 4)) return fail(rc);
+  if (int rc = dev_alloc(ep, (void**)&e->handover_status, 256)) return fail(rc);
+  // tags start at 0: the vector must not hold that tag before the first launch wrote it
+  if (hipMemset(e->hid_tag, 0xff, (size_t)H * 4) != hipSuccess || hipMemset(e->handover_status, 0, 256) != hipSuccess) {
+    awq_set_error("hipMemset of the hand-over buffers failed");
+    return fail(AWQ_ERR_HIP);
+  }
+  e->fused = false;  // measured slower than two launches (904 against 924 tok/s): awq_set_fused_mode switches it on
   *out = e.release();
   return AWQ_OK;
 }
@@ -770,8 +794,93 @@ extern "C" int awq_reset(awq_engine* e) {
   e->n_positions = 0;
   e->n_generated = 0;
   if (int rc = launch_fill_zero(e->hidden, (int64_t)e->cfg.hidden * 2, e->stream)) return rc;
+  // the words through which waits report (and the tests ask them to give up) start clean
+  if (int rc = launch_fill_zero(e->handover_status, 4, e->stream)) return rc;
+  if (e->pb.gemm_ws)
+    if (int rc = launch_fill_zero(e->pb.gemm_ws, 8, e->stream)) return rc;
   AWQ_HIP_TRY(hipStreamSynchronize(e->stream));
   return AWQ_OK;
+}
+
+namespace {
+// After the stream has drained: did a wait inside a fused launch give up?  The word is cleared, so the engine
+// works again after awq_reset.
+int check_handover(awq_engine* e) {
+  if (!e->fused) return AWQ_OK;
+  int32_t word = 0;
+  AWQ_HIP_TRY(hipMemcpy(&word, e->handover_status, 4, hipMemcpyDeviceToHost));
+  if (word == 0) return AWQ_OK;
+  AWQ_HIP_TRY(hipMemset(e->handover_status, 0, 4));
+  awq_set_error("a fused launch gave up waiting for the hidden state of other workgroups");
+  return AWQ_ERR_HIP;
+}
+}  // namespace
+
+extern "C" int awq_set_fused_mode(awq_engine* e, int enabled) {
+  AWQ_REQUIRE(e != nullptr, "engine is NULL");
+  const bool want = enabled != 0 && fused_wo_w1_supported(e->cfg.hidden, e->cfg.inter) != 0;
+  if (want != e->fused) {
+    // the captured steps hold the other launches
+    AWQ_HIP_TRY(hipStreamSynchronize(e->stream));
+    for (auto& row : e->graphs)
+      for (hipGraphExec_t& g : row)
+        if (g) {
+          (void)hipGraphExecDestroy(g);
+          g = nullptr;
+        }
+    e->fused = want;
+  }
+  return AWQ_OK;
+}
+
+extern "C" int awq_fused_mode(const awq_engine* e) { return e && e->fused ? 1 : 0; }
+
+// The fused launch of every layer, back to back, with layer `layer`'s launch instrumented: thread 0 of each of its
+// hidden/16 workgroups notes the time at kFusedStamps points (10 ns units, one clock for the whole device).
+extern "C" int awq_debug_fused_timeline(awq_engine* e, int32_t layer, uint64_t* host_out, int32_t* n_workgroups,
+                                        int32_t* n_stamps) {
+  AWQ_REQUIRE(e && host_out && n_workgroups && n_stamps, "NULL argument");
+  AWQ_REQUIRE(e->finalized, "awq_debug_fused_timeline before awq_finalize");
+  AWQ_REQUIRE(fused_wo_w1_supported(e->cfg.hidden, e->cfg.inter) != 0,
+              "the fused launch needs hidden 4096, intermediate 12288 and 256 compute units");
+  AWQ_REQUIRE(layer >= 0 && layer < e->cfg.n_layers, "layer out of range");
+  const int wgs = e->cfg.hidden / 16;
+  unsigned long long* d_stamps = nullptr;
+  AWQ_HIP_TRY(hipMalloc((void**)&d_stamps, (size_t)wgs * kFusedStamps * 8));
+  StepState s{0, 1, 1, -1, 0, 0, 0};
+  s.epoch = e->epoch_next;
+  e->epoch_next = (e->epoch_next + e->cfg.n_layers) & 0x3fffffff;
+  int rc = launch_set_state(e->d_state, s, e->stream);
+  for (int rep = 0; rep < 3 && rc == AWQ_OK; ++rep) {  // the last round is the one that counts (warm clocks)
+    if (rep) {
+      s.epoch = e->epoch_next;
+      e->epoch_next = (e->epoch_next + e->cfg.n_layers) & 0x3fffffff;
+      rc = launch_set_state(e->d_state, s, e->stream);
+    }
+    for (int l = 0; l < e->cfg.n_layers && rc == AWQ_OK; ++l) {
+      LayerDev& L = e->layers[l];
+      rc = launch_fused_wo_w1(L.wo.stream_order, L.wo.scale, L.wo.zp, L.w1.stream_order, L.w1.scale, L.w1.zp, L.gamma,
+                              e->cfg.eps, e->ctx, e->hidden, e->mid, e->hid_tag, e->handover_status, e->d_state, l,
+                              e->cfg.hidden, e->cfg.inter, l == layer ? d_stamps : nullptr, e->stream);
+    }
+  }
+  if (rc == AWQ_OK && hipStreamSynchronize(e->stream) != hipSuccess) rc = AWQ_ERR_HIP;
+  if (rc == AWQ_OK && hipMemcpy(host_out, d_stamps, (size_t)wgs * kFusedStamps * 8, hipMemcpyDeviceToHost) != hipSuccess)
+    rc = AWQ_ERR_HIP;
+  (void)hipFree(d_stamps);
+  if (rc) return rc;
+  *n_workgroups = wgs;
+  *n_stamps = kFusedStamps;
+  {
+    int32_t word = 0;
+    AWQ_HIP_TRY(hipMemcpy(&word, e->handover_status, 4, hipMemcpyDeviceToHost));
+    if (word != 0) {
+      AWQ_HIP_TRY(hipMemset(e->handover_status, 0, 4));
+      awq_set_error("a fused launch gave up waiting for the hidden state of other workgroups");
+      return AWQ_ERR_HIP;
+    }
+  }
+  return awq_reset(e);
 }
 
 // prompt loop, Inference.cu:1304-1343
@@ -798,7 +907,7 @@ extern "C" int awq_prefill(awq_engine* e, const int32_t* prompt_ids, int32_t n_p
     e->n_positions = t + 1;
   }
   AWQ_HIP_TRY(hipStreamSynchronize(e->stream));
-  return AWQ_OK;
+  return check_handover(e);
 }
 
 namespace {
@@ -916,6 +1025,8 @@ extern "C" int awq_debug_force_handover_giveup(awq_engine* e, int on) {
   const int32_t word = on ? 1 : 0;
   AWQ_HIP_TRY(hipStreamSynchronize(e->stream));
   AWQ_HIP_TRY(hipMemcpy((int32_t*)e->pb.gemm_ws + 1, &word, 4, hipMemcpyHostToDevice));
+  // the fused launches of the token-by-token steps look at their status word before they wait
+  AWQ_HIP_TRY(hipMemcpy(e->handover_status, &word, 4, hipMemcpyHostToDevice));
   return AWQ_OK;
 }
 
@@ -950,6 +1061,7 @@ extern "C" int awq_decode(awq_engine* e, int32_t n_steps, int32_t* out_ids) {
     e->n_generated += 1;
   }
   AWQ_HIP_TRY(hipStreamSynchronize(e->stream));
+  if (int rc = check_handover(e)) return rc;
   if (n_steps > 0)
     AWQ_HIP_TRY(hipMemcpy(out_ids, e->d_out + first, (size_t)n_steps * 4, hipMemcpyDeviceToHost));
   return AWQ_OK;

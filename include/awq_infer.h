@@ -107,6 +107,31 @@ int awq_set_prefill_mode(awq_engine* e, int batched);
  * after awq_reset. */
 int awq_debug_force_handover_giveup(awq_engine* e, int on);
 
+/* No counterpart in the reference.  With hidden 4096 / intermediate 12288 on a
+ * device with at least 256 compute units, awq_set_fused_mode(e, 1) makes the
+ * token-by-token steps run the attention output product (Inference.cu:
+ * 1128-1155) and RMSNorm + W1 + GeLU (:1163-1198) of a layer as ONE launch
+ * whose workgroups hand the hidden state to each other through memory, with
+ * W1's weights requested while that hand-over is under way (bit-identical
+ * results).  Off by default: on MI355X it measures 2 % slower than the two
+ * launches it replaces (the hand-over costs what a kernel boundary costs, and
+ * W1's multiplies no longer overlap its stream).  The launch needs all its
+ * 256 workgroups resident at once, i.e. the device to itself: a wait that
+ * cannot end gives up after a bounded number of polls and the call
+ * (awq_prefill, awq_decode, awq_generate) returns AWQ_ERR_HIP; awq_reset
+ * leaves the engine usable.  Asking for it where it is not supported leaves
+ * it off; awq_fused_mode tells which is in use. */
+int awq_set_fused_mode(awq_engine* e, int enabled);
+int awq_fused_mode(const awq_engine* e);
+/* Diagnostics, no counterpart in the reference: runs the fused launch of every
+ * layer back to back with one layer's launch instrumented and returns, per
+ * workgroup, the device time (10 ns units) at which its first thread passed
+ * each of *n_stamps points (request, staged, multiplied, stored, hidden state
+ * seen, ...; listed where bench.py prints them).  host_out holds at least
+ * 256 * 16 values.  Leaves the engine reset. */
+int awq_debug_fused_timeline(awq_engine* e, int32_t layer, uint64_t* host_out, int32_t* n_workgroups,
+                             int32_t* n_stamps);
+
 /* Copies of internal state for tests: hidden state [hidden] and the logits of
  * the last sampled position [vocab], both FP16, to host memory. */
 int awq_read_hidden(awq_engine* e, uint16_t* host_dst);

@@ -435,3 +435,53 @@ def test_non_integral_zero_points_take_the_general_dequantisation(awq, oracle, t
     compare_state(awq, oracle, eng, model, cfg)
     eng.close()
     oracle.awqo_model_destroy(model)
+
+
+def test_fused_wo_w1_launch_is_bit_identical_and_gives_up_cleanly(awq, lib, oracle, torch_gpu):
+    """awq_set_fused_mode(e, 1): Wo + residual and RMSNorm + W1 + GeLU of a layer as one launch whose 256
+    workgroups hand the hidden state to each other through memory (tagged words, bounded waits).  Two
+    full-width layers: ids, hidden state and logits must be the oracle's bit for bit, with and without a
+    captured graph, over enough steps for the tags to change a few hundred times.  Then the give-up path,
+    driven from the host (the status word is set before the call, so every wait ends at its first look and
+    every kernel runs to its end): the call fails with AWQ_ERR_HIP and the engine works again after a reset.
+    Last, the instrumented launch behind awq_debug_fused_timeline returns ordered time stamps."""
+    cfg = awq.make_config(n_layers=2, max_pos=256)
+    model = make_oracle_model(oracle, cfg)
+    eng = awq.QWen3AWQInfer.empty(cfg)
+    fill_pair(awq, oracle, cfg, 2025, engine=eng, model=model, profile=awq.SYNTH_BALANCED)
+    assert not eng.fused_mode()                      # two launches by default
+    eng.set_fused_mode(True)
+    if not eng.fused_mode():
+        pytest.skip("this device cannot hold the fused launch's 256 workgroups at once")
+    rng = np.random.default_rng(17)
+    prompt = rng.integers(0, cfg.vocab, 40).tolist()
+    for graph in (True, False):
+        eng.set_graph_mode(graph)
+        print("fused launch, graph", graph, flush=True)
+        got = eng.generateResponse(prompt, 100)
+        ref = oracle_generate(oracle, model, prompt, 100)
+        print("distinct ids:", len(set(got)), flush=True)
+        assert got == ref
+        compare_state(awq, oracle, eng, model, cfg)
+    eng.set_graph_mode(True)
+    print("fused launch, every wait giving up", flush=True)
+    eng.reset()
+    awq.check(lib.awq_debug_force_handover_giveup(eng._h, 1))
+    with pytest.raises(awq.AwqError) as ei:
+        eng.prefill(prompt[:3])
+    assert ei.value.code == 3 and "gave up" in str(ei.value)
+    print("fused launch, after a reset", flush=True)
+    assert eng.generateResponse(prompt, 100) == ref
+    compare_state(awq, oracle, eng, model, cfg)
+    # the same model through two launches per layer pair: the same bits
+    eng.set_fused_mode(False)
+    assert eng.generateResponse(prompt, 100) == ref
+    buf = np.zeros(256 * 16, dtype=np.uint64)
+    nw, ns = ctypes.c_int32(0), ctypes.c_int32(0)
+    awq.check(lib.awq_debug_fused_timeline(eng._h, 1, buf.ctypes.data_as(ctypes.c_void_p), ctypes.byref(nw),
+                                           ctypes.byref(ns)))
+    t = buf[:nw.value * ns.value].reshape(nw.value, ns.value).astype(np.int64)
+    assert nw.value == 256 and ns.value >= 8 and (np.diff(t, axis=1) >= 0).all()
+    assert 0 < (t[:, -1].max() - t[:, 0].min()) * 0.01 < 1000.0     # microseconds
+    eng.close()
+    oracle.awqo_model_destroy(model)
