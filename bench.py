@@ -53,7 +53,13 @@ def mode_attention(args):
     q = torch.randn(H * 128, dtype=torch.float16, device="cuda")
     ctx = torch.empty(H * 128, dtype=torch.float16, device="cuda")
     ws = torch.zeros(lib.awq_attention_workspace_bytes(H, MP), dtype=torch.uint8, device="cuda")
-    for L in (128, 256, 512, 576, 577, 768, 1024, 1025, 1536, 2048, 2049, 4096, 8192, 16384, 40960):
+    # a 1 GiB copy first: under `rocprofv3 --pmc FETCH_SIZE` its known size calibrates the counter's unit
+    src = torch.full((1 << 28,), 1.0, dtype=torch.float32, device="cuda")
+    dst = torch.empty_like(src)
+    dst.copy_(src)
+    torch.cuda.synchronize()
+    del src, dst
+    for L in [int(v) for v in args.att_lengths.split(",")]:
         def run(i):
             awq.check(lib.awq_decode_attention(q.data_ptr(), kcs[i % NL].data_ptr(), vcs[i % NL].data_ptr(),
                                                ctx.data_ptr(), H, MP, L, ws.data_ptr(), st))
@@ -191,6 +197,8 @@ def main():
     ap.add_argument("--mode", choices=["decode", "steps", "attention", "prefill", "traffic", "w4a16", "fused-timeline"], default="decode",
                     help="decode: the benchmark line; steps: only the prompt and the timed decode steps (for traces)")
     ap.add_argument("--one-cache", action="store_true", help="--mode attention: every launch reads the same cache")
+    ap.add_argument("--att-lengths", default="128,256,512,576,577,768,1024,1025,1536,2048,2049,4096,8192,16384,40960",
+                    help="--mode attention: attended lengths")
     ap.add_argument("--lengths", default="32,128,256,576,1024,1280,2040,4096,8192,30000", help="--mode prefill")
     ap.add_argument("--tokens", default="1,4,16,64,128,512,2048", help="--mode w4a16: token counts")
     ap.add_argument("--shapes", default="w1,w2", help="--mode w4a16: of w1 (12288x4096), w2 (4096x12288), wo (4096x4096)")
