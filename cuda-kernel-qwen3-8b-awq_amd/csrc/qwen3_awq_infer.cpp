@@ -11,8 +11,9 @@ static void die_on(int rc, const char* what) {
   std::exit(1);
 }
 
-QWen3AWQInfer::QWen3AWQInfer(const std::string& weight_dir) : engine_(nullptr) {
+QWen3AWQInfer::QWen3AWQInfer(const std::string& weight_dir, PromptMode prompt_mode) : engine_(nullptr) {
   die_on(awq_create(weight_dir.c_str(), nullptr, &engine_), "QWen3AWQInfer");
+  if (prompt_mode == PromptMode::Batched) setBatchedPrefill(true);
 }
 
 QWen3AWQInfer::~QWen3AWQInfer() { awq_destroy(engine_); }
