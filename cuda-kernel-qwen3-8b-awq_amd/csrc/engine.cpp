@@ -236,9 +236,12 @@ DevLinear* find_linear(awq_engine* e, int layer, int kind) {
   return nullptr;
 }
 
-int alloc_linear(awq_engine* e, DevLinear& t, int kind) {
+// with_packed false: the file-order bytes of this tensor never rest on the device (the directory loader reorders
+// them out of a staging buffer)
+int alloc_linear(awq_engine* e, DevLinear& t, int kind, bool with_packed = true) {
   awq_tensor_dims(e->cfg, kind, &t.m, &t.k);
-  if (int rc = dev_alloc(e, (void**)&t.packed, part_bytes(e->cfg, kind, AWQ_P_PACKED))) return rc;
+  if (with_packed)
+    if (int rc = dev_alloc(e, (void**)&t.packed, part_bytes(e->cfg, kind, AWQ_P_PACKED))) return rc;
   if (int rc = dev_alloc(e, (void**)&t.scale, part_bytes(e->cfg, kind, AWQ_P_SCALE))) return rc;
   if (int rc = dev_alloc(e, (void**)&t.zp, part_bytes(e->cfg, kind, AWQ_P_ZP))) return rc;
   return AWQ_OK;
@@ -460,7 +463,16 @@ thread_local double g_last_load_seconds = 0.0;
 
 }  // namespace
 
+namespace {
+int create_engine(const awq_config* cfg_in, awq_engine** out, bool packed_on_device);
+}
 extern "C" int awq_create_empty(const awq_config* cfg_in, awq_engine** out) {
+  return create_engine(cfg_in, out, true);
+}
+namespace {
+// packed_on_device: every linear layer gets a device buffer for its file-order bytes (awq_upload fills it,
+// awq_finalize reorders it and frees it); without, only the embedding does (it is gathered from in file order)
+int create_engine(const awq_config* cfg_in, awq_engine** out, bool packed_on_device) {
   AWQ_REQUIRE(out != nullptr, "out is NULL");
   *out = nullptr;
   awq_config cfg;
@@ -490,16 +502,16 @@ extern "C" int awq_create_empty(const awq_config* cfg_in, awq_engine** out) {
   const int64_t kv_bytes = (int64_t)e->n_heads * ((cfg.max_pos + 63) / 64 * 64) * AWQ_HEAD_DIM * 2;
   for (int l = 0; l < cfg.n_layers; ++l) {
     LayerDev& L = e->layers[l];
-    if (int rc = alloc_linear(ep, L.wqkv, AWQ_T_WQKV)) return fail(rc);
-    if (int rc = alloc_linear(ep, L.wo, AWQ_T_WO)) return fail(rc);
-    if (int rc = alloc_linear(ep, L.w1, AWQ_T_W1)) return fail(rc);
-    if (int rc = alloc_linear(ep, L.w2, AWQ_T_W2)) return fail(rc);
+    if (int rc = alloc_linear(ep, L.wqkv, AWQ_T_WQKV, packed_on_device)) return fail(rc);
+    if (int rc = alloc_linear(ep, L.wo, AWQ_T_WO, packed_on_device)) return fail(rc);
+    if (int rc = alloc_linear(ep, L.w1, AWQ_T_W1, packed_on_device)) return fail(rc);
+    if (int rc = alloc_linear(ep, L.w2, AWQ_T_W2, packed_on_device)) return fail(rc);
     if (int rc = dev_alloc(ep, (void**)&L.gamma, H * 2)) return fail(rc);
     if (int rc = dev_alloc(ep, (void**)&L.kcache, kv_bytes)) return fail(rc);
     if (int rc = dev_alloc(ep, (void**)&L.vcache, kv_bytes)) return fail(rc);
   }
   if (int rc = alloc_linear(ep, e->embed, AWQ_T_EMBED)) return fail(rc);
-  if (int rc = alloc_linear(ep, e->unembed, AWQ_T_UNEMBED)) return fail(rc);
+  if (int rc = alloc_linear(ep, e->unembed, AWQ_T_UNEMBED, packed_on_device)) return fail(rc);
   const int64_t table_bytes = (int64_t)cfg.max_pos * (AWQ_HEAD_DIM / 2) * 2;
   if (int rc = dev_alloc(ep, (void**)&e->cos_t, table_bytes)) return fail(rc);
   if (int rc = dev_alloc(ep, (void**)&e->sin_t, table_bytes)) return fail(rc);
@@ -526,6 +538,7 @@ extern "C" int awq_create_empty(const awq_config* cfg_in, awq_engine** out) {
   *out = e.release();
   return AWQ_OK;
 }
+}  // namespace
 
 extern "C" int awq_upload(awq_engine* e, int layer, int kind, int part, const void* host_src, int64_t bytes) {
   AWQ_REQUIRE(e && host_src, "NULL argument");
@@ -586,16 +599,18 @@ extern "C" int awq_finalize(awq_engine* e) {
     all.push_back(&L.w2);
   }
   all.push_back(&e->unembed);
-  for (DevLinear* t : all) {
+  for (DevLinear* t : all)
     if (!t->reordered) {
       if (int rc = stream_alloc(e, &t->stream_order, t->m * (t->k / 2))) return rc;
       if (int rc = launch_repack(t->packed, t->stream_order, t->m, t->k, st)) return rc;
       t->reordered = true;
     }
-    AWQ_HIP_TRY(hipStreamSynchronize(st));
-    if (int rc = dev_free(e, t->packed)) return rc;
-    t->packed = nullptr;
-  }
+  AWQ_HIP_TRY(hipStreamSynchronize(st));
+  for (DevLinear* t : all)
+    if (t->packed) {
+      if (int rc = dev_free(e, t->packed)) return rc;
+      t->packed = nullptr;
+    }
   // rotary tables, Inference.cu:443-464
   {
     std::vector<uint16_t> c((size_t)e->cfg.max_pos * 64), s(c.size());
@@ -630,10 +645,20 @@ extern "C" int awq_create(const char* weight_dir, const awq_config* cfg_in, awq_
   // look at the directory before touching the GPU
   if (int rc = awq_validate_weight_dir(weight_dir, cfg_in)) return rc;
   awq_engine* e = nullptr;
-  if (int rc = awq_create_empty(cfg_in, &e)) return rc;
+  if (int rc = create_engine(cfg_in, &e, false)) return rc;
   const std::vector<WeightFile> files = awq_weight_files(e->cfg);
-  int64_t largest = 0;
-  for (const WeightFile& wf : files) largest = std::max(largest, wf.bytes);
+  int64_t largest = 0, largest_reordered = 0;
+  for (const WeightFile& wf : files) {
+    largest = std::max(largest, wf.bytes);
+    if (wf.part == AWQ_P_PACKED && wf.kind != AWQ_T_EMBED && wf.kind != AWQ_T_GAMMA)
+      largest_reordered = std::max(largest_reordered, wf.bytes);
+  }
+  // The file-order bytes of a linear layer pass through one of two device buffers on their way into the
+  // reordered stream: the engine's stream runs copy, reorder, copy, reorder, ... in order, so a buffer is free
+  // again when its turn comes two matrices later.  (One device buffer per matrix, freed after the last
+  // reordering, held a second copy of all weights until the end of the load.)
+  void* dstage[2] = {nullptr, nullptr};
+  int n_staged = 0;
   const auto t_begin = std::chrono::steady_clock::now();
 
   struct Slot {
@@ -648,6 +673,11 @@ extern "C" int awq_create(const char* weight_dir, const awq_config* cfg_in, awq_
   std::condition_variable cv;
   bool stop = false;
   int rc = AWQ_OK;
+  for (void*& d : dstage)
+    if (rc == AWQ_OK && hipMalloc(&d, (size_t)std::max<int64_t>(largest_reordered, 4)) != hipSuccess) {
+      awq_set_error("hipMalloc of a device staging buffer failed");
+      rc = AWQ_ERR_HIP;
+    }
   for (Slot& s : slot) {
     if (rc == AWQ_OK && hipHostMalloc(&s.host, (size_t)largest, hipHostMallocDefault) != hipSuccess) {
       awq_set_error("hipHostMalloc of a staging buffer failed");
@@ -700,6 +730,7 @@ extern "C" int awq_create(const char* weight_dir, const awq_config* cfg_in, awq_
         e->layers[wf.layer].have_gamma = true;
       } else {
         t = find_linear(e, wf.layer, wf.kind);
+        if (wf.part == AWQ_P_PACKED && wf.kind != AWQ_T_EMBED) t->packed = (uint8_t*)dstage[n_staged++ & 1];
         dst = wf.part == AWQ_P_PACKED ? (void*)t->packed : wf.part == AWQ_P_SCALE ? (void*)t->scale : (void*)t->zp;
         if (wf.part == AWQ_P_ZP) t->zp_integral = zp_all_integral((const uint16_t*)s.host, wf.bytes / 2);
         t->have[wf.part] = true;
@@ -711,7 +742,10 @@ extern "C" int awq_create(const char* weight_dir, const awq_config* cfg_in, awq_
         break;
       }
       // the embedding is only ever gathered from, so it stays in file order
-      if (t && wf.part == AWQ_P_PACKED && wf.kind != AWQ_T_EMBED) rc = reorder_now(e, t);
+      if (t && wf.part == AWQ_P_PACKED && wf.kind != AWQ_T_EMBED) {
+        rc = reorder_now(e, t);
+        t->packed = nullptr;  // the staging buffer is not the tensor's
+      }
       {
         std::lock_guard<std::mutex> lock(mu);
         s.state = 2;
@@ -753,6 +787,8 @@ extern "C" int awq_create(const char* weight_dir, const awq_config* cfg_in, awq_
     if (s.copied) (void)hipEventDestroy(s.copied);
     if (s.host) (void)hipHostFree(s.host);
   }
+  for (void* d : dstage)
+    if (d) (void)hipFree(d);
   if (rc == AWQ_OK) g_last_load_seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - t_begin).count();
   if (rc == AWQ_OK) rc = awq_finalize(e);
   if (rc) {
