@@ -342,11 +342,13 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
   // microseconds late (measured: 7.9 -> 7.45 us per launch at 12288 x 4096).
   __syncthreads();
   // With the fused norm (the model's own launches: three workgroups per compute unit) only the first block of a
-  // lane is requested here and the others behind the norm's second barrier.  A wavefront passes a barrier only
-  // once the memory pipeline has accepted all its requests, and a compute unit accepts about 37 KB before it
-  // makes the next wavefront wait: with all 96 KB of its three workgroups asked for up front, the norm of the
-  // second and third workgroup stood at its barriers until most of the stream was through (12288 x 4096:
-  // 6.67 -> 6.37 us per launch; all blocks behind the barriers: 6.53, the stream then starts late).
+  // lane is requested here and the others behind the barrier that ends the staging of x.  A wavefront passes a
+  // barrier only once the memory pipeline has accepted all its requests, and a compute unit accepts about 37 KB
+  // before it makes the next wavefront wait: with all 96 KB of its three workgroups asked for up front, the norm
+  // of the second and third workgroup stood at its barriers until most of the stream was through.  12288 x 4096,
+  // launches of this shape back to back: 6.67 us with all four blocks here, 6.37 with three of them behind the
+  // norm's second barrier, 6.20 behind the staging barrier (921 / 935 / 938 tok/s); two blocks here and two
+  // behind the staging barrier 7.0 us, nothing here 6.95 us (the stream then starts late).
   constexpr int kEarly = (PRO == PRO_RMSNORM && NWC > 0 && !MULTI && G > 1) ? 1 : G;
 #pragma unroll
   for (int b = 0; b < kEarly; ++b) w[b] = __builtin_nontemporal_load(wp + b * 16);
@@ -384,8 +386,6 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
       part[pi] = acc;
     }
     __syncthreads();
-#pragma unroll
-    for (int b = kEarly; b < G; ++b) w[b] = __builtin_nontemporal_load(wp + b * 16);
     // the tree of Inference.cu:130-135, by every wavefront for itself: lane t of a
     // row of 16 takes part[t + 16 j]; strides 128..16 are then additions in its own
     // registers and strides 8..1 exchanges within the row (a + b == b + a, so
@@ -452,6 +452,8 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
     }
   }
   __syncthreads();  // the planes, the blocks' constants and the table
+#pragma unroll
+  for (int b = kEarly; b < G; ++b) w[b] = __builtin_nontemporal_load(wp + b * 16);
   float xcb[G], xSb[G];
   if (G >= 4) {
 #pragma unroll
