@@ -20,6 +20,10 @@
 // a packed pair of binary16 values.
 #include "common.hpp"
 #include "gemv_device.hpp"
+
+#ifndef AWQ_GEMV_MFMA
+#define AWQ_GEMV_MFMA 1
+#endif
 #include <stdlib.h>
 
 #include <algorithm>
@@ -269,6 +273,8 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
   const int epi = EPI >= 0 ? EPI : epi_arg;
   const int n_waves = NWC ? NWC : p.n_waves;
   constexpr int Q = 64 / RH;  // lanes that share a row = consecutive block ranges of a wavefront
+  // 16 rows per wavefront: the lanes (q, r) are the matrix instruction's (k-group, column) as they stand
+  constexpr bool MM = RH == 16 && G <= 4 && AWQ_GEMV_MFMA;
   static_assert(RH == 16 || (RH == 8 && !PERIODIC), "half row groups are for one scale group per 16 rows");
   const int k = NWC ? NWC * Q * 32 * G : p.k;
   const int nblk = NWC ? NWC * Q * G : p.nblk;
@@ -425,10 +431,17 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
     const int unit = tid + u * nthreads;
     if (!stager) continue;
     const uint32_t h[4] = {xu[u].x, xu[u].y, xu[u].z, xu[u].w};
-    u32x4 planes;
     float c, S;
-    stage_unit8(h, planes, c, S);
-    *reinterpret_cast<u32x4*>(xs + (size_t)(unit + (unit / (4 * G))) * 16) = planes;
+    if (MM) {
+      uint32_t lo0, lo1, hi0, hi1;
+      stage_unit8_bytes(h, lo0, lo1, hi0, hi1, c, S);
+      uint32_t* blk = reinterpret_cast<uint32_t*>(xs + (size_t)(unit >> 2) * 64) + (unit & 3);
+      blk[0] = lo0, blk[4] = lo1, blk[8] = hi0, blk[12] = hi1;
+    } else {
+      u32x4 planes;
+      stage_unit8(h, planes, c, S);
+      *reinterpret_cast<u32x4*>(xs + (size_t)(unit + (unit / (4 * G))) * 16) = planes;
+    }
     if ((tid & 3) == 0) {
       xc[unit >> 2] = c;
       xS[unit >> 2] = S;
@@ -469,6 +482,17 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
   }
   // the G blocks of this lane in LDS: 64 bytes each, the lane group's skew included
   const unsigned char* xl = xs + (size_t)(blk0 * 4 + blk0 / G) * 16;
+  // on the matrix cores: this lane's share of the input operand of its wavefront's G block columns, kept in
+  // registers for all row groups of the workgroup
+  u32x4 a_lo[MM ? G : 1], a_hi[MM ? G : 1];
+  if (MM) {
+#pragma unroll
+    for (int b = 0; b < G; ++b) load_planes(xs + (size_t)(blk0 + b) * 64, lane, a_lo[b], a_hi[b]);
+  }
+  auto dot = [&](const u32x4& wv, int b) -> float {
+    if (MM) return block_dot_mfma(wv, a_lo[b], a_hi[b]);
+    return block_dot(wv, xl + 64 * b);
+  };
   unsigned long long best_here = 0;  // EPI_ARGMAX: best candidate among this lane's rows
 
   // the weights of one row group, and (one scale group per 16 rows) its scale and zero-point
@@ -508,7 +532,7 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
 #pragma unroll
       for (int b = 0; b < G; ++b) {
         const GroupConst& gb = gc[UFAST > 0 ? b / UFAST : 0];
-        bs[b] = __builtin_fmaf(gb.zn, xSb[b], block_dot(wc[b], xl + 64 * b)) * (gb.s * xcb[b]);
+        bs[b] = __builtin_fmaf(gb.zn, xSb[b], dot(wc[b], b)) * (gb.s * xcb[b]);
       }
     } else {
 #pragma unroll
@@ -520,7 +544,7 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
             cls_left = U;
           }
         }
-        bs[b] = __builtin_fmaf(g.zn, xSb[b], block_dot(wc[b], xl + 64 * b)) * (g.s * xcb[b]);
+        bs[b] = __builtin_fmaf(g.zn, xSb[b], dot(wc[b], b)) * (g.s * xcb[b]);
       }
     }
     // adjacent-pair tree: this lane's G blocks, then the four quarters of the

@@ -158,4 +158,80 @@ __device__ __forceinline__ void stage_unit8(const uint32_t h[4], u32x4& planes, 
   planes.w = __builtin_amdgcn_perm(B1, B0, 0x07030501u);
 }
 
+// ---------------------------------------------------------------------------
+// The same block products on the matrix cores.  v_mfma_i32_16x16x64_i8 multiplies a 16 x 64 byte
+// operand by a 64 x 16 one; lane (g = lane / 16, n = lane % 16) supplies 16 consecutive k-bytes (group g)
+// of row n of the first operand and of column n of the second, and receives rows 4g..4g+3 of column n.
+// A lane's four weight dwords are 16 bytes of two nibbles each, so the second operand is the weights as
+// they were loaded, once masked to the low nibbles and once to the high ones: lane (q, r) supplies k-group
+// q of column r.  The first operand carries the inputs: row 4q' + p is plane p of the block of lane group
+// q' in k-group q' and zero elsewhere, so that the sum over all 64 k-bytes picks one block, and lane (q, r)
+// receives in its own four results exactly the planes of its own block against its own row.  Planes: the
+// 16-bit integers I = lo + 256 hi, lo - 128 as a signed byte (plane 0), hi as a signed byte (plane 1), and
+// all ones (plane 2, sum q):  D = sum q I = C0 + 256 C1 + 128 C2.  Three instructions per 8 weights to
+// unpack and two matrix instructions per 64 (block, row) pairs instead of five dot products per 8 weights;
+// the integers are the same, so every result keeps its bits.
+// ---------------------------------------------------------------------------
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+
+// Byte planes of 8 consecutive block-order inputs (stage_unit8's arguments): the unit's dword of plane 0 and
+// plane 1 of the inputs under the low nibbles (lo0, lo1) and of those under the high nibbles (hi0, hi1).
+// Byte i of a weight dword holds element {0, 4, 1, 5}[i] in its low and {2, 6, 3, 7}[i] in its high nibble.
+__device__ __forceinline__ void stage_unit8_bytes(const uint32_t h[4], uint32_t& lo0, uint32_t& lo1, uint32_t& hi0,
+                                                  uint32_t& hi1, float& c, float& S) {
+  uint32_t mm = pk_max_u16(pk_max_u16(h[0] & 0x7fff7fffu, h[1] & 0x7fff7fffu),
+                           pk_max_u16(h[2] & 0x7fff7fffu, h[3] & 0x7fff7fffu));
+  mm = max(mm & 0xffffu, mm >> 16);
+  mm = max(mm, dpp_u<kDppXor1>(mm));
+  mm = max(mm, dpp_u<kDppXor2>(mm));
+  const uint32_t e = mm >> 10;
+  const uint32_t cbits = (max(e, 1u) + 98u) << 23;
+  c = __builtin_bit_cast(float, e == 31u ? 0x7fc00000u : cbits);
+  const float inv = __builtin_bit_cast(float, 0x7f000000u - cbits);
+  // x/c + 1.5 * 2^23 rounds to an integer (nearest even) whose low 16 bits are I in two's complement
+  const float magic = 12582912.0f;
+  uint32_t P[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const half2_t x2 = as_half2(h[i]);
+    const uint32_t lo = __builtin_bit_cast(uint32_t, __builtin_fmaf((float)x2.x, inv, magic));
+    const uint32_t hi = __builtin_bit_cast(uint32_t, __builtin_fmaf((float)x2.y, inv, magic));
+    P[i] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);  // I of element 2i | I of element 2i+1 << 16
+  }
+  typedef short short2_t __attribute__((ext_vector_type(2)));
+  int su = 0;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) su = __builtin_amdgcn_sdot2(__builtin_bit_cast(short2_t, P[i]), short2_t{1, 1}, su, false);
+  su += (int)dpp_u<kDppXor1>((uint32_t)su);
+  su += (int)dpp_u<kDppXor2>((uint32_t)su);
+  S = (float)su;
+  lo0 = __builtin_amdgcn_perm(P[2], P[0], 0x06020400u) ^ 0x80808080u;  // low bytes of elements 0, 4, 1, 5, less 128
+  lo1 = __builtin_amdgcn_perm(P[2], P[0], 0x07030501u);                // their high bytes
+  hi0 = __builtin_amdgcn_perm(P[3], P[1], 0x06020400u) ^ 0x80808080u;  // elements 2, 6, 3, 7
+  hi1 = __builtin_amdgcn_perm(P[3], P[1], 0x07030501u);
+}
+
+// The first operands of a lane for one block column of its wavefront: LDS holds per block 64 bytes,
+// [plane 0 | plane 1] of the inputs under the low nibbles, then the same under the high nibbles.  blocks:
+// the 64 bytes of the block of this lane's own k-group (lane / 16).
+__device__ __forceinline__ void load_planes(const unsigned char* block, int lane, u32x4& a_lo, u32x4& a_hi) {
+  const int row = lane & 15, p = row & 3;
+  const bool mine = (row >> 2) == (lane >> 4);
+  const u32x4 zero = {0u, 0u, 0u, 0u}, ones = {0x01010101u, 0x01010101u, 0x01010101u, 0x01010101u};
+  a_lo = a_hi = mine && p == 2 ? ones : zero;
+  if (mine && p < 2) {
+    a_lo = *reinterpret_cast<const u32x4*>(block + 16 * p);
+    a_hi = *reinterpret_cast<const u32x4*>(block + 32 + 16 * p);
+  }
+}
+
+// D of this lane's (block, row) as a float (exact); every lane of the wavefront must be here
+__device__ __forceinline__ float block_dot_mfma(const u32x4& w, const u32x4& a_lo, const u32x4& a_hi) {
+  const u32x4 lo = w & 0x0f0f0f0fu, hi = (w >> 4) & 0x0f0f0f0fu;
+  i32x4 acc = {0, 0, 0, 0};
+  acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, a_lo), __builtin_bit_cast(i32x4, lo), acc, 0, 0, 0);
+  acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, a_hi), __builtin_bit_cast(i32x4, hi), acc, 0, 0, 0);
+  return (float)(acc.x + (acc.y << 8) + (acc.z << 7));
+}
+
 }  // namespace
