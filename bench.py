@@ -327,11 +327,15 @@ def main():
     if os.path.exists(tpath):
         import hashlib
         rec = json.load(open(tpath))
-        src = os.path.join(ROOT, awq.__name__, "csrc", "gemv.hip")
-        if os.path.exists(src) and hashlib.sha256(open(src, "rb").read()).hexdigest() == rec.get("gemv_hip_sha256"):
+        h = hashlib.sha256()
+        for name in ("gemv.hip", "gemv_device.hpp"):  # the kernel and its device helpers
+            src = os.path.join(ROOT, awq.__name__, "csrc", name)
+            h.update(open(src, "rb").read() if os.path.exists(src) else b"missing")
+        if h.hexdigest() == rec.get("gemv_sources_sha256"):
             traffic = rec.get("hbm_bytes_per_launch")
         else:
-            log("profiles/gemv_w1_traffic.json was measured on another version of csrc/gemv.hip: traffic = null")
+            log("profiles/gemv_w1_traffic.json was measured on another version of csrc/gemv.hip, "
+                "csrc/gemv_device.hpp: traffic = null")
     w1 = kernels["w1"]
     roofline = {"bound": "hbm", "kernel": "gemv_kernel (int4 dequant + GEMV, m=12288 k=4096, GeLU epilogue)",
                 "achieved": w1["GBs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",

@@ -13,17 +13,16 @@
 // 16*rg + r; a wavefront load is four contiguous 256-byte pieces, and the G
 // loads of a lane walk 256*G contiguous bytes per quarter.  Inside the 16
 // bytes, dword c holds elements 8c..8c+7 with nibble positions
-// {0,16,4,20,8,24,12,28}[t & 7].  The decode kernel multiplies a dword as it
-// is (eight 4-bit weights against eight 4-bit digits of the inputs, laid out the
-// same way, in one v_dot8_u32_u4); the matrix-core kernels mask with 0x000f000f /
-// 0x00f000f0 (and the same after one shift by 8) to get two weights at a time as
-// a packed pair of binary16 values.
+// {0,16,4,20,8,24,12,28}[t & 7].  The decode kernel hands a lane's 16 bytes to
+// v_mfma_i32_16x16x64_i8 as they stand but for two masks (low nibbles, high
+// nibbles) against byte planes of the inputs, or, for half row groups and eight
+// blocks per lane, multiplies a dword as it is in v_dot8_u32_u4 (eight 4-bit
+// weights against eight 4-bit digits of the inputs laid out the same way); the
+// many-token kernels mask with 0x000f000f / 0x00f000f0 (and the same after one
+// shift by 8) to get two weights at a time as a packed pair of binary16 values.
 #include "common.hpp"
 #include "gemv_device.hpp"
 
-#ifndef AWQ_GEMV_MFMA
-#define AWQ_GEMV_MFMA 1
-#endif
 #include <stdlib.h>
 
 #include <algorithm>
@@ -250,7 +249,8 @@ __global__ __launch_bounds__(256) void sample_finish_kernel(SampleFinish f) {
 // compile time and divides G, so that a lane's G blocks are G/UFAST whole classes
 // whose constants it reads once per row group; 0 = look the class up per block.
 //
-// Dynamic LDS: x in block order as nibble planes, 2 bytes per input (skewed 16 bytes per lane group) | the
+// Dynamic LDS: x in block order, 2 bytes per input, as byte planes for the matrix cores (64 bytes per block)
+// or as nibble planes for the dot products (skewed 16 bytes per lane group) | the
 // blocks' powers of two, k/32 floats | the blocks' integer sums, k/32 floats | periodic matrices: group
 // constants per (pass, class) | several row groups per workgroup: the finished sums, RH floats per pass |
 // with the fused norm, x in natural order (k halves).
@@ -273,8 +273,12 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
   const int epi = EPI >= 0 ? EPI : epi_arg;
   const int n_waves = NWC ? NWC : p.n_waves;
   constexpr int Q = 64 / RH;  // lanes that share a row = consecutive block ranges of a wavefront
-  // 16 rows per wavefront: the lanes (q, r) are the matrix instruction's (k-group, column) as they stand
-  constexpr bool MM = RH == 16 && G <= 4 && AWQ_GEMV_MFMA;
+  // The block products on the matrix cores.  16 rows per wavefront: the lanes (q, r) are the matrix
+  // instruction's (k-group, column) as they stand.  Not with eight blocks per lane (the input operands of a
+  // lane's blocks stay in registers, 8 per block: that spills), nor for half row groups (a k-group then holds
+  // two lanes' blocks; with rows for both and the sum of q from a second product or from dot products it
+  // measured 6.6 against 6.4 us at 4096 x 12288).
+  constexpr bool MM = RH == 16 && G <= 4;
   static_assert(RH == 16 || (RH == 8 && !PERIODIC), "half row groups are for one scale group per 16 rows");
   const int k = NWC ? NWC * Q * 32 * G : p.k;
   const int nblk = NWC ? NWC * Q * G : p.nblk;
