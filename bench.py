@@ -488,8 +488,9 @@ def main():
         "metric": "decode tok/s @bs1, 8B-shape AWQ; int4 GEMV achieved HBM GB/s vs peak",
         "value": round(tok_s, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "int4 weights; f16 activations held as 16-bit block fixed point per 32 inputs; exact integer dot "
-                 "products; f32 per-block scaling and accumulation; f16 outputs",
+        "dtype": "int4 weights; f16 activations held as 16-bit block fixed point per 32 inputs; exact integer block "
+                 "products (int8 matrix cores on byte planes, 4-bit dot products for w2); f32 per-block scaling and "
+                 "accumulation; f16 outputs",
         "data": "synthetic (seeded random-init; nibbles uniform 0..15; %s)" % (
             "value: scale U[0.0025,0.004], zero-point 7 or 8 so that activations stay finite; value_spec_profile: the "
             "benchmark definition's scale U[0.002,0.02], zero-point 0..15, whose activations overflow FP16"
