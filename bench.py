@@ -193,7 +193,7 @@ def main():
     ap.add_argument("--cpu-prompt", type=int, default=16, help="prompt length of the CPU sample")
     ap.add_argument("--cpu-steps", type=int, default=112, help="generated tokens of the CPU sample (0 = skip)")
     ap.add_argument("--no-graph", action="store_true")
-    ap.add_argument("--no-fused", action="store_true", help="one launch per product (Wo and W1 are one launch by default)")
+    ap.add_argument("--no-fused", action="store_true", help="kept for old command lines: one launch per product is the default")
     ap.add_argument("--mode", choices=["decode", "steps", "attention", "prefill", "traffic", "w4a16", "fused-timeline"], default="decode",
                     help="decode: the benchmark line; steps: only the prompt and the timed decode steps (for traces)")
     ap.add_argument("--one-cache", action="store_true", help="--mode attention: every launch reads the same cache")
