@@ -152,6 +152,50 @@ def mode_fused_timeline(args):
     eng.close()
 
 
+def mode_qkv_timeline(args):
+    """Where the time of the fused Wqkv + attention launch goes: the launch of every layer of the 36-layer model
+    back to back, one of them instrumented -- thread 0 of each of its 256 workgroups notes the device time at 11
+    points.  Printed per point: minimum, median, 90th percentile and maximum over the workgroups, in
+    microseconds after the first workgroup started.  Next to it the decode rate with one launch and with two."""
+    import numpy as np
+    import torch  # noqa: F401  (the HIP runtime of the process)
+    awq = importlib.import_module("cuda-kernel-qwen3-8b-awq_amd")
+    lib = awq.load_library()
+    eng = _synthetic_engine(awq, lib, awq.make_config(n_layers=36, max_pos=768), 1, awq.SYNTH_BALANCED)
+    names = ["workgroup starts", "x, gamma, state, scales, Q weights requested", "x normalised and staged (wavefront 0)",
+             "... (all wavefronts); K and V weights and the cache rows requested now",
+             "Q, K, V multiplied (wavefront 0: its weights have arrived)", "... (all wavefronts)",
+             "this workgroup's Q, K, V rotated and stored", "... and in LDS for all wavefronts",
+             "wavefront 0 past the partial scores (the streaming wavefronts publish theirs about now)",
+             "all partial scores of the head seen, scores finished", "softmax, context of 16 dimensions, end"]
+    for pos in (200, 600):
+        for layer in (9, 27):
+            buf = np.zeros(256 * 16, dtype=np.uint64)
+            nw, ns = ctypes.c_int32(0), ctypes.c_int32(0)
+            awq.check(lib.awq_debug_qkv_attention_timeline(eng._h, layer, pos, buf.ctypes.data_as(ctypes.c_void_p),
+                                                           ctypes.byref(nw), ctypes.byref(ns)))
+            t = buf[:nw.value * ns.value].reshape(nw.value, ns.value).astype(np.int64)
+            us = (t - t[:, 0].min()) * 0.01
+            print("fused Wqkv + attention launch of layer %d at position %d, %d workgroups: microseconds after the first "
+                  "workgroup's start" % (layer, pos, nw.value))
+            print("  %-72s %7s %7s %7s %7s" % ("point", "min", "median", "p90", "max"))
+            for k in range(ns.value):
+                v = np.sort(us[:, k])
+                print("  %-72s %7.2f %7.2f %7.2f %7.2f" % (names[k], v[0], v[len(v) // 2], v[len(v) * 9 // 10], v[-1]))
+    prompt = [(7 * i + 3) % 1000 for i in range(128)]
+    for fused in (0, 2, 0, 2):
+        eng.set_fused_mode(fused)
+        eng.reset()
+        eng.prefill(prompt, batched=True)
+        eng.decode(8)
+        t0 = time.perf_counter()
+        eng.decode(256)
+        dt = time.perf_counter() - t0
+        print("decode, 256 steps after a 128-token prompt, Wqkv and attention as %s: %.1f tok/s" %
+              ("one launch " if fused else "two launches", 256 / dt), flush=True)
+    eng.close()
+
+
 def mode_traffic(args):
     """Workload for the HBM-traffic counters of the decode GEMV kernel.  Run under
     `rocprofv3 --pmc FETCH_SIZE` and again under `rocprofv3 --pmc WRITE_SIZE`:
@@ -193,8 +237,10 @@ def main():
     ap.add_argument("--cpu-prompt", type=int, default=16, help="prompt length of the CPU sample")
     ap.add_argument("--cpu-steps", type=int, default=112, help="generated tokens of the CPU sample (0 = skip)")
     ap.add_argument("--no-graph", action="store_true")
-    ap.add_argument("--no-fused", action="store_true", help="kept for old command lines: one launch per product is the default")
-    ap.add_argument("--mode", choices=["decode", "steps", "attention", "prefill", "traffic", "w4a16", "fused-timeline"], default="decode",
+    ap.add_argument("--no-fused", action="store_true", help="one launch per product: no pair of a layer's launches runs as one")
+    ap.add_argument("--fused", type=int, default=None,
+                    help="which pairs of a layer's launches run as one: 1 Wo + W1, 2 Wqkv + attention, 3 both (default: the engine's)")
+    ap.add_argument("--mode", choices=["decode", "steps", "attention", "prefill", "traffic", "w4a16", "fused-timeline", "qkv-timeline"], default="decode",
                     help="decode: the benchmark line; steps: only the prompt and the timed decode steps (for traces)")
     ap.add_argument("--one-cache", action="store_true", help="--mode attention: every launch reads the same cache")
     ap.add_argument("--att-lengths", default="128,256,512,576,577,768,1024,1025,1536,2048,2049,4096,8192,16384,40960",
@@ -218,7 +264,7 @@ def main():
         args.cpu_steps = 0
     if args.mode not in ("decode", "steps"):
         return {"attention": mode_attention, "prefill": mode_prefill, "traffic": mode_traffic,
-                "fused-timeline": mode_fused_timeline,
+                "fused-timeline": mode_fused_timeline, "qkv-timeline": mode_qkv_timeline,
                 "w4a16": mode_w4a16}[args.mode](args)
 
     import numpy as np
@@ -250,8 +296,10 @@ def main():
         eng = _synthetic_engine(awq, lib, cfg, args.seed, profile)
     eng.set_graph_mode(not args.no_graph)
     if args.no_fused:
-        eng.set_fused_mode(False)
-    log("fused Wo + W1 launch: %s" % eng.fused_mode())
+        eng.set_fused_mode(0)
+    elif args.fused is not None:
+        eng.set_fused_mode(args.fused)
+    log("fused launches (1 Wo + W1, 2 Wqkv + attention): %d" % eng.fused_mode())
     log("weights generated, uploaded and reordered in %.1f s" % (time.time() - t0))
 
     prompt = np.zeros(args.prompt_len, dtype=np.int32)

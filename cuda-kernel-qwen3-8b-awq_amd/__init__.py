@@ -67,9 +67,15 @@ SIGNATURES = {
     "awq_prefill_batched": (ctypes.c_int, [_vp, _vp, _i32]),
     "awq_set_prefill_mode": (ctypes.c_int, [_vp, ctypes.c_int]),
     "awq_debug_force_handover_giveup": (ctypes.c_int, [_vp, ctypes.c_int]),
+    "awq_qkv_attention_workspace_bytes": (_i64, [ctypes.c_int32]),
+    "awq_qkv_attention_supported": (ctypes.c_int, [_i64, ctypes.c_int32, _vp]),
+    "awq_qkv_attention": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, ctypes.c_float, _vp, _vp, _vp, _vp, _i64, ctypes.c_int32,
+                                         _i64, _i64, _vp, _vp, _vp, ctypes.c_int32, _vp]),
+    "awq_qkv_attention_status": (ctypes.c_int, [_vp, _vp]),
     "awq_set_fused_mode": (ctypes.c_int, [_vp, ctypes.c_int]),
     "awq_fused_mode": (ctypes.c_int, [_vp]),
     "awq_debug_fused_timeline": (ctypes.c_int, [_vp, ctypes.c_int32, _vp, _vp, _vp]),
+    "awq_debug_qkv_attention_timeline": (ctypes.c_int, [_vp, ctypes.c_int32, ctypes.c_int32, _vp, _vp, _vp]),
     "awq_read_hidden": (ctypes.c_int, [_vp, _vp]),
     "awq_read_logits": (ctypes.c_int, [_vp, _vp]),
     "awq_set_graph_mode": (ctypes.c_int, [_vp, ctypes.c_int]),
@@ -256,12 +262,16 @@ class QWen3AWQInfer:
         check(self._lib.awq_decode(self._h, n_steps, out))
         return [int(out[i]) for i in range(n_steps)]
 
-    def set_fused_mode(self, enabled):
-        """Wo and W1 of a layer as one launch (the default where the device allows it) or as two."""
-        check(self._lib.awq_set_fused_mode(self._h, 1 if enabled else 0))
+    FUSED_WO_W1 = 1      # Wo + residual and RMSNorm + W1 + GeLU of a layer as one launch
+    FUSED_QKV_ATTN = 2   # RMSNorm + Wqkv + rotary + KV append and the attention of a layer as one launch
+
+    def set_fused_mode(self, mode):
+        """Which pairs of a layer's launches run as one (a sum of FUSED_*; True means FUSED_WO_W1, False or 0
+        none).  A pair the device cannot run fused stays two launches: fused_mode() tells what is on."""
+        check(self._lib.awq_set_fused_mode(self._h, int(mode)))
 
     def fused_mode(self):
-        return bool(self._lib.awq_fused_mode(self._h))
+        return int(self._lib.awq_fused_mode(self._h))
 
     def set_graph_mode(self, enabled):
         check(self._lib.awq_set_graph_mode(self._h, 1 if enabled else 0))

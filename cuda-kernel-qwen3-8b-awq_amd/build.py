@@ -15,7 +15,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libawq_infer.so")
 CLI = os.path.join(HERE, "qwen3_awq_infer")
 
-HIP_SOURCES = ["gemv.hip", "gemm.hip", "ops.hip", "prefill.hip", "attention.hip", "fused.hip", "engine.cpp", "synth.cpp"]
+HIP_SOURCES = ["gemv.hip", "gemm.hip", "ops.hip", "prefill.hip", "attention.hip", "fused.hip", "qkv_attn.hip", "engine.cpp", "synth.cpp"]
 
 # -ffp-contract=off: every fma in the sources is written out; a contracted
 #   a*b-c*d would break bit parity with the reference's __hmul/__hsub sequence.

@@ -211,5 +211,14 @@ int launch_fused_wo_w1(const void* wo, const half_t* wo_scale, const half_t* wo_
                        half_t* hidden, half_t* mid, uint32_t* hid_tag, int32_t* status, const StepState* dyn, int layer,
                        int64_t hidden_size, int64_t inter, unsigned long long* stamps, hipStream_t st);
 constexpr int kFusedStamps = 13;  // time stamps per workgroup of the instrumented fused launch
+// RMSNorm + Wqkv + rotary + KV append and the attention of one layer in one launch (qkv_attn.hip), for attended
+// lengths up to kAttnOneWorkgroupMax
+int fused_qkv_attn_supported(int64_t hidden, int n_heads, hipStream_t st);
+int64_t fused_qkv_attn_exchange_bytes(int n_heads);
+int launch_fused_qkv_attn(const void* wq, const half_t* scale, const half_t* zp, int64_t m, const half_t* x,
+                          const half_t* gamma, float eps, const half_t* cos_t, const half_t* sin_t, half_t* k_cache,
+                          half_t* v_cache, KvLayout kv, half_t* q_out, half_t* ctx, uint32_t* score_tag, int32_t* status, const StepState* dyn, int layer,
+                          int use_len_hi, int n_heads, unsigned long long* stamps, hipStream_t st);
+constexpr int kQkvStamps = 11;  // time stamps per workgroup of the instrumented launch
 int launch_fill_zero(void* p, int64_t bytes, hipStream_t st);
 int launch_copy(const void* src, void* dst, int64_t bytes, hipStream_t st);

@@ -180,6 +180,10 @@ struct awq_engine {
   // through which a wait that gave up reports
   bool fused = false;
   uint32_t* hid_tag = nullptr;
+  // Wqkv and the attention of a layer as one launch (qkv_attn.hip): the partial scores as tagged words, handed
+  // between the eight workgroups of a head
+  bool fused_qkv = false;
+  uint32_t* score_tag = nullptr;
   int32_t* handover_status = nullptr;
   int32_t epoch_next = 0;  // the epoch of the next step (mirrors what the device adds per step)
   std::vector<void*> allocations;
@@ -294,11 +298,19 @@ int enqueue_wqkv(awq_engine* e, int l) {
 int enqueue_layer(awq_engine* e, int l, int use_len_hi, int64_t len_bound) {
   LayerDev& L = e->layers[l];
   hipStream_t st = e->stream;
-  if (int rc = enqueue_wqkv(e, l)) return rc;
-  if (int rc = launch_attention(e->q, L.kcache, L.vcache, e->ctx, e->n_heads, e->cfg.max_pos,
-                                kv_blocked(e->n_heads), 0, e->d_state,
-                                use_len_hi, len_bound, e->attn_ws, st))
-    return rc;  // :1110
+  if (e->fused_qkv && len_bound <= kAttnOneWorkgroupMax) {  // :1040-1110 in one launch
+    if (int rc = launch_fused_qkv_attn(L.wqkv.stream_order, L.wqkv.scale, L.wqkv.zp, L.wqkv.m, e->hidden, L.gamma,
+                                       e->cfg.eps, e->cos_t, e->sin_t, L.kcache, L.vcache, kv_blocked(e->n_heads),
+                                       e->q, e->ctx, e->score_tag, e->handover_status, e->d_state, l,
+                                       use_len_hi, e->n_heads, nullptr, st))
+      return rc;
+  } else {
+    if (int rc = enqueue_wqkv(e, l)) return rc;
+    if (int rc = launch_attention(e->q, L.kcache, L.vcache, e->ctx, e->n_heads, e->cfg.max_pos,
+                                  kv_blocked(e->n_heads), 0, e->d_state,
+                                  use_len_hi, len_bound, e->attn_ws, st))
+      return rc;  // :1110
+  }
   if (e->fused) {  // :1128-1198 in one launch
     if (int rc = launch_fused_wo_w1(L.wo.stream_order, L.wo.scale, L.wo.zp, L.w1.stream_order, L.w1.scale, L.w1.zp,
                                     L.gamma, e->cfg.eps, e->ctx, e->hidden, e->mid, e->hid_tag, e->handover_status,
@@ -529,8 +541,12 @@ int create_engine(const awq_config* cfg_in, awq_engine** out, bool packed_on_dev
   if (int rc = dev_alloc(ep, (void**)&e->d_out, (int64_t)cfg.max_pos * 4)) return fail(rc);
   if (int rc = dev_alloc(ep, (void**)&e->hid_tag, H * 4)) return fail(rc);
   if (int rc = dev_alloc(ep, (void**)&e->handover_status, 256)) return fail(rc);
-  // tags start at 0: the vector must not hold that tag before the first launch wrote it
-  if (hipMemset(e->hid_tag, 0xff, (size_t)H * 4) != hipSuccess || hipMemset(e->handover_status, 0, 256) != hipSuccess) {
+  const int64_t xch_bytes = fused_qkv_attn_exchange_bytes(e->n_heads);
+  if (int rc = dev_alloc(ep, (void**)&e->score_tag, xch_bytes)) return fail(rc);
+  // tags start at 0 (Wo + W1) resp. never are 0 (Wqkv + attention): the vectors must not hold a launch's tag
+  // before the launch wrote it
+  if (hipMemset(e->hid_tag, 0xff, (size_t)H * 4) != hipSuccess || hipMemset(e->handover_status, 0, 256) != hipSuccess ||
+      hipMemset(e->score_tag, 0, (size_t)xch_bytes) != hipSuccess) {
     awq_set_error("hipMemset of the hand-over buffers failed");
     return fail(AWQ_ERR_HIP);
   }
@@ -832,6 +848,9 @@ extern "C" int awq_reset(awq_engine* e) {
   if (int rc = launch_fill_zero(e->hidden, (int64_t)e->cfg.hidden * 2, e->stream)) return rc;
   // the words through which waits report (and the tests ask them to give up) start clean
   if (int rc = launch_fill_zero(e->handover_status, 4, e->stream)) return rc;
+  // scores of an earlier sequence must not meet their tag again
+  if (e->fused_qkv)
+    if (int rc = launch_fill_zero(e->score_tag, fused_qkv_attn_exchange_bytes(e->n_heads), e->stream)) return rc;
   if (e->pb.gemm_ws)
     if (int rc = launch_fill_zero(e->pb.gemm_ws, 8, e->stream)) return rc;
   AWQ_HIP_TRY(hipStreamSynchronize(e->stream));
@@ -842,20 +861,23 @@ namespace {
 // After the stream has drained: did a wait inside a fused launch give up?  The word is cleared, so the engine
 // works again after awq_reset.
 int check_handover(awq_engine* e) {
-  if (!e->fused) return AWQ_OK;
+  if (!e->fused && !e->fused_qkv) return AWQ_OK;
   int32_t word = 0;
   AWQ_HIP_TRY(hipMemcpy(&word, e->handover_status, 4, hipMemcpyDeviceToHost));
   if (word == 0) return AWQ_OK;
   AWQ_HIP_TRY(hipMemset(e->handover_status, 0, 4));
-  awq_set_error("a fused launch gave up waiting for the hidden state of other workgroups");
+  awq_set_error("a fused launch gave up waiting for what other workgroups hand over");
   return AWQ_ERR_HIP;
 }
 }  // namespace
 
 extern "C" int awq_set_fused_mode(awq_engine* e, int enabled) {
   AWQ_REQUIRE(e != nullptr, "engine is NULL");
-  const bool want = enabled != 0 && fused_wo_w1_supported(e->cfg.hidden, e->cfg.inter) != 0;
-  if (want != e->fused) {
+  // bit 0: Wo + W1 as one launch; bit 1: Wqkv + attention as one launch; each only where the device can run it
+  const bool want = (enabled & 1) != 0 && fused_wo_w1_supported(e->cfg.hidden, e->cfg.inter) != 0;
+  const bool want_qkv = (enabled & 2) != 0 && e->cfg.hidden / AWQ_HEAD_DIM == e->n_heads &&
+                        fused_qkv_attn_supported(e->cfg.hidden, e->n_heads, e->stream) != 0;
+  if (want != e->fused || want_qkv != e->fused_qkv) {
     // the captured steps hold the other launches
     AWQ_HIP_TRY(hipStreamSynchronize(e->stream));
     for (auto& row : e->graphs)
@@ -865,11 +887,12 @@ extern "C" int awq_set_fused_mode(awq_engine* e, int enabled) {
           g = nullptr;
         }
     e->fused = want;
+    e->fused_qkv = want_qkv;
   }
   return AWQ_OK;
 }
 
-extern "C" int awq_fused_mode(const awq_engine* e) { return e && e->fused ? 1 : 0; }
+extern "C" int awq_fused_mode(const awq_engine* e) { return e ? (e->fused ? 1 : 0) | (e->fused_qkv ? 2 : 0) : 0; }
 
 // The fused launch of every layer, back to back, with layer `layer`'s launch instrumented: thread 0 of each of its
 // hidden/16 workgroups notes the time at kFusedStamps points (10 ns units, one clock for the whole device).
@@ -1053,6 +1076,51 @@ extern "C" int awq_prefill_batched(awq_engine* e, const int32_t* prompt_ids, int
     e->n_positions = (int)(pos0 + M);
   }
   return AWQ_OK;
+}
+
+// The same for the fused Wqkv + attention launch (kQkvStamps points), position `pos` attending pos + 1 positions.
+extern "C" int awq_debug_qkv_attention_timeline(awq_engine* e, int32_t layer, int32_t pos, uint64_t* host_out,
+                                                int32_t* n_workgroups, int32_t* n_stamps) {
+  AWQ_REQUIRE(e && host_out && n_workgroups && n_stamps, "NULL argument");
+  AWQ_REQUIRE(e->finalized, "awq_debug_qkv_attention_timeline before awq_finalize");
+  AWQ_REQUIRE(fused_qkv_attn_supported(e->cfg.hidden, e->n_heads, e->stream) != 0,
+              "the fused launch needs hidden 4096, 32 heads and 256 compute units");
+  AWQ_REQUIRE(layer >= 0 && layer < e->cfg.n_layers, "layer out of range");
+  AWQ_REQUIRE(pos >= 0 && pos < e->cfg.max_pos && pos + 1 <= kAttnOneWorkgroupMax, "pos out of range");
+  const int wgs = e->n_heads * 8;
+  unsigned long long* d_stamps = nullptr;
+  AWQ_HIP_TRY(hipMalloc((void**)&d_stamps, (size_t)wgs * kQkvStamps * 8));
+  StepState s{pos, pos + 1, pos + 1, -1, 0, 0, 0};
+  int rc = launch_fill_zero(e->score_tag, fused_qkv_attn_exchange_bytes(e->n_heads), e->stream);
+  for (int rep = 0; rep < 3 && rc == AWQ_OK; ++rep) {  // the last round is the one that counts (warm clocks)
+    s.epoch = e->epoch_next;
+    e->epoch_next = (e->epoch_next + e->cfg.n_layers) & 0x3fffffff;
+    rc = launch_set_state(e->d_state, s, e->stream);
+    for (int l = 0; l < e->cfg.n_layers && rc == AWQ_OK; ++l) {
+      LayerDev& L = e->layers[l];
+      rc = launch_fused_qkv_attn(L.wqkv.stream_order, L.wqkv.scale, L.wqkv.zp, L.wqkv.m, e->hidden, L.gamma, e->cfg.eps,
+                                 e->cos_t, e->sin_t, L.kcache, L.vcache, kv_blocked(e->n_heads), e->q, e->ctx,
+                                 e->score_tag, e->handover_status, e->d_state, l, 1, e->n_heads,
+                                 l == layer ? d_stamps : nullptr, e->stream);
+    }
+  }
+  if (rc == AWQ_OK && hipStreamSynchronize(e->stream) != hipSuccess) rc = AWQ_ERR_HIP;
+  if (rc == AWQ_OK && hipMemcpy(host_out, d_stamps, (size_t)wgs * kQkvStamps * 8, hipMemcpyDeviceToHost) != hipSuccess)
+    rc = AWQ_ERR_HIP;
+  (void)hipFree(d_stamps);
+  if (rc) return rc;
+  *n_workgroups = wgs;
+  *n_stamps = kQkvStamps;
+  {
+    int32_t word = 0;
+    AWQ_HIP_TRY(hipMemcpy(&word, e->handover_status, 4, hipMemcpyDeviceToHost));
+    if (word != 0) {
+      AWQ_HIP_TRY(hipMemset(e->handover_status, 0, 4));
+      awq_set_error("a fused launch gave up waiting for what other workgroups hand over");
+      return AWQ_ERR_HIP;
+    }
+  }
+  return awq_reset(e);
 }
 
 extern "C" int awq_debug_force_handover_giveup(awq_engine* e, int on) {
@@ -1289,6 +1357,58 @@ extern "C" int awq_gemv_fused(const awq_linear_args* u, void* stream) {
   a.kv = kv_head_major(u->max_pos);
   a.out_token = (int32_t*)u->out_token;
   return launch_gemv(a, (hipStream_t)stream);
+}
+
+// workspace of awq_qkv_attention: the step state the launch reads, the status word, then the exchange buffers
+namespace {
+constexpr int64_t kQkvWsHeader = 256;  // StepState at 0, status word at 128
+}
+extern "C" int64_t awq_qkv_attention_workspace_bytes(int32_t n_heads) {
+  if (n_heads <= 0) return -1;
+  return kQkvWsHeader + fused_qkv_attn_exchange_bytes(n_heads);
+}
+
+extern "C" int awq_qkv_attention_supported(int64_t hidden, int32_t n_heads, void* stream) {
+  return fused_qkv_attn_supported(hidden, n_heads, (hipStream_t)stream);
+}
+
+extern "C" int awq_qkv_attention(const void* wqkv_repacked, const void* scale, const void* zp, const void* x,
+                                 const void* gamma, float eps, const void* cos_t, const void* sin_t, void* k_cache,
+                                 void* v_cache, int64_t max_pos, int32_t n_heads, int64_t pos, int64_t L, void* q_out,
+                                 void* ctx, void* workspace, int32_t call_tag, void* stream) {
+  AWQ_REQUIRE(workspace != nullptr, "workspace is NULL");
+  AWQ_REQUIRE(n_heads == 32, "the fused launch is built for 32 heads of 128");
+  AWQ_REQUIRE(max_pos > 0 && pos >= 0 && pos < max_pos, "pos out of range");
+  AWQ_REQUIRE(L >= 0 && L <= pos + 1 && L <= kAttnOneWorkgroupMax, "attended length out of range for the fused launch");
+  AWQ_REQUIRE(call_tag >= 1 && call_tag < (1 << 30), "call_tag must be in [1, 2^30)");
+  hipStream_t st = (hipStream_t)stream;
+  char* ws = (char*)workspace;
+  StepState s{};
+  s.pos = (int32_t)pos;
+  s.len_lo = s.len_hi = (int32_t)L;
+  s.token = -1;
+  s.epoch = call_tag;
+  if (int rc = launch_set_state((StepState*)ws, s, st)) return rc;
+  const int64_t hidden = (int64_t)n_heads * AWQ_HEAD_DIM;
+  uint32_t* score_tag = (uint32_t*)(ws + kQkvWsHeader);
+  // the words of an earlier call must not meet their tag again
+  if (int rc = launch_fill_zero(score_tag, fused_qkv_attn_exchange_bytes(n_heads), st)) return rc;
+  return launch_fused_qkv_attn(wqkv_repacked, (const half_t*)scale, (const half_t*)zp, 3 * hidden, (const half_t*)x,
+                               (const half_t*)gamma, eps, (const half_t*)cos_t, (const half_t*)sin_t, (half_t*)k_cache,
+                               (half_t*)v_cache, kv_head_major(max_pos), (half_t*)q_out, (half_t*)ctx, score_tag,
+                               (int32_t*)(ws + 128), (const StepState*)ws, 0, 0, n_heads, nullptr, st);
+}
+
+// after the stream has drained: 0, or AWQ_ERR_HIP when a wait of the last launches gave up (the word is cleared)
+extern "C" int awq_qkv_attention_status(void* workspace, void* stream) {
+  AWQ_REQUIRE(workspace != nullptr, "workspace is NULL");
+  AWQ_HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+  int32_t word = 0;
+  AWQ_HIP_TRY(hipMemcpy(&word, (char*)workspace + 128, 4, hipMemcpyDeviceToHost));
+  if (word == 0) return AWQ_OK;
+  AWQ_HIP_TRY(hipMemset((char*)workspace + 128, 0, 4));
+  awq_set_error("a fused launch gave up waiting for what other workgroups hand over");
+  return AWQ_ERR_HIP;
 }
 
 extern "C" int awq_gemv(const void* repacked, const void* scale, const void* zp, int64_t m, int64_t k, const void* x,

@@ -1,0 +1,579 @@
+// The first two launches of a decoder layer as ONE: RMSNorm + Wqkv + rotary + KV append (Inference.cu:1040-1103)
+// and the attention over the cache (Inference.cu:1110, attentionKernel :182-267), for attended lengths that the
+// one-launch attention covers (kAttnOneWorkgroupMax).
+//
+// Of all the boundaries between a layer's launches this is the one across which the data dependence is local:
+// the attention of head h needs rows 128 h .. 128 h + 127 of Q and of K and nothing else of the product.  A
+// head is given to eight workgroups ON ONE DIE -- workgroups are handed to the eight dies in turn, so those
+// whose indices agree modulo 8 share a die and its L2 -- and what they owe each other travels through that L2:
+// nontemporal stores and loads go past the compute unit's own cache and meet in the L2, a quarter of a
+// microsecond from store to load where a kernel boundary costs 1.6 us and the first loads behind it a memory
+// round trip more.  One hand-over per launch:
+//   every workgroup computes 16 of the head's 128 dimensions of Q, K and V (three 16-row groups of the product,
+//   x normalised and staged once for all three), rotates its Q and K and appends K and V to the cache.  With its
+//   16 dimensions of Q it forms, for every attended position, the sum over its 16 dimensions of the score's dot
+//   product -- two chains of eight and their sum, which is exactly one node of the dot product's adjacent-pair
+//   tree -- and publishes these partial scores as tagged words (the halves of the binary32 pattern next to a
+//   16-bit tag: only a 4-byte word is seen whole by a load that races with the store -- an 8-byte (score, tag)
+//   pair was observed with the new tag next to the old score).  All eight workgroups read all eight partial
+//   scores of every position, finish the tree, and normalise for themselves (the same instructions on the same
+//   data: the same bits); each forms the context of its own 16 dimensions, for which it needs only its own V.
+//   (A first version handed Q and K round first and the finished scores of an eighth of the positions second:
+//   two hand-overs, 0.5 and 0.75 us.)
+// The keys and values a workgroup needs from the cache (its 16 dimensions of every attended position, 32 bytes
+// per row) are requested right behind its weights.  The new position's key and value come from the workgroup's
+// own product, not from the cache rows just written.
+//
+// Every wait is bounded and looks at the status word the other fused launch uses: a workgroup that gives up
+// sets it and stores no context, the others follow, the launch ends, and the host finds the word after the
+// step.  A tag that never arrives (a stale line in another die's L2, were workgroups ever placed otherwise)
+// therefore ends in an error, never in a wrong token.
+//
+// Arithmetic: the product is gemv_kernel's (awq_canon_math.h: block fixed point, canonical tree -- the same
+// tree for 16 wavefronts of two blocks per lane as for 8 of four), the attention is attention_kernel's (dot
+// products as 16 lanes x 8 fma chains and an adjacent-pair tree, chunks of 64 positions, four interleaved
+// chains per chunk and dimension, chunk results added in order), so the bits are those of the two launches.
+#include "common.hpp"
+#include "gemv_device.hpp"
+
+namespace {
+
+constexpr int kWaves = 16;
+constexpr int kThreads = kWaves * 64;
+constexpr int kK = 4096;            // inputs of the product
+constexpr int kBlocks = kK / 32;    // 128 blocks of 32 inputs
+constexpr int kG = 2;               // blocks per lane and row group
+constexpr int kParts = 8;           // workgroups per head
+constexpr int kDP = AWQ_HEAD_DIM / kParts;  // dimensions per workgroup: one 16-row group each of Q, K and V
+constexpr int kMaxLen = (int)kAttnOneWorkgroupMax;
+constexpr int kChunkCap = 16;       // chunks of 64 positions: one per wavefront
+constexpr int kScoreStride = kChunkCap * 64;  // (score, tag) pairs per head in the exchange buffer
+static_assert(kDP == 16 && kMaxLen <= kChunkCap * 64 && kMaxLen <= kScoreStride, "shape of the fused launch");
+// Wavefront 0 finishes the product (rotary, stores); the other kAttnWaves stream the cache: what queues behind
+// bulk requests in the compute unit's memory pipeline waits for them.
+constexpr int kAttnWave0 = 1;
+constexpr int kAttnWaves = kWaves - kAttnWave0;
+static_assert((kMaxLen + 63) / 64 <= kAttnWaves, "one chunk of keys and values per wavefront");
+
+struct QkvAttnArgs {
+  const u32x4* wq;
+  const half_t* scale;
+  const half_t* zp;
+  const half_t* x;        // [4096] hidden state
+  const half_t* gamma;
+  const half_t* cos_t;
+  const half_t* sin_t;
+  half_t* k_cache;
+  half_t* v_cache;
+  half_t* q_out;          // [4096] rotated Q, as the separate launch leaves it
+  half_t* ctx;            // [4096] attention output
+  uint32_t* score_tag;    // [heads][8 workgroups][kScoreStride][2] the halves of a partial score as (half | tag << 16)
+  int32_t* status;        // [0] != 0: a wait gave up (or the host asks every wait to)
+  const StepState* dyn;
+  KvLayout kv;
+  int32_t layer;
+  int32_t use_len_hi;
+  int32_t spin_limit;
+  int32_t mg;             // m / 128 of the matrix
+  float eps;
+  unsigned long long* stamps;  // STAMPS: [workgroup][kQkvStamps] times of thread 0, 10 ns units
+};
+
+typedef _Float16 half8v_t __attribute__((ext_vector_type(8)));
+
+// 16 bytes past the compute unit's cache, complete on return (the wait also covers every load the wavefront
+// issued before: they return in order)
+__device__ __forceinline__ u32x4 load_l2_16(const void* p) {
+  u32x4 v;
+  asm volatile("global_load_dwordx4 %0, %1, off nt\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory");
+  return v;
+}
+
+// eight 8-byte pieces `stride` bytes apart the same way
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void load_l2_8x8(const char* p, u32x2 (&v)[8]) {
+  static_assert(kScoreStride * 8 == 8192, "piece stride in the instruction offsets below");
+  const char* p2 = p + 4 * 8192;
+  asm volatile(
+      "global_load_dwordx2 %0, %8, off nt\n\tglobal_load_dwordx2 %1, %9, off nt\n\t"
+      "global_load_dwordx2 %2, %10, off nt\n\tglobal_load_dwordx2 %3, %11, off nt\n\t"
+      "global_load_dwordx2 %4, %12, off nt\n\tglobal_load_dwordx2 %5, %13, off nt\n\t"
+      "global_load_dwordx2 %6, %14, off nt\n\tglobal_load_dwordx2 %7, %15, off nt\n\ts_waitcnt vmcnt(0)"
+      : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]), "=&v"(v[6]), "=&v"(v[7])
+      : "v"(p), "v"(p + 8192), "v"(p + 2 * 8192), "v"(p + 3 * 8192), "v"(p2), "v"(p2 + 8192), "v"(p2 + 2 * 8192), "v"(p2 + 3 * 8192)
+      : "memory");
+}
+
+template <int CTRL>
+__device__ __forceinline__ float add_dpp(float v) {
+  return v + dpp_f<CTRL>(v);
+}
+constexpr int kDppMirror = 0x140;  // lane i <-> 15 - i within 16
+// sum over the 16 lanes of a row, adjacent pairs first (attention_kernel's row16_tree_sum)
+__device__ __forceinline__ float row16_sum(float v) {
+  v = add_dpp<kDppXor1>(v);
+  v = add_dpp<kDppXor2>(v);
+  v = add_dpp<kDppHalfMirror>(v);
+  v = add_dpp<kDppMirror>(v);
+  return v;
+}
+__device__ __forceinline__ float add_swap16(float v) {
+  float a = v, b = v;
+  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+  return a + b;
+}
+__device__ __forceinline__ float add_swap32(float v) {
+  float a = v, b = v;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+  return a + b;
+}
+__device__ __forceinline__ float wave_sum(float v) { return add_swap32(add_swap16(row16_sum(v))); }
+__device__ __forceinline__ float wave_maxf(float v) {
+  v = fmaxf(v, dpp_f<kDppXor1>(v));
+  v = fmaxf(v, dpp_f<kDppXor2>(v));
+  v = fmaxf(v, dpp_f<kDppHalfMirror>(v));
+  v = fmaxf(v, dpp_f<kDppMirror>(v));
+  float a = v, b = v;
+  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+  v = fmaxf(a, b);
+  a = v, b = v;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+  return fmaxf(a, b);
+}
+
+// the canonical tree over the 16 wavefronts' sums of one row
+__device__ __forceinline__ float sum_16_waves(const float (*rd)[16], int r) {
+  float t[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) t[i] = rd[i][r];
+#pragma unroll
+  for (int n = 8; n >= 1; n >>= 1) {
+#pragma unroll
+    for (int i = 0; i < n; ++i) t[i] = t[2 * i] + t[2 * i + 1];
+  }
+  return t[0];
+}
+
+// workgroup -> (head, part): the eight parts of a head are the workgroups idx = 8 g .. 8 g + 7 of one residue
+// class w % 8 (one die); head = 8 g + class
+__device__ __forceinline__ void head_of(int w, int& head, int& part) {
+  const int cls = w & 7, idx = w >> 3;
+  head = (idx >> 3) * 8 + cls;
+  part = idx & 7;
+}
+
+__global__ __launch_bounds__(64) void die_probe_kernel(int32_t* die_of) {
+  if (threadIdx.x == 0) die_of[blockIdx.x] = __builtin_amdgcn_s_getreg((20) | (0 << 6) | ((4 - 1) << 11)) & 15;  // XCC_ID
+}
+
+template <bool STAMPS>
+__global__ __launch_bounds__(kThreads) void qkv_attn_kernel(QkvAttnArgs a) {
+  __shared__ __attribute__((aligned(16))) unsigned char xs[kBlocks * 64];  // byte planes, 64 bytes per block
+  __shared__ __attribute__((aligned(16))) float xc[kBlocks];
+  __shared__ __attribute__((aligned(16))) float xS[kBlocks];
+  __shared__ __attribute__((aligned(16))) half_t xn[kK];
+  __shared__ float red[3][16][16];
+  __shared__ __attribute__((aligned(16))) float part_sum[256];
+  __shared__ __attribute__((aligned(16))) half_t own[3 * kDP];  // this workgroup's 16 dimensions of the rotated Q, of the new key and of the new value
+  __shared__ float s[kChunkCap * 64];
+  __shared__ float ex[kChunkCap * 64];  // the exponentials (a second array: no barrier between maximum and exponentials)
+  __shared__ __attribute__((aligned(16))) half_t vt[kAttnWaves][64 * kDP];  // a wavefront's chunk of values, [position][dimension]
+  __shared__ float cs[kChunkCap];
+  __shared__ float cv[kChunkCap * kDP];
+  __shared__ int lost;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int q = lane >> 4, r = lane & 15;
+  const int tq = q, dl = r;  // the attention's names: position within a group of four, lane of a row
+  const int blk0 = (4 * wave + q) * kG;
+  const bool stager = tid < kThreads / 2;  // 512 units of eight inputs
+  int head, part;
+  head_of((int)blockIdx.x, head, part);
+  if (tid == 0) lost = 0;
+  int n_stamp = 0;
+  auto stamp = [&]() {
+    if (STAMPS && tid == 0) a.stamps[(size_t)blockIdx.x * kQkvStamps + n_stamp++] = wall_clock64();
+  };
+  stamp();  // 0 start
+
+  // ---- requests, in the order the compute unit's memory pipeline should serve them
+  uint4 xu = uint4{0, 0, 0, 0}, gu = uint4{0, 0, 0, 0};
+  if (stager) {
+    xu = reinterpret_cast<const uint4*>(a.x)[tid];
+    gu = reinterpret_cast<const uint4*>(a.gamma)[tid];
+  }
+  const int32_t pos = a.dyn->pos;
+  // (the launcher's bound is kMaxLen; the clamp keeps every index inside the arrays whatever the state says)
+  const int32_t L = min(a.use_len_hi ? a.dyn->len_hi : a.dyn->len_lo, kChunkCap * 64);
+  const int32_t epoch = a.dyn->epoch;
+  const int32_t gave_up_before = __hip_atomic_load(a.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  // the three row groups of this workgroup: dimensions 16 part .. + 15 of the head's Q, K and V
+  int rg[3];
+  half_t gs[3], gz[3];
+#pragma unroll
+  for (int i = 0; i < 3; ++i) {
+    rg[i] = i * (kK / 16) + head * kParts + part;
+    const unsigned gi = ((unsigned)(rg[i] * 16 >> 7) % (unsigned)(kK / 128)) % (unsigned)a.mg;
+    gs[i] = a.scale[gi];
+    gz[i] = a.zp[gi];
+  }
+  __syncthreads();  // every request for x is out before any request for weights
+  u32x4 wr[3][kG];
+  auto request_w = [&](int i) {
+    const u32x4* wp = a.wq + ((int64_t)rg[i] * kBlocks + blk0) * 16 + r;
+#pragma unroll
+    for (int b = 0; b < kG; ++b) wr[i][b] = __builtin_nontemporal_load(wp + b * 16);
+  };
+  // the first row group now (32 KB: what a compute unit accepts at once), the others behind the staging:
+  // a wavefront passes a barrier only once the memory pipeline has accepted all its requests
+  request_w(0);
+  stamp();  // 1 first requests issued
+  // 1 .. 65535: never the 0 of a cleared buffer.  Q and K words are all rewritten by every launch, so a word
+  // holds the previous launch's tag until then; score words beyond the attended length are not, which is why
+  // the buffer is cleared when a sequence starts (a sequence stays below 65535 launches of this kind)
+  const uint32_t tag16 = 1u + (uint32_t)(epoch + a.layer) % 65535u;
+
+  // ---- rmsNormKernel, Inference.cu:111-145: x in natural order for the 256 strided partial sums
+  if (stager) reinterpret_cast<uint4*>(xn)[tid] = xu;
+  __syncthreads();
+  if (tid < 256) {
+    half_t hv[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) hv[j] = xn[tid + 256 * j];
+    float acc = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      const float v = (float)hv[j];
+      acc = __builtin_fmaf(v, v, acc);
+    }
+    part_sum[tid] = acc;
+  }
+  __syncthreads();
+  {
+    // the tree of Inference.cu:130-135, by every wavefront for itself (see gemv_kernel)
+    float pv[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) pv[j] = part_sum[(lane & 15) + 16 * j];
+#pragma unroll
+    for (int n = 8; n >= 1; n >>= 1) {
+#pragma unroll
+      for (int j = 0; j < n; ++j) pv[j] += pv[j + n];
+    }
+    float tot = pv[0];
+    tot += dpp_f<kDppRor8>(tot);
+    tot += dpp_f<kDppRor4>(tot);
+    tot += dpp_f<kDppXor2>(tot);
+    tot += dpp_f<kDppXor1>(tot);
+    tot = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, tot)));
+    const half_t sc = rsqrt_half(tot / (float)kK + a.eps);
+    const half2_t sc2 = half2_t{sc, sc};
+    uint32_t* d = reinterpret_cast<uint32_t*>(&xu);
+    const uint32_t* g = reinterpret_cast<const uint32_t*>(&gu);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      half2_t t = as_half2(d[i]) * sc2;
+      t = t * as_half2(g[i]);
+      d[i] = __builtin_bit_cast(uint32_t, t);
+    }
+  }
+  // x in block fixed point: byte planes, the power of two and the integer sum of every block
+  if (stager) {
+    const uint32_t h[4] = {xu.x, xu.y, xu.z, xu.w};
+    uint32_t lo0, lo1, hi0, hi1;
+    float cc, S;
+    stage_unit8_bytes(h, lo0, lo1, hi0, hi1, cc, S);
+    uint32_t* blk = reinterpret_cast<uint32_t*>(xs + (size_t)(tid >> 2) * 64) + (tid & 3);
+    blk[0] = lo0, blk[4] = lo1, blk[8] = hi0, blk[12] = hi1;
+    if ((tid & 3) == 0) {
+      xc[tid >> 2] = cc;
+      xS[tid >> 2] = S;
+    }
+  }
+  stamp();  // 2 x normalised and staged (this wavefront)
+  __syncthreads();
+  stamp();  // 3 ... by all wavefronts
+  request_w(1);
+  request_w(2);
+  // ---- what the attention needs from the cache, requested right behind the weights so that it arrives right
+  // behind them: one chunk of 64 positions per wavefront, this workgroup's 16 dimensions of every key and
+  // value row as two 16-byte pieces (lane = (position % 32, piece))
+  const int nchunks = (L + 63) >> 6;
+  const int aw = wave - kAttnWave0;  // index among the streaming wavefronts
+  const bool streams = aw >= 0 && aw < nchunks;
+  half8v_t kraw[2], vraw[2];
+  if (streams) {
+    const int64_t col = kDP * part + 8 * (lane & 1);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int t = (aw << 6) + 32 * j + (lane >> 1);
+      if (t < L) {
+        const int64_t row = kv_row(a.kv, head, t) + col;
+        kraw[j] = *reinterpret_cast<const half8v_t*>(a.k_cache + row);
+        vraw[j] = *reinterpret_cast<const half8v_t*>(a.v_cache + row);
+      }
+    }
+  }
+
+  // ---- the three products (Inference.cu:1052)
+  {
+    u32x4 a_lo[kG], a_hi[kG];
+    float cb[kG], Sb[kG];
+#pragma unroll
+    for (int b = 0; b < kG; ++b) {
+      load_planes(xs + (size_t)(blk0 + b) * 64, lane, a_lo[b], a_hi[b]);
+      cb[b] = xc[blk0 + b];
+      Sb[b] = xS[blk0 + b];
+    }
+#pragma unroll
+    for (int i = 0; i < 3; ++i) {
+      const GroupConst g = make_group(gs[i], gz[i]);
+      float bs[kG];
+#pragma unroll
+      for (int b = 0; b < kG; ++b)
+        bs[b] = __builtin_fmaf(g.zn, Sb[b], block_dot_mfma(wr[i][b], a_lo[b], a_hi[b])) * (g.s * cb[b]);
+      const float v = sum_rows_of_16(bs[0] + bs[1]);
+      if (q == 0) red[i][wave][r] = v;
+    }
+  }
+
+  // the wavefront that finishes the product asks for its rotary constants now
+  half_t rc = (half_t)0.0f, rs = (half_t)0.0f;
+  if (tid < 2 * kDP) {
+    const int d = kDP * part + r;
+    rc = a.cos_t[(int64_t)pos * 64 + (d >> 1)];
+    rs = a.sin_t[(int64_t)pos * 64 + (d >> 1)];
+  }
+  // the sums below add all kChunkCap entries unconditionally: zeros where there is no chunk (x + 0 is x for the
+  // non-negative sums and for the chunk vectors, which are never -0: every chain starts at +0)
+  if (tid >= nchunks && tid < kChunkCap) cs[tid] = 0.0f;
+  if (tid < kChunkCap * kDP && (tid >> 4) >= nchunks) cv[tid] = 0.0f;
+  stamp();  // 4 products multiplied (this wavefront: its weights have arrived)
+  __syncthreads();
+  stamp();  // 5 ... by all wavefronts
+
+  // ---- split, rotary, KV append (Inference.cu:1070-1103) and the first hand-over
+  if (tid < 3 * kDP) {
+    const int sec = tid >> 4;  // 0 Q, 1 K, 2 V
+    const half_t v = (half_t)sum_16_waves(red[sec], r);
+    const int d = kDP * part + r;
+    const half_t other = __builtin_bit_cast(half_t, (unsigned short)__shfl_xor((int)__builtin_bit_cast(unsigned short, v), 1, 64));
+    half_t out = v;
+    if (sec < 2) {  // pairs (2i, 2i + 1) are rotated (Inference.cu:158-176)
+      const half_t av = (r & 1) ? other : v, bv = (r & 1) ? v : other;
+      if (r & 1) {
+        half_t as = av * rs, bc = bv * rc;
+        out = as + bc;
+      } else {
+        half_t ac = av * rc, bs = bv * rs;
+        out = ac - bs;
+      }
+    }
+    own[tid] = out;
+    if (sec == 0) a.q_out[head * AWQ_HEAD_DIM + d] = out;
+    else if (sec == 1) a.k_cache[kv_row(a.kv, head, pos) + d] = out;
+    else a.v_cache[kv_row(a.kv, head, pos) + d] = out;
+  }
+  stamp();  // 6 this workgroup's Q, K, V rotated and stored
+  __syncthreads();
+  stamp();  // 7 ... and in LDS for all wavefronts
+
+  // ---- this workgroup's share of every score (Inference.cu:202-226): lane (position, piece) runs the chain of
+  // eight dimensions of its piece, the two pieces of a position are added (the first level of the dot
+  // product's adjacent-pair tree), and the sum is published
+  if (streams) {
+    float qf[8];
+    const half8v_t qv = *reinterpret_cast<const half8v_t*>(own + 8 * (lane & 1));
+    const half8v_t knew = *reinterpret_cast<const half8v_t*>(own + kDP + 8 * (lane & 1));
+#pragma unroll
+    for (int i = 0; i < 8; ++i) qf[i] = (float)qv[i];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int t = (aw << 6) + 32 * j + (lane >> 1);
+      const half8v_t kv = t == pos ? knew : kraw[j];  // not from the row just written
+      float pt = 0.0f;
+      if (t < L) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) pt = __builtin_fmaf(qf[i], (float)kv[i], pt);
+      }
+      pt = add_dpp<kDppXor1>(pt);
+      if (t < L && (lane & 1) == 0) {
+        const uint32_t bits = __builtin_bit_cast(uint32_t, pt);
+        uint32_t* dst = a.score_tag + (((size_t)head * kParts + part) * kScoreStride + t) * 2;
+        __builtin_nontemporal_store((bits & 0xffffu) | (tag16 << 16), dst);
+        __builtin_nontemporal_store((bits >> 16) | (tag16 << 16), dst + 1);
+      }
+      // this wavefront's chunk of values into the order of the sums: [position][dimension]
+      if (t < L) *reinterpret_cast<half8v_t*>(&vt[aw][(32 * j + (lane >> 1)) * kDP + 8 * (lane & 1)]) = vraw[j];
+    }
+  }
+  stamp();  // 8 partial scores published (this wavefront)
+  if ((wave << 6) < L) {
+    // the eight partial scores of position tid: the rest of the tree (Inference.cu:218 scales the sum)
+    const bool mine = tid < L;
+    const char* src = reinterpret_cast<const char*>(a.score_tag + ((size_t)head * kParts * kScoreStride + tid) * 2);
+    const float scale = 1.0f / sqrtf((float)AWQ_HEAD_DIM);
+    int spins = 0;
+    bool dead = gave_up_before != 0;
+    while (!dead) {
+      int32_t st = 0;
+      const bool look = (spins & 7) == 7;  // every eighth poll also reads the status word
+      if (look) st = __hip_atomic_load(a.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      u32x2 w[8];
+      bool ok = true;
+      if (mine) {
+        load_l2_8x8(src, w);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) ok = ok && (w[i].x >> 16) == tag16 && (w[i].y >> 16) == tag16;
+      }
+      if (__builtin_amdgcn_ballot_w64(!ok) == 0) {
+        if (mine) {
+          float p8[8];
+#pragma unroll
+          for (int i = 0; i < 8; ++i) p8[i] = __builtin_bit_cast(float, (w[i].x & 0xffffu) | (w[i].y << 16));
+          const float tot = ((p8[0] + p8[1]) + (p8[2] + p8[3])) + ((p8[4] + p8[5]) + (p8[6] + p8[7]));
+          s[tid] = tot * scale;
+        }
+        break;
+      }
+      if (++spins > a.spin_limit) {
+        if (lane == 0) __hip_atomic_store(a.status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        dead = true;
+      }
+      if (look && st != 0) dead = true;
+    }
+    if (dead && lane == 0) lost = 1;
+  }
+  __syncthreads();
+  stamp();  // 9 all scores of the head seen
+  if (lost) return;
+
+  // ---- maximum (Inference.cu:229-233; it does not depend on the order), by every wavefront for itself
+  float mx = -1e9f;
+  for (int c = 0; c < nchunks; ++c) {
+    const int t = (c << 6) + lane;
+    if (t < L) mx = fmaxf(mx, s[t]);
+  }
+  mx = wave_maxf(mx);
+
+  // ---- exponentials and their sum (Inference.cu:239-249), one wavefront per chunk
+  if (streams) {
+    const int t = (aw << 6) + lane;
+    float e = 0.0f;
+    if (t < L) {
+      e = awq_expf(s[t] - mx);
+      ex[t] = e;
+    }
+    e = wave_sum(e);
+    if (lane == 0) cs[aw] = e;
+  }
+  __syncthreads();
+  float Z;
+  {
+    float zc[kChunkCap];
+#pragma unroll
+    for (int c = 0; c < kChunkCap; ++c) zc[c] = cs[c];
+    Z = zc[0];
+#pragma unroll
+    for (int c = 1; c < kChunkCap; ++c) Z += zc[c];
+  }
+
+  // ---- weighted sum of V (Inference.cu:251-265), one wavefront per chunk: lane (tq, dl) runs the chain of
+  // positions 4 nl + tq for dimension dl
+  if (streams) {
+    const int base = aw << 6;
+    half_t vv[16];
+#pragma unroll
+    for (int nl = 0; nl < 16; ++nl) vv[nl] = vt[aw][(4 * nl + tq) * kDP + dl];
+    const float p_lane = base + lane < L ? ex[base + lane] / Z : 0.0f;
+    float acc = 0.0f;
+    float pp[16];
+#pragma unroll
+    for (int nl = 0; nl < 16; ++nl) pp[nl] = __shfl(p_lane, 4 * nl + tq, 64);
+#pragma unroll
+    for (int nl = 0; nl < 16; ++nl) {
+      const int t = base + 4 * nl + tq;
+      const half_t val = t == pos ? own[2 * kDP + dl] : vv[nl];  // the new row from this workgroup's own product
+      const float rr = __builtin_fmaf(pp[nl], (float)val, acc);
+      acc = t < L ? rr : acc;
+    }
+    acc = add_swap16(acc);
+    acc = add_swap32(acc);
+    if (tq == 0) cv[aw * kDP + dl] = acc;
+  }
+  __syncthreads();
+  if (tid < kDP) {
+    float oc[kChunkCap];
+#pragma unroll
+    for (int c = 0; c < kChunkCap; ++c) oc[c] = cv[c * kDP + tid];
+    float out = oc[0];
+#pragma unroll
+    for (int c = 1; c < kChunkCap; ++c) out += oc[c];
+    a.ctx[head * AWQ_HEAD_DIM + kDP * part + tid] = (half_t)out;
+  }
+  stamp();  // 10 end
+}
+
+}  // namespace
+
+// hidden 4096 with 32 heads of 128, every workgroup resident at once, and workgroups whose indices agree
+// modulo 8 on one die (checked with a probe launch of the same grid: 0 = not so, or not known)
+int fused_qkv_attn_supported(int64_t hidden, int n_heads, hipStream_t st) {
+  if (hidden != kK || n_heads != kK / AWQ_HEAD_DIM) return 0;
+  int dev = 0, cus = 0, occ = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 0;
+  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, qkv_attn_kernel<false>, kThreads, 0) != hipSuccess) return 0;
+  const int n_wg = n_heads * kParts;
+  if (occ < 1 || (int64_t)cus * occ < n_wg) return 0;
+  int32_t* d = nullptr;
+  if (hipMalloc((void**)&d, n_wg * sizeof(int32_t)) != hipSuccess) return 0;
+  int32_t h[kK / AWQ_HEAD_DIM * kParts];
+  bool ok = true;
+  for (int round = 0; round < 2 && ok; ++round) {
+    hipLaunchKernelGGL(die_probe_kernel, dim3((unsigned)n_wg), dim3(64), 0, st, d);
+    ok = hipGetLastError() == hipSuccess && hipStreamSynchronize(st) == hipSuccess &&
+         hipMemcpy(h, d, sizeof(h), hipMemcpyDeviceToHost) == hipSuccess;
+    for (int w = 8; w < n_wg && ok; ++w) ok = h[w] == h[w & 7];
+  }
+  (void)hipFree(d);
+  return ok ? 1 : 0;
+}
+
+int launch_fused_qkv_attn(const void* wq, const half_t* scale, const half_t* zp, int64_t m, const half_t* x,
+                          const half_t* gamma, float eps, const half_t* cos_t, const half_t* sin_t, half_t* k_cache,
+                          half_t* v_cache, KvLayout kv, half_t* q_out, half_t* ctx, uint32_t* score_tag, int32_t* status, const StepState* dyn, int layer,
+                          int use_len_hi, int n_heads, unsigned long long* stamps, hipStream_t st) {
+  AWQ_REQUIRE(m == 3 * kK && n_heads == kK / AWQ_HEAD_DIM, "the fused launch is built for hidden 4096 and 32 heads");
+  AWQ_REQUIRE(wq && x && gamma && cos_t && sin_t && k_cache && v_cache && q_out && ctx && score_tag && status && dyn,
+              "NULL pointer");
+  QkvAttnArgs a;
+  a.wq = (const u32x4*)wq;
+  a.scale = scale;
+  a.zp = zp;
+  a.x = x;
+  a.gamma = gamma;
+  a.cos_t = cos_t;
+  a.sin_t = sin_t;
+  a.k_cache = k_cache;
+  a.v_cache = v_cache;
+  a.q_out = q_out;
+  a.ctx = ctx;
+  a.score_tag = score_tag;
+  a.status = status;
+  a.dyn = dyn;
+  a.kv = kv;
+  a.layer = layer;
+  a.use_len_hi = use_len_hi;
+  a.spin_limit = 1 << 20;
+  a.mg = (int32_t)(m / 128);
+  a.eps = eps;
+  a.stamps = stamps;
+  if (stamps) hipLaunchKernelGGL(qkv_attn_kernel<true>, dim3((unsigned)(n_heads * kParts)), dim3(kThreads), 0, st, a);
+  else hipLaunchKernelGGL(qkv_attn_kernel<false>, dim3((unsigned)(n_heads * kParts)), dim3(kThreads), 0, st, a);
+  AWQ_HIP_TRY(hipGetLastError());
+  return AWQ_OK;
+}
+
+int64_t fused_qkv_attn_exchange_bytes(int n_heads) {
+  return (int64_t)n_heads * kScoreStride * kParts * 8;
+}

@@ -107,20 +107,29 @@ int awq_set_prefill_mode(awq_engine* e, int batched);
  * after awq_reset. */
 int awq_debug_force_handover_giveup(awq_engine* e, int on);
 
-/* No counterpart in the reference.  With hidden 4096 / intermediate 12288 on a
- * device with at least 256 compute units, awq_set_fused_mode(e, 1) makes the
- * token-by-token steps run the attention output product (Inference.cu:
- * 1128-1155) and RMSNorm + W1 + GeLU (:1163-1198) of a layer as ONE launch
- * whose workgroups hand the hidden state to each other through memory, with
- * W1's weights requested while that hand-over is under way (bit-identical
- * results).  Off by default: on MI355X it measures 2 % slower than the two
- * launches it replaces (the hand-over costs what a kernel boundary costs, and
- * W1's multiplies no longer overlap its stream).  The launch needs all its
- * 256 workgroups resident at once, i.e. the device to itself: a wait that
- * cannot end gives up after a bounded number of polls and the call
- * (awq_prefill, awq_decode, awq_generate) returns AWQ_ERR_HIP; awq_reset
- * leaves the engine usable.  Asking for it where it is not supported leaves
- * it off; awq_fused_mode tells which is in use. */
+/* No counterpart in the reference: pairs of a layer's launches as ONE launch,
+ * with bit-identical results.  `enabled` is a sum of
+ *   1  the attention output product (Inference.cu:1128-1155) and RMSNorm + W1 +
+ *      GeLU (:1163-1198): 256 workgroups hand the hidden state to each other
+ *      through memory, W1's weights requested while that hand-over is under way
+ *      (hidden 4096 / intermediate 12288);
+ *   2  RMSNorm + Wqkv + rotary + KV append (:1040-1103) and the attention
+ *      (:1110) up to 704 attended positions: the eight workgroups of a head sit
+ *      on one die and hand partial scores to each other through its L2 (hidden
+ *      4096, 32 heads; longer sequences keep the two launches).
+ * Both are off by default: on MI355X the first measures 2 % slower than the two
+ * launches it replaces (a hand-over between all workgroups costs what a kernel
+ * boundary costs), the second level with them (967 against 964-966 tok/s: what
+ * the missing boundary saves, the wait for the slowest of a head's eight
+ * workgroups and one workgroup per compute unit give back).  A fused launch
+ * needs all its 256 workgroups resident at once, i.e. a device of at least 256
+ * compute units to itself, and the second one workgroups whose indices agree
+ * modulo 8 on one die (probed with a launch of the same grid when it is
+ * switched on).  A wait that cannot end gives up after a bounded number of
+ * polls and the call (awq_prefill, awq_decode, awq_generate) returns
+ * AWQ_ERR_HIP, never a wrong token; awq_reset leaves the engine usable.  Asking
+ * for a launch where it is not supported leaves it off; awq_fused_mode tells
+ * which are in use. */
 int awq_set_fused_mode(awq_engine* e, int enabled);
 int awq_fused_mode(const awq_engine* e);
 /* Diagnostics, no counterpart in the reference: runs the fused launch of every
@@ -131,6 +140,10 @@ int awq_fused_mode(const awq_engine* e);
  * 256 * 16 values.  Leaves the engine reset. */
 int awq_debug_fused_timeline(awq_engine* e, int32_t layer, uint64_t* host_out, int32_t* n_workgroups,
                              int32_t* n_stamps);
+/* The same for the fused Wqkv + attention launch, at position `pos` attending
+ * pos + 1 positions (pos < 704). */
+int awq_debug_qkv_attention_timeline(awq_engine* e, int32_t layer, int32_t pos, uint64_t* host_out,
+                                     int32_t* n_workgroups, int32_t* n_stamps);
 
 /* Copies of internal state for tests: hidden state [hidden] and the logits of
  * the last sampled position [vocab], both FP16, to host memory. */
@@ -316,6 +329,29 @@ int awq_decode_attention(const void* q, const void* k_cache, const void* v_cache
  * capture. */
 int awq_decode_attention_static(const void* q, const void* k_cache, const void* v_cache, void* ctx, int32_t n_heads,
                                 int64_t max_pos, int64_t L, void* stream);
+
+/* No counterpart in the reference: awq_gemv_fused(RMSNorm, Wqkv, rotary + KV
+ * append) and awq_decode_attention as ONE launch for hidden 4096 and 32 heads
+ * (wqkv_repacked is the 12288 x 4096 matrix from awq_linear_repack; caches
+ * [head][max_pos][128]; x, gamma [4096]; q_out, ctx [4096]), position `pos`
+ * attending the first L positions, L <= pos + 1 and L <= 704.  Same bits as the
+ * two calls.  Every head is given to eight workgroups that the device places on
+ * one die (awq_qkv_attention_supported probes that and that all 256 workgroups
+ * are resident at once: 1 = yes); they hand partial scores to each other through
+ * that die's L2, in words that carry a tag derived from call_tag: any value in
+ * [1, 2^30) that differs from the previous call's on the same workspace.
+ * workspace: awq_qkv_attention_workspace_bytes(n_heads) bytes, zero-filled once;
+ * calls on one workspace must not overlap.  A wait that cannot end gives up
+ * after a bounded number of polls and leaves ctx unwritten:
+ * awq_qkv_attention_status (synchronises the stream) then returns AWQ_ERR_HIP
+ * once and clears the condition. */
+int64_t awq_qkv_attention_workspace_bytes(int32_t n_heads);
+int awq_qkv_attention_supported(int64_t hidden, int32_t n_heads, void* stream);
+int awq_qkv_attention(const void* wqkv_repacked, const void* scale, const void* zp, const void* x, const void* gamma,
+                      float eps, const void* cos_t, const void* sin_t, void* k_cache, void* v_cache, int64_t max_pos,
+                      int32_t n_heads, int64_t pos, int64_t L, void* q_out, void* ctx, void* workspace,
+                      int32_t call_tag, void* stream);
+int awq_qkv_attention_status(void* workspace, void* stream);
 
 /* The same attention for n_tokens consecutive prompt positions pos0 ..
  * pos0 + n_tokens - 1 at once (their keys and values already appended): q and

@@ -485,3 +485,57 @@ def test_fused_wo_w1_launch_is_bit_identical_and_gives_up_cleanly(awq, lib, orac
     assert 0 < (t[:, -1].max() - t[:, 0].min()) * 0.01 < 1000.0     # microseconds
     eng.close()
     oracle.awqo_model_destroy(model)
+
+
+def test_fused_qkv_attention_launch_is_bit_identical_and_gives_up_cleanly(awq, lib, oracle, torch_gpu):
+    """awq_set_fused_mode(e, 2): RMSNorm + Wqkv + rotary + KV append and the attention of a layer as one launch
+    (eight workgroups per head on one die, partial scores handed over through its L2, bounded waits).  Two
+    full-width layers, a 40-token prompt token by token and 100 generated tokens (attended lengths on both sides
+    of 128): ids, hidden state and logits must be the oracle's bit for bit, with and without a captured graph,
+    also together with the fused Wo + W1 launch.  Then the give-up path, driven from the host (the status word
+    is set before the call, so every wait ends at its first look and every kernel runs to its end): the call
+    fails with AWQ_ERR_HIP and the engine works again after a reset.  Last, the instrumented launch behind
+    awq_debug_qkv_attention_timeline returns ordered time stamps."""
+    cfg = awq.make_config(n_layers=2, max_pos=1024)
+    model = make_oracle_model(oracle, cfg)
+    eng = awq.QWen3AWQInfer.empty(cfg)
+    fill_pair(awq, oracle, cfg, 2025, engine=eng, model=model, profile=awq.SYNTH_BALANCED)
+    assert eng.fused_mode() == 0                     # one launch per product by default
+    eng.set_fused_mode(eng.FUSED_QKV_ATTN)
+    if not eng.fused_mode() & eng.FUSED_QKV_ATTN:
+        pytest.skip("this device cannot run the fused launch")
+    rng = np.random.default_rng(17)
+    prompt = rng.integers(0, cfg.vocab, 40).tolist()
+    ref = oracle_generate(oracle, model, prompt, 100)
+    for graph in (True, False):
+        eng.set_graph_mode(graph)
+        print("fused Wqkv + attention launch, graph", graph, flush=True)
+        assert eng.generateResponse(prompt, 100) == ref
+        compare_state(awq, oracle, eng, model, cfg)
+    eng.set_graph_mode(True)
+    eng.set_fused_mode(eng.FUSED_QKV_ATTN | eng.FUSED_WO_W1)
+    if eng.fused_mode() == 3:
+        print("both fused launches", flush=True)
+        assert eng.generateResponse(prompt, 100) == ref
+        compare_state(awq, oracle, eng, model, cfg)
+    eng.set_fused_mode(eng.FUSED_QKV_ATTN)
+    print("fused Wqkv + attention launch, every wait giving up", flush=True)
+    eng.reset()
+    awq.check(lib.awq_debug_force_handover_giveup(eng._h, 1))
+    with pytest.raises(awq.AwqError) as ei:
+        eng.prefill(prompt[:3])
+    assert ei.value.code == 3 and "gave up" in str(ei.value)
+    print("fused Wqkv + attention launch, after a reset", flush=True)
+    assert eng.generateResponse(prompt, 100) == ref
+    compare_state(awq, oracle, eng, model, cfg)
+    buf = np.zeros(256 * 16, dtype=np.uint64)
+    nw, ns = ctypes.c_int32(0), ctypes.c_int32(0)
+    awq.check(lib.awq_debug_qkv_attention_timeline(eng._h, 1, 200, buf.ctypes.data_as(ctypes.c_void_p),
+                                                   ctypes.byref(nw), ctypes.byref(ns)))
+    t = buf[:nw.value * ns.value].reshape(nw.value, ns.value).astype(np.int64)
+    assert nw.value == 256 and ns.value >= 8 and (np.diff(t, axis=1) >= 0).all()
+    assert 0 < (t[:, -1].max() - t[:, 0].min()) * 0.01 < 1000.0     # microseconds
+    eng.set_fused_mode(0)
+    assert eng.generateResponse(prompt, 100) == ref
+    eng.close()
+    oracle.awqo_model_destroy(model)

@@ -592,6 +592,83 @@ def test_gemv_fused_norm_unembed_argmax(awq, lib, oracle, torch_gpu, m, k):
     assert int(keep["ws"].to(torch.int32).abs().sum().item()) == 0  # sampler workspace left zeroed
 
 
+# ----------------------------------------------------------------------------- Wqkv + attention as one launch
+@pytest.mark.parametrize("pos,L", [(0, 1), (1, 1), (2, 2), (2, 3), (5, 5), (63, 64), (70, 71), (300, 301), (640, 640),
+                                   (703, 704)])
+def test_fused_qkv_attention_launch_against_the_two_launches_and_the_oracle(awq, lib, oracle, torch_gpu, pos, L):
+    """awq_qkv_attention: RMSNorm + Wqkv + rotary + KV append and the attention over the cache in one launch whose
+    eight workgroups per head hand partial scores to each other through the L2 of their die.  Q, the caches and
+    the context must be those of awq_gemv_fused + awq_decode_attention and of the oracle, bit for bit, on two
+    calls in a row (the tags change; the second call finds the first one's words in the exchange buffer)."""
+    torch = torch_gpu
+    H = 4096
+    m, k, nh, mp = 3 * H, H, H // 128, 768
+    if not lib.awq_qkv_attention_supported(H, nh, stream(torch)):
+        pytest.skip("this device cannot run the fused launch")
+    rng = np.random.default_rng(pos * 1000 + L)
+    packed, scale, zp, a, keep = fused_setup(awq, lib, torch, rng, m, k)
+    hidden = rng.standard_normal(k).astype(np.float16)
+    gamma = (1 + 0.02 * rng.standard_normal(k)).astype(np.float16)
+    cos_t, sin_t = np.zeros((mp, 64), np.float16), np.zeros((mp, 64), np.float16)
+    oracle.awqo_rope_tables(ptr(cos_t), ptr(sin_t), mp)
+    kc = (rng.standard_normal(nh * mp * 128) * 0.3).astype(np.float16)
+    vc = rng.standard_normal(nh * mp * 128).astype(np.float16)
+    d_h, d_g, d_c, d_s = dev(torch, hidden), dev(torch, gamma), dev(torch, cos_t), dev(torch, sin_t)
+    # the oracle
+    normed = np.zeros(k, dtype=np.float16)
+    oracle.awqo_rmsnorm(ptr(hidden), ptr(gamma), ptr(normed), k, 1e-6)
+    qkv = np.zeros(m, dtype=np.float16)
+    oracle.awqo_linear(ptr(packed), ptr(scale), ptr(zp), m, k, ptr(normed), ptr(qkv), 1)
+    q_ref, k_ref, v_ref = qkv[:H].copy(), qkv[H:2 * H].copy(), qkv[2 * H:].copy()
+    oracle.awqo_rotary(ptr(q_ref), ptr(cos_t), ptr(sin_t), nh, pos)
+    oracle.awqo_rotary(ptr(k_ref), ptr(cos_t), ptr(sin_t), nh, pos)
+    kc_ref, vc_ref = kc.copy(), vc.copy()
+    oracle.awqo_kv_append(ptr(kc_ref), ptr(k_ref), nh, mp, pos)
+    oracle.awqo_kv_append(ptr(vc_ref), ptr(v_ref), nh, mp, pos)
+    ctx_ref = np.zeros(H, dtype=np.float16)
+    oracle.awqo_attention(ptr(q_ref), ptr(kc_ref), ptr(vc_ref), ptr(ctx_ref), nh, mp, L, None)
+    # two launches
+    d_kc, d_vc = dev(torch, kc), dev(torch, vc)
+    d_q = torch.zeros(H, dtype=torch.float16, device="cuda")
+    d_o = torch.zeros(H, dtype=torch.float16, device="cuda")
+    a.x, a.y, a.gamma, a.eps = d_h.data_ptr(), d_q.data_ptr(), d_g.data_ptr(), 1e-6
+    a.prologue, a.epilogue = awq.PRO_RMSNORM, awq.EPI_QKV_ROPE
+    a.cos_t, a.sin_t, a.k_cache, a.v_cache = d_c.data_ptr(), d_s.data_ptr(), d_kc.data_ptr(), d_vc.data_ptr()
+    a.hidden, a.max_pos, a.pos = H, mp, pos
+    awq.check(lib.awq_gemv_fused(ctypes.byref(a), stream(torch)))
+    ws = torch.zeros(lib.awq_attention_workspace_bytes(nh, mp), dtype=torch.uint8, device="cuda")
+    awq.check(lib.awq_decode_attention(d_q.data_ptr(), d_kc.data_ptr(), d_vc.data_ptr(), d_o.data_ptr(), nh, mp, L,
+                                       ws.data_ptr(), stream(torch)))
+    torch.cuda.synchronize()
+    assert np.array_equal(d_o.cpu().numpy().view(np.uint16), ctx_ref.view(np.uint16))
+    # one launch
+    f_kc, f_vc = dev(torch, kc), dev(torch, vc)
+    f_q = torch.zeros(H, dtype=torch.float16, device="cuda")
+    f_o = torch.zeros(H, dtype=torch.float16, device="cuda")
+    fws = torch.zeros(lib.awq_qkv_attention_workspace_bytes(nh), dtype=torch.uint8, device="cuda")
+    print("fused launch pos", pos, "L", L, flush=True)
+    for call in (1, 2):
+        f_o.zero_()
+        awq.check(lib.awq_qkv_attention(keep["d_w"].data_ptr(), keep["d_s"].data_ptr(), keep["d_z"].data_ptr(),
+                                        d_h.data_ptr(), d_g.data_ptr(), 1e-6, d_c.data_ptr(), d_s.data_ptr(),
+                                        f_kc.data_ptr(), f_vc.data_ptr(), mp, nh, pos, L, f_q.data_ptr(), f_o.data_ptr(),
+                                        fws.data_ptr(), call, stream(torch)))
+        awq.check(lib.awq_qkv_attention_status(fws.data_ptr(), stream(torch)))
+        assert np.array_equal(f_q.cpu().numpy().view(np.uint16), q_ref.view(np.uint16))
+        assert np.array_equal(f_kc.cpu().numpy().view(np.uint16), kc_ref.view(np.uint16))
+        assert np.array_equal(f_vc.cpu().numpy().view(np.uint16), vc_ref.view(np.uint16))
+        assert np.array_equal(f_o.cpu().numpy().view(np.uint16), ctx_ref.view(np.uint16))
+        assert np.array_equal(f_o.cpu().numpy().view(np.uint16), d_o.cpu().numpy().view(np.uint16))
+    # arguments the launch is not built for are refused before anything runs
+    args = [keep["d_w"].data_ptr(), keep["d_s"].data_ptr(), keep["d_z"].data_ptr(), d_h.data_ptr(), d_g.data_ptr(), 1e-6,
+            d_c.data_ptr(), d_s.data_ptr(), f_kc.data_ptr(), f_vc.data_ptr(), mp, nh, pos, L, f_q.data_ptr(),
+            f_o.data_ptr(), fws.data_ptr(), 3, stream(torch)]
+    for idx, bad in ((11, 16), (12, mp), (13, pos + 2), (17, 0)):
+        wrong = list(args)
+        wrong[idx] = bad
+        assert lib.awq_qkv_attention(*wrong) != 0
+
+
 # ----------------------------------------------------------------------------- W4A16 GEMM on the matrix cores
 @pytest.mark.parametrize("m,k,M,zp_int", [(256, 512, 3, True), (256, 512, 17, False), (384, 1536, 130, True),
                                           (12288, 4096, 16, True), (12288, 4096, 200, True), (4096, 12288, 64, False),
