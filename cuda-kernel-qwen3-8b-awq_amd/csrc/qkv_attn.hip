@@ -179,6 +179,7 @@ __global__ __launch_bounds__(kThreads) void qkv_attn_kernel(QkvAttnArgs a) {
   __shared__ float ex[kChunkCap * 64];  // the exponentials (a second array: no barrier between maximum and exponentials)
   __shared__ __attribute__((aligned(16))) half_t vt[kAttnWaves][64 * kDP];  // a wavefront's chunk of values, [position][dimension]
   __shared__ float cs[kChunkCap];
+  __shared__ float wmax[kWaves];
   __shared__ float cv[kChunkCap * kDP];
   __shared__ int lost;
   const int tid = threadIdx.x;
@@ -352,6 +353,7 @@ __global__ __launch_bounds__(kThreads) void qkv_attn_kernel(QkvAttnArgs a) {
   stamp();  // 5 ... by all wavefronts
 
   // ---- split, rotary, KV append (Inference.cu:1070-1103) and the first hand-over
+  half_t fin_out = (half_t)0.0f;
   if (tid < 3 * kDP) {
     const int sec = tid >> 4;  // 0 Q, 1 K, 2 V
     const half_t v = (half_t)sum_16_waves(red[sec], r);
@@ -369,13 +371,17 @@ __global__ __launch_bounds__(kThreads) void qkv_attn_kernel(QkvAttnArgs a) {
       }
     }
     own[tid] = out;
-    if (sec == 0) a.q_out[head * AWQ_HEAD_DIM + d] = out;
-    else if (sec == 1) a.k_cache[kv_row(a.kv, head, pos) + d] = out;
-    else a.v_cache[kv_row(a.kv, head, pos) + d] = out;
+    fin_out = out;
   }
-  stamp();  // 6 this workgroup's Q, K, V rotated and stored
+  stamp();  // 6 this workgroup's Q, K, V rotated
   __syncthreads();
   stamp();  // 7 ... and in LDS for all wavefronts
+  if (tid < 3 * kDP) {  // the stores, off the path of the scores
+    const int sec = tid >> 4, d = kDP * part + r;
+    if (sec == 0) a.q_out[head * AWQ_HEAD_DIM + d] = fin_out;
+    else if (sec == 1) a.k_cache[kv_row(a.kv, head, pos) + d] = fin_out;
+    else a.v_cache[kv_row(a.kv, head, pos) + d] = fin_out;
+  }
 
   // ---- this workgroup's share of every score (Inference.cu:202-226): lane (position, piece) runs the chain of
   // eight dimensions of its piece, the two pieces of a position are added (the first level of the dot
@@ -414,6 +420,7 @@ __global__ __launch_bounds__(kThreads) void qkv_attn_kernel(QkvAttnArgs a) {
     const float scale = 1.0f / sqrtf((float)AWQ_HEAD_DIM);
     int spins = 0;
     bool dead = gave_up_before != 0;
+    float my_score = -1e9f;
     while (!dead) {
       int32_t st = 0;
       const bool look = (spins & 7) == 7;  // every eighth poll also reads the status word
@@ -431,7 +438,8 @@ __global__ __launch_bounds__(kThreads) void qkv_attn_kernel(QkvAttnArgs a) {
 #pragma unroll
           for (int i = 0; i < 8; ++i) p8[i] = __builtin_bit_cast(float, (w[i].x & 0xffffu) | (w[i].y << 16));
           const float tot = ((p8[0] + p8[1]) + (p8[2] + p8[3])) + ((p8[4] + p8[5]) + (p8[6] + p8[7]));
-          s[tid] = tot * scale;
+          my_score = tot * scale;
+          s[tid] = my_score;
         }
         break;
       }
@@ -442,17 +450,17 @@ __global__ __launch_bounds__(kThreads) void qkv_attn_kernel(QkvAttnArgs a) {
       if (look && st != 0) dead = true;
     }
     if (dead && lane == 0) lost = 1;
+    // maximum (Inference.cu:229-233; it does not depend on the order): this wavefront's positions
+    my_score = wave_maxf(my_score);
+    if (lane == 0) wmax[wave] = my_score;
+  } else if (lane == 0) {
+    wmax[wave] = -1e9f;
   }
   __syncthreads();
   stamp();  // 9 all scores of the head seen
   if (lost) return;
 
-  // ---- maximum (Inference.cu:229-233; it does not depend on the order), by every wavefront for itself
-  float mx = -1e9f;
-  for (int c = 0; c < nchunks; ++c) {
-    const int t = (c << 6) + lane;
-    if (t < L) mx = fmaxf(mx, s[t]);
-  }
+  float mx = lane < kWaves ? wmax[lane] : -1e9f;
   mx = wave_maxf(mx);
 
   // ---- exponentials and their sum (Inference.cu:239-249), one wavefront per chunk

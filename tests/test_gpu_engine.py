@@ -449,9 +449,9 @@ def test_fused_wo_w1_launch_is_bit_identical_and_gives_up_cleanly(awq, lib, orac
     model = make_oracle_model(oracle, cfg)
     eng = awq.QWen3AWQInfer.empty(cfg)
     fill_pair(awq, oracle, cfg, 2025, engine=eng, model=model, profile=awq.SYNTH_BALANCED)
-    assert not eng.fused_mode()                      # two launches by default
-    eng.set_fused_mode(True)
-    if not eng.fused_mode():
+    assert not eng.fused_mode() & eng.FUSED_WO_W1    # Wo and W1 are two launches by default
+    eng.set_fused_mode(eng.FUSED_WO_W1)
+    if not eng.fused_mode() & eng.FUSED_WO_W1:
         pytest.skip("this device cannot hold the fused launch's 256 workgroups at once")
     rng = np.random.default_rng(17)
     prompt = rng.integers(0, cfg.vocab, 40).tolist()
@@ -500,10 +500,9 @@ def test_fused_qkv_attention_launch_is_bit_identical_and_gives_up_cleanly(awq, l
     model = make_oracle_model(oracle, cfg)
     eng = awq.QWen3AWQInfer.empty(cfg)
     fill_pair(awq, oracle, cfg, 2025, engine=eng, model=model, profile=awq.SYNTH_BALANCED)
-    assert eng.fused_mode() == 0                     # one launch per product by default
-    eng.set_fused_mode(eng.FUSED_QKV_ATTN)
-    if not eng.fused_mode() & eng.FUSED_QKV_ATTN:
+    if not eng.fused_mode() & eng.FUSED_QKV_ATTN:    # the default where the device can run it
         pytest.skip("this device cannot run the fused launch")
+    eng.set_fused_mode(eng.FUSED_QKV_ATTN)
     rng = np.random.default_rng(17)
     prompt = rng.integers(0, cfg.vocab, 40).tolist()
     ref = oracle_generate(oracle, model, prompt, 100)
