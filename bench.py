@@ -165,7 +165,7 @@ def mode_qkv_timeline(args):
     names = ["workgroup starts", "x, gamma, state, scales, Q weights requested", "x normalised and staged (wavefront 0)",
              "... (all wavefronts); K and V weights and the cache rows requested now",
              "Q, K, V multiplied (wavefront 0: its weights have arrived)", "... (all wavefronts)",
-             "this workgroup's Q, K, V rotated and stored", "... and in LDS for all wavefronts",
+             "this workgroup's Q, K, V rotated", "... and in LDS for all wavefronts (the cache appends follow)",
              "wavefront 0 past the partial scores (the streaming wavefronts publish theirs about now)",
              "all partial scores of the head seen, scores finished", "softmax, context of 16 dimensions, end"]
     for pos in (200, 600):

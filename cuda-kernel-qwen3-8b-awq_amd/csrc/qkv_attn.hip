@@ -176,7 +176,6 @@ __global__ __launch_bounds__(kThreads) void qkv_attn_kernel(QkvAttnArgs a) {
   __shared__ __attribute__((aligned(16))) float part_sum[256];
   __shared__ __attribute__((aligned(16))) half_t own[3 * kDP];  // this workgroup's 16 dimensions of the rotated Q, of the new key and of the new value
   __shared__ float s[kChunkCap * 64];
-  __shared__ float ex[kChunkCap * 64];  // the exponentials (a second array: no barrier between maximum and exponentials)
   __shared__ __attribute__((aligned(16))) half_t vt[kAttnWaves][64 * kDP];  // a wavefront's chunk of values, [position][dimension]
   __shared__ float cs[kChunkCap];
   __shared__ float wmax[kWaves];
@@ -464,15 +463,18 @@ __global__ __launch_bounds__(kThreads) void qkv_attn_kernel(QkvAttnArgs a) {
   mx = wave_maxf(mx);
 
   // ---- exponentials and their sum (Inference.cu:239-249), one wavefront per chunk
+  float e_lane = 0.0f;  // the exponential of position 64 aw + lane stays in its register
   if (streams) {
     const int t = (aw << 6) + lane;
-    float e = 0.0f;
-    if (t < L) {
-      e = awq_expf(s[t] - mx);
-      ex[t] = e;
-    }
-    e = wave_sum(e);
+    if (t < L) e_lane = awq_expf(s[t] - mx);
+    const float e = wave_sum(e_lane);
     if (lane == 0) cs[aw] = e;
+  }
+  // this lane's values of its chunk, read before the barrier: they do not depend on the normaliser
+  half_t vv[16];
+  if (streams) {
+#pragma unroll
+    for (int nl = 0; nl < 16; ++nl) vv[nl] = vt[aw][(4 * nl + tq) * kDP + dl];
   }
   __syncthreads();
   float Z;
@@ -489,10 +491,7 @@ __global__ __launch_bounds__(kThreads) void qkv_attn_kernel(QkvAttnArgs a) {
   // positions 4 nl + tq for dimension dl
   if (streams) {
     const int base = aw << 6;
-    half_t vv[16];
-#pragma unroll
-    for (int nl = 0; nl < 16; ++nl) vv[nl] = vt[aw][(4 * nl + tq) * kDP + dl];
-    const float p_lane = base + lane < L ? ex[base + lane] / Z : 0.0f;
+    const float p_lane = base + lane < L ? e_lane / Z : 0.0f;
     float acc = 0.0f;
     float pp[16];
 #pragma unroll
