@@ -298,7 +298,7 @@ int enqueue_wqkv(awq_engine* e, int l) {
 int enqueue_layer(awq_engine* e, int l, int use_len_hi, int64_t len_bound) {
   LayerDev& L = e->layers[l];
   hipStream_t st = e->stream;
-  if (e->fused_qkv && len_bound <= kAttnOneWorkgroupMax) {  // :1040-1110 in one launch
+  if (e->fused_qkv && len_bound <= kFusedQkvAttnMax) {  // :1040-1110 in one launch
     if (int rc = launch_fused_qkv_attn(L.wqkv.stream_order, L.wqkv.scale, L.wqkv.zp, L.wqkv.m, e->hidden, L.gamma,
                                        e->cfg.eps, e->cos_t, e->sin_t, L.kcache, L.vcache, kv_blocked(e->n_heads),
                                        e->q, e->ctx, e->score_tag, e->handover_status, e->d_state, l,
@@ -1089,7 +1089,7 @@ extern "C" int awq_debug_qkv_attention_timeline(awq_engine* e, int32_t layer, in
   AWQ_REQUIRE(fused_qkv_attn_supported(e->cfg.hidden, e->n_heads, e->stream) != 0,
               "the fused launch needs hidden 4096, 32 heads and 256 compute units");
   AWQ_REQUIRE(layer >= 0 && layer < e->cfg.n_layers, "layer out of range");
-  AWQ_REQUIRE(pos >= 0 && pos < e->cfg.max_pos && pos + 1 <= kAttnOneWorkgroupMax, "pos out of range");
+  AWQ_REQUIRE(pos >= 0 && pos < e->cfg.max_pos && pos + 1 <= kFusedQkvAttnMax, "pos out of range");
   const int wgs = e->n_heads * 8;
   unsigned long long* d_stamps = nullptr;
   AWQ_HIP_TRY(hipMalloc((void**)&d_stamps, (size_t)wgs * kQkvStamps * 8));
@@ -1382,7 +1382,7 @@ extern "C" int awq_qkv_attention(const void* wqkv_repacked, const void* scale, c
   AWQ_REQUIRE(workspace != nullptr, "workspace is NULL");
   AWQ_REQUIRE(n_heads == 32, "the fused launch is built for 32 heads of 128");
   AWQ_REQUIRE(max_pos > 0 && pos >= 0 && pos < max_pos, "pos out of range");
-  AWQ_REQUIRE(L >= 0 && L <= pos + 1 && L <= kAttnOneWorkgroupMax, "attended length out of range for the fused launch");
+  AWQ_REQUIRE(L >= 0 && L <= pos + 1 && L <= kFusedQkvAttnMax, "attended length out of range for the fused launch");
   AWQ_REQUIRE(call_tag >= 1 && call_tag < (1 << 30), "call_tag must be in [1, 2^30)");
   hipStream_t st = (hipStream_t)stream;
   char* ws = (char*)workspace;

@@ -1,6 +1,6 @@
 // The first two launches of a decoder layer as ONE: RMSNorm + Wqkv + rotary + KV append (Inference.cu:1040-1103)
 // and the attention over the cache (Inference.cu:1110, attentionKernel :182-267), for attended lengths that the
-// one-launch attention covers (kAttnOneWorkgroupMax).
+// attention covers in at most two launches of its own (kFusedQkvAttnMax = kAttnTwoLaunchMax).
 //
 // Of all the boundaries between a layer's launches this is the one across which the data dependence is local:
 // the attention of head h needs rows 128 h .. 128 h + 127 of Q and of K and nothing else of the product.  A
@@ -45,15 +45,14 @@ constexpr int kBlocks = kK / 32;    // 128 blocks of 32 inputs
 constexpr int kG = 2;               // blocks per lane and row group
 constexpr int kParts = 8;           // workgroups per head
 constexpr int kDP = AWQ_HEAD_DIM / kParts;  // dimensions per workgroup: one 16-row group each of Q, K and V
-constexpr int kMaxLen = (int)kAttnOneWorkgroupMax;
+constexpr int kMaxLen = (int)kFusedQkvAttnMax;
 constexpr int kChunkCap = 16;       // chunks of 64 positions: one per wavefront
 constexpr int kScoreStride = kChunkCap * 64;  // (score, tag) pairs per head in the exchange buffer
 static_assert(kDP == 16 && kMaxLen <= kChunkCap * 64 && kMaxLen <= kScoreStride, "shape of the fused launch");
-// Wavefront 0 finishes the product (rotary, stores); the other kAttnWaves stream the cache: what queues behind
-// bulk requests in the compute unit's memory pipeline waits for them.
-constexpr int kAttnWave0 = 1;
-constexpr int kAttnWaves = kWaves - kAttnWave0;
-static_assert((kMaxLen + 63) / 64 <= kAttnWaves, "one chunk of keys and values per wavefront");
+// Wavefront 0 finishes the product (rotary, stores): what queues behind bulk requests in the compute unit's
+// memory pipeline waits for them, so the chunks of the cache go to the wavefronts from the last one down and
+// wavefront 0 streams one only beyond 960 attended positions.
+static_assert((kMaxLen + 63) / 64 <= kWaves, "one chunk of keys and values per wavefront");
 
 struct QkvAttnArgs {
   const u32x4* wq;
@@ -176,7 +175,7 @@ __global__ __launch_bounds__(kThreads) void qkv_attn_kernel(QkvAttnArgs a) {
   __shared__ __attribute__((aligned(16))) float part_sum[256];
   __shared__ __attribute__((aligned(16))) half_t own[3 * kDP];  // this workgroup's 16 dimensions of the rotated Q, of the new key and of the new value
   __shared__ float s[kChunkCap * 64];
-  __shared__ __attribute__((aligned(16))) half_t vt[kAttnWaves][64 * kDP];  // a wavefront's chunk of values, [position][dimension]
+  __shared__ __attribute__((aligned(16))) half_t vt[kWaves][64 * kDP];  // a wavefront's chunk of values, [position][dimension]
   __shared__ float cs[kChunkCap];
   __shared__ float wmax[kWaves];
   __shared__ float cv[kChunkCap * kDP];
@@ -298,8 +297,8 @@ __global__ __launch_bounds__(kThreads) void qkv_attn_kernel(QkvAttnArgs a) {
   // behind them: one chunk of 64 positions per wavefront, this workgroup's 16 dimensions of every key and
   // value row as two 16-byte pieces (lane = (position % 32, piece))
   const int nchunks = (L + 63) >> 6;
-  const int aw = wave - kAttnWave0;  // index among the streaming wavefronts
-  const bool streams = aw >= 0 && aw < nchunks;
+  const int aw = kWaves - 1 - wave;  // the chunk of this wavefront
+  const bool streams = aw < nchunks;
   half8v_t kraw[2], vraw[2];
   if (streams) {
     const int64_t col = kDP * part + 8 * (lane & 1);

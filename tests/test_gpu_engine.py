@@ -534,6 +534,13 @@ def test_fused_qkv_attention_launch_is_bit_identical_and_gives_up_cleanly(awq, l
     t = buf[:nw.value * ns.value].reshape(nw.value, ns.value).astype(np.int64)
     assert nw.value == 256 and ns.value >= 8 and (np.diff(t, axis=1) >= 0).all()
     assert 0 < (t[:, -1].max() - t[:, 0].min()) * 0.01 < 1000.0     # microseconds
+    # a long prompt token by token: attended lengths up to 760, across the 704 at which the separate attention
+    # switches from one launch to two (the fused launch covers both)
+    eng.set_fused_mode(eng.FUSED_QKV_ATTN)
+    long_prompt = rng.integers(0, cfg.vocab, 700).tolist()
+    print("fused Wqkv + attention launch, 700-token prompt", flush=True)
+    assert eng.generateResponse(long_prompt, 60) == oracle_generate(oracle, model, long_prompt, 60)
+    compare_state(awq, oracle, eng, model, cfg)
     eng.set_fused_mode(0)
     assert eng.generateResponse(prompt, 100) == ref
     eng.close()
