@@ -179,9 +179,9 @@ constexpr int64_t kAttnShortMax = 128;
 constexpr int64_t kAttnOneWorkgroupMax = 704;
 constexpr int64_t kAttnTwoLaunchMax = 1024;
 constexpr int64_t kAttnMergedMax = 2048;
-// the fused Wqkv + attention launch (qkv_attn.hip) covers attended lengths up to here: one 64-position chunk per
+// the fused Wqkv + attention launch (qkv_attn.hip) covers attended lengths up to here: two 64-position chunks per
 // wavefront of its workgroups
-constexpr int64_t kFusedQkvAttnMax = kAttnTwoLaunchMax;
+constexpr int64_t kFusedQkvAttnMax = kAttnMergedMax;
 int64_t attention_workspace_bytes(int n_heads, int64_t max_pos);
 int launch_attention(const half_t* q, const half_t* kc, const half_t* vc, half_t* ctx, int n_heads, int64_t max_pos,
                      KvLayout kv, int64_t L, const StepState* dyn, int use_len_hi, int64_t len_bound, void* ws,
@@ -221,7 +221,7 @@ int64_t fused_qkv_attn_exchange_bytes(int n_heads);
 int launch_fused_qkv_attn(const void* wq, const half_t* scale, const half_t* zp, int64_t m, const half_t* x,
                           const half_t* gamma, float eps, const half_t* cos_t, const half_t* sin_t, half_t* k_cache,
                           half_t* v_cache, KvLayout kv, half_t* q_out, half_t* ctx, uint32_t* score_tag, int32_t* status, const StepState* dyn, int layer,
-                          int use_len_hi, int n_heads, unsigned long long* stamps, hipStream_t st);
+                          int use_len_hi, int64_t len_bound, int n_heads, unsigned long long* stamps, hipStream_t st);
 constexpr int kQkvStamps = 11;  // time stamps per workgroup of the instrumented launch
 int launch_fill_zero(void* p, int64_t bytes, hipStream_t st);
 int launch_copy(const void* src, void* dst, int64_t bytes, hipStream_t st);

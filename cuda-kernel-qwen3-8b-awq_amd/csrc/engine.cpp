@@ -302,7 +302,7 @@ int enqueue_layer(awq_engine* e, int l, int use_len_hi, int64_t len_bound) {
     if (int rc = launch_fused_qkv_attn(L.wqkv.stream_order, L.wqkv.scale, L.wqkv.zp, L.wqkv.m, e->hidden, L.gamma,
                                        e->cfg.eps, e->cos_t, e->sin_t, L.kcache, L.vcache, kv_blocked(e->n_heads),
                                        e->q, e->ctx, e->score_tag, e->handover_status, e->d_state, l,
-                                       use_len_hi, e->n_heads, nullptr, st))
+                                       use_len_hi, len_bound, e->n_heads, nullptr, st))
       return rc;
   } else {
     if (int rc = enqueue_wqkv(e, l)) return rc;
@@ -1103,7 +1103,7 @@ extern "C" int awq_debug_qkv_attention_timeline(awq_engine* e, int32_t layer, in
       LayerDev& L = e->layers[l];
       rc = launch_fused_qkv_attn(L.wqkv.stream_order, L.wqkv.scale, L.wqkv.zp, L.wqkv.m, e->hidden, L.gamma, e->cfg.eps,
                                  e->cos_t, e->sin_t, L.kcache, L.vcache, kv_blocked(e->n_heads), e->q, e->ctx,
-                                 e->score_tag, e->handover_status, e->d_state, l, 1, e->n_heads,
+                                 e->score_tag, e->handover_status, e->d_state, l, 1, pos + 1, e->n_heads,
                                  l == layer ? d_stamps : nullptr, e->stream);
     }
   }
@@ -1399,7 +1399,7 @@ extern "C" int awq_qkv_attention(const void* wqkv_repacked, const void* scale, c
   return launch_fused_qkv_attn(wqkv_repacked, (const half_t*)scale, (const half_t*)zp, 3 * hidden, (const half_t*)x,
                                (const half_t*)gamma, eps, (const half_t*)cos_t, (const half_t*)sin_t, (half_t*)k_cache,
                                (half_t*)v_cache, kv_head_major(max_pos), (half_t*)q_out, (half_t*)ctx, score_tag,
-                               (int32_t*)(ws + 128), (const StepState*)ws, 0, 0, n_heads, nullptr, st);
+                               (int32_t*)(ws + 128), (const StepState*)ws, 0, 0, L > 0 ? L : 1, n_heads, nullptr, st);
 }
 
 // after the stream has drained: 0, or AWQ_ERR_HIP when a wait of the last launches gave up (the word is cleared)

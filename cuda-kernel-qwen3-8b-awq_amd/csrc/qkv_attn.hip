@@ -1,6 +1,6 @@
 // The first two launches of a decoder layer as ONE: RMSNorm + Wqkv + rotary + KV append (Inference.cu:1040-1103)
 // and the attention over the cache (Inference.cu:1110, attentionKernel :182-267), for attended lengths that the
-// attention covers in at most two launches of its own (kFusedQkvAttnMax = kAttnTwoLaunchMax).
+// attention covers in at most three launches of its own (kFusedQkvAttnMax = kAttnMergedMax).
 //
 // Of all the boundaries between a layer's launches this is the one across which the data dependence is local:
 // the attention of head h needs rows 128 h .. 128 h + 127 of Q and of K and nothing else of the product.  A
@@ -46,13 +46,16 @@ constexpr int kG = 2;               // blocks per lane and row group
 constexpr int kParts = 8;           // workgroups per head
 constexpr int kDP = AWQ_HEAD_DIM / kParts;  // dimensions per workgroup: one 16-row group each of Q, K and V
 constexpr int kMaxLen = (int)kFusedQkvAttnMax;
-constexpr int kChunkCap = 16;       // chunks of 64 positions: one per wavefront
+constexpr int kMaxCPW = 2;          // chunks of 64 positions per wavefront: 1 up to 1024 attended positions, 2 beyond
+constexpr int kChunkCap = kMaxCPW * kWaves;
 constexpr int kScoreStride = kChunkCap * 64;  // (score, tag) pairs per head in the exchange buffer
 static_assert(kDP == 16 && kMaxLen <= kChunkCap * 64 && kMaxLen <= kScoreStride, "shape of the fused launch");
 // Wavefront 0 finishes the product (rotary, stores): what queues behind bulk requests in the compute unit's
-// memory pipeline waits for them, so the chunks of the cache go to the wavefronts from the last one down and
-// wavefront 0 streams one only beyond 960 attended positions.
-static_assert((kMaxLen + 63) / 64 <= kWaves, "one chunk of keys and values per wavefront");
+// memory pipeline waits for them, so chunk c of the cache goes to wavefront 1 + c % 16 for c % 16 < 15 and
+// wavefront 0 streams one only beyond 960 attended positions.  (Handing the chunks out from the last wavefront
+// down instead measured 981 against 987 tok/s.)
+static_assert((kMaxLen + 63) / 64 <= kChunkCap, "kMaxCPW chunks of keys and values per wavefront");
+static_assert(kChunkCap * 64 * sizeof(float) == kK * sizeof(half_t), "the scores take the place of x in natural order");
 
 struct QkvAttnArgs {
   const u32x4* wq;
@@ -91,15 +94,15 @@ __device__ __forceinline__ u32x4 load_l2_16(const void* p) {
 // eight 8-byte pieces `stride` bytes apart the same way
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ void load_l2_8x8(const char* p, u32x2 (&v)[8]) {
-  static_assert(kScoreStride * 8 == 8192, "piece stride in the instruction offsets below");
-  const char* p2 = p + 4 * 8192;
+  constexpr int kPiece = kScoreStride * 8;  // bytes between the workgroups' pieces of one position
+  const char* p2 = p + 4 * kPiece;
   asm volatile(
       "global_load_dwordx2 %0, %8, off nt\n\tglobal_load_dwordx2 %1, %9, off nt\n\t"
       "global_load_dwordx2 %2, %10, off nt\n\tglobal_load_dwordx2 %3, %11, off nt\n\t"
       "global_load_dwordx2 %4, %12, off nt\n\tglobal_load_dwordx2 %5, %13, off nt\n\t"
       "global_load_dwordx2 %6, %14, off nt\n\tglobal_load_dwordx2 %7, %15, off nt\n\ts_waitcnt vmcnt(0)"
       : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]), "=&v"(v[6]), "=&v"(v[7])
-      : "v"(p), "v"(p + 8192), "v"(p + 2 * 8192), "v"(p + 3 * 8192), "v"(p2), "v"(p2 + 8192), "v"(p2 + 2 * 8192), "v"(p2 + 3 * 8192)
+      : "v"(p), "v"(p + kPiece), "v"(p + 2 * kPiece), "v"(p + 3 * kPiece), "v"(p2), "v"(p2 + kPiece), "v"(p2 + 2 * kPiece), "v"(p2 + 3 * kPiece)
       : "memory");
 }
 
@@ -165,16 +168,18 @@ __global__ __launch_bounds__(64) void die_probe_kernel(int32_t* die_of) {
   if (threadIdx.x == 0) die_of[blockIdx.x] = __builtin_amdgcn_s_getreg((20) | (0 << 6) | ((4 - 1) << 11)) & 15;  // XCC_ID
 }
 
-template <bool STAMPS>
+// kCPW: chunks per wavefront (the launcher's bound on the attended length is 1024 kCPW)
+template <bool STAMPS, int kCPW>
 __global__ __launch_bounds__(kThreads) void qkv_attn_kernel(QkvAttnArgs a) {
+  constexpr int kChunks = kCPW * kWaves;  // of this instance; the LDS arrays and the exchange buffer are laid out for kChunkCap
   __shared__ __attribute__((aligned(16))) unsigned char xs[kBlocks * 64];  // byte planes, 64 bytes per block
   __shared__ __attribute__((aligned(16))) float xc[kBlocks];
   __shared__ __attribute__((aligned(16))) float xS[kBlocks];
-  __shared__ __attribute__((aligned(16))) half_t xn[kK];
+  __shared__ __attribute__((aligned(16))) float s[kChunkCap * 64];  // the scores; before them, x in natural order
+  half_t* const xn = reinterpret_cast<half_t*>(s);
   __shared__ float red[3][16][16];
   __shared__ __attribute__((aligned(16))) float part_sum[256];
   __shared__ __attribute__((aligned(16))) half_t own[3 * kDP];  // this workgroup's 16 dimensions of the rotated Q, of the new key and of the new value
-  __shared__ float s[kChunkCap * 64];
   __shared__ __attribute__((aligned(16))) half_t vt[kWaves][64 * kDP];  // a wavefront's chunk of values, [position][dimension]
   __shared__ float cs[kChunkCap];
   __shared__ float wmax[kWaves];
@@ -203,7 +208,7 @@ __global__ __launch_bounds__(kThreads) void qkv_attn_kernel(QkvAttnArgs a) {
   }
   const int32_t pos = a.dyn->pos;
   // (the launcher's bound is kMaxLen; the clamp keeps every index inside the arrays whatever the state says)
-  const int32_t L = min(a.use_len_hi ? a.dyn->len_hi : a.dyn->len_lo, kChunkCap * 64);
+  const int32_t L = min(a.use_len_hi ? a.dyn->len_hi : a.dyn->len_lo, kChunks * 64);
   const int32_t epoch = a.dyn->epoch;
   const int32_t gave_up_before = __hip_atomic_load(a.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   // the three row groups of this workgroup: dimensions 16 part .. + 15 of the head's Q, K and V
@@ -297,20 +302,21 @@ __global__ __launch_bounds__(kThreads) void qkv_attn_kernel(QkvAttnArgs a) {
   // behind them: one chunk of 64 positions per wavefront, this workgroup's 16 dimensions of every key and
   // value row as two 16-byte pieces (lane = (position % 32, piece))
   const int nchunks = (L + 63) >> 6;
-  const int aw = kWaves - 1 - wave;  // the chunk of this wavefront
-  const bool streams = aw < nchunks;
-  half8v_t kraw[2], vraw[2];
-  if (streams) {
+  const int aw = wave == 0 ? kWaves - 1 : wave - 1;  // this wavefront's chunks are aw, aw + 16
+  half8v_t kraw[kCPW][2], vraw[kCPW][2];
+  {
     const int64_t col = kDP * part + 8 * (lane & 1);
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int t = (aw << 6) + 32 * j + (lane >> 1);
-      if (t < L) {
-        const int64_t row = kv_row(a.kv, head, t) + col;
-        kraw[j] = *reinterpret_cast<const half8v_t*>(a.k_cache + row);
-        vraw[j] = *reinterpret_cast<const half8v_t*>(a.v_cache + row);
+    for (int i = 0; i < kCPW; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int t = ((aw + kWaves * i) << 6) + 32 * j + (lane >> 1);
+        if (t < L) {
+          const int64_t row = kv_row(a.kv, head, t) + col;
+          kraw[i][j] = *reinterpret_cast<const half8v_t*>(a.k_cache + row);
+          vraw[i][j] = *reinterpret_cast<const half8v_t*>(a.v_cache + row);
+        }
       }
-    }
   }
 
   // ---- the three products (Inference.cu:1052)
@@ -344,8 +350,8 @@ __global__ __launch_bounds__(kThreads) void qkv_attn_kernel(QkvAttnArgs a) {
   }
   // the sums below add all kChunkCap entries unconditionally: zeros where there is no chunk (x + 0 is x for the
   // non-negative sums and for the chunk vectors, which are never -0: every chain starts at +0)
-  if (tid >= nchunks && tid < kChunkCap) cs[tid] = 0.0f;
-  if (tid < kChunkCap * kDP && (tid >> 4) >= nchunks) cv[tid] = 0.0f;
+  if (tid >= nchunks && tid < kChunks) cs[tid] = 0.0f;
+  if (tid < kChunks * kDP && (tid >> 4) >= nchunks) cv[tid] = 0.0f;
   stamp();  // 4 products multiplied (this wavefront: its weights have arrived)
   __syncthreads();
   stamp();  // 5 ... by all wavefronts
@@ -384,73 +390,89 @@ __global__ __launch_bounds__(kThreads) void qkv_attn_kernel(QkvAttnArgs a) {
   // ---- this workgroup's share of every score (Inference.cu:202-226): lane (position, piece) runs the chain of
   // eight dimensions of its piece, the two pieces of a position are added (the first level of the dot
   // product's adjacent-pair tree), and the sum is published
-  if (streams) {
+  if (aw < nchunks) {
     float qf[8];
     const half8v_t qv = *reinterpret_cast<const half8v_t*>(own + 8 * (lane & 1));
     const half8v_t knew = *reinterpret_cast<const half8v_t*>(own + kDP + 8 * (lane & 1));
 #pragma unroll
     for (int i = 0; i < 8; ++i) qf[i] = (float)qv[i];
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int t = (aw << 6) + 32 * j + (lane >> 1);
-      const half8v_t kv = t == pos ? knew : kraw[j];  // not from the row just written
-      float pt = 0.0f;
-      if (t < L) {
+    for (int i = 0; i < kCPW; ++i)
 #pragma unroll
-        for (int i = 0; i < 8; ++i) pt = __builtin_fmaf(qf[i], (float)kv[i], pt);
+      for (int j = 0; j < 2; ++j) {
+        const int t = ((aw + kWaves * i) << 6) + 32 * j + (lane >> 1);
+        const half8v_t kv = t == pos ? knew : kraw[i][j];  // not from the row just written
+        float pt = 0.0f;
+        if (t < L) {
+#pragma unroll
+          for (int d = 0; d < 8; ++d) pt = __builtin_fmaf(qf[d], (float)kv[d], pt);
+        }
+        pt = add_dpp<kDppXor1>(pt);
+        if (t < L && (lane & 1) == 0) {
+          const uint32_t bits = __builtin_bit_cast(uint32_t, pt);
+          uint32_t* dst = a.score_tag + (((size_t)head * kParts + part) * kScoreStride + t) * 2;
+          __builtin_nontemporal_store((bits & 0xffffu) | (tag16 << 16), dst);
+          __builtin_nontemporal_store((bits >> 16) | (tag16 << 16), dst + 1);
+        }
       }
-      pt = add_dpp<kDppXor1>(pt);
-      if (t < L && (lane & 1) == 0) {
-        const uint32_t bits = __builtin_bit_cast(uint32_t, pt);
-        uint32_t* dst = a.score_tag + (((size_t)head * kParts + part) * kScoreStride + t) * 2;
-        __builtin_nontemporal_store((bits & 0xffffu) | (tag16 << 16), dst);
-        __builtin_nontemporal_store((bits >> 16) | (tag16 << 16), dst + 1);
-      }
-      // this wavefront's chunk of values into the order of the sums: [position][dimension]
-      if (t < L) *reinterpret_cast<half8v_t*>(&vt[aw][(32 * j + (lane >> 1)) * kDP + 8 * (lane & 1)]) = vraw[j];
-    }
   }
+  // this wavefront's first chunk of values into the order of the sums, [position][dimension], while the other
+  // workgroups' partial scores are on their way
+  auto values_to_lds = [&](int i) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int t = ((aw + kWaves * i) << 6) + 32 * j + (lane >> 1);
+      if (t < L) *reinterpret_cast<half8v_t*>(&vt[wave][(32 * j + (lane >> 1)) * kDP + 8 * (lane & 1)]) = vraw[i][j];
+    }
+  };
+  if (aw < nchunks) values_to_lds(0);
   stamp();  // 8 partial scores published (this wavefront)
   if ((wave << 6) < L) {
-    // the eight partial scores of position tid: the rest of the tree (Inference.cu:218 scales the sum)
-    const bool mine = tid < L;
-    const char* src = reinterpret_cast<const char*>(a.score_tag + ((size_t)head * kParts * kScoreStride + tid) * 2);
+    // the eight partial scores of positions tid and tid + 1024: the rest of the tree (Inference.cu:218 scales the sum)
     const float scale = 1.0f / sqrtf((float)AWQ_HEAD_DIM);
-    int spins = 0;
     bool dead = gave_up_before != 0;
-    float my_score = -1e9f;
-    while (!dead) {
-      int32_t st = 0;
-      const bool look = (spins & 7) == 7;  // every eighth poll also reads the status word
-      if (look) st = __hip_atomic_load(a.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      u32x2 w[8];
-      bool ok = true;
-      if (mine) {
-        load_l2_8x8(src, w);
+    float my_max = -1e9f;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) ok = ok && (w[i].x >> 16) == tag16 && (w[i].y >> 16) == tag16;
-      }
-      if (__builtin_amdgcn_ballot_w64(!ok) == 0) {
+    for (int i = 0; i < kCPW; ++i) {
+      const int t = tid + kThreads * i;
+      if ((wave << 6) + kThreads * i >= L) break;  // the same for the whole wavefront
+      const bool mine = t < L;
+      const char* src = reinterpret_cast<const char*>(a.score_tag + ((size_t)head * kParts * kScoreStride + t) * 2);
+      int spins = 0;
+      while (!dead) {
+        int32_t st = 0;
+        const bool look = (spins & 7) == 7;  // every eighth poll also reads the status word
+        if (look) st = __hip_atomic_load(a.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        u32x2 w[8];
+        bool ok = true;
         if (mine) {
-          float p8[8];
+          load_l2_8x8(src, w);
 #pragma unroll
-          for (int i = 0; i < 8; ++i) p8[i] = __builtin_bit_cast(float, (w[i].x & 0xffffu) | (w[i].y << 16));
-          const float tot = ((p8[0] + p8[1]) + (p8[2] + p8[3])) + ((p8[4] + p8[5]) + (p8[6] + p8[7]));
-          my_score = tot * scale;
-          s[tid] = my_score;
+          for (int j = 0; j < 8; ++j) ok = ok && (w[j].x >> 16) == tag16 && (w[j].y >> 16) == tag16;
         }
-        break;
+        if (__builtin_amdgcn_ballot_w64(!ok) == 0) {
+          if (mine) {
+            float p8[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) p8[j] = __builtin_bit_cast(float, (w[j].x & 0xffffu) | (w[j].y << 16));
+            const float tot = ((p8[0] + p8[1]) + (p8[2] + p8[3])) + ((p8[4] + p8[5]) + (p8[6] + p8[7]));
+            const float sc = tot * scale;
+            s[t] = sc;
+            my_max = fmaxf(my_max, sc);
+          }
+          break;
+        }
+        if (++spins > a.spin_limit) {
+          if (lane == 0) __hip_atomic_store(a.status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          dead = true;
+        }
+        if (look && st != 0) dead = true;
       }
-      if (++spins > a.spin_limit) {
-        if (lane == 0) __hip_atomic_store(a.status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        dead = true;
-      }
-      if (look && st != 0) dead = true;
     }
     if (dead && lane == 0) lost = 1;
     // maximum (Inference.cu:229-233; it does not depend on the order): this wavefront's positions
-    my_score = wave_maxf(my_score);
-    if (lane == 0) wmax[wave] = my_score;
+    my_max = wave_maxf(my_max);
+    if (lane == 0) wmax[wave] = my_max;
   } else if (lane == 0) {
     wmax[wave] = -1e9f;
   }
@@ -461,36 +483,54 @@ __global__ __launch_bounds__(kThreads) void qkv_attn_kernel(QkvAttnArgs a) {
   float mx = lane < kWaves ? wmax[lane] : -1e9f;
   mx = wave_maxf(mx);
 
-  // ---- exponentials and their sum (Inference.cu:239-249), one wavefront per chunk
-  float e_lane = 0.0f;  // the exponential of position 64 aw + lane stays in its register
-  if (streams) {
-    const int t = (aw << 6) + lane;
-    if (t < L) e_lane = awq_expf(s[t] - mx);
-    const float e = wave_sum(e_lane);
-    if (lane == 0) cs[aw] = e;
-  }
-  // this lane's values of its chunk, read before the barrier: they do not depend on the normaliser
-  half_t vv[16];
-  if (streams) {
+  // ---- exponentials and their sum (Inference.cu:239-249), a chunk at a time; the exponential of position
+  // 64 chunk + lane stays in its register
+  float e_lane[kCPW];
 #pragma unroll
-    for (int nl = 0; nl < 16; ++nl) vv[nl] = vt[aw][(4 * nl + tq) * kDP + dl];
+  for (int i = 0; i < kCPW; ++i) {
+    const int c = aw + kWaves * i;
+    e_lane[i] = 0.0f;
+    if (c < nchunks) {
+      const int t = (c << 6) + lane;
+      if (t < L) e_lane[i] = awq_expf(s[t] - mx);
+      const float e = wave_sum(e_lane[i]);
+      if (lane == 0) cs[c] = e;
+    }
   }
+  // this lane's part of the first chunk's values back, ahead of the barrier: it does not depend on the normaliser
+  auto values_of = [&](half_t (&vv)[16]) {
+#pragma unroll
+    for (int nl = 0; nl < 16; ++nl) vv[nl] = vt[wave][(4 * nl + tq) * kDP + dl];
+  };
+  half_t vv0[16];
+  if (aw < nchunks) values_of(vv0);
   __syncthreads();
   float Z;
   {
-    float zc[kChunkCap];
+    float zc[kChunks];
 #pragma unroll
-    for (int c = 0; c < kChunkCap; ++c) zc[c] = cs[c];
+    for (int c = 0; c < kChunks; ++c) zc[c] = cs[c];
     Z = zc[0];
 #pragma unroll
-    for (int c = 1; c < kChunkCap; ++c) Z += zc[c];
+    for (int c = 1; c < kChunks; ++c) Z += zc[c];
   }
 
-  // ---- weighted sum of V (Inference.cu:251-265), one wavefront per chunk: lane (tq, dl) runs the chain of
-  // positions 4 nl + tq for dimension dl
-  if (streams) {
-    const int base = aw << 6;
-    const float p_lane = base + lane < L ? e_lane / Z : 0.0f;
+  // ---- weighted sum of V (Inference.cu:251-265), a chunk at a time: lane (tq, dl) runs the chain of positions
+  // 4 nl + tq for dimension dl
+#pragma unroll
+  for (int i = 0; i < kCPW; ++i) {
+    const int c = aw + kWaves * i;
+    if (c >= nchunks) break;  // the same for the whole wavefront
+    const int base = c << 6;
+    half_t vv[16];
+    if (i == 0) {
+#pragma unroll
+      for (int nl = 0; nl < 16; ++nl) vv[nl] = vv0[nl];
+    } else {
+      values_to_lds(i);  // the wavefront's LDS accesses execute in order: the slot is free again
+      values_of(vv);
+    }
+    const float p_lane = base + lane < L ? e_lane[i] / Z : 0.0f;
     float acc = 0.0f;
     float pp[16];
 #pragma unroll
@@ -504,16 +544,16 @@ __global__ __launch_bounds__(kThreads) void qkv_attn_kernel(QkvAttnArgs a) {
     }
     acc = add_swap16(acc);
     acc = add_swap32(acc);
-    if (tq == 0) cv[aw * kDP + dl] = acc;
+    if (tq == 0) cv[c * kDP + dl] = acc;
   }
   __syncthreads();
   if (tid < kDP) {
-    float oc[kChunkCap];
+    float oc[kChunks];
 #pragma unroll
-    for (int c = 0; c < kChunkCap; ++c) oc[c] = cv[c * kDP + tid];
+    for (int c = 0; c < kChunks; ++c) oc[c] = cv[c * kDP + tid];
     float out = oc[0];
 #pragma unroll
-    for (int c = 1; c < kChunkCap; ++c) out += oc[c];
+    for (int c = 1; c < kChunks; ++c) out += oc[c];
     a.ctx[head * AWQ_HEAD_DIM + kDP * part + tid] = (half_t)out;
   }
   stamp();  // 10 end
@@ -528,7 +568,7 @@ int fused_qkv_attn_supported(int64_t hidden, int n_heads, hipStream_t st) {
   int dev = 0, cus = 0, occ = 0;
   if (hipGetDevice(&dev) != hipSuccess) return 0;
   if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
-  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, qkv_attn_kernel<false>, kThreads, 0) != hipSuccess) return 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, qkv_attn_kernel<false, kMaxCPW>, kThreads, 0) != hipSuccess) return 0;
   const int n_wg = n_heads * kParts;
   if (occ < 1 || (int64_t)cus * occ < n_wg) return 0;
   int32_t* d = nullptr;
@@ -548,7 +588,7 @@ int fused_qkv_attn_supported(int64_t hidden, int n_heads, hipStream_t st) {
 int launch_fused_qkv_attn(const void* wq, const half_t* scale, const half_t* zp, int64_t m, const half_t* x,
                           const half_t* gamma, float eps, const half_t* cos_t, const half_t* sin_t, half_t* k_cache,
                           half_t* v_cache, KvLayout kv, half_t* q_out, half_t* ctx, uint32_t* score_tag, int32_t* status, const StepState* dyn, int layer,
-                          int use_len_hi, int n_heads, unsigned long long* stamps, hipStream_t st) {
+                          int use_len_hi, int64_t len_bound, int n_heads, unsigned long long* stamps, hipStream_t st) {
   AWQ_REQUIRE(m == 3 * kK && n_heads == kK / AWQ_HEAD_DIM, "the fused launch is built for hidden 4096 and 32 heads");
   AWQ_REQUIRE(wq && x && gamma && cos_t && sin_t && k_cache && v_cache && q_out && ctx && score_tag && status && dyn,
               "NULL pointer");
@@ -574,8 +614,15 @@ int launch_fused_qkv_attn(const void* wq, const half_t* scale, const half_t* zp,
   a.mg = (int32_t)(m / 128);
   a.eps = eps;
   a.stamps = stamps;
-  if (stamps) hipLaunchKernelGGL(qkv_attn_kernel<true>, dim3((unsigned)(n_heads * kParts)), dim3(kThreads), 0, st, a);
-  else hipLaunchKernelGGL(qkv_attn_kernel<false>, dim3((unsigned)(n_heads * kParts)), dim3(kThreads), 0, st, a);
+  AWQ_REQUIRE(len_bound > 0 && len_bound <= kMaxLen, "attended length beyond what the fused launch covers");
+  const dim3 grid((unsigned)(n_heads * kParts)), block(kThreads);
+  if (len_bound <= 64 * kWaves) {
+    if (stamps) hipLaunchKernelGGL((qkv_attn_kernel<true, 1>), grid, block, 0, st, a);
+    else hipLaunchKernelGGL((qkv_attn_kernel<false, 1>), grid, block, 0, st, a);
+  } else {
+    if (stamps) hipLaunchKernelGGL((qkv_attn_kernel<true, 2>), grid, block, 0, st, a);
+    else hipLaunchKernelGGL((qkv_attn_kernel<false, 2>), grid, block, 0, st, a);
+  }
   AWQ_HIP_TRY(hipGetLastError());
   return AWQ_OK;
 }

@@ -114,7 +114,7 @@ int awq_debug_force_handover_giveup(awq_engine* e, int on);
  *      through memory, W1's weights requested while that hand-over is under way
  *      (hidden 4096 / intermediate 12288);
  *   2  RMSNorm + Wqkv + rotary + KV append (:1040-1103) and the attention
- *      (:1110) up to 1024 attended positions: the eight workgroups of a head sit
+ *      (:1110) up to 2048 attended positions: the eight workgroups of a head sit
  *      on one die and hand partial scores to each other through its L2 (hidden
  *      4096, 32 heads; longer sequences keep the two launches).
  * Both are off by default: on MI355X the first measures 2 % slower than the two
@@ -141,7 +141,7 @@ int awq_fused_mode(const awq_engine* e);
 int awq_debug_fused_timeline(awq_engine* e, int32_t layer, uint64_t* host_out, int32_t* n_workgroups,
                              int32_t* n_stamps);
 /* The same for the fused Wqkv + attention launch, at position `pos` attending
- * pos + 1 positions (pos < 1024). */
+ * pos + 1 positions (pos < 2048). */
 int awq_debug_qkv_attention_timeline(awq_engine* e, int32_t layer, int32_t pos, uint64_t* host_out,
                                      int32_t* n_workgroups, int32_t* n_stamps);
 
@@ -334,7 +334,7 @@ int awq_decode_attention_static(const void* q, const void* k_cache, const void* 
  * append) and awq_decode_attention as ONE launch for hidden 4096 and 32 heads
  * (wqkv_repacked is the 12288 x 4096 matrix from awq_linear_repack; caches
  * [head][max_pos][128]; x, gamma [4096]; q_out, ctx [4096]), position `pos`
- * attending the first L positions, L <= pos + 1 and L <= 1024.  Same bits as the
+ * attending the first L positions, L <= pos + 1 and L <= 2048.  Same bits as the
  * two calls.  Every head is given to eight workgroups that the device places on
  * one die (awq_qkv_attention_supported probes that and that all 256 workgroups
  * are resident at once: 1 = yes); they hand partial scores to each other through

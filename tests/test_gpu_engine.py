@@ -496,7 +496,7 @@ def test_fused_qkv_attention_launch_is_bit_identical_and_gives_up_cleanly(awq, l
     is set before the call, so every wait ends at its first look and every kernel runs to its end): the call
     fails with AWQ_ERR_HIP and the engine works again after a reset.  Last, the instrumented launch behind
     awq_debug_qkv_attention_timeline returns ordered time stamps."""
-    cfg = awq.make_config(n_layers=2, max_pos=1024)
+    cfg = awq.make_config(n_layers=2, max_pos=1152)
     model = make_oracle_model(oracle, cfg)
     eng = awq.QWen3AWQInfer.empty(cfg)
     fill_pair(awq, oracle, cfg, 2025, engine=eng, model=model, profile=awq.SYNTH_BALANCED)
@@ -534,12 +534,13 @@ def test_fused_qkv_attention_launch_is_bit_identical_and_gives_up_cleanly(awq, l
     t = buf[:nw.value * ns.value].reshape(nw.value, ns.value).astype(np.int64)
     assert nw.value == 256 and ns.value >= 8 and (np.diff(t, axis=1) >= 0).all()
     assert 0 < (t[:, -1].max() - t[:, 0].min()) * 0.01 < 1000.0     # microseconds
-    # a long prompt token by token: attended lengths up to 760, across the 704 at which the separate attention
-    # switches from one launch to two (the fused launch covers both)
+    # a long prompt token by token: attended lengths up to 1060, across the 704 and the 1024 at which the separate
+    # attention switches from one launch to two and to three (the fused launch covers all of them, with a second
+    # chunk of 64 positions per wavefront beyond 1024)
     eng.set_fused_mode(eng.FUSED_QKV_ATTN)
-    long_prompt = rng.integers(0, cfg.vocab, 700).tolist()
-    print("fused Wqkv + attention launch, 700-token prompt", flush=True)
-    assert eng.generateResponse(long_prompt, 60) == oracle_generate(oracle, model, long_prompt, 60)
+    long_prompt = rng.integers(0, cfg.vocab, 1010).tolist()
+    print("fused Wqkv + attention launch, 1010-token prompt", flush=True)
+    assert eng.generateResponse(long_prompt, 50) == oracle_generate(oracle, model, long_prompt, 50)
     compare_state(awq, oracle, eng, model, cfg)
     eng.set_fused_mode(0)
     assert eng.generateResponse(prompt, 100) == ref

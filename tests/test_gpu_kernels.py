@@ -594,7 +594,8 @@ def test_gemv_fused_norm_unembed_argmax(awq, lib, oracle, torch_gpu, m, k):
 
 # ----------------------------------------------------------------------------- Wqkv + attention as one launch
 @pytest.mark.parametrize("pos,L", [(0, 1), (1, 1), (2, 2), (2, 3), (5, 5), (63, 64), (70, 71), (300, 301), (640, 640),
-                                   (703, 704), (704, 705), (959, 960), (960, 961), (1023, 1023), (1023, 1024)])
+                                   (703, 704), (704, 705), (959, 960), (960, 961), (1023, 1023), (1023, 1024),
+                                   (1024, 1025), (1500, 1501), (1984, 1985), (2047, 2048)])
 def test_fused_qkv_attention_launch_against_the_two_launches_and_the_oracle(awq, lib, oracle, torch_gpu, pos, L):
     """awq_qkv_attention: RMSNorm + Wqkv + rotary + KV append and the attention over the cache in one launch whose
     eight workgroups per head hand partial scores to each other through the L2 of their die.  Q, the caches and
@@ -602,7 +603,7 @@ def test_fused_qkv_attention_launch_against_the_two_launches_and_the_oracle(awq,
     calls in a row (the tags change; the second call finds the first one's words in the exchange buffer)."""
     torch = torch_gpu
     H = 4096
-    m, k, nh, mp = 3 * H, H, H // 128, 1088
+    m, k, nh, mp = 3 * H, H, H // 128, 2112
     if not lib.awq_qkv_attention_supported(H, nh, stream(torch)):
         pytest.skip("this device cannot run the fused launch")
     rng = np.random.default_rng(pos * 1000 + L)
@@ -663,7 +664,7 @@ def test_fused_qkv_attention_launch_against_the_two_launches_and_the_oracle(awq,
     args = [keep["d_w"].data_ptr(), keep["d_s"].data_ptr(), keep["d_z"].data_ptr(), d_h.data_ptr(), d_g.data_ptr(), 1e-6,
             d_c.data_ptr(), d_s.data_ptr(), f_kc.data_ptr(), f_vc.data_ptr(), mp, nh, pos, L, f_q.data_ptr(),
             f_o.data_ptr(), fws.data_ptr(), 3, stream(torch)]
-    for idx, bad in ((11, 16), (12, mp), (13, pos + 2), (17, 0)) + (((13, 1025),) if pos >= 1024 else ()):
+    for idx, bad in ((11, 16), (12, mp), (13, pos + 2), (17, 0)) + (((13, 2049),) if pos >= 2048 else ()):
         wrong = list(args)
         wrong[idx] = bad
         assert lib.awq_qkv_attention(*wrong) != 0
