@@ -69,8 +69,10 @@ SIGNATURES = {
     "awq_debug_force_handover_giveup": (ctypes.c_int, [_vp, ctypes.c_int]),
     "awq_qkv_attention_workspace_bytes": (_i64, [ctypes.c_int32]),
     "awq_qkv_attention_supported": (ctypes.c_int, [_i64, ctypes.c_int32, _vp]),
-    "awq_qkv_attention": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, ctypes.c_float, _vp, _vp, _vp, _vp, _i64, ctypes.c_int32,
-                                         _i64, _i64, _vp, _vp, _vp, ctypes.c_int32, _vp]),
+    "awq_kv_parts_bytes": (_i64, [ctypes.c_int32, _i64]),
+    "awq_kv_cache_to_parts": (ctypes.c_int, [_vp, _vp, _i64, ctypes.c_int32, _vp, _vp, _i64, _i64, _i64, _vp]),
+    "awq_qkv_attention": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, ctypes.c_float, _vp, _vp, _vp, _vp, _i64, _vp, _vp, _i64,
+                                         ctypes.c_int32, _i64, _i64, _vp, _vp, _vp, ctypes.c_int32, _vp]),
     "awq_qkv_attention_status": (ctypes.c_int, [_vp, _vp]),
     "awq_set_fused_mode": (ctypes.c_int, [_vp, ctypes.c_int]),
     "awq_fused_mode": (ctypes.c_int, [_vp]),

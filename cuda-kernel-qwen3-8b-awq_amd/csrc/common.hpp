@@ -220,8 +220,13 @@ int fused_qkv_attn_supported(int64_t hidden, int n_heads, hipStream_t st);
 int64_t fused_qkv_attn_exchange_bytes(int n_heads);
 int launch_fused_qkv_attn(const void* wq, const half_t* scale, const half_t* zp, int64_t m, const half_t* x,
                           const half_t* gamma, float eps, const half_t* cos_t, const half_t* sin_t, half_t* k_cache,
-                          half_t* v_cache, KvLayout kv, half_t* q_out, half_t* ctx, uint32_t* score_tag, int32_t* status, const StepState* dyn, int layer,
+                          half_t* v_cache, KvLayout kv, half_t* k_parts, half_t* v_parts, int parts_pos, half_t* q_out,
+                          half_t* ctx, uint32_t* score_tag, int32_t* status, const StepState* dyn, int layer,
                           int use_len_hi, int64_t len_bound, int n_heads, unsigned long long* stamps, hipStream_t st);
+// the caches a second time in the order the fused launch reads them: [head][8][parts_pos][16]
+int64_t fused_qkv_attn_parts_bytes(int n_heads, int64_t parts_pos);
+int launch_kv_to_parts(const half_t* k_cache, const half_t* v_cache, KvLayout kv, half_t* k_parts, half_t* v_parts,
+                       int n_heads, int parts_pos, int64_t pos0, int64_t n, hipStream_t st);
 constexpr int kQkvStamps = 11;  // time stamps per workgroup of the instrumented launch
 int launch_fill_zero(void* p, int64_t bytes, hipStream_t st);
 int launch_copy(const void* src, void* dst, int64_t bytes, hipStream_t st);

@@ -139,6 +139,9 @@ struct LayerDev {
   bool have_gamma = false;
   half_t* kcache = nullptr;
   half_t* vcache = nullptr;
+  // the first parts_pos positions of both a second time, in the order the fused Wqkv + attention launch reads them
+  half_t* kparts = nullptr;
+  half_t* vparts = nullptr;
 };
 
 }  // namespace
@@ -184,6 +187,7 @@ struct awq_engine {
   // between the eight workgroups of a head
   bool fused_qkv = false;
   uint32_t* score_tag = nullptr;
+  int parts_pos = 0;  // positions the layers' parts arrays hold (0: none allocated, the launch is not available)
   int32_t* handover_status = nullptr;
   int32_t epoch_next = 0;  // the epoch of the next step (mirrors what the device adds per step)
   std::vector<void*> allocations;
@@ -298,10 +302,11 @@ int enqueue_wqkv(awq_engine* e, int l) {
 int enqueue_layer(awq_engine* e, int l, int use_len_hi, int64_t len_bound) {
   LayerDev& L = e->layers[l];
   hipStream_t st = e->stream;
-  if (e->fused_qkv && len_bound <= kFusedQkvAttnMax) {  // :1040-1110 in one launch
+  if (e->fused_qkv && len_bound <= e->parts_pos) {  // :1040-1110 in one launch
     if (int rc = launch_fused_qkv_attn(L.wqkv.stream_order, L.wqkv.scale, L.wqkv.zp, L.wqkv.m, e->hidden, L.gamma,
                                        e->cfg.eps, e->cos_t, e->sin_t, L.kcache, L.vcache, kv_blocked(e->n_heads),
-                                       e->q, e->ctx, e->score_tag, e->handover_status, e->d_state, l,
+                                       L.kparts, L.vparts, e->parts_pos, e->q, e->ctx, e->score_tag,
+                                       e->handover_status, e->d_state, l,
                                        use_len_hi, len_bound, e->n_heads, nullptr, st))
       return rc;
   } else {
@@ -551,9 +556,17 @@ int create_engine(const awq_config* cfg_in, awq_engine** out, bool packed_on_dev
     return fail(AWQ_ERR_HIP);
   }
   e->fused = false;  // measured slower than two launches (904 against 924 tok/s): awq_set_fused_mode switches it on
-  // Wqkv + attention as one launch where the device can run it (985 against 963 tok/s); awq_set_fused_mode(e, 0)
-  // switches it off
+  // Wqkv + attention as one launch where the device can run it (992 against 966 tok/s); awq_set_fused_mode(e, 0)
+  // switches it off.  The launch reads the caches from a second copy in its own order.
   e->fused_qkv = cfg.hidden / AWQ_HEAD_DIM == e->n_heads && fused_qkv_attn_supported(cfg.hidden, e->n_heads, e->stream) != 0;
+  if (e->fused_qkv) {
+    e->parts_pos = (int)std::min<int64_t>((cfg.max_pos + 63) / 64 * 64, kFusedQkvAttnMax);
+    const int64_t parts_bytes = fused_qkv_attn_parts_bytes(e->n_heads, e->parts_pos);
+    for (auto& L : e->layers) {
+      if (int rc = dev_alloc(ep, (void**)&L.kparts, parts_bytes)) return fail(rc);
+      if (int rc = dev_alloc(ep, (void**)&L.vparts, parts_bytes)) return fail(rc);
+    }
+  }
   *out = e.release();
   return AWQ_OK;
 }
@@ -642,6 +655,11 @@ extern "C" int awq_finalize(awq_engine* e) {
   for (auto& L : e->layers) {
     if (int rc = launch_fill_zero(L.kcache, kv_bytes, st)) return rc;
     if (int rc = launch_fill_zero(L.vcache, kv_bytes, st)) return rc;
+    if (L.kparts) {
+      const int64_t parts_bytes = fused_qkv_attn_parts_bytes(e->n_heads, e->parts_pos);
+      if (int rc = launch_fill_zero(L.kparts, parts_bytes, st)) return rc;
+      if (int rc = launch_fill_zero(L.vparts, parts_bytes, st)) return rc;
+    }
   }
   if (int rc = launch_fill_zero(e->sample_ws, gemv_workspace_bytes(e->cfg.vocab, e->cfg.hidden), st)) return rc;
   if (int rc = launch_embed_rows((const uint8_t*)e->embed.packed, e->embed_rows, e->cfg.hidden, e->cfg.vocab, st)) return rc;
@@ -878,7 +896,8 @@ extern "C" int awq_set_fused_mode(awq_engine* e, int enabled) {
   AWQ_REQUIRE(e != nullptr, "engine is NULL");
   // bit 0: Wo + W1 as one launch; bit 1: Wqkv + attention as one launch; each only where the device can run it
   const bool want = (enabled & 1) != 0 && fused_wo_w1_supported(e->cfg.hidden, e->cfg.inter) != 0;
-  const bool want_qkv = (enabled & 2) != 0 && e->cfg.hidden / AWQ_HEAD_DIM == e->n_heads &&
+  // (the parts arrays exist if the launch was available when the engine was created)
+  const bool want_qkv = (enabled & 2) != 0 && e->parts_pos > 0 &&
                         fused_qkv_attn_supported(e->cfg.hidden, e->n_heads, e->stream) != 0;
   if (want != e->fused || want_qkv != e->fused_qkv) {
     // the captured steps hold the other launches
@@ -889,6 +908,15 @@ extern "C" int awq_set_fused_mode(awq_engine* e, int enabled) {
           (void)hipGraphExecDestroy(g);
           g = nullptr;
         }
+    if (want_qkv && !e->fused_qkv && e->n_positions > 0) {
+      // the rows appended while the launch was off
+      const int64_t n = std::min<int64_t>(e->n_positions, e->parts_pos);
+      for (auto& L : e->layers)
+        if (int rc = launch_kv_to_parts(L.kcache, L.vcache, kv_blocked(e->n_heads), L.kparts, L.vparts, e->n_heads,
+                                        e->parts_pos, 0, n, e->stream))
+          return rc;
+      AWQ_HIP_TRY(hipStreamSynchronize(e->stream));
+    }
     e->fused = want;
     e->fused_qkv = want_qkv;
   }
@@ -1013,6 +1041,10 @@ int enqueue_layer_batch(awq_engine* e, int l, int64_t pos0, int64_t M) {
   if (int rc = launch_rope_kv_append_batch(b.qkv, e->cos_t, e->sin_t, b.q, L.kcache, L.vcache, e->n_heads,
                                            e->cfg.max_pos, kv_blocked(e->n_heads), pos0, M, st))
     return rc;  // :1070-1103
+  if (e->fused_qkv && pos0 < e->parts_pos)  // the rows just appended, for the fused launch of the steps that follow
+    if (int rc = launch_kv_to_parts(L.kcache, L.vcache, kv_blocked(e->n_heads), L.kparts, L.vparts, e->n_heads,
+                                    e->parts_pos, pos0, std::min<int64_t>(M, e->parts_pos - pos0), st))
+      return rc;
   if (int rc = launch_prefill_attention(b.q, L.kcache, L.vcache, b.ctx, e->n_heads, e->cfg.max_pos,
                                         kv_blocked(e->n_heads), pos0, M, l >= 1,
                                         st))
@@ -1086,10 +1118,10 @@ extern "C" int awq_debug_qkv_attention_timeline(awq_engine* e, int32_t layer, in
                                                 int32_t* n_workgroups, int32_t* n_stamps) {
   AWQ_REQUIRE(e && host_out && n_workgroups && n_stamps, "NULL argument");
   AWQ_REQUIRE(e->finalized, "awq_debug_qkv_attention_timeline before awq_finalize");
-  AWQ_REQUIRE(fused_qkv_attn_supported(e->cfg.hidden, e->n_heads, e->stream) != 0,
+  AWQ_REQUIRE(e->parts_pos > 0 && fused_qkv_attn_supported(e->cfg.hidden, e->n_heads, e->stream) != 0,
               "the fused launch needs hidden 4096, 32 heads and 256 compute units");
   AWQ_REQUIRE(layer >= 0 && layer < e->cfg.n_layers, "layer out of range");
-  AWQ_REQUIRE(pos >= 0 && pos < e->cfg.max_pos && pos + 1 <= kFusedQkvAttnMax, "pos out of range");
+  AWQ_REQUIRE(pos >= 0 && pos < e->cfg.max_pos && pos + 1 <= e->parts_pos, "pos out of range");
   const int wgs = e->n_heads * 8;
   unsigned long long* d_stamps = nullptr;
   AWQ_HIP_TRY(hipMalloc((void**)&d_stamps, (size_t)wgs * kQkvStamps * 8));
@@ -1102,8 +1134,8 @@ extern "C" int awq_debug_qkv_attention_timeline(awq_engine* e, int32_t layer, in
     for (int l = 0; l < e->cfg.n_layers && rc == AWQ_OK; ++l) {
       LayerDev& L = e->layers[l];
       rc = launch_fused_qkv_attn(L.wqkv.stream_order, L.wqkv.scale, L.wqkv.zp, L.wqkv.m, e->hidden, L.gamma, e->cfg.eps,
-                                 e->cos_t, e->sin_t, L.kcache, L.vcache, kv_blocked(e->n_heads), e->q, e->ctx,
-                                 e->score_tag, e->handover_status, e->d_state, l, 1, pos + 1, e->n_heads,
+                                 e->cos_t, e->sin_t, L.kcache, L.vcache, kv_blocked(e->n_heads), L.kparts, L.vparts,
+                                 e->parts_pos, e->q, e->ctx, e->score_tag, e->handover_status, e->d_state, l, 1, pos + 1, e->n_heads,
                                  l == layer ? d_stamps : nullptr, e->stream);
     }
   }
@@ -1375,14 +1407,30 @@ extern "C" int awq_qkv_attention_supported(int64_t hidden, int32_t n_heads, void
   return fused_qkv_attn_supported(hidden, n_heads, (hipStream_t)stream);
 }
 
+extern "C" int64_t awq_kv_parts_bytes(int32_t n_heads, int64_t parts_pos) {
+  if (n_heads <= 0 || parts_pos <= 0) return -1;
+  return fused_qkv_attn_parts_bytes(n_heads, parts_pos);
+}
+
+extern "C" int awq_kv_cache_to_parts(const void* k_cache, const void* v_cache, int64_t max_pos, int32_t n_heads,
+                                     void* k_parts, void* v_parts, int64_t parts_pos, int64_t pos0, int64_t n,
+                                     void* stream) {
+  AWQ_REQUIRE(max_pos > 0 && pos0 >= 0 && n >= 0 && pos0 + n <= max_pos && parts_pos > 0 && parts_pos < (1ll << 30),
+              "positions out of range");
+  return launch_kv_to_parts((const half_t*)k_cache, (const half_t*)v_cache, kv_head_major(max_pos), (half_t*)k_parts,
+                            (half_t*)v_parts, n_heads, (int)parts_pos, pos0, n, (hipStream_t)stream);
+}
+
 extern "C" int awq_qkv_attention(const void* wqkv_repacked, const void* scale, const void* zp, const void* x,
                                  const void* gamma, float eps, const void* cos_t, const void* sin_t, void* k_cache,
-                                 void* v_cache, int64_t max_pos, int32_t n_heads, int64_t pos, int64_t L, void* q_out,
-                                 void* ctx, void* workspace, int32_t call_tag, void* stream) {
+                                 void* v_cache, int64_t max_pos, void* k_parts, void* v_parts, int64_t parts_pos,
+                                 int32_t n_heads, int64_t pos, int64_t L, void* q_out, void* ctx, void* workspace,
+                                 int32_t call_tag, void* stream) {
   AWQ_REQUIRE(workspace != nullptr, "workspace is NULL");
   AWQ_REQUIRE(n_heads == 32, "the fused launch is built for 32 heads of 128");
   AWQ_REQUIRE(max_pos > 0 && pos >= 0 && pos < max_pos, "pos out of range");
   AWQ_REQUIRE(L >= 0 && L <= pos + 1 && L <= kFusedQkvAttnMax, "attended length out of range for the fused launch");
+  AWQ_REQUIRE(parts_pos > 0 && parts_pos < (1ll << 30) && L <= parts_pos, "the parts arrays do not hold the attended positions");
   AWQ_REQUIRE(call_tag >= 1 && call_tag < (1 << 30), "call_tag must be in [1, 2^30)");
   hipStream_t st = (hipStream_t)stream;
   char* ws = (char*)workspace;
@@ -1398,7 +1446,8 @@ extern "C" int awq_qkv_attention(const void* wqkv_repacked, const void* scale, c
   if (int rc = launch_fill_zero(score_tag, fused_qkv_attn_exchange_bytes(n_heads), st)) return rc;
   return launch_fused_qkv_attn(wqkv_repacked, (const half_t*)scale, (const half_t*)zp, 3 * hidden, (const half_t*)x,
                                (const half_t*)gamma, eps, (const half_t*)cos_t, (const half_t*)sin_t, (half_t*)k_cache,
-                               (half_t*)v_cache, kv_head_major(max_pos), (half_t*)q_out, (half_t*)ctx, score_tag,
+                               (half_t*)v_cache, kv_head_major(max_pos), (half_t*)k_parts, (half_t*)v_parts, (int)parts_pos,
+                               (half_t*)q_out, (half_t*)ctx, score_tag,
                                (int32_t*)(ws + 128), (const StepState*)ws, 0, 0, L > 0 ? L : 1, n_heads, nullptr, st);
 }
 

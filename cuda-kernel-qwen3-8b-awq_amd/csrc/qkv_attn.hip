@@ -20,9 +20,12 @@
 //   data: the same bits); each forms the context of its own 16 dimensions, for which it needs only its own V.
 //   (A first version handed Q and K round first and the finished scores of an eighth of the positions second:
 //   two hand-overs, 0.5 and 0.75 us.)
-// The keys and values a workgroup needs from the cache (its 16 dimensions of every attended position, 32 bytes
-// per row) are requested right behind its weights.  The new position's key and value come from the workgroup's
-// own product, not from the cache rows just written.
+// The keys and values a workgroup needs from the cache are its 16 dimensions of every attended position: 32
+// bytes of every 256-byte row, for which the L2 hands over whole lines.  They are therefore kept a second time
+// in the order of this launch, [head][workgroup of the head][position][16 dimensions] (the "parts" arrays, for
+// positions below their capacity), where a chunk of 64 positions is 2 KB in a row: the launch appends to both
+// forms and reads the second, requested right behind its weights.  The new position's key and value come from
+// the workgroup's own product, not from the rows just written.
 //
 // Every wait is bounded and looks at the status word the other fused launch uses: a workgroup that gives up
 // sets it and stores no context, the others follow, the launch ends, and the host finds the word after the
@@ -67,6 +70,8 @@ struct QkvAttnArgs {
   const half_t* sin_t;
   half_t* k_cache;
   half_t* v_cache;
+  half_t* k_parts;        // [heads][8][parts_pos][16]: the same rows in the order this launch reads them
+  half_t* v_parts;
   half_t* q_out;          // [4096] rotated Q, as the separate launch leaves it
   half_t* ctx;            // [4096] attention output
   uint32_t* score_tag;    // [heads][8 workgroups][kScoreStride][2] the halves of a partial score as (half | tag << 16)
@@ -77,6 +82,7 @@ struct QkvAttnArgs {
   int32_t use_len_hi;
   int32_t spin_limit;
   int32_t mg;             // m / 128 of the matrix
+  int32_t parts_pos;      // positions the parts arrays hold
   float eps;
   unsigned long long* stamps;  // STAMPS: [workgroup][kQkvStamps] times of thread 0, 10 ns units
 };
@@ -166,6 +172,21 @@ __device__ __forceinline__ void head_of(int w, int& head, int& part) {
 
 __global__ __launch_bounds__(64) void die_probe_kernel(int32_t* die_of) {
   if (threadIdx.x == 0) die_of[blockIdx.x] = __builtin_amdgcn_s_getreg((20) | (0 << 6) | ((4 - 1) << 11)) & 15;  // XCC_ID
+}
+
+// rows [pos0, pos0 + n) of both caches into the parts arrays: a thread moves 16 bytes
+__global__ __launch_bounds__(256) void kv_to_parts_kernel(const half_t* __restrict__ kc, const half_t* __restrict__ vc,
+                                                          KvLayout lay, half_t* __restrict__ kp, half_t* __restrict__ vp,
+                                                          int n_heads, int parts_pos, int pos0, int n) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;  // (head, position, piece of 8 dimensions)
+  if (idx >= (int64_t)n_heads * n * 16) return;
+  const int piece = (int)(idx & 15);
+  const int pos = pos0 + (int)((idx >> 4) % n);
+  const int head = (int)((idx >> 4) / n);
+  const int64_t src = kv_row(lay, head, pos) + 8 * piece;
+  const int64_t dst = (((int64_t)head * kParts + (piece >> 1)) * parts_pos + pos) * kDP + 8 * (piece & 1);
+  *reinterpret_cast<uint4*>(kp + dst) = *reinterpret_cast<const uint4*>(kc + src);
+  *reinterpret_cast<uint4*>(vp + dst) = *reinterpret_cast<const uint4*>(vc + src);
 }
 
 // kCPW: chunks per wavefront (the launcher's bound on the attended length is 1024 kCPW)
@@ -305,16 +326,15 @@ __global__ __launch_bounds__(kThreads) void qkv_attn_kernel(QkvAttnArgs a) {
   const int aw = wave == 0 ? kWaves - 1 : wave - 1;  // this wavefront's chunks are aw, aw + 16
   half8v_t kraw[kCPW][2], vraw[kCPW][2];
   {
-    const int64_t col = kDP * part + 8 * (lane & 1);
+    const int64_t base = ((int64_t)head * kParts + part) * a.parts_pos * kDP + 8 * (lane & 1);
 #pragma unroll
     for (int i = 0; i < kCPW; ++i)
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
         const int t = ((aw + kWaves * i) << 6) + 32 * j + (lane >> 1);
         if (t < L) {
-          const int64_t row = kv_row(a.kv, head, t) + col;
-          kraw[i][j] = *reinterpret_cast<const half8v_t*>(a.k_cache + row);
-          vraw[i][j] = *reinterpret_cast<const half8v_t*>(a.v_cache + row);
+          kraw[i][j] = *reinterpret_cast<const half8v_t*>(a.k_parts + base + (int64_t)t * kDP);
+          vraw[i][j] = *reinterpret_cast<const half8v_t*>(a.v_parts + base + (int64_t)t * kDP);
         }
       }
   }
@@ -382,9 +402,16 @@ __global__ __launch_bounds__(kThreads) void qkv_attn_kernel(QkvAttnArgs a) {
   stamp();  // 7 ... and in LDS for all wavefronts
   if (tid < 3 * kDP) {  // the stores, off the path of the scores
     const int sec = tid >> 4, d = kDP * part + r;
-    if (sec == 0) a.q_out[head * AWQ_HEAD_DIM + d] = fin_out;
-    else if (sec == 1) a.k_cache[kv_row(a.kv, head, pos) + d] = fin_out;
-    else a.v_cache[kv_row(a.kv, head, pos) + d] = fin_out;
+    const int64_t prow = (((int64_t)head * kParts + part) * a.parts_pos + pos) * kDP + r;
+    if (sec == 0) {
+      a.q_out[head * AWQ_HEAD_DIM + d] = fin_out;
+    } else if (sec == 1) {
+      a.k_cache[kv_row(a.kv, head, pos) + d] = fin_out;
+      if (pos < a.parts_pos) a.k_parts[prow] = fin_out;
+    } else {
+      a.v_cache[kv_row(a.kv, head, pos) + d] = fin_out;
+      if (pos < a.parts_pos) a.v_parts[prow] = fin_out;
+    }
   }
 
   // ---- this workgroup's share of every score (Inference.cu:202-226): lane (position, piece) runs the chain of
@@ -587,11 +614,14 @@ int fused_qkv_attn_supported(int64_t hidden, int n_heads, hipStream_t st) {
 
 int launch_fused_qkv_attn(const void* wq, const half_t* scale, const half_t* zp, int64_t m, const half_t* x,
                           const half_t* gamma, float eps, const half_t* cos_t, const half_t* sin_t, half_t* k_cache,
-                          half_t* v_cache, KvLayout kv, half_t* q_out, half_t* ctx, uint32_t* score_tag, int32_t* status, const StepState* dyn, int layer,
+                          half_t* v_cache, KvLayout kv, half_t* k_parts, half_t* v_parts, int parts_pos, half_t* q_out,
+                          half_t* ctx, uint32_t* score_tag, int32_t* status, const StepState* dyn, int layer,
                           int use_len_hi, int64_t len_bound, int n_heads, unsigned long long* stamps, hipStream_t st) {
   AWQ_REQUIRE(m == 3 * kK && n_heads == kK / AWQ_HEAD_DIM, "the fused launch is built for hidden 4096 and 32 heads");
-  AWQ_REQUIRE(wq && x && gamma && cos_t && sin_t && k_cache && v_cache && q_out && ctx && score_tag && status && dyn,
+  AWQ_REQUIRE(wq && x && gamma && cos_t && sin_t && k_cache && v_cache && k_parts && v_parts && q_out && ctx && score_tag &&
+                  status && dyn,
               "NULL pointer");
+  AWQ_REQUIRE(parts_pos > 0 && len_bound <= parts_pos, "the parts arrays do not hold the attended positions");
   QkvAttnArgs a;
   a.wq = (const u32x4*)wq;
   a.scale = scale;
@@ -602,6 +632,9 @@ int launch_fused_qkv_attn(const void* wq, const half_t* scale, const half_t* zp,
   a.sin_t = sin_t;
   a.k_cache = k_cache;
   a.v_cache = v_cache;
+  a.k_parts = k_parts;
+  a.v_parts = v_parts;
+  a.parts_pos = parts_pos;
   a.q_out = q_out;
   a.ctx = ctx;
   a.score_tag = score_tag;
@@ -629,4 +662,18 @@ int launch_fused_qkv_attn(const void* wq, const half_t* scale, const half_t* zp,
 
 int64_t fused_qkv_attn_exchange_bytes(int n_heads) {
   return (int64_t)n_heads * kScoreStride * kParts * 8;
+}
+
+int64_t fused_qkv_attn_parts_bytes(int n_heads, int64_t parts_pos) { return (int64_t)n_heads * AWQ_HEAD_DIM * parts_pos * 2; }
+
+int launch_kv_to_parts(const half_t* k_cache, const half_t* v_cache, KvLayout kv, half_t* k_parts, half_t* v_parts,
+                       int n_heads, int parts_pos, int64_t pos0, int64_t n, hipStream_t st) {
+  AWQ_REQUIRE(k_cache && v_cache && k_parts && v_parts, "NULL pointer");
+  AWQ_REQUIRE(n_heads > 0 && parts_pos > 0 && pos0 >= 0 && n >= 0 && pos0 + n <= parts_pos, "positions beyond the parts arrays");
+  if (n == 0) return AWQ_OK;
+  const int64_t threads = (int64_t)n_heads * n * 16;
+  hipLaunchKernelGGL(kv_to_parts_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st, k_cache, v_cache, kv,
+                     k_parts, v_parts, n_heads, parts_pos, (int)pos0, (int)n);
+  AWQ_HIP_TRY(hipGetLastError());
+  return AWQ_OK;
 }

@@ -340,6 +340,12 @@ int awq_decode_attention_static(const void* q, const void* k_cache, const void* 
  * are resident at once: 1 = yes); they hand partial scores to each other through
  * that die's L2, in words that carry a tag derived from call_tag: any value in
  * [1, 2^30) that differs from the previous call's on the same workspace.
+ * Each workgroup reads 16 of a cached row's 128 dimensions, so the launch reads
+ * the caches from a second copy in its own order, k_parts and v_parts,
+ * [head][8][parts_pos][16] FP16 (awq_kv_parts_bytes(n_heads, parts_pos) bytes
+ * each, L <= parts_pos): it appends the new position to the caches AND to
+ * these; rows that got into the caches another way are copied with
+ * awq_kv_cache_to_parts (positions pos0 .. pos0 + n - 1).
  * workspace: awq_qkv_attention_workspace_bytes(n_heads) bytes, zero-filled once;
  * calls on one workspace must not overlap.  A wait that cannot end gives up
  * after a bounded number of polls and leaves ctx unwritten:
@@ -347,10 +353,13 @@ int awq_decode_attention_static(const void* q, const void* k_cache, const void* 
  * once and clears the condition. */
 int64_t awq_qkv_attention_workspace_bytes(int32_t n_heads);
 int awq_qkv_attention_supported(int64_t hidden, int32_t n_heads, void* stream);
+int64_t awq_kv_parts_bytes(int32_t n_heads, int64_t parts_pos);
+int awq_kv_cache_to_parts(const void* k_cache, const void* v_cache, int64_t max_pos, int32_t n_heads, void* k_parts,
+                          void* v_parts, int64_t parts_pos, int64_t pos0, int64_t n, void* stream);
 int awq_qkv_attention(const void* wqkv_repacked, const void* scale, const void* zp, const void* x, const void* gamma,
                       float eps, const void* cos_t, const void* sin_t, void* k_cache, void* v_cache, int64_t max_pos,
-                      int32_t n_heads, int64_t pos, int64_t L, void* q_out, void* ctx, void* workspace,
-                      int32_t call_tag, void* stream);
+                      void* k_parts, void* v_parts, int64_t parts_pos, int32_t n_heads, int64_t pos, int64_t L,
+                      void* q_out, void* ctx, void* workspace, int32_t call_tag, void* stream);
 int awq_qkv_attention_status(void* workspace, void* stream);
 
 /* The same attention for n_tokens consecutive prompt positions pos0 ..

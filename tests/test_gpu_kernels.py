@@ -647,27 +647,42 @@ def test_fused_qkv_attention_launch_against_the_two_launches_and_the_oracle(awq,
     f_q = torch.zeros(H, dtype=torch.float16, device="cuda")
     f_o = torch.zeros(H, dtype=torch.float16, device="cuda")
     fws = torch.zeros(lib.awq_qkv_attention_workspace_bytes(nh), dtype=torch.uint8, device="cuda")
+    # the caches a second time in the launch's own order, [head][8][pp][16]: the rows before pos are copied, the
+    # launch appends row pos itself
+    pp = 2048
+    assert lib.awq_kv_parts_bytes(nh, pp) == nh * 128 * pp * 2
+    f_kp = torch.full((nh * 8 * pp * 16,), 7.0, dtype=torch.float16, device="cuda")
+    f_vp = torch.full((nh * 8 * pp * 16,), 7.0, dtype=torch.float16, device="cuda")
+    awq.check(lib.awq_kv_cache_to_parts(f_kc.data_ptr(), f_vc.data_ptr(), mp, nh, f_kp.data_ptr(), f_vp.data_ptr(), pp, 0,
+                                        pos, stream(torch)))
     print("fused launch pos", pos, "L", L, flush=True)
+    args = [keep["d_w"].data_ptr(), keep["d_s"].data_ptr(), keep["d_z"].data_ptr(), d_h.data_ptr(), d_g.data_ptr(), 1e-6,
+            d_c.data_ptr(), d_s.data_ptr(), f_kc.data_ptr(), f_vc.data_ptr(), mp, f_kp.data_ptr(), f_vp.data_ptr(), pp, nh,
+            pos, L, f_q.data_ptr(), f_o.data_ptr(), fws.data_ptr(), 3, stream(torch)]
     for call in (1, 2):
         f_o.zero_()
-        awq.check(lib.awq_qkv_attention(keep["d_w"].data_ptr(), keep["d_s"].data_ptr(), keep["d_z"].data_ptr(),
-                                        d_h.data_ptr(), d_g.data_ptr(), 1e-6, d_c.data_ptr(), d_s.data_ptr(),
-                                        f_kc.data_ptr(), f_vc.data_ptr(), mp, nh, pos, L, f_q.data_ptr(), f_o.data_ptr(),
-                                        fws.data_ptr(), call, stream(torch)))
+        args[20] = call
+        awq.check(lib.awq_qkv_attention(*args))
         awq.check(lib.awq_qkv_attention_status(fws.data_ptr(), stream(torch)))
         assert np.array_equal(f_q.cpu().numpy().view(np.uint16), q_ref.view(np.uint16))
         assert np.array_equal(f_kc.cpu().numpy().view(np.uint16), kc_ref.view(np.uint16))
         assert np.array_equal(f_vc.cpu().numpy().view(np.uint16), vc_ref.view(np.uint16))
         assert np.array_equal(f_o.cpu().numpy().view(np.uint16), ctx_ref.view(np.uint16))
         assert np.array_equal(f_o.cpu().numpy().view(np.uint16), d_o.cpu().numpy().view(np.uint16))
+        # the second copy: rows 0..pos of the caches, dimension 16 p + d of head h at [h][p][position][d]; nothing else written
+        for parts, ref in ((f_kp, kc_ref), (f_vp, vc_ref)):
+            got = parts.cpu().numpy().view(np.uint16).reshape(nh, 8, pp, 16)
+            want = ref.view(np.uint16).reshape(nh, mp, 8, 16)[:, :pos + 1].transpose(0, 2, 1, 3)
+            assert np.array_equal(got[:, :, :pos + 1], want)
+            assert (got[:, :, pos + 1:] == np.float16(7.0).view(np.uint16)).all()
     # arguments the launch is not built for are refused before anything runs
-    args = [keep["d_w"].data_ptr(), keep["d_s"].data_ptr(), keep["d_z"].data_ptr(), d_h.data_ptr(), d_g.data_ptr(), 1e-6,
-            d_c.data_ptr(), d_s.data_ptr(), f_kc.data_ptr(), f_vc.data_ptr(), mp, nh, pos, L, f_q.data_ptr(),
-            f_o.data_ptr(), fws.data_ptr(), 3, stream(torch)]
-    for idx, bad in ((11, 16), (12, mp), (13, pos + 2), (17, 0)) + (((13, 2049),) if pos >= 2048 else ()):
+    args[20] = 3
+    for idx, bad in ((14, 16), (15, mp), (16, pos + 2), (20, 0), (13, L - 1)):
         wrong = list(args)
         wrong[idx] = bad
         assert lib.awq_qkv_attention(*wrong) != 0
+    assert lib.awq_kv_cache_to_parts(f_kc.data_ptr(), f_vc.data_ptr(), mp, nh, f_kp.data_ptr(), f_vp.data_ptr(), pp, pp - 1,
+                                     2, stream(torch)) != 0
 
 
 # ----------------------------------------------------------------------------- W4A16 GEMM on the matrix cores
