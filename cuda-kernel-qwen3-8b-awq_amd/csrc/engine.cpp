@@ -170,7 +170,7 @@ struct awq_engine {
   int n_generated = 0;
   bool finalized = false;
   bool graph_mode = true;
-  hipGraphExec_t graphs[2][5] = {};  // [prompt|gen][length bound]
+  hipGraphExec_t graphs[2][6] = {};  // [prompt|gen][length bound]
   // activations of the batched prompt pass, [chunk][n] each; allocated at first use
   struct {
     half_t *hidden = nullptr, *norm = nullptr, *qkv = nullptr, *q = nullptr, *ctx = nullptr, *mid = nullptr;
@@ -411,7 +411,7 @@ int run_step(awq_engine* e, bool gen, StepState s, bool write_state = true) {
   // the attention launches are specialised by an upper bound of the attended
   // length (one workgroup per head, or two to four launches cut along the
   // sequence); one captured graph per bound
-  static const int64_t kBounds[5] = {kAttnShortMax, kAttnOneWorkgroupMax, kAttnTwoLaunchMax, kAttnMergedMax, 1 << 30};
+  static const int64_t kBounds[6] = {kAttnShortMax, kAttnOneWorkgroupMax, kAttnTwoLaunchMax, kAttnMergedMax, kFusedQkvAttnMax, 1 << 30};
   int bucket = 0;
   while (s.len_hi > kBounds[bucket]) ++bucket;
   const int64_t len_bound = kBounds[bucket] < e->cfg.max_pos ? kBounds[bucket] : e->cfg.max_pos;

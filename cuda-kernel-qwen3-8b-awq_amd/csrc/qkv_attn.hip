@@ -1,6 +1,6 @@
 // The first two launches of a decoder layer as ONE: RMSNorm + Wqkv + rotary + KV append (Inference.cu:1040-1103)
 // and the attention over the cache (Inference.cu:1110, attentionKernel :182-267), for attended lengths that the
-// attention covers in at most three launches of its own (kFusedQkvAttnMax = kAttnMergedMax).
+// attention covers in at most three launches of its own, and twice as far (kFusedQkvAttnMax).
 //
 // Of all the boundaries between a layer's launches this is the one across which the data dependence is local:
 // the attention of head h needs rows 128 h .. 128 h + 127 of Q and of K and nothing else of the product.  A
@@ -49,7 +49,7 @@ constexpr int kG = 2;               // blocks per lane and row group
 constexpr int kParts = 8;           // workgroups per head
 constexpr int kDP = AWQ_HEAD_DIM / kParts;  // dimensions per workgroup: one 16-row group each of Q, K and V
 constexpr int kMaxLen = (int)kFusedQkvAttnMax;
-constexpr int kMaxCPW = 2;          // chunks of 64 positions per wavefront: 1 up to 1024 attended positions, 2 beyond
+constexpr int kMaxCPW = 3;          // chunks of 64 positions per wavefront: 1 up to 1024 attended positions, 2 up to 2048, 3 beyond
 constexpr int kChunkCap = kMaxCPW * kWaves;
 constexpr int kScoreStride = kChunkCap * 64;  // (score, tag) pairs per head in the exchange buffer
 static_assert(kDP == 16 && kMaxLen <= kChunkCap * 64 && kMaxLen <= kScoreStride, "shape of the fused launch");
@@ -58,7 +58,7 @@ static_assert(kDP == 16 && kMaxLen <= kChunkCap * 64 && kMaxLen <= kScoreStride,
 // wavefront 0 streams one only beyond 960 attended positions.  (Handing the chunks out from the last wavefront
 // down instead measured 981 against 987 tok/s.)
 static_assert((kMaxLen + 63) / 64 <= kChunkCap, "kMaxCPW chunks of keys and values per wavefront");
-static_assert(kChunkCap * 64 * sizeof(float) == kK * sizeof(half_t), "the scores take the place of x in natural order");
+static_assert(kChunkCap * 64 * sizeof(float) >= kK * sizeof(half_t), "the scores take the place of x in natural order");
 
 struct QkvAttnArgs {
   const u32x4* wq;
@@ -204,7 +204,8 @@ __global__ __launch_bounds__(kThreads) void qkv_attn_kernel(QkvAttnArgs a) {
   __shared__ __attribute__((aligned(16))) half_t vt[kWaves][64 * kDP];  // a wavefront's chunk of values, [position][dimension]
   __shared__ float cs[kChunkCap];
   __shared__ float wmax[kWaves];
-  __shared__ float cv[kChunkCap * kDP];
+  float* const cv = reinterpret_cast<float*>(xs);  // [kChunkCap][kDP] chunk vectors, once the products have read the planes
+  static_assert(sizeof(xs) >= kChunkCap * kDP * sizeof(float), "the chunk vectors take the place of the byte planes");
   __shared__ int lost;
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -324,20 +325,20 @@ __global__ __launch_bounds__(kThreads) void qkv_attn_kernel(QkvAttnArgs a) {
   // value row as two 16-byte pieces (lane = (position % 32, piece))
   const int nchunks = (L + 63) >> 6;
   const int aw = wave == 0 ? kWaves - 1 : wave - 1;  // this wavefront's chunks are aw, aw + 16
+  // (the values of a third chunk are requested once the keys' registers are free)
+  constexpr int kVEarly = kCPW < 2 ? kCPW : 2;
   half8v_t kraw[kCPW][2], vraw[kCPW][2];
-  {
-    const int64_t base = ((int64_t)head * kParts + part) * a.parts_pos * kDP + 8 * (lane & 1);
+  const int64_t parts_base = ((int64_t)head * kParts + part) * a.parts_pos * kDP + 8 * (lane & 1);
 #pragma unroll
-    for (int i = 0; i < kCPW; ++i)
+  for (int i = 0; i < kCPW; ++i)
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const int t = ((aw + kWaves * i) << 6) + 32 * j + (lane >> 1);
-        if (t < L) {
-          kraw[i][j] = *reinterpret_cast<const half8v_t*>(a.k_parts + base + (int64_t)t * kDP);
-          vraw[i][j] = *reinterpret_cast<const half8v_t*>(a.v_parts + base + (int64_t)t * kDP);
-        }
+    for (int j = 0; j < 2; ++j) {
+      const int t = ((aw + kWaves * i) << 6) + 32 * j + (lane >> 1);
+      if (t < L) {
+        kraw[i][j] = *reinterpret_cast<const half8v_t*>(a.k_parts + parts_base + (int64_t)t * kDP);
+        if (i < kVEarly) vraw[i][j] = *reinterpret_cast<const half8v_t*>(a.v_parts + parts_base + (int64_t)t * kDP);
       }
-  }
+    }
 
   // ---- the three products (Inference.cu:1052)
   {
@@ -371,10 +372,10 @@ __global__ __launch_bounds__(kThreads) void qkv_attn_kernel(QkvAttnArgs a) {
   // the sums below add all kChunkCap entries unconditionally: zeros where there is no chunk (x + 0 is x for the
   // non-negative sums and for the chunk vectors, which are never -0: every chain starts at +0)
   if (tid >= nchunks && tid < kChunks) cs[tid] = 0.0f;
-  if (tid < kChunks * kDP && (tid >> 4) >= nchunks) cv[tid] = 0.0f;
   stamp();  // 4 products multiplied (this wavefront: its weights have arrived)
   __syncthreads();
   stamp();  // 5 ... by all wavefronts
+  if (tid < kChunks * kDP && (tid >> 4) >= nchunks) cv[tid] = 0.0f;  // (every wavefront is done with the planes)
 
   // ---- split, rotary, KV append (Inference.cu:1070-1103) and the first hand-over
   half_t fin_out = (half_t)0.0f;
@@ -452,6 +453,13 @@ __global__ __launch_bounds__(kThreads) void qkv_attn_kernel(QkvAttnArgs a) {
       if (t < L) *reinterpret_cast<half8v_t*>(&vt[wave][(32 * j + (lane >> 1)) * kDP + 8 * (lane & 1)]) = vraw[i][j];
     }
   };
+#pragma unroll
+  for (int i = kVEarly; i < kCPW; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int t = ((aw + kWaves * i) << 6) + 32 * j + (lane >> 1);
+      if (t < L) vraw[i][j] = *reinterpret_cast<const half8v_t*>(a.v_parts + parts_base + (int64_t)t * kDP);
+    }
   if (aw < nchunks) values_to_lds(0);
   stamp();  // 8 partial scores published (this wavefront)
   if ((wave << 6) < L) {
@@ -652,9 +660,12 @@ int launch_fused_qkv_attn(const void* wq, const half_t* scale, const half_t* zp,
   if (len_bound <= 64 * kWaves) {
     if (stamps) hipLaunchKernelGGL((qkv_attn_kernel<true, 1>), grid, block, 0, st, a);
     else hipLaunchKernelGGL((qkv_attn_kernel<false, 1>), grid, block, 0, st, a);
-  } else {
+  } else if (len_bound <= 2 * 64 * kWaves) {
     if (stamps) hipLaunchKernelGGL((qkv_attn_kernel<true, 2>), grid, block, 0, st, a);
     else hipLaunchKernelGGL((qkv_attn_kernel<false, 2>), grid, block, 0, st, a);
+  } else {
+    if (stamps) hipLaunchKernelGGL((qkv_attn_kernel<true, 3>), grid, block, 0, st, a);
+    else hipLaunchKernelGGL((qkv_attn_kernel<false, 3>), grid, block, 0, st, a);
   }
   AWQ_HIP_TRY(hipGetLastError());
   return AWQ_OK;

@@ -546,3 +546,47 @@ def test_fused_qkv_attention_launch_is_bit_identical_and_gives_up_cleanly(awq, l
     assert eng.generateResponse(prompt, 100) == ref
     eng.close()
     oracle.awqo_model_destroy(model)
+
+
+def test_fused_qkv_attention_launch_across_its_length_bounds(awq, lib, torch_gpu):
+    """The fused Wqkv + attention launch against the two launches it replaces (those are checked against the oracle
+    at these lengths elsewhere) on sequences that cross 2048 positions (a third chunk of 64 positions per
+    wavefront) and 3072 (where the engine goes back to two launches): a batched prompt pass fills the caches and
+    the launch's second copy of them, then generation steps.  Ids, last hidden state and logits bit for bit."""
+    cfg = awq.make_config(n_layers=2, max_pos=3200)
+    eng = awq.QWen3AWQInfer.empty(cfg)
+    for layer, kind, part in awq.tensor_list(cfg):
+        count = cfg.part_count(kind, part)
+        nbytes = count if (part == awq.P_PACKED and kind != awq.T_GAMMA) else 2 * count
+        buf = (ctypes.c_uint8 * nbytes)()
+        awq.check(lib.awq_synth_fill_profile(awq.SYNTH_BALANCED, 77, layer, kind, part, buf, count))
+        eng.upload(layer, kind, part, buf, nbytes)
+    eng.finalize()
+    if not eng.fused_mode() & eng.FUSED_QKV_ATTN:
+        pytest.skip("this device cannot run the fused launch")
+    rng = np.random.default_rng(5)
+    for n_prompt, n_new in ((2020, 60), (3040, 60)):
+        prompt = rng.integers(0, cfg.vocab, n_prompt).tolist()
+        out = []
+        for mode in (0, eng.FUSED_QKV_ATTN):
+            print("prompt", n_prompt, "fused mode", mode, flush=True)
+            eng.reset()
+            eng.set_fused_mode(mode)
+            eng.prefill(prompt, batched=True)
+            ids = eng.decode(n_new)
+            out.append((list(ids), np.ctypeslib.as_array(eng.read_hidden()).copy(),
+                        np.ctypeslib.as_array(eng.read_logits()).copy()))
+        assert out[0][0] == out[1][0] and len(set(out[0][0])) > 1
+        assert np.array_equal(out[0][1], out[1][1]) and np.array_equal(out[0][2], out[1][2])
+    # the mode switched on in the middle of a sequence: the rows the two launches appended are copied over
+    eng.reset()
+    eng.set_fused_mode(0)
+    eng.prefill(prompt[:2500], batched=True)
+    a = list(eng.decode(20))
+    eng.set_fused_mode(eng.FUSED_QKV_ATTN)
+    b = list(eng.decode(20))
+    eng.reset()
+    eng.set_fused_mode(0)
+    eng.prefill(prompt[:2500], batched=True)
+    assert list(eng.decode(40)) == a + b
+    eng.close()
