@@ -186,6 +186,8 @@ struct awq_engine {
   // Wqkv and the attention of a layer as one launch (qkv_attn.hip): the partial scores as tagged words, handed
   // between the eight workgroups of a head
   bool fused_qkv = false;
+  bool handover_gave_up = false;  // a fused launch's wait gave up since awq_generate last cleared this
+  bool giveup_after_reset = false;  // test hook: the next awq_reset leaves the status word set
   uint32_t* score_tag = nullptr;
   int parts_pos = 0;  // positions the layers' parts arrays hold (0: none allocated, the launch is not available)
   int32_t* handover_status = nullptr;
@@ -875,6 +877,11 @@ extern "C" int awq_reset(awq_engine* e) {
   if (e->pb.gemm_ws)
     if (int rc = launch_fill_zero(e->pb.gemm_ws, 8, e->stream)) return rc;
   AWQ_HIP_TRY(hipStreamSynchronize(e->stream));
+  if (e->giveup_after_reset) {  // awq_debug_force_handover_giveup(e, 2): the sequence that starts here meets the condition
+    e->giveup_after_reset = false;
+    const int32_t word = 1;
+    AWQ_HIP_TRY(hipMemcpy(e->handover_status, &word, 4, hipMemcpyHostToDevice));
+  }
   return AWQ_OK;
 }
 
@@ -887,6 +894,7 @@ int check_handover(awq_engine* e) {
   AWQ_HIP_TRY(hipMemcpy(&word, e->handover_status, 4, hipMemcpyDeviceToHost));
   if (word == 0) return AWQ_OK;
   AWQ_HIP_TRY(hipMemset(e->handover_status, 0, 4));
+  e->handover_gave_up = true;
   awq_set_error("a fused launch gave up waiting for what other workgroups hand over");
   return AWQ_ERR_HIP;
 }
@@ -1162,6 +1170,7 @@ extern "C" int awq_debug_force_handover_giveup(awq_engine* e, int on) {
   AWQ_REQUIRE(e != nullptr, "engine is NULL");
   if (int rc = ensure_prefill_buffers(e)) return rc;
   const int32_t word = on ? 1 : 0;
+  e->giveup_after_reset = on == 2;
   AWQ_HIP_TRY(hipStreamSynchronize(e->stream));
   AWQ_HIP_TRY(hipMemcpy((int32_t*)e->pb.gemm_ws + 1, &word, 4, hipMemcpyHostToDevice));
   // the fused launches of the token-by-token steps look at their status word before they wait
@@ -1211,10 +1220,22 @@ extern "C" int awq_generate(awq_engine* e, const int32_t* prompt_ids, int32_t n_
   AWQ_REQUIRE(e != nullptr, "engine is NULL");
   AWQ_REQUIRE(n_prompt >= 0 && max_new_tokens >= 0, "negative count");
   AWQ_REQUIRE((int64_t)n_prompt + max_new_tokens <= e->cfg.max_pos, "prompt + new tokens exceed max_pos");
-  if (int rc = awq_reset(e)) return rc;
-  if (int rc = e->batched_prefill ? awq_prefill_batched(e, prompt_ids, n_prompt) : awq_prefill(e, prompt_ids, n_prompt))
-    return rc;
-  return awq_decode(e, max_new_tokens, out_ids);
+  auto once = [&]() -> int {
+    if (int rc = awq_reset(e)) return rc;
+    if (int rc = e->batched_prefill ? awq_prefill_batched(e, prompt_ids, n_prompt) : awq_prefill(e, prompt_ids, n_prompt))
+      return rc;
+    return awq_decode(e, max_new_tokens, out_ids);
+  };
+  e->handover_gave_up = false;
+  int rc = once();
+  if (rc == AWQ_ERR_HIP && e->handover_gave_up && (e->fused || e->fused_qkv)) {
+    // A fused launch needs all its workgroups resident at once.  Where that does not hold (the device shared
+    // with other work) its bounded waits give up; the whole request is then run again with every launch on its
+    // own, as the reference has them, and the engine stays that way until awq_set_fused_mode is called again.
+    if (int rc2 = awq_set_fused_mode(e, 0)) return rc2;
+    rc = once();
+  }
+  return rc;
 }
 
 extern "C" int awq_read_hidden(awq_engine* e, uint16_t* host_dst) {

@@ -104,7 +104,10 @@ int awq_set_prefill_mode(awq_engine* e, int batched);
  * wait (see awq_gemm).  With `on` non-zero every such wait of the next
  * awq_prefill_batched call gives up before its first poll: all kernels end
  * normally, the call returns AWQ_ERR_HIP, and the engine is usable again
- * after awq_reset. */
+ * after awq_reset.  The fused launches of the token-by-token steps (see
+ * awq_set_fused_mode) take the same path; with `on` == 2 their condition is
+ * set again by the next awq_reset, once, so that a whole awq_generate call
+ * (which starts with a reset) meets it. */
 int awq_debug_force_handover_giveup(awq_engine* e, int on);
 
 /* No counterpart in the reference: pairs of a layer's launches as ONE launch,
@@ -129,8 +132,10 @@ int awq_debug_force_handover_giveup(awq_engine* e, int on);
  * compute units to itself, and the second one workgroups whose indices agree
  * modulo 8 on one die (probed with a launch of the same grid when it is
  * switched on).  A wait that cannot end gives up after a bounded number of
- * polls and the call (awq_prefill, awq_decode, awq_generate) returns
- * AWQ_ERR_HIP, never a wrong token; awq_reset leaves the engine usable.  Asking
+ * polls and the call (awq_prefill, awq_decode) returns AWQ_ERR_HIP, never a
+ * wrong token; awq_reset leaves the engine usable.  awq_generate (the drop-in
+ * call) then switches the fused launches off and runs the whole request again
+ * with every launch on its own; they stay off until this is called again.  Asking
  * for a launch where it is not supported leaves it off; awq_fused_mode tells
  * which are in use. */
 int awq_set_fused_mode(awq_engine* e, int enabled);

@@ -527,6 +527,17 @@ def test_fused_qkv_attention_launch_is_bit_identical_and_gives_up_cleanly(awq, l
     print("fused Wqkv + attention launch, after a reset", flush=True)
     assert eng.generateResponse(prompt, 100) == ref
     compare_state(awq, oracle, eng, model, cfg)
+    # the drop-in call does not fail where the reference would not: after a give-up it runs the request again
+    # with every launch on its own and leaves the fused launches off
+    print("generateResponse over a give-up", flush=True)
+    awq.check(lib.awq_debug_force_handover_giveup(eng._h, 2))
+    assert eng.generateResponse(prompt, 100) == ref
+    compare_state(awq, oracle, eng, model, cfg)
+    assert eng.fused_mode() == 0
+    awq.check(lib.awq_debug_force_handover_giveup(eng._h, 0))
+    eng.set_fused_mode(eng.FUSED_QKV_ATTN)
+    assert eng.fused_mode() == eng.FUSED_QKV_ATTN
+    assert eng.generateResponse(prompt, 100) == ref
     buf = np.zeros(256 * 16, dtype=np.uint64)
     nw, ns = ctypes.c_int32(0), ctypes.c_int32(0)
     awq.check(lib.awq_debug_qkv_attention_timeline(eng._h, 1, 200, buf.ctypes.data_as(ctypes.c_void_p),
