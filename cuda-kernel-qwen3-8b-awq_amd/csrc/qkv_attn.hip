@@ -383,7 +383,7 @@ __global__ __launch_bounds__(kThreads) void qkv_attn_kernel(QkvAttnArgs a) {
     const int sec = tid >> 4;  // 0 Q, 1 K, 2 V
     const half_t v = (half_t)sum_16_waves(red[sec], r);
     const int d = kDP * part + r;
-    const half_t other = __builtin_bit_cast(half_t, (unsigned short)__shfl_xor((int)__builtin_bit_cast(unsigned short, v), 1, 64));
+    const half_t other = __builtin_bit_cast(half_t, (unsigned short)__builtin_bit_cast(uint32_t, dpp_f<kDppXor1>(__builtin_bit_cast(float, (uint32_t)__builtin_bit_cast(unsigned short, v)))));
     half_t out = v;
     if (sec < 2) {  // pairs (2i, 2i + 1) are rotated (Inference.cu:158-176)
       const half_t av = (r & 1) ? other : v, bv = (r & 1) ? v : other;
@@ -568,8 +568,13 @@ __global__ __launch_bounds__(kThreads) void qkv_attn_kernel(QkvAttnArgs a) {
     const float p_lane = base + lane < L ? e_lane[i] / Z : 0.0f;
     float acc = 0.0f;
     float pp[16];
+    // through the chunk's own slots of the scores (this wavefront alone reads them, and has): position 4 nl + tq at 16 tq + nl
+    s[base + 16 * (lane & 3) + (lane >> 2)] = p_lane;
 #pragma unroll
-    for (int nl = 0; nl < 16; ++nl) pp[nl] = __shfl(p_lane, 4 * nl + tq, 64);
+    for (int j = 0; j < 4; ++j) {
+      const float4 v = *reinterpret_cast<const float4*>(&s[base + 16 * tq + 4 * j]);
+      pp[4 * j] = v.x, pp[4 * j + 1] = v.y, pp[4 * j + 2] = v.z, pp[4 * j + 3] = v.w;
+    }
 #pragma unroll
     for (int nl = 0; nl < 16; ++nl) {
       const int t = base + 4 * nl + tq;
