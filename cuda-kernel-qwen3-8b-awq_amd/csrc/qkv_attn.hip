@@ -445,12 +445,14 @@ __global__ __launch_bounds__(kThreads) void qkv_attn_kernel(QkvAttnArgs a) {
       }
   }
   // this wavefront's first chunk of values into the order of the sums, [position][dimension], while the other
-  // workgroups' partial scores are on their way
+  // workgroups' partial scores are on their way; the new position's row comes from this workgroup's own product,
+  // not from the row just written
+  const half8v_t vnew = *reinterpret_cast<const half8v_t*>(own + 2 * kDP + 8 * (lane & 1));
   auto values_to_lds = [&](int i) {
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       const int t = ((aw + kWaves * i) << 6) + 32 * j + (lane >> 1);
-      if (t < L) *reinterpret_cast<half8v_t*>(&vt[wave][(32 * j + (lane >> 1)) * kDP + 8 * (lane & 1)]) = vraw[i][j];
+      if (t < L) *reinterpret_cast<half8v_t*>(&vt[wave][(32 * j + (lane >> 1)) * kDP + 8 * (lane & 1)]) = t == pos ? vnew : vraw[i][j];
     }
   };
 #pragma unroll
@@ -578,8 +580,7 @@ __global__ __launch_bounds__(kThreads) void qkv_attn_kernel(QkvAttnArgs a) {
 #pragma unroll
     for (int nl = 0; nl < 16; ++nl) {
       const int t = base + 4 * nl + tq;
-      const half_t val = t == pos ? own[2 * kDP + dl] : vv[nl];  // the new row from this workgroup's own product
-      const float rr = __builtin_fmaf(pp[nl], (float)val, acc);
+      const float rr = __builtin_fmaf(pp[nl], (float)vv[nl], acc);
       acc = t < L ? rr : acc;
     }
     acc = add_swap16(acc);
