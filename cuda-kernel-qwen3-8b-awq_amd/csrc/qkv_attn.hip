@@ -81,7 +81,6 @@ struct QkvAttnArgs {
   int32_t layer;
   int32_t use_len_hi;
   int32_t spin_limit;
-  int32_t mg;             // m / 128 of the matrix
   int32_t parts_pos;      // positions the parts arrays hold
   float eps;
   unsigned long long* stamps;  // STAMPS: [workgroup][kQkvStamps] times of thread 0, 10 ns units
@@ -189,9 +188,14 @@ __global__ __launch_bounds__(256) void kv_to_parts_kernel(const half_t* __restri
   *reinterpret_cast<uint4*>(vp + dst) = *reinterpret_cast<const uint4*>(vc + src);
 }
 
-// kCPW: chunks per wavefront (the launcher's bound on the attended length is 1024 kCPW)
+// kCPW: chunks per wavefront (the launcher's bound on the attended length is 1024 kCPW).  The pointers a workgroup
+// needs first are arguments of their own ahead of the struct: the first 14 dwords of the arguments are in scalar
+// registers when a wavefront starts (kernarg preload), the rest takes a memory round trip.
 template <bool STAMPS, int kCPW>
-__global__ __launch_bounds__(kThreads) void qkv_attn_kernel(QkvAttnArgs a) {
+__global__ __launch_bounds__(kThreads) void qkv_attn_kernel(const half_t* __restrict__ hot_x, const half_t* __restrict__ hot_gamma,
+                                                            const StepState* __restrict__ hot_dyn, int32_t* hot_status,
+                                                            const u32x4* __restrict__ hot_wq, const half_t* __restrict__ hot_scale,
+                                                            const half_t* __restrict__ hot_zp, QkvAttnArgs a) {
   constexpr int kChunks = kCPW * kWaves;  // of this instance; the LDS arrays and the exchange buffer are laid out for kChunkCap
   __shared__ __attribute__((aligned(16))) unsigned char xs[kBlocks * 64];  // byte planes, 64 bytes per block
   __shared__ __attribute__((aligned(16))) float xc[kBlocks];
@@ -225,28 +229,28 @@ __global__ __launch_bounds__(kThreads) void qkv_attn_kernel(QkvAttnArgs a) {
   // ---- requests, in the order the compute unit's memory pipeline should serve them
   uint4 xu = uint4{0, 0, 0, 0}, gu = uint4{0, 0, 0, 0};
   if (stager) {
-    xu = reinterpret_cast<const uint4*>(a.x)[tid];
-    gu = reinterpret_cast<const uint4*>(a.gamma)[tid];
+    xu = reinterpret_cast<const uint4*>(hot_x)[tid];
+    gu = reinterpret_cast<const uint4*>(hot_gamma)[tid];
   }
-  const int32_t pos = a.dyn->pos;
+  const int32_t pos = hot_dyn->pos;
   // (the launcher's bound is kMaxLen; the clamp keeps every index inside the arrays whatever the state says)
-  const int32_t L = min(a.use_len_hi ? a.dyn->len_hi : a.dyn->len_lo, kChunks * 64);
-  const int32_t epoch = a.dyn->epoch;
-  const int32_t gave_up_before = __hip_atomic_load(a.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  const int32_t L = min(a.use_len_hi ? hot_dyn->len_hi : hot_dyn->len_lo, kChunks * 64);
+  const int32_t epoch = hot_dyn->epoch;
+  const int32_t gave_up_before = __hip_atomic_load(hot_status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   // the three row groups of this workgroup: dimensions 16 part .. + 15 of the head's Q, K and V
   int rg[3];
   half_t gs[3], gz[3];
 #pragma unroll
   for (int i = 0; i < 3; ++i) {
     rg[i] = i * (kK / 16) + head * kParts + part;
-    const unsigned gi = ((unsigned)(rg[i] * 16 >> 7) % (unsigned)(kK / 128)) % (unsigned)a.mg;
-    gs[i] = a.scale[gi];
-    gz[i] = a.zp[gi];
+    const unsigned gi = (unsigned)(rg[i] * 16 >> 7) % (unsigned)(kK / 128);  // (... % (m / 128) of Inference.cu:90 changes nothing: m / 128 = 96 > 31)
+    gs[i] = hot_scale[gi];
+    gz[i] = hot_zp[gi];
   }
   __syncthreads();  // every request for x is out before any request for weights
   u32x4 wr[3][kG];
   auto request_w = [&](int i) {
-    const u32x4* wp = a.wq + ((int64_t)rg[i] * kBlocks + blk0) * 16 + r;
+    const u32x4* wp = hot_wq + ((int64_t)rg[i] * kBlocks + blk0) * 16 + r;
 #pragma unroll
     for (int b = 0; b < kG; ++b) wr[i][b] = __builtin_nontemporal_load(wp + b * 16);
   };
@@ -479,7 +483,7 @@ __global__ __launch_bounds__(kThreads) void qkv_attn_kernel(QkvAttnArgs a) {
       while (!dead) {
         int32_t st = 0;
         const bool look = (spins & 7) == 7;  // every eighth poll also reads the status word
-        if (look) st = __hip_atomic_load(a.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (look) st = __hip_atomic_load(hot_status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         u32x2 w[8];
         bool ok = true;
         if (mine) {
@@ -500,7 +504,7 @@ __global__ __launch_bounds__(kThreads) void qkv_attn_kernel(QkvAttnArgs a) {
           break;
         }
         if (++spins > a.spin_limit) {
-          if (lane == 0) __hip_atomic_store(a.status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          if (lane == 0) __hip_atomic_store(hot_status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           dead = true;
         }
         if (look && st != 0) dead = true;
@@ -658,21 +662,22 @@ int launch_fused_qkv_attn(const void* wq, const half_t* scale, const half_t* zp,
   a.layer = layer;
   a.use_len_hi = use_len_hi;
   a.spin_limit = 1 << 20;
-  a.mg = (int32_t)(m / 128);
   a.eps = eps;
   a.stamps = stamps;
   AWQ_REQUIRE(len_bound > 0 && len_bound <= kMaxLen, "attended length beyond what the fused launch covers");
+#define QKV_HOT_ARGS a.x, a.gamma, a.dyn, a.status, a.wq, a.scale, a.zp
   const dim3 grid((unsigned)(n_heads * kParts)), block(kThreads);
   if (len_bound <= 64 * kWaves) {
-    if (stamps) hipLaunchKernelGGL((qkv_attn_kernel<true, 1>), grid, block, 0, st, a);
-    else hipLaunchKernelGGL((qkv_attn_kernel<false, 1>), grid, block, 0, st, a);
+    if (stamps) hipLaunchKernelGGL((qkv_attn_kernel<true, 1>), grid, block, 0, st, QKV_HOT_ARGS, a);
+    else hipLaunchKernelGGL((qkv_attn_kernel<false, 1>), grid, block, 0, st, QKV_HOT_ARGS, a);
   } else if (len_bound <= 2 * 64 * kWaves) {
-    if (stamps) hipLaunchKernelGGL((qkv_attn_kernel<true, 2>), grid, block, 0, st, a);
-    else hipLaunchKernelGGL((qkv_attn_kernel<false, 2>), grid, block, 0, st, a);
+    if (stamps) hipLaunchKernelGGL((qkv_attn_kernel<true, 2>), grid, block, 0, st, QKV_HOT_ARGS, a);
+    else hipLaunchKernelGGL((qkv_attn_kernel<false, 2>), grid, block, 0, st, QKV_HOT_ARGS, a);
   } else {
-    if (stamps) hipLaunchKernelGGL((qkv_attn_kernel<true, 3>), grid, block, 0, st, a);
-    else hipLaunchKernelGGL((qkv_attn_kernel<false, 3>), grid, block, 0, st, a);
+    if (stamps) hipLaunchKernelGGL((qkv_attn_kernel<true, 3>), grid, block, 0, st, QKV_HOT_ARGS, a);
+    else hipLaunchKernelGGL((qkv_attn_kernel<false, 3>), grid, block, 0, st, QKV_HOT_ARGS, a);
   }
+#undef QKV_HOT_ARGS
   AWQ_HIP_TRY(hipGetLastError());
   return AWQ_OK;
 }
