@@ -78,8 +78,6 @@ struct QkvAttnArgs {
   int32_t* status;        // [0] != 0: a wait gave up (or the host asks every wait to)
   const StepState* dyn;
   KvLayout kv;
-  int32_t layer;
-  int32_t use_len_hi;
   int32_t spin_limit;
   int32_t parts_pos;      // positions the parts arrays hold
   float eps;
@@ -193,9 +191,9 @@ __global__ __launch_bounds__(256) void kv_to_parts_kernel(const half_t* __restri
 // registers when a wavefront starts (kernarg preload), the rest takes a memory round trip.
 template <bool STAMPS, int kCPW>
 __global__ __launch_bounds__(kThreads) void qkv_attn_kernel(const half_t* __restrict__ hot_x, const half_t* __restrict__ hot_gamma,
-                                                            const StepState* __restrict__ hot_dyn, int32_t* hot_status,
+                                                            const StepState* __restrict__ hot_dyn,
                                                             const u32x4* __restrict__ hot_wq, const half_t* __restrict__ hot_scale,
-                                                            const half_t* __restrict__ hot_zp, QkvAttnArgs a) {
+                                                            const half_t* __restrict__ hot_zp, int hot_use_len_hi, int hot_layer, QkvAttnArgs a) {
   constexpr int kChunks = kCPW * kWaves;  // of this instance; the LDS arrays and the exchange buffer are laid out for kChunkCap
   __shared__ __attribute__((aligned(16))) unsigned char xs[kBlocks * 64];  // byte planes, 64 bytes per block
   __shared__ __attribute__((aligned(16))) float xc[kBlocks];
@@ -234,9 +232,8 @@ __global__ __launch_bounds__(kThreads) void qkv_attn_kernel(const half_t* __rest
   }
   const int32_t pos = hot_dyn->pos;
   // (the launcher's bound is kMaxLen; the clamp keeps every index inside the arrays whatever the state says)
-  const int32_t L = min(a.use_len_hi ? hot_dyn->len_hi : hot_dyn->len_lo, kChunks * 64);
+  const int32_t L = min(hot_use_len_hi ? hot_dyn->len_hi : hot_dyn->len_lo, kChunks * 64);
   const int32_t epoch = hot_dyn->epoch;
-  const int32_t gave_up_before = __hip_atomic_load(hot_status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   // the three row groups of this workgroup: dimensions 16 part .. + 15 of the head's Q, K and V
   int rg[3];
   half_t gs[3], gz[3];
@@ -261,7 +258,7 @@ __global__ __launch_bounds__(kThreads) void qkv_attn_kernel(const half_t* __rest
   // 1 .. 65535: never the 0 of a cleared buffer.  Q and K words are all rewritten by every launch, so a word
   // holds the previous launch's tag until then; score words beyond the attended length are not, which is why
   // the buffer is cleared when a sequence starts (a sequence stays below 65535 launches of this kind)
-  const uint32_t tag16 = 1u + (uint32_t)(epoch + a.layer) % 65535u;
+  const uint32_t tag16 = 1u + (uint32_t)(epoch + hot_layer) % 65535u;
 
   // ---- rmsNormKernel, Inference.cu:111-145: x in natural order for the 256 strided partial sums
   if (stager) reinterpret_cast<uint4*>(xn)[tid] = xu;
@@ -343,6 +340,10 @@ __global__ __launch_bounds__(kThreads) void qkv_attn_kernel(const half_t* __rest
         if (i < kVEarly) vraw[i][j] = *reinterpret_cast<const half8v_t*>(a.v_parts + parts_base + (int64_t)t * kDP);
       }
     }
+
+  // a wait that gave up in an earlier launch: this one does not wait at all (asked for behind the bulk requests,
+  // needed long after them)
+  const int32_t gave_up_before = __hip_atomic_load(a.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 
   // ---- the three products (Inference.cu:1052)
   {
@@ -483,7 +484,7 @@ __global__ __launch_bounds__(kThreads) void qkv_attn_kernel(const half_t* __rest
       while (!dead) {
         int32_t st = 0;
         const bool look = (spins & 7) == 7;  // every eighth poll also reads the status word
-        if (look) st = __hip_atomic_load(hot_status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (look) st = __hip_atomic_load(a.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         u32x2 w[8];
         bool ok = true;
         if (mine) {
@@ -504,7 +505,7 @@ __global__ __launch_bounds__(kThreads) void qkv_attn_kernel(const half_t* __rest
           break;
         }
         if (++spins > a.spin_limit) {
-          if (lane == 0) __hip_atomic_store(hot_status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          if (lane == 0) __hip_atomic_store(a.status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           dead = true;
         }
         if (look && st != 0) dead = true;
@@ -659,13 +660,11 @@ int launch_fused_qkv_attn(const void* wq, const half_t* scale, const half_t* zp,
   a.status = status;
   a.dyn = dyn;
   a.kv = kv;
-  a.layer = layer;
-  a.use_len_hi = use_len_hi;
   a.spin_limit = 1 << 20;
   a.eps = eps;
   a.stamps = stamps;
   AWQ_REQUIRE(len_bound > 0 && len_bound <= kMaxLen, "attended length beyond what the fused launch covers");
-#define QKV_HOT_ARGS a.x, a.gamma, a.dyn, a.status, a.wq, a.scale, a.zp
+#define QKV_HOT_ARGS a.x, a.gamma, a.dyn, a.wq, a.scale, a.zp, use_len_hi, layer
   const dim3 grid((unsigned)(n_heads * kParts)), block(kThreads);
   if (len_bound <= 64 * kWaves) {
     if (stamps) hipLaunchKernelGGL((qkv_attn_kernel<true, 1>), grid, block, 0, st, QKV_HOT_ARGS, a);
