@@ -232,6 +232,16 @@ __global__ __launch_bounds__(256) void sample_finish_kernel(SampleFinish f) {
     *f.best = 0ull;
   }
 }
+// (row / 128 % (k / 128)) % (m / 128), the group of a row (Inference.cu:90 with the index wrapped to the m / 128
+// stored entries), without a division where there is nothing to divide: row / 128 < m / 128, so with
+// k / 128 >= m / 128 both remainders change nothing, and otherwise the second one does not.  (The divisions stood
+// between the requests for x and the first request for weights.)  A row group past the matrix gets a valid index.
+__device__ __forceinline__ unsigned group_index(int row_over_128, int kg, int mg) {
+  const unsigned g = min((unsigned)row_over_128, (unsigned)mg - 1u);
+  if (kg >= mg) return g;
+  return (kg & (kg - 1)) == 0 ? g & (unsigned)(kg - 1) : g % (unsigned)kg;
+}
+
 
 // A workgroup takes row groups blockIdx.x, blockIdx.x + gridDim.x, ... (16
 // output rows x all of k each).  n_waves wavefronts; lane (w, q, r) owns blocks
@@ -342,7 +352,7 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
   // the m/128 stored entries): requested with x, so that they are there when the first block is done
   half_t gs = (half_t)0.0f, gz = (half_t)0.0f;
   if (!PERIODIC) {
-    const unsigned gi = ((unsigned)(rg * RH >> 7) % (unsigned)kg) % (unsigned)mg;
+    const unsigned gi = group_index(rg * RH >> 7, kg, mg);
     gs = scale[gi];
     gz = zp[gi];
   }
@@ -505,7 +515,7 @@ __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
 #pragma unroll
     for (int b = 0; b < G; ++b) dst[b] = __builtin_nontemporal_load(src + b * 16);
     if (!PERIODIC) {
-      const unsigned gi = ((unsigned)(row_group * RH >> 7) % (unsigned)kg) % (unsigned)mg;
+      const unsigned gi = group_index(row_group * RH >> 7, kg, mg);
       s_out = scale[gi];
       z_out = zp[gi];
     }
