@@ -277,10 +277,13 @@ __device__ __forceinline__ unsigned group_index(int row_over_128, int kg, int mg
 template <int G, bool PERIODIC, int UFAST = 0, int NWC = 0, bool MULTI = true, int RH = 16, int PRO = -1, int EPI = -1>
 __global__ __launch_bounds__(NWC ? NWC * 64 : 1024) void gemv_kernel(
     const u32x4* __restrict__ wq, const half_t* __restrict__ x, const half_t* __restrict__ gamma,
-    const half_t* __restrict__ scale, const half_t* __restrict__ zp, int32_t mg, int32_t kg, int32_t prologue_arg,
-    int32_t epi_arg, int32_t m, float eps, GemvParams p) {
-  const int prologue = PRO >= 0 ? PRO : prologue_arg;
-  const int epi = EPI >= 0 ? EPI : epi_arg;
+    const half_t* __restrict__ scale, const half_t* __restrict__ zp, int32_t mg, int32_t kg, float eps,
+    int32_t pro_epi, GemvParams p) {
+  // (14 dwords up to here: what is preloaded.  The norm's epsilon among them: read from the argument block it was
+  // a memory round trip between the norm's statistic and its reciprocal square root.)
+  const int prologue = PRO >= 0 ? PRO : (pro_epi & 0xff);
+  const int epi = EPI >= 0 ? EPI : (pro_epi >> 8);
+  const int m = mg * 128;
   const int n_waves = NWC ? NWC : p.n_waves;
   constexpr int Q = 64 / RH;  // lanes that share a row = consecutive block ranges of a wavefront
   // The block products on the matrix cores.  16 rows per wavefront: the lanes (q, r) are the matrix
@@ -681,7 +684,7 @@ bool plan_gemv(int64_t m, int64_t k, GemvPlan* out) {
   return found;
 }
 
-#define GEMV_HOT_ARGS p.wq, p.x, p.gamma, p.scale, p.zp, p.mg, p.kg, p.prologue, p.epilogue, p.m, p.eps
+#define GEMV_HOT_ARGS p.wq, p.x, p.gamma, p.scale, p.zp, p.mg, p.kg, p.eps, (p.prologue | (p.epilogue << 8))
 template <int G>
 void launch_g(const GemvParams& p, bool periodic, bool multi, int rh, dim3 grid, dim3 block, size_t lds, hipStream_t st) {
   if (rh == 8) {  // plan_gemv: four blocks per lane, not periodic, one row group per workgroup
