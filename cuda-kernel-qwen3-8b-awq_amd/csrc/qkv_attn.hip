@@ -335,10 +335,15 @@ __global__ __launch_bounds__(kThreads) void qkv_attn_kernel(const half_t* __rest
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       const int t = ((aw + kWaves * i) << 6) + 32 * j + (lane >> 1);
-      if (t < L) {
-        kraw[i][j] = *reinterpret_cast<const half8v_t*>(a.k_parts + parts_base + (int64_t)t * kDP);
-        if (i < kVEarly) vraw[i][j] = *reinterpret_cast<const half8v_t*>(a.v_parts + parts_base + (int64_t)t * kDP);
-      }
+      if (t < L) kraw[i][j] = *reinterpret_cast<const half8v_t*>(a.k_parts + parts_base + (int64_t)t * kDP);
+    }
+  // (the keys first: the partial scores wait for them alone)
+#pragma unroll
+  for (int i = 0; i < kVEarly; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int t = ((aw + kWaves * i) << 6) + 32 * j + (lane >> 1);
+      if (t < L) vraw[i][j] = *reinterpret_cast<const half8v_t*>(a.v_parts + parts_base + (int64_t)t * kDP);
     }
 
   // a wait that gave up in an earlier launch: this one does not wait at all (asked for behind the bulk requests,
