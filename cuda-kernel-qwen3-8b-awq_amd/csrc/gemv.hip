@@ -134,10 +134,10 @@ __device__ __forceinline__ void epilogue(const GemvParams& p, int epi, int row, 
   half_t v = (half_t)acc;
   switch (epi) {
     case EPI_RESIDUAL:  // Inference.cu:1149-1155
-      p.y[row] = res + v;
+      store_through(p.y + row, res + v);
       return;
     case EPI_GELU:  // Inference.cu:271-279
-      p.y[row] = to_half_rn(awq_gelu_f32((float)v));
+      store_through(p.y + row, to_half_rn(awq_gelu_f32((float)v)));
       return;
     case EPI_QKV_ROPE: {
       // Inference.cu:1070-1103: rows [0,H) are Q, [H,2H) K, [2H,3H) V.  Q and K

@@ -605,7 +605,7 @@ __global__ __launch_bounds__(kThreads) void qkv_attn_kernel(const half_t* __rest
     float out = oc[0];
 #pragma unroll
     for (int c = 1; c < kChunks; ++c) out += oc[c];
-    a.ctx[head * AWQ_HEAD_DIM + kDP * part + tid] = (half_t)out;
+    store_through(a.ctx + head * AWQ_HEAD_DIM + kDP * part + tid, (half_t)out);
   }
   stamp();  // 10 end
 }
