@@ -126,7 +126,7 @@ int awq_debug_force_handover_giveup(awq_engine* e, int on);
  * The first is off by default: on MI355X it measures 2 % slower than the two
  * launches it replaces (a hand-over between all workgroups costs what a kernel
  * boundary costs).  The second is on by default where the device can run it
- * (992 against 967 tok/s at 137..392 positions, 713 against 625 at 2104..2144,
+ * (1033 against 987 tok/s at 137..392 positions, 713 against 625 at 2104..2144,
  * 629 against 594 at 3004..3044).  A fused launch
  * needs all its 256 workgroups resident at once, i.e. a device of at least 256
  * compute units to itself, and the second one workgroups whose indices agree
