@@ -525,9 +525,9 @@ __global__ __launch_bounds__(kThreads) void qkv_attn_kernel(const half_t* __rest
   }
   __syncthreads();
   stamp();  // 9 all scores of the head seen
-  if (lost) return;
-
-  float mx = lane < kWaves ? wmax[lane] : -1e9f;
+  float mx = lane < kWaves ? wmax[lane] : -1e9f;  // (read together with the flag: one LDS round trip, not two)
+  const int gave_up = lost;
+  if (gave_up) return;
   mx = wave_maxf(mx);
 
   // ---- exponentials and their sum (Inference.cu:239-249), a chunk at a time; the exponential of position
