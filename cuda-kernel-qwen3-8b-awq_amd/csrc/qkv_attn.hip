@@ -1,6 +1,6 @@
 // The first two launches of a decoder layer as ONE: RMSNorm + Wqkv + rotary + KV append (Inference.cu:1040-1103)
 // and the attention over the cache (Inference.cu:1110, attentionKernel :182-267), for attended lengths that the
-// attention covers in at most three launches of its own, and twice as far (kFusedQkvAttnMax).
+// attention covers in at most three launches of its own, and half as far again (kFusedQkvAttnMax = 3072).
 //
 // Of all the boundaries between a layer's launches this is the one across which the data dependence is local:
 // the attention of head h needs rows 128 h .. 128 h + 127 of Q and of K and nothing else of the product.  A
