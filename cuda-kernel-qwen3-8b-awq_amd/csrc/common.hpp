@@ -179,11 +179,11 @@ constexpr int64_t kAttnShortMax = 128;
 constexpr int64_t kAttnOneWorkgroupMax = 704;
 constexpr int64_t kAttnTwoLaunchMax = 1024;
 constexpr int64_t kAttnMergedMax = 2048;
-// the fused Wqkv + attention launch (qkv_attn.hip) covers attended lengths up to here: three 64-position chunks per
-// wavefront of its workgroups.  (With four it still wins at 3000 positions, 631 against 597 tok/s, and loses at
-// 4050, 549 against 562: every workgroup reads all eight partial scores of every position, as many bytes as its
-// share of the cache rows.)
-constexpr int64_t kFusedQkvAttnMax = 3072;
+// the fused Wqkv + attention launch (qkv_attn.hip) covers attended lengths up to here: four 64-position chunks per
+// wavefront of its workgroups (606 against 574 tok/s at 3500 positions, 564 against 558 at 4050: every workgroup
+// reads all eight partial scores of every position, as many bytes as its share of the cache rows, so the gain
+// ends here)
+constexpr int64_t kFusedQkvAttnMax = 4096;
 int64_t attention_workspace_bytes(int n_heads, int64_t max_pos);
 int launch_attention(const half_t* q, const half_t* kc, const half_t* vc, half_t* ctx, int n_heads, int64_t max_pos,
                      KvLayout kv, int64_t L, const StepState* dyn, int use_len_hi, int64_t len_bound, void* ws,

@@ -170,7 +170,7 @@ struct awq_engine {
   int n_generated = 0;
   bool finalized = false;
   bool graph_mode = true;
-  hipGraphExec_t graphs[3][6] = {};  // [prompt | generation step | kStepsPerGraph generation steps][length bound]
+  hipGraphExec_t graphs[3][7] = {};  // [prompt | generation step | kStepsPerGraph generation steps][length bound]
   // activations of the batched prompt pass, [chunk][n] each; allocated at first use
   struct {
     half_t *hidden = nullptr, *norm = nullptr, *qkv = nullptr, *q = nullptr, *ctx = nullptr, *mid = nullptr;
@@ -391,7 +391,8 @@ int enqueue_step_body(awq_engine* e, bool gen, int64_t len_bound) {
 
 // the attention launches are specialised by an upper bound of the attended length (one workgroup per head, or two
 // to four launches cut along the sequence; the fused launch's chunks per wavefront); one captured graph per bound
-constexpr int64_t kLengthBounds[6] = {kAttnShortMax, kAttnOneWorkgroupMax, kAttnTwoLaunchMax, kAttnMergedMax, kFusedQkvAttnMax, 1 << 30};
+constexpr int64_t kLengthBounds[7] = {kAttnShortMax, kAttnOneWorkgroupMax, kAttnTwoLaunchMax, kAttnMergedMax, 3072, kFusedQkvAttnMax, 1 << 30};
+static_assert(kFusedQkvAttnMax == 4096, "the fused launch's instances: three chunks of 64 positions per wavefront up to 3072 positions, four beyond");
 int length_bucket(int64_t len) {
   int bucket = 0;
   while (len > kLengthBounds[bucket]) ++bucket;

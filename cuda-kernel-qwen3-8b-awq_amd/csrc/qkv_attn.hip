@@ -49,7 +49,7 @@ constexpr int kG = 2;               // blocks per lane and row group
 constexpr int kParts = 8;           // workgroups per head
 constexpr int kDP = AWQ_HEAD_DIM / kParts;  // dimensions per workgroup: one 16-row group each of Q, K and V
 constexpr int kMaxLen = (int)kFusedQkvAttnMax;
-constexpr int kMaxCPW = 3;          // chunks of 64 positions per wavefront: 1 up to 1024 attended positions, 2 up to 2048, 3 beyond
+constexpr int kMaxCPW = 4;          // chunks of 64 positions per wavefront: 1 up to 1024 attended positions, 2 up to 2048, 3 beyond
 constexpr int kChunkCap = kMaxCPW * kWaves;
 constexpr int kScoreStride = kChunkCap * 64;  // (score, tag) pairs per head in the exchange buffer
 static_assert(kDP == 16 && kMaxLen <= kChunkCap * 64 && kMaxLen <= kScoreStride, "shape of the fused launch");
@@ -682,9 +682,12 @@ int launch_fused_qkv_attn(const void* wq, const half_t* scale, const half_t* zp,
   } else if (len_bound <= 2 * 64 * kWaves) {
     if (stamps) hipLaunchKernelGGL((qkv_attn_kernel<true, 2>), grid, block, 0, st, QKV_HOT_ARGS, a);
     else hipLaunchKernelGGL((qkv_attn_kernel<false, 2>), grid, block, 0, st, QKV_HOT_ARGS, a);
-  } else {
+  } else if (len_bound <= 3 * 64 * kWaves) {
     if (stamps) hipLaunchKernelGGL((qkv_attn_kernel<true, 3>), grid, block, 0, st, QKV_HOT_ARGS, a);
     else hipLaunchKernelGGL((qkv_attn_kernel<false, 3>), grid, block, 0, st, QKV_HOT_ARGS, a);
+  } else {
+    if (stamps) hipLaunchKernelGGL((qkv_attn_kernel<true, 4>), grid, block, 0, st, QKV_HOT_ARGS, a);
+    else hipLaunchKernelGGL((qkv_attn_kernel<false, 4>), grid, block, 0, st, QKV_HOT_ARGS, a);
   }
 #undef QKV_HOT_ARGS
   AWQ_HIP_TRY(hipGetLastError());

@@ -117,17 +117,17 @@ int awq_debug_force_handover_giveup(awq_engine* e, int on);
  *      through memory, W1's weights requested while that hand-over is under way
  *      (hidden 4096 / intermediate 12288);
  *   2  RMSNorm + Wqkv + rotary + KV append (:1040-1103) and the attention
- *      (:1110) up to 3072 attended positions: the eight workgroups of a head sit
+ *      (:1110) up to 4096 attended positions: the eight workgroups of a head sit
  *      on one die and hand partial scores to each other through its L2 (hidden
  *      4096, 32 heads; longer sequences keep the two launches).  The launch
  *      reads the caches from a second copy that the engine keeps for it, the
- *      first min(max_pos, 3072) positions as [head][8][position][16] (2 x 25 MB
- *      per layer at 3072 positions).
+ *      first min(max_pos, 4096) positions as [head][8][position][16] (2 x 33.5 MB
+ *      per layer at 4096 positions).
  * The first is off by default: on MI355X it measures 2 % slower than the two
  * launches it replaces (a hand-over between all workgroups costs what a kernel
  * boundary costs).  The second is on by default where the device can run it
- * (1033 against 987 tok/s at 137..392 positions, 713 against 625 at 2104..2144,
- * 629 against 594 at 3004..3044).  A fused launch
+ * (1049 against 987 tok/s at 137..392 positions, 764 against 625 at 2104..2144,
+ * 676 against 594 at 3004..3044, 606 against 574 at 3504..3544).  A fused launch
  * needs all its 256 workgroups resident at once, i.e. a device of at least 256
  * compute units to itself, and the second one workgroups whose indices agree
  * modulo 8 on one die (probed with a launch of the same grid when it is
@@ -149,7 +149,7 @@ int awq_fused_mode(const awq_engine* e);
 int awq_debug_fused_timeline(awq_engine* e, int32_t layer, uint64_t* host_out, int32_t* n_workgroups,
                              int32_t* n_stamps);
 /* The same for the fused Wqkv + attention launch, at position `pos` attending
- * pos + 1 positions (pos < min(max_pos, 3072)). */
+ * pos + 1 positions (pos < min(max_pos, 4096)). */
 int awq_debug_qkv_attention_timeline(awq_engine* e, int32_t layer, int32_t pos, uint64_t* host_out,
                                      int32_t* n_workgroups, int32_t* n_stamps);
 
@@ -342,7 +342,7 @@ int awq_decode_attention_static(const void* q, const void* k_cache, const void* 
  * append) and awq_decode_attention as ONE launch for hidden 4096 and 32 heads
  * (wqkv_repacked is the 12288 x 4096 matrix from awq_linear_repack; caches
  * [head][max_pos][128]; x, gamma [4096]; q_out, ctx [4096]), position `pos`
- * attending the first L positions, L <= pos + 1 and L <= 3072.  Same bits as the
+ * attending the first L positions, L <= pos + 1 and L <= 4096.  Same bits as the
  * two calls.  Every head is given to eight workgroups that the device places on
  * one die (awq_qkv_attention_supported probes that and that all 256 workgroups
  * are resident at once: 1 = yes); they hand partial scores to each other through

@@ -561,10 +561,10 @@ def test_fused_qkv_attention_launch_is_bit_identical_and_gives_up_cleanly(awq, l
 
 def test_fused_qkv_attention_launch_across_its_length_bounds(awq, lib, torch_gpu):
     """The fused Wqkv + attention launch against the two launches it replaces (those are checked against the oracle
-    at these lengths elsewhere) on sequences that cross 2048 positions (a third chunk of 64 positions per
-    wavefront) and 3072 (where the engine goes back to two launches): a batched prompt pass fills the caches and
+    at these lengths elsewhere) on sequences that cross 2048 and 3072 positions (a third and a fourth chunk of 64
+    positions per wavefront) and 4096 (where the engine goes back to two launches): a batched prompt pass fills the caches and
     the launch's second copy of them, then generation steps.  Ids, last hidden state and logits bit for bit."""
-    cfg = awq.make_config(n_layers=2, max_pos=3200)
+    cfg = awq.make_config(n_layers=2, max_pos=4224)
     eng = awq.QWen3AWQInfer.empty(cfg)
     for layer, kind, part in awq.tensor_list(cfg):
         count = cfg.part_count(kind, part)
@@ -576,7 +576,7 @@ def test_fused_qkv_attention_launch_across_its_length_bounds(awq, lib, torch_gpu
     if not eng.fused_mode() & eng.FUSED_QKV_ATTN:
         pytest.skip("this device cannot run the fused launch")
     rng = np.random.default_rng(5)
-    for n_prompt, n_new in ((2020, 60), (3040, 60)):
+    for n_prompt, n_new in ((2020, 60), (3040, 60), (4070, 60)):
         prompt = rng.integers(0, cfg.vocab, n_prompt).tolist()
         out = []
         for mode in (0, eng.FUSED_QKV_ATTN):

@@ -596,7 +596,7 @@ def test_gemv_fused_norm_unembed_argmax(awq, lib, oracle, torch_gpu, m, k):
 @pytest.mark.parametrize("pos,L", [(0, 1), (1, 1), (2, 2), (2, 3), (5, 5), (63, 64), (70, 71), (300, 301), (640, 640),
                                    (703, 704), (704, 705), (959, 960), (960, 961), (1023, 1023), (1023, 1024),
                                    (1024, 1025), (1500, 1501), (1984, 1985), (2047, 2048), (2048, 2049), (3000, 2950),
-                                   (3007, 3008), (3071, 3072)])
+                                   (3007, 3008), (3071, 3072), (3072, 3073), (4031, 4032), (4095, 4096)])
 def test_fused_qkv_attention_launch_against_the_two_launches_and_the_oracle(awq, lib, oracle, torch_gpu, pos, L):
     """awq_qkv_attention: RMSNorm + Wqkv + rotary + KV append and the attention over the cache in one launch whose
     eight workgroups per head hand partial scores to each other through the L2 of their die.  Q, the caches and
@@ -604,7 +604,7 @@ def test_fused_qkv_attention_launch_against_the_two_launches_and_the_oracle(awq,
     calls in a row (the tags change; the second call finds the first one's words in the exchange buffer)."""
     torch = torch_gpu
     H = 4096
-    m, k, nh, mp = 3 * H, H, H // 128, (2112 if pos < 2112 else 3136)
+    m, k, nh, mp = 3 * H, H, H // 128, (2112 if pos < 2112 else 4160)
     if not lib.awq_qkv_attention_supported(H, nh, stream(torch)):
         pytest.skip("this device cannot run the fused launch")
     rng = np.random.default_rng(pos * 1000 + L)
@@ -650,7 +650,7 @@ def test_fused_qkv_attention_launch_against_the_two_launches_and_the_oracle(awq,
     fws = torch.zeros(lib.awq_qkv_attention_workspace_bytes(nh), dtype=torch.uint8, device="cuda")
     # the caches a second time in the launch's own order, [head][8][pp][16]: the rows before pos are copied, the
     # launch appends row pos itself
-    pp = 2048 if pos < 2048 else 3072
+    pp = 2048 if pos < 2048 else 4096
     assert lib.awq_kv_parts_bytes(nh, pp) == nh * 128 * pp * 2
     f_kp = torch.full((nh * 8 * pp * 16,), 7.0, dtype=torch.float16, device="cuda")
     f_vp = torch.full((nh * 8 * pp * 16,), 7.0, dtype=torch.float16, device="cuda")
