@@ -559,6 +559,37 @@ def test_fused_qkv_attention_launch_is_bit_identical_and_gives_up_cleanly(awq, l
     oracle.awqo_model_destroy(model)
 
 
+def test_fused_qkv_attention_launch_over_the_wrap_of_its_tags(awq, lib, torch_gpu):
+    """The partial scores travel as words that carry a 16-bit tag, 1 + (launch counter mod 65535): the 36-layer
+    model uses 36 tags per step, so a sequence of 1900 generated tokens passes the wrap (and the length bounds at
+    128, 704 and 1024 positions, four steps per graph launch).  Ids, last hidden state and logits are those of the
+    same sequence with Wqkv and the attention as separate launches, bit for bit."""
+    cfg = awq.make_config(n_layers=36, max_pos=2048)
+    eng = awq.QWen3AWQInfer.empty(cfg)
+    for layer, kind, part in awq.tensor_list(cfg):
+        count = cfg.part_count(kind, part)
+        nbytes = count if (part == awq.P_PACKED and kind != awq.T_GAMMA) else 2 * count
+        buf = (ctypes.c_uint8 * nbytes)()
+        awq.check(lib.awq_synth_fill_profile(awq.SYNTH_BALANCED, 31, layer, kind, part, buf, count))
+        eng.upload(layer, kind, part, buf, nbytes)
+    eng.finalize()
+    if not eng.fused_mode() & eng.FUSED_QKV_ATTN:
+        pytest.skip("this device cannot run the fused launch")
+    prompt = [11, 7, 1999, 3, 150000, 42, 8, 77]
+    out = []
+    for mode in (eng.FUSED_QKV_ATTN, 0):
+        print("1900 generated tokens, fused mode", mode, flush=True)
+        eng.set_fused_mode(mode)
+        eng.reset()
+        eng.prefill(prompt, batched=True)
+        ids = eng.decode(1900)
+        out.append((list(ids), np.ctypeslib.as_array(eng.read_hidden()).copy(),
+                    np.ctypeslib.as_array(eng.read_logits()).copy()))
+    assert out[0][0] == out[1][0] and len(set(out[0][0])) > 1
+    assert np.array_equal(out[0][1], out[1][1]) and np.array_equal(out[0][2], out[1][2])
+    eng.close()
+
+
 def test_fused_qkv_attention_launch_across_its_length_bounds(awq, lib, torch_gpu):
     """The fused Wqkv + attention launch against the two launches it replaces (those are checked against the oracle
     at these lengths elsewhere) on sequences that cross 2048 and 3072 positions (a third and a fourth chunk of 64
