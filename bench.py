@@ -299,7 +299,8 @@ def main():
         eng.set_fused_mode(0)
     elif args.fused is not None:
         eng.set_fused_mode(args.fused)
-    log("fused launches (1 Wo + W1, 2 Wqkv + attention): %d" % eng.fused_mode())
+    eng_fused_mode = eng.fused_mode()
+    log("fused launches (1 Wo + W1, 2 Wqkv + attention): %d" % eng_fused_mode)
     log("weights generated, uploaded and reordered in %.1f s" % (time.time() - t0))
 
     prompt = np.zeros(args.prompt_len, dtype=np.int32)
@@ -548,7 +549,8 @@ def main():
                                "intermediate 12288, vocab 151936, int4 g=128; %d-token prompt, batch-1 greedy decode"
                                % (cfg.n_layers, args.prompt_len),
                    "attended_positions": "%d..%d" % (args.prompt_len + args.warmup, args.prompt_len + args.warmup + args.steps),
-                   "max_pos": cfg.max_pos, "graph": not args.no_graph},
+                   "max_pos": cfg.max_pos, "graph": not args.no_graph,
+                   "steps_per_graph_launch": 1 if args.no_graph else 4, "fused_launches": eng_fused_mode},
         "step_algorithmic_bytes": int(step_bytes),
         "step_hbm_frac": round(step_bytes * tok_s / (HBM_PEAK_GBS * 1e9), 4),
         "greedy_tokens_identical_to_cpu": tokens_match,

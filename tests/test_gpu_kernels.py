@@ -684,6 +684,21 @@ def test_fused_qkv_attention_launch_against_the_two_launches_and_the_oracle(awq,
         assert lib.awq_qkv_attention(*wrong) != 0
     assert lib.awq_kv_cache_to_parts(f_kc.data_ptr(), f_vc.data_ptr(), mp, nh, f_kp.data_ptr(), f_vp.data_ptr(), pp, pp - 1,
                                      2, stream(torch)) != 0
+    # the copy by itself: no rows is no work; rows from the middle land where they belong and nowhere else
+    if pos >= 70:
+        t_kp = torch.full_like(f_kp, 3.0)
+        t_vp = torch.full_like(f_vp, 3.0)
+        awq.check(lib.awq_kv_cache_to_parts(f_kc.data_ptr(), f_vc.data_ptr(), mp, nh, t_kp.data_ptr(), t_vp.data_ptr(), pp, 5, 0,
+                                            stream(torch)))
+        assert (t_kp == 3.0).all() and (t_vp == 3.0).all()
+        awq.check(lib.awq_kv_cache_to_parts(f_kc.data_ptr(), f_vc.data_ptr(), mp, nh, t_kp.data_ptr(), t_vp.data_ptr(), pp, 5, 60,
+                                            stream(torch)))
+        for parts, ref in ((t_kp, kc_ref), (t_vp, vc_ref)):
+            got = parts.cpu().numpy().view(np.uint16).reshape(nh, 8, pp, 16)
+            want = ref.view(np.uint16).reshape(nh, mp, 8, 16)[:, 5:65].transpose(0, 2, 1, 3)
+            assert np.array_equal(got[:, :, 5:65], want)
+            three = np.float16(3.0).view(np.uint16)
+            assert (got[:, :, :5] == three).all() and (got[:, :, 65:] == three).all()
 
 
 # ----------------------------------------------------------------------------- W4A16 GEMM on the matrix cores
