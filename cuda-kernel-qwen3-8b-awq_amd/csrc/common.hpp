@@ -198,7 +198,8 @@ int launch_rmsnorm_batch(const half_t* x, const half_t* gamma, half_t* out, int6
                          hipStream_t st);
 int launch_rope_kv_append_batch(const half_t* qkv, const half_t* cos_t, const half_t* sin_t, half_t* q_out,
                                 half_t* kc, half_t* vc, int n_heads, int64_t max_pos, KvLayout kv, int64_t pos0,
-                                int64_t M, hipStream_t st);
+                                int64_t M, hipStream_t st, half_t* k_parts = nullptr, half_t* v_parts = nullptr,
+                                int parts_pos = 0);
 int launch_residual(const half_t* a, const half_t* b, half_t* out, int64_t n, hipStream_t st);
 int launch_gelu(half_t* x, int64_t n, hipStream_t st);
 int64_t argmax_workspace_bytes(int64_t n);

@@ -1054,13 +1054,12 @@ int enqueue_layer_batch(awq_engine* e, int l, int64_t pos0, int64_t M) {
   auto& b = e->pb;
   if (int rc = launch_rmsnorm_batch(b.hidden, L.gamma, b.norm, H, M, e->cfg.eps, st)) return rc;  // :1040
   if (int rc = gemm_of(e, L.wqkv, b.norm, b.qkv, M)) return rc;                                    // :1052
+  // (with the fused launch on, the appended rows also go into its second copy of the caches)
   if (int rc = launch_rope_kv_append_batch(b.qkv, e->cos_t, e->sin_t, b.q, L.kcache, L.vcache, e->n_heads,
-                                           e->cfg.max_pos, kv_blocked(e->n_heads), pos0, M, st))
+                                           e->cfg.max_pos, kv_blocked(e->n_heads), pos0, M, st,
+                                           e->fused_qkv ? L.kparts : nullptr, e->fused_qkv ? L.vparts : nullptr,
+                                           e->parts_pos))
     return rc;  // :1070-1103
-  if (e->fused_qkv && pos0 < e->parts_pos)  // the rows just appended, for the fused launch of the steps that follow
-    if (int rc = launch_kv_to_parts(L.kcache, L.vcache, kv_blocked(e->n_heads), L.kparts, L.vparts, e->n_heads,
-                                    e->parts_pos, pos0, std::min<int64_t>(M, e->parts_pos - pos0), st))
-      return rc;
   if (int rc = launch_prefill_attention(b.q, L.kcache, L.vcache, b.ctx, e->n_heads, e->cfg.max_pos,
                                         kv_blocked(e->n_heads), pos0, M, l >= 1,
                                         st))

@@ -77,7 +77,8 @@ __global__ __launch_bounds__(256) void rope_kv_batch_kernel(const half_t* __rest
                                                            const half_t* __restrict__ sin_t,
                                                            half_t* __restrict__ q_out, half_t* __restrict__ kc,
                                                            half_t* __restrict__ vc, int n_heads, KvLayout kv,
-                                                           int pos0) {
+                                                           int pos0, half_t* __restrict__ kp,
+                                                           half_t* __restrict__ vp, int parts_pos) {
   const int tok = blockIdx.y, pos = pos0 + tok;
   const int hd = blockIdx.x * 4 + (threadIdx.x >> 6), i = threadIdx.x & 63;
   if (hd >= n_heads) return;
@@ -93,14 +94,22 @@ __global__ __launch_bounds__(256) void rope_kv_batch_kernel(const half_t* __rest
     q_out[e] = ac - bs;
     q_out[e + 1] = as + bc;
   }
+  // the same rows a second time in the order the fused Wqkv + attention launch of the decode steps reads them,
+  // [head][dimension / 16][position][dimension % 16], for the positions that copy holds
+  const bool parts = kp != nullptr && pos < parts_pos;
+  const int64_t dst_p = (((int64_t)hd * 8 + (i >> 3)) * parts_pos + pos) * 16 + 2 * (i & 7);
   {
     const half_t a = qkv[H + e], b = qkv[H + e + 1];
     const half_t ac = a * c, bs = b * s, as = a * s, bc = b * c;
-    kc[dst] = ac - bs;
-    kc[dst + 1] = as + bc;
+    const half_t k0 = ac - bs, k1 = as + bc;
+    kc[dst] = k0;
+    kc[dst + 1] = k1;
+    if (parts) kp[dst_p] = k0, kp[dst_p + 1] = k1;
   }
-  vc[dst] = qkv[2 * H + e];
-  vc[dst + 1] = qkv[2 * H + e + 1];
+  const half_t v0 = qkv[2 * H + e], v1 = qkv[2 * H + e + 1];
+  vc[dst] = v0;
+  vc[dst + 1] = v1;
+  if (parts) vp[dst_p] = v0, vp[dst_p + 1] = v1;
 }
 
 
@@ -323,11 +332,12 @@ int launch_rmsnorm_batch(const half_t* x, const half_t* gamma, half_t* out, int6
 
 int launch_rope_kv_append_batch(const half_t* qkv, const half_t* cos_t, const half_t* sin_t, half_t* q_out,
                                 half_t* kc, half_t* vc, int n_heads, int64_t max_pos, KvLayout kv, int64_t pos0,
-                                int64_t M, hipStream_t st) {
+                                int64_t M, hipStream_t st, half_t* k_parts, half_t* v_parts, int parts_pos) {
   AWQ_REQUIRE(n_heads > 0 && max_pos > 0, "n_heads and max_pos must be positive");
+  AWQ_REQUIRE((k_parts == nullptr) == (v_parts == nullptr) && (k_parts == nullptr || parts_pos > 0), "parts arrays: both or none");
   AWQ_REQUIRE(M >= 1 && M <= 65535 && pos0 >= 0 && pos0 + M <= max_pos, "positions out of range");
   hipLaunchKernelGGL(rope_kv_batch_kernel, dim3((unsigned)((n_heads + 3) / 4), (unsigned)M), dim3(256), 0, st, qkv, cos_t, sin_t,
-                     q_out, kc, vc, n_heads, kv, (int)pos0);
+                     q_out, kc, vc, n_heads, kv, (int)pos0, k_parts, v_parts, parts_pos);
   AWQ_HIP_TRY(hipGetLastError());
   return AWQ_OK;
 }
