@@ -184,6 +184,9 @@ def test_gemm_plan_for_the_model_matrices(lib):
     assert [plan(w2, M) for M in (640, 1024, 1280)] == [ROWS_CUT] * 3   # long k, 80..160 tiles
     assert plan(w2, 1024, 0) == ROWS                                    # no workspace: no hand-over
     assert [plan(w2, M) for M in (2048, 4096)] == [ROWS] * 2
-    assert [plan(wo, M) for M in (128, 512)] == [K_SPLIT] * 2
+    assert [plan(wo, M) for M in (17, 32, 33, 64)] == [6] * 4           # tokens shared through LDS
+    assert plan((4096, 2048), 40) == 6 and plan((4096, 8192), 40) == K_SPLIT and plan((8192, 4096), 40) == K_SPLIT
+    assert lib.awq_gemm_workspace_bytes(4096, 4096, 40) == 0
+    assert [plan(wo, M) for M in (65, 128, 512)] == [K_SPLIT] * 3
     assert [plan(wo, M) for M in (576, 1024, 1280)] == [ROWS_64] * 3
     assert plan(wo, 2048) == ROWS and plan(wo, 2560) == ROWS_64 and plan(wo, 4096) == ROWS

@@ -717,7 +717,12 @@ def test_fused_qkv_attention_launch_against_the_two_launches_and_the_oracle(awq,
                                           # workgroup of two; two; one), k of 128, 256 and 384 blocks
                                           (12288, 4096, 5, False), (16384, 4096, 11, True), (4096, 8192, 9, False),
                                           (8192, 8192, 13, True), (4096, 12288, 7, True), (4096, 4096, 16, False),
-                                          (2048, 16384, 10, True), (4096, 4096, 2, True), (1024, 4096, 3, False)])
+                                          (2048, 16384, 10, True), (4096, 4096, 2, True), (1024, 4096, 3, False),
+                                          # 17..64 tokens on 4096 rows, the token tile shared through LDS: two
+                                          # and four 16-token tiles, k of 16 and of 8 steps
+                                          (4096, 4096, 17, True), (4096, 4096, 32, False), (4096, 4096, 33, True),
+                                          (4096, 4096, 64, False), (4096, 2048, 20, True), (4096, 2048, 49, False),
+                                          (12288, 4096, 33, True), (8192, 4096, 49, False)])
 def test_gemm_matches_fp32_accumulate_reference(awq, lib, oracle, torch_gpu, m, k, M, zp_int):
     """config 5: dequant-on-load MFMA product; 1e-2 relative against the sequential FP32-accumulate
     reference, and the weights it multiplies are the bit-exact dequantised ones (one-hot check below).
