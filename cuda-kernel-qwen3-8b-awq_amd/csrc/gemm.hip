@@ -1006,7 +1006,7 @@ __global__ __launch_bounds__(256, (MODE == WIDE_K && TT == 4) ? 1 : ((MODE == WI
   } while (CUT && --tile >= tile_first);
 }
 
-// 17..64 tokens on the 12288 x 4096 matrices: gemm_shared_kernel's scheme -- all weights requested at the start,
+// 17..256 tokens on the 12288 x 4096 matrices: gemm_shared_kernel's scheme -- all weights requested at the start,
 // the tokens through four rotating LDS tiles behind them, k split over eight wavefronts by 32-input block -- on
 // RP pairs of 16-row groups per workgroup (64 rows: 192 workgroups) and v_mfma_f32_32x32x16_f16, twice the rate
 // of the 16x16x32 shape, which holds gemm_shared_kernel at 0.39 us per step with three row groups.  A block is
@@ -1028,18 +1028,6 @@ __global__ __launch_bounds__(512) void gemm_shared32_kernel(GemmParams p) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int h = lane >> 5, n = lane & 31;
   const int rg0 = blockIdx.x * (2 * RP);
-  const half_t* src[TD];
-#pragma unroll
-  for (int i = 0; i < TD; ++i) {
-    const int row = 2 * (wave * TD + i) + (lane >> 5);
-    const int piece = (lane & 31) ^ (row & 31);
-    src[i] = p.x + (int64_t)min(row, p.M - 1) * p.k + piece * 8;
-  }
-  auto request = [&](int s) __attribute__((always_inline)) {
-    half_t* const tile = tiles + (s % NSLOT) * kTile + wave * TD * 512;
-#pragma unroll
-    for (int i = 0; i < TD; ++i) __builtin_amdgcn_global_load_lds((gptr_t)(src[i] + s * 256), (lptr_t)(tile + i * 512), 16, 0, 0);
-  };
   // the request order and the counts at the barriers are gemm_shared_kernel's
   uint32_t sc_raw, zz_raw;
   u32x2_t w[NS][RP];
@@ -1048,110 +1036,140 @@ __global__ __launch_bounds__(512) void gemm_shared32_kernel(GemmParams p) {
     asm volatile("global_load_ushort %0, %1, off" : "=v"(sc_raw) : "v"(p.scale + gi) : "memory");
     asm volatile("global_load_ushort %0, %1, off" : "=v"(zz_raw) : "v"(p.zp + gi) : "memory");
   }
-#pragma unroll
-  for (int s = 0; s < A; ++s) request(s);
-  asm volatile("" ::: "memory");
-#pragma unroll
-  for (int s = 0; s < NS; ++s)
-#pragma unroll
-    for (int a = 0; a < RP; ++a) {
-      const int rg = rg0 + 2 * a + (n >> 4);
-      const uint32_t* at = p.wq + (((int64_t)rg * p.nblk + wave + 8 * s) * 16 + (n & 15)) * 4 + 2 * h;
-      asm volatile("global_load_dwordx2 %0, %1, off nt" : "=v"(w[s][a]) : "v"(at) : "memory");
-    }
-  f32x16_t acc[RP][TT32];
-#pragma unroll
-  for (int a = 0; a < RP; ++a)
-#pragma unroll
-    for (int t = 0; t < TT32; ++t)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) acc[a][t][e] = 0.0f;
-  __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0((NS - 1) * RP));  // the scales, the tiles ahead, the first weights
-  __builtin_amdgcn_s_barrier();
-  asm volatile("" ::: "memory");
-  asm volatile("" : "+v"(sc_raw), "+v"(zz_raw));
-  const half_t sc = __builtin_bit_cast(half_t, (unsigned short)sc_raw), zz = __builtin_bit_cast(half_t, (unsigned short)zz_raw);
+  half_t sc, zz;
   // the operands of token tile t: row 32 t + n, pieces 4 wave + 2 h and + 1 of the step
   const int xoff0 = n * 256 + (((4 * wave + 2 * h) ^ n) << 3), xoff1 = n * 256 + (((4 * wave + 2 * h + 1) ^ n) << 3);
-  half8_t xr[2][TT32][2], wop[2][RP][2];
+  // More than 32 TT32 tokens: one slab of 32 TT32 tokens after the other against the same weights, which stay in
+  // their registers.  Only the first slab has weights in flight next to its tiles.
+  auto slab = [&](auto FIRST, int t0) __attribute__((always_inline)) {
+    constexpr bool first = decltype(FIRST)::value;
+    const half_t* src[TD];
 #pragma unroll
-  for (int t = 0; t < TT32; ++t) {
-    xr[0][t][0] = *reinterpret_cast<const half8_t*>(tiles + t * 32 * 256 + xoff0);
-    xr[0][t][1] = *reinterpret_cast<const half8_t*>(tiles + t * 32 * 256 + xoff1);
-  }
+    for (int i = 0; i < TD; ++i) {
+      const int row = 2 * (wave * TD + i) + (lane >> 5);
+      const int piece = (lane & 31) ^ (row & 31);
+      src[i] = p.x + (int64_t)min(t0 + row, p.M - 1) * p.k + piece * 8;
+    }
+    auto request = [&](int s) __attribute__((always_inline)) {
+      half_t* const tile = tiles + (s % NSLOT) * kTile + wave * TD * 512;
 #pragma unroll
-  for (int a = 0; a < RP; ++a) {
-    asm volatile("" : "+v"(w[0][a]));
-    wop[0][a][0] = dequant8<ZINT, false>(w[0][a].x, sc, zz);
-    wop[0][a][1] = dequant8<ZINT, false>(w[0][a].y, sc, zz);
-  }
-  static_for<NS>([&](auto S) __attribute__((always_inline)) {
-    constexpr int s = decltype(S)::value, c = s & 1, nx = c ^ 1;
-    // Tile s + 1 and the weights of step s + 1.  A tile requested before the loop is ahead of the weights: the
-    // later steps' weights and the tiles requested by the steps so far may be out.  A tile requested by a step is
-    // behind all the weights: the tiles requested since may be out.
-    constexpr int since = A - 2 < NS - 2 - s ? A - 2 : (NS - 2 - s > 0 ? NS - 2 - s : 0);
-    constexpr int so_far = s < NS - A ? s : NS - A;
-    __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(s + 1 < A ? (NS - 2 - s) * RP + so_far * TD : since * TD));
+      for (int i = 0; i < TD; ++i) __builtin_amdgcn_global_load_lds((gptr_t)(src[i] + s * 256), (lptr_t)(tile + i * 512), 16, 0, 0);
+    };
+#pragma unroll
+    for (int s = 0; s < A; ++s) request(s);
+    asm volatile("" ::: "memory");
+    if constexpr (first) {
+#pragma unroll
+      for (int s = 0; s < NS; ++s)
+#pragma unroll
+        for (int a = 0; a < RP; ++a) {
+          const int rg = rg0 + 2 * a + (n >> 4);
+          const uint32_t* at = p.wq + (((int64_t)rg * p.nblk + wave + 8 * s) * 16 + (n & 15)) * 4 + 2 * h;
+          asm volatile("global_load_dwordx2 %0, %1, off nt" : "=v"(w[s][a]) : "v"(at) : "memory");
+        }
+    }
+    f32x16_t acc[RP][TT32];
+#pragma unroll
+    for (int a = 0; a < RP; ++a)
+#pragma unroll
+      for (int t = 0; t < TT32; ++t)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[a][t][e] = 0.0f;
+    // the scales, the tiles ahead and the first weights; a later slab: tile 0
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(first ? (NS - 1) * RP : (A - 1) * TD));
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    if constexpr (s + 1 < NS) {
-#pragma unroll
-      for (int a = 0; a < RP; ++a) asm volatile("" : "+v"(w[s + 1][a]));  // not read before the wait above
+    if constexpr (first) {
+      asm volatile("" : "+v"(sc_raw), "+v"(zz_raw));
+      sc = __builtin_bit_cast(half_t, (unsigned short)sc_raw);
+      zz = __builtin_bit_cast(half_t, (unsigned short)zz_raw);
     }
-    // (what this step multiplies is not touched before the barrier: its products would wait for the reads there)
+    half8_t xr[2][TT32][2], wop[2][RP][2];
 #pragma unroll
-    for (int t = 0; t < TT32; ++t) asm volatile("" : "+v"(xr[c][t][0]), "+v"(xr[c][t][1]));
-#pragma unroll
-    for (int a = 0; a < RP; ++a) asm volatile("" : "+v"(wop[c][a][0]), "+v"(wop[c][a][1]));
-    if constexpr (s + A < NS) request(s + A);
-    if constexpr (s + 1 < NS) {
-#pragma unroll
-      for (int t = 0; t < TT32; ++t) {
-        xr[nx][t][0] = *reinterpret_cast<const half8_t*>(tiles + ((s + 1) % NSLOT) * kTile + t * 32 * 256 + xoff0);
-        xr[nx][t][1] = *reinterpret_cast<const half8_t*>(tiles + ((s + 1) % NSLOT) * kTile + t * 32 * 256 + xoff1);
-      }
+    for (int t = 0; t < TT32; ++t) {
+      xr[0][t][0] = *reinterpret_cast<const half8_t*>(tiles + t * 32 * 256 + xoff0);
+      xr[0][t][1] = *reinterpret_cast<const half8_t*>(tiles + t * 32 * 256 + xoff1);
     }
 #pragma unroll
     for (int a = 0; a < RP; ++a) {
+      asm volatile("" : "+v"(w[0][a]));
+      wop[0][a][0] = dequant8<ZINT, false>(w[0][a].x, sc, zz);
+      wop[0][a][1] = dequant8<ZINT, false>(w[0][a].y, sc, zz);
+    }
+    static_for<NS>([&](auto S) __attribute__((always_inline)) {
+      constexpr int s = decltype(S)::value, c = s & 1, nx = c ^ 1;
+      // Tile s + 1 and the weights of step s + 1.  A tile requested before the loop of the first slab is ahead
+      // of the weights: the later steps' weights and the tiles requested by the steps so far may be out.  A tile
+      // requested by a step is behind all the weights, and a later slab has none in flight: the tiles requested
+      // since may be out.
+      constexpr int since = A - 2 < NS - 2 - s ? A - 2 : (NS - 2 - s > 0 ? NS - 2 - s : 0);
+      constexpr int so_far = s < NS - A ? s : NS - A;
+      __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(first && s + 1 < A ? (NS - 2 - s) * RP + so_far * TD : since * TD));
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
       if constexpr (s + 1 < NS) {
-        wop[nx][a][0] = dequant8<ZINT, false>(w[s + 1][a].x, sc, zz);
-        wop[nx][a][1] = dequant8<ZINT, false>(w[s + 1][a].y, sc, zz);
+#pragma unroll
+        for (int a = 0; a < RP; ++a) asm volatile("" : "+v"(w[s + 1][a]));  // not read before the wait above
+      }
+      // (what this step multiplies is not touched before the barrier: its products would wait for the reads there)
+#pragma unroll
+      for (int t = 0; t < TT32; ++t) asm volatile("" : "+v"(xr[c][t][0]), "+v"(xr[c][t][1]));
+#pragma unroll
+      for (int a = 0; a < RP; ++a) asm volatile("" : "+v"(wop[c][a][0]), "+v"(wop[c][a][1]));
+      if constexpr (s + A < NS) request(s + A);
+      if constexpr (s + 1 < NS) {
+#pragma unroll
+        for (int t = 0; t < TT32; ++t) {
+          xr[nx][t][0] = *reinterpret_cast<const half8_t*>(tiles + ((s + 1) % NSLOT) * kTile + t * 32 * 256 + xoff0);
+          xr[nx][t][1] = *reinterpret_cast<const half8_t*>(tiles + ((s + 1) % NSLOT) * kTile + t * 32 * 256 + xoff1);
+        }
       }
 #pragma unroll
-      for (int kk = 0; kk < 2; ++kk)
+      for (int a = 0; a < RP; ++a) {
+        if constexpr (s + 1 < NS) {
+          wop[nx][a][0] = dequant8<ZINT, false>(w[s + 1][a].x, sc, zz);
+          wop[nx][a][1] = dequant8<ZINT, false>(w[s + 1][a].y, sc, zz);
+        }
 #pragma unroll
-        for (int t = 0; t < TT32; ++t)
-          acc[a][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xr[c][t][kk], wop[c][a][kk], acc[a][t], 0, 0, 0);
-    }
-  });
-  __syncthreads();  // every wavefront has read its operands: the tiles make room for the sums
-  float4_t* red = reinterpret_cast<float4_t*>(shared32_lds);  // [wavefront][pair][token tile][quarter][lane]
+        for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
-  for (int a = 0; a < RP; ++a)
-#pragma unroll
-    for (int t = 0; t < TT32; ++t)
-#pragma unroll
-      for (int g = 0; g < 4; ++g)
-        red[(((wave * RP + a) * TT32 + t) * 4 + g) * 64 + lane] =
-            float4_t{acc[a][t][4 * g], acc[a][t][4 * g + 1], acc[a][t][4 * g + 2], acc[a][t][4 * g + 3]};
-  __syncthreads();
-  // D[token 8 g + 4 (lane / 32) + e][row lane % 32] sits in element 4 g + e of the lane
-  const float scf = (float)sc;
-  with_epilogue(p, [&](auto E) {
-#pragma unroll
-    for (int idx = tid; idx < RP * TT32 * 256; idx += 512) {
-      const int a = idx / (TT32 * 256), t = (idx >> 8) % TT32, g = (idx >> 6) & 3;
-      float4_t v = red[idx];
-#pragma unroll
-      for (int wv = 1; wv < 8; ++wv) v += red[wv * (RP * TT32 * 256) + idx];
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int tok = 32 * t + 8 * g + 4 * h + e;
-        if (tok < p.M) store_out<decltype(E)::value, true>(p, tok, (rg0 + 2 * a) * 16 + n, v[e] * scf);
+          for (int t = 0; t < TT32; ++t)
+            acc[a][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xr[c][t][kk], wop[c][a][kk], acc[a][t], 0, 0, 0);
       }
-    }
-  });
+    });
+    __syncthreads();  // every wavefront has read its operands: the tiles make room for the sums
+    float4_t* red = reinterpret_cast<float4_t*>(shared32_lds);  // [wavefront][pair][token tile][quarter][lane]
+#pragma unroll
+    for (int a = 0; a < RP; ++a)
+#pragma unroll
+      for (int t = 0; t < TT32; ++t)
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+          red[(((wave * RP + a) * TT32 + t) * 4 + g) * 64 + lane] =
+              float4_t{acc[a][t][4 * g], acc[a][t][4 * g + 1], acc[a][t][4 * g + 2], acc[a][t][4 * g + 3]};
+    __syncthreads();
+    // D[token 8 g + 4 (lane / 32) + e][row lane % 32] sits in element 4 g + e of the lane
+    const float scf = (float)sc;
+    with_epilogue(p, [&](auto E) {
+#pragma unroll
+      for (int idx = tid; idx < RP * TT32 * 256; idx += 512) {
+        const int a = idx / (TT32 * 256), t = (idx >> 8) % TT32, g = (idx >> 6) & 3;
+        float4_t v = red[idx];
+#pragma unroll
+        for (int wv = 1; wv < 8; ++wv) v += red[wv * (RP * TT32 * 256) + idx];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int tok = t0 + 32 * t + 8 * g + 4 * h + e;
+          if (tok < p.M) store_out<decltype(E)::value, true>(p, tok, (rg0 + 2 * a) * 16 + n, v[e] * scf);
+        }
+      }
+    });
+  };
+  slab(std::true_type{}, 0);
+  for (int t0 = 32 * TT32; t0 < p.M; t0 += 32 * TT32) {
+    __syncthreads();  // the sums of the slab before have been read: its place takes tiles again
+    slab(std::false_type{}, t0);
+  }
 }
 
 // k cut over several workgroups: the chunks' FP32 partial sums are added in
@@ -1279,10 +1297,11 @@ int launch_shared(const GemmParams& p, bool zint, hipStream_t st) {
   return AWQ_OK;
 }
 
-// 17..64 tokens on 10240..16384 rows and k of 2048 or 4096 (the model's 12288 x 4096): gemm_shared32_kernel, 64
-// rows per workgroup
+// 17..256 tokens on 10240..16384 rows and k of 2048 or 4096 (the model's 12288 x 4096): gemm_shared32_kernel, 64
+// rows per workgroup, slabs of 64 tokens (12288 x 4096: 22.9 us at 128 tokens, 31.5 at 192, 39.5 at 256 against
+// 24.6 / 45.0 / 44.8 of the k-split and rows-split workgroups; 48.1 against 44.9 at 320)
 bool shared32_takes(int64_t m, int64_t k, int64_t M) {
-  return M >= 17 && M <= 64 && (k == 2048 || k == 4096) && m % 128 == 0 && m >= 10240 && m <= 16384;
+  return M >= 17 && M <= 256 && (k == 2048 || k == 4096) && m % 128 == 0 && m >= 10240 && m <= 16384;
 }
 template <int TT32, int NS>
 int launch_shared32(const GemmParams& p, bool zint, hipStream_t st) {
@@ -1340,7 +1359,7 @@ static WidePlan plan_wide(int64_t m, int64_t k, int64_t M, bool has_workspace) {
 // the shape awq_gemm takes for a product (diagnostics and tests): 0 few tokens, 1 k split, 2 rows split
 // with a tile per workgroup, 3 rows split with 64 tokens per workgroup, 4 rows split with the work cut evenly,
 // 5 up to 16 tokens with several row groups per workgroup, 6 17..64 tokens on 4096 rows with the tokens shared
-// through LDS, 7 the same on 10240..16384 rows with 64 rows per workgroup
+// through LDS, 7 17..256 tokens on 10240..16384 rows the same way with 64 rows per workgroup
 int gemm_plan(int64_t m, int64_t k, int64_t M, int has_workspace) {
   if (M >= 2 && mid_row_groups(m, k, M)) return 5;
   if (shared_takes(m, k, M)) return 6;

@@ -302,8 +302,9 @@ int64_t awq_gemm_workspace_bytes(int64_t m, int64_t k, int64_t M);
  * (needs the workspace), 5 two to sixteen tokens on a k that is a multiple of 4096 (up to 16384):
  * 16 wavefronts share up to three 16-row groups and split k, 6 17..64 tokens on 4096 rows and a k of
  * 2048 or 4096: one 16-row group per workgroup, all weights requested at the start, the tokens
- * streamed through LDS, 7 the same for 10240 to 16384 rows: 64 rows per workgroup on the 32 x 32 x 16
- * matrix instruction. */
+ * streamed through LDS, 7 17 to 256 tokens on 10240 to 16384 rows the same way: 64 rows per
+ * workgroup on the 32 x 32 x 16 matrix instruction, 64 tokens after the other against weights
+ * that stay in registers. */
 int awq_gemm_plan(int64_t m, int64_t k, int64_t M, int has_workspace);
 int awq_gemm(const void* repacked, const void* scale, const void* zp, int64_t m, int64_t k, const void* x, void* y,
              int64_t M, int32_t zp_integral, void* workspace, void* stream);

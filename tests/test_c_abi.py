@@ -175,10 +175,9 @@ def test_gemm_plan_for_the_model_matrices(lib):
     plan = lambda shape, M, ws=1: lib.awq_gemm_plan(shape[0], shape[1], M, ws)
     assert plan(w1, 1) == 0 and plan((256, 512), 4) == 0 and plan((256, 512), 5) == K_SPLIT
     assert [plan(s, M) for s in (w1, w2, wo) for M in (2, 4, 16)] == [5] * 9   # k a multiple of 4096
-    assert [plan(w1, M) for M in (17, 32, 33, 64)] == [7] * 4             # 64-row workgroups, tokens shared through LDS
+    assert [plan(w1, M) for M in (17, 32, 33, 64, 65, 128, 200, 256)] == [7] * 8   # 64-row workgroups, tokens shared through LDS
     assert plan((12288, 2048), 50) == 7 and plan((12288, 8192), 50) == K_SPLIT and plan((8192, 4096), 50) == K_SPLIT
-    assert [plan(w1, M) for M in (65, 128)] == [K_SPLIT] * 2
-    assert [plan(w1, M) for M in (256, 384)] == [ROWS_64] * 2           # 96..144 tiles: units would idle
+    assert [plan(w1, M) for M in (257, 384)] == [ROWS_64] * 2           # 96..144 tiles: units would idle
     assert [plan(w1, M) for M in (512, 640)] == [ROWS] * 2              # 192..240 tiles, one per unit
     assert [plan(w1, M) for M in (704, 1024)] == [ROWS_64] * 2          # 288..384 tiles: three per unit in one round
     assert [plan(w1, M) for M in (1280, 2048, 4096)] == [ROWS] * 3
