@@ -1012,6 +1012,8 @@ __global__ __launch_bounds__(256, (MODE == WIDE_K && TT == 4) ? 1 : ((MODE == WI
 // of the 16x16x32 shape, which holds gemm_shared_kernel at 0.39 us per step with three row groups.  A block is
 // two matrix instructions of 16 inputs: lane (h, n) holds dwords 2 h and 2 h + 1 of weight row n of the pair
 // (one 8-byte request) and reads the token pieces 2 h and 2 h + 1 of the block.  The 64 rows share one scale.
+// On 4096 x 12288 k is cut over four workgroups as well (256 workgroups of 12 steps): their FP32 sums go to the
+// workspace and a second launch adds them in slice order.
 template <int TT32, int RP, int NS, int A, bool ZINT>
 __global__ __launch_bounds__(512) void gemm_shared32_kernel(GemmParams p) {
   typedef __attribute__((address_space(1))) const void* gptr_t;
@@ -1028,6 +1030,7 @@ __global__ __launch_bounds__(512) void gemm_shared32_kernel(GemmParams p) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int h = lane >> 5, n = lane & 31;
   const int rg0 = blockIdx.x * (2 * RP);
+  const int step0 = blockIdx.y * NS;  // k cut over p.kz workgroups: NS steps each, their FP32 sums to p.part
   // the request order and the counts at the barriers are gemm_shared_kernel's
   uint32_t sc_raw, zz_raw;
   u32x2_t w[NS][RP];
@@ -1048,7 +1051,7 @@ __global__ __launch_bounds__(512) void gemm_shared32_kernel(GemmParams p) {
     for (int i = 0; i < TD; ++i) {
       const int row = 2 * (wave * TD + i) + (lane >> 5);
       const int piece = (lane & 31) ^ (row & 31);
-      src[i] = p.x + (int64_t)min(t0 + row, p.M - 1) * p.k + piece * 8;
+      src[i] = p.x + (int64_t)min(t0 + row, p.M - 1) * p.k + piece * 8 + step0 * 256;
     }
     auto request = [&](int s) __attribute__((always_inline)) {
       half_t* const tile = tiles + (s % NSLOT) * kTile + wave * TD * 512;
@@ -1064,7 +1067,7 @@ __global__ __launch_bounds__(512) void gemm_shared32_kernel(GemmParams p) {
 #pragma unroll
         for (int a = 0; a < RP; ++a) {
           const int rg = rg0 + 2 * a + (n >> 4);
-          const uint32_t* at = p.wq + (((int64_t)rg * p.nblk + wave + 8 * s) * 16 + (n & 15)) * 4 + 2 * h;
+          const uint32_t* at = p.wq + (((int64_t)rg * p.nblk + wave + 8 * (step0 + s)) * 16 + (n & 15)) * 4 + 2 * h;
           asm volatile("global_load_dwordx2 %0, %1, off nt" : "=v"(w[s][a]) : "v"(at) : "memory");
         }
     }
@@ -1159,8 +1162,10 @@ __global__ __launch_bounds__(512) void gemm_shared32_kernel(GemmParams p) {
         for (int wv = 1; wv < 8; ++wv) v += red[wv * (RP * TT32 * 256) + idx];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          const int tok = t0 + 32 * t + 8 * g + 4 * h + e;
-          if (tok < p.M) store_out<decltype(E)::value, true>(p, tok, (rg0 + 2 * a) * 16 + n, v[e] * scf);
+          const int tok = t0 + 32 * t + 8 * g + 4 * h + e, row = (rg0 + 2 * a) * 16 + n;
+          if (tok >= p.M) continue;
+          if (p.kz > 1) p.part[((int64_t)blockIdx.y * p.M + tok) * p.m + row] = v[e] * scf;  // finished by reduce_parts_kernel
+          else store_out<decltype(E)::value, true>(p, tok, row, v[e] * scf);
         }
       }
     });
@@ -1303,6 +1308,10 @@ int launch_shared(const GemmParams& p, bool zint, hipStream_t st) {
 bool shared32_takes(int64_t m, int64_t k, int64_t M) {
   return M >= 17 && M <= 256 && (k == 2048 || k == 4096) && m % 128 == 0 && m >= 10240 && m <= 16384;
 }
+// ... and 128..320 tokens on 4096 x 12288 with k cut over four workgroups (needs the workspace for their sums):
+// 25.9 us at 128 tokens, 35.2 at 192, 43.3 at 256, 52.1 at 320 against 26.8 / 45.0 / 47.2 / 57.9 of the k-split
+// and rows-split workgroups (slower than those below 128 and from 384 on, and on 4096 x 4096 throughout)
+bool shared32_kcut_takes(int64_t m, int64_t k, int64_t M) { return M >= 128 && M <= 320 && k == 12288 && m == 4096; }
 template <int TT32, int NS>
 int launch_shared32(const GemmParams& p, bool zint, hipStream_t st) {
   // tiles requested ahead of the weights (and kept ahead of the steps): 64 tokens 13.8 us with three, 14.2 with
@@ -1322,7 +1331,11 @@ int launch_shared32(const GemmParams& p, bool zint, hipStream_t st) {
       raised[zint].fetch_or(bit, std::memory_order_relaxed);
     }
   }
-  hipLaunchKernelGGL(kern, dim3((unsigned)(p.m / 64)), dim3(512), lds, st, p);
+  hipLaunchKernelGGL(kern, dim3((unsigned)(p.m / 64), (unsigned)p.kz), dim3(512), lds, st, p);
+  if (p.kz > 1) {
+    const int64_t total = (int64_t)p.M * p.m;
+    hipLaunchKernelGGL(reduce_parts_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, p);
+  }
   return AWQ_OK;
 }
 
@@ -1359,11 +1372,13 @@ static WidePlan plan_wide(int64_t m, int64_t k, int64_t M, bool has_workspace) {
 // the shape awq_gemm takes for a product (diagnostics and tests): 0 few tokens, 1 k split, 2 rows split
 // with a tile per workgroup, 3 rows split with 64 tokens per workgroup, 4 rows split with the work cut evenly,
 // 5 up to 16 tokens with several row groups per workgroup, 6 17..64 tokens on 4096 rows with the tokens shared
-// through LDS, 7 17..256 tokens on 10240..16384 rows the same way with 64 rows per workgroup
+// through LDS, 7 17..256 tokens on 10240..16384 rows the same way with 64 rows per workgroup, 8 the same with k
+// cut over four workgroups (4096 x 12288 at 128..320 tokens)
 int gemm_plan(int64_t m, int64_t k, int64_t M, int has_workspace) {
   if (M >= 2 && mid_row_groups(m, k, M)) return 5;
   if (shared_takes(m, k, M)) return 6;
   if (shared32_takes(m, k, M)) return 7;
+  if (has_workspace && shared32_kcut_takes(m, k, M)) return 8;
   if (M <= 4) return 0;
   switch (plan_wide(m, k, M, has_workspace != 0)) {
     case PLAN_K: return 1;
@@ -1374,6 +1389,7 @@ int gemm_plan(int64_t m, int64_t k, int64_t M, int has_workspace) {
 }
 
 int64_t gemm_workspace_bytes(int64_t m, int64_t k, int64_t M) {
+  if (shared32_kcut_takes(m, k, M)) return kSkHeaderBytes + 4 * M * m * 4;
   if (M <= 4 || mid_row_groups(m, k, M) || shared_takes(m, k, M) || shared32_takes(m, k, M)) return 0;
   switch (plan_wide(m, k, M, true)) {
     case PLAN_ROWS_CUT: return kSkHeaderBytes + (int64_t)kSkWgs * kSkTileFloats * 4;
@@ -1414,6 +1430,13 @@ int launch_gemm(const void* wq, const half_t* scale, const half_t* zp, int64_t m
   p.nr = p.n_tiles = 0;
   p.sk_head = nullptr;
   p.sk_part = nullptr;
+  if (shared32_kcut_takes(m, k, M) && workspace && kSkHeaderBytes + 4 * M * m * 4 <= workspace_bytes) {
+    p.kz = 4;
+    p.part = (float*)((char*)workspace + kSkHeaderBytes);
+    if (int rc = launch_shared32<2, 12>(p, zp_integral, st)) return rc;
+    AWQ_HIP_TRY(hipGetLastError());
+    return AWQ_OK;
+  }
   if (shared32_takes(m, k, M)) {
     int rc;
     if (k == 4096) rc = M <= 32 ? launch_shared32<1, 16>(p, zp_integral, st) : launch_shared32<2, 16>(p, zp_integral, st);

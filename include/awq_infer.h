@@ -304,7 +304,8 @@ int64_t awq_gemm_workspace_bytes(int64_t m, int64_t k, int64_t M);
  * 2048 or 4096: one 16-row group per workgroup, all weights requested at the start, the tokens
  * streamed through LDS, 7 17 to 256 tokens on 10240 to 16384 rows the same way: 64 rows per
  * workgroup on the 32 x 32 x 16 matrix instruction, 64 tokens after the other against weights
- * that stay in registers. */
+ * that stay in registers, 8 the same with k cut over four workgroups and a second launch that adds
+ * their FP32 sums (4096 x 12288 at 128 to 320 tokens; needs the workspace). */
 int awq_gemm_plan(int64_t m, int64_t k, int64_t M, int has_workspace);
 int awq_gemm(const void* repacked, const void* scale, const void* zp, int64_t m, int64_t k, const void* x, void* y,
              int64_t M, int32_t zp_integral, void* workspace, void* stream);

@@ -181,7 +181,9 @@ def test_gemm_plan_for_the_model_matrices(lib):
     assert [plan(w1, M) for M in (512, 640)] == [ROWS] * 2              # 192..240 tiles, one per unit
     assert [plan(w1, M) for M in (704, 1024)] == [ROWS_64] * 2          # 288..384 tiles: three per unit in one round
     assert [plan(w1, M) for M in (1280, 2048, 4096)] == [ROWS] * 3
-    assert [plan(w2, M) for M in (128, 512)] == [K_SPLIT] * 2
+    assert [plan(w2, M) for M in (64, 127, 512)] == [K_SPLIT] * 3
+    assert [plan(w2, M) for M in (128, 192, 320)] == [8] * 3 and plan(w2, 192, 0) != 8   # k cut, sums in the workspace
+    assert lib.awq_gemm_workspace_bytes(4096, 12288, 192) == 4096 + 4 * 192 * 4096 * 4
     assert [plan(w2, M) for M in (640, 1024, 1280)] == [ROWS_CUT] * 3   # long k, 80..160 tiles
     assert plan(w2, 1024, 0) == ROWS                                    # no workspace: no hand-over
     assert [plan(w2, M) for M in (2048, 4096)] == [ROWS] * 2

@@ -726,7 +726,9 @@ def test_fused_qkv_attention_launch_against_the_two_launches_and_the_oracle(awq,
                                           (12288, 4096, 20, False), (12288, 2048, 40, True), (10240, 2048, 31, False),
                                           # ... and 64 tokens after the other: two slabs, a ragged third, four
                                           (12288, 4096, 65, True), (12288, 4096, 128, False), (12288, 2048, 150, True),
-                                          (12288, 4096, 256, True)])
+                                          (12288, 4096, 256, True),
+                                          # ... with k cut over four workgroups and a second launch
+                                          (4096, 12288, 130, False), (4096, 12288, 192, True), (4096, 12288, 320, True)])
 def test_gemm_matches_fp32_accumulate_reference(awq, lib, oracle, torch_gpu, m, k, M, zp_int):
     """config 5: dequant-on-load MFMA product; 1e-2 relative against the sequential FP32-accumulate
     reference, and the weights it multiplies are the bit-exact dequantised ones (one-hot check below).
