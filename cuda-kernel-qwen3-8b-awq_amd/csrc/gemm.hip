@@ -11,10 +11,13 @@
 // rounding fewer per weight than the reference).
 //
 // Same weight stream as the decode kernel: [16-row group][32-wide block][row][16 B],
-// dword c of a row holding elements 8c..8c+7 of the block.  Three kernels:
+// dword c of a row holding elements 8c..8c+7 of the block.  The kernels:
 //   up to 4 tokens   the decode kernel's decomposition, products on v_mfma_f32_16x16x32_f16
 //   up to 16 tokens, k a multiple of 4096 (taken first)
 //                    the same operand shapes, 16 wavefronts sharing up to three row groups
+//   17..64 tokens on 4096 rows, 17..256 on 10240..16384 rows (k of 2048 or 4096), 128..320 on 4096 x 12288
+//                    16 or 64 rows per workgroup, all its weights requested at the start into registers, the
+//                    tokens shared by eight wavefronts through rotating LDS tiles
 //   more tokens      64 rows x 32..128 tokens per wavefront on v_mfma_f32_32x32x16_f16,
 //                    tokens staged through LDS
 #include "common.hpp"
@@ -351,9 +354,10 @@ constexpr int waitcnt_vm_lgkm0(int n) { return (n & 15) | (7 << 4) | ((n >> 4) <
 // piece ^ (row & 15) so that the operand reads of sixteen rows hit all banks), wavefront v multiplies block v
 // of the step against the TT token tiles, v_mfma_f32_16x16x32_f16 with the tokens as the first operand.  The
 // eight wavefronts' sums meet in LDS, in the place of the tiles.  No hand-over between workgroups, no second
-// launch.  (RG row groups per workgroup: written for up to three, which the 12288-row matrices would take, and
-// measured there at the time of the rows-split kernel, 15.7 us at 64 tokens -- the matrix instructions and the
-// weights' 4 us are not hidden behind the tokens -- so only RG = 1 is launched.)
+// launch.  (RG row groups per workgroup: written for up to three, which the 12288-row matrices would take;
+// there it took 15.7 us at 64 tokens, as long as the k-split workgroups -- 12 of these half-rate matrix
+// instructions per wavefront and step are 0.32 us of a 0.39 us step -- so only RG = 1 is launched, and those
+// matrices go to gemm_shared32_kernel.)
 template <int TT, int RG, int NS, bool ZINT>
 __global__ __launch_bounds__(512) void gemm_shared_kernel(GemmParams p, int n_rg) {
   typedef __attribute__((address_space(1))) const void* gptr_t;
