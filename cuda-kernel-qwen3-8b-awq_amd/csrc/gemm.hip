@@ -1415,6 +1415,8 @@ int launch_gemm(const void* wq, const half_t* scale, const half_t* zp, int64_t m
   AWQ_REQUIRE(M >= 1 && M <= (1 << 20), "M out of range");
   AWQ_REQUIRE(awq_group_period(m, k) == 1, "matrices whose scale group depends on the input index are not supported here");
   AWQ_REQUIRE(m < (1ll << 31) && k < (1ll << 31), "shape too large");
+  // the kernels read the weights and the tokens 16 bytes at a time (the tokens also straight into LDS)
+  AWQ_REQUIRE(((uintptr_t)wq & 15) == 0 && ((uintptr_t)x & 15) == 0, "the weights and x must be 16-byte aligned");
   GemmParams p;
   p.wq = (const uint32_t*)wq;
   p.scale = scale;

@@ -273,7 +273,8 @@ int awq_gemv_fused(const awq_linear_args* args, void* stream);
 
 /* The same product for M tokens at once (prefill, batched decode): the
  * reference's cublasGemmEx with n = M, ldb = k, ldc = m (it only ever calls it
- * with n = 1, Inference.cu:1056).  x [M][k], y [M][m] row-major FP16.  Weights
+ * with n = 1, Inference.cu:1056).  x [M][k], y [M][m] row-major FP16, x and the
+ * weights 16-byte aligned (AWQ_ERR_ARG otherwise).  Weights
  * are dequantised on load and contracted on the matrix cores with FP32
  * accumulation: within rounding noise of awq_gemv applied to each token, not
  * bit-identical to it.  Matrices whose scale group depends on the input index

@@ -82,6 +82,19 @@ def test_bad_configs_are_rejected(awq, lib, tmp_path):
         assert lib.awq_validate_weight_dir(str(tmp_path).encode(), ctypes.byref(cfg)) == 1, kw
 
 
+def test_gemm_rejects_bad_arguments_before_any_gpu_call(lib):
+    """awq_gemm's host checks (shape, alignment) fail with AWQ_ERR_ARG and a message; nothing is launched"""
+    buf = ctypes.create_string_buffer(4096 + 64)
+    base = (ctypes.addressof(buf) + 63) & ~63
+    call = lambda wq, x, m, k, M: lib.awq_gemm(ctypes.c_void_p(wq), ctypes.c_void_p(base), ctypes.c_void_p(base), m, k,
+                                              ctypes.c_void_p(x), ctypes.c_void_p(base), M, 1, None, None)
+    assert call(base, base + 2, 4096, 4096, 40) == 1 and b"16-byte aligned" in lib.awq_last_error()
+    assert call(base + 8, base, 12288, 4096, 40) == 1 and b"16-byte aligned" in lib.awq_last_error()
+    assert call(base, base, 4096, 4000, 40) == 1 and b"multiples of 128" in lib.awq_last_error()
+    assert call(base, base, 4096, 4096, 0) == 1 and b"M out of range" in lib.awq_last_error()
+    assert call(base, base, 6144, 4096, 40) == 1 and b"scale group" in lib.awq_last_error()
+
+
 def test_cli_usage_error():
     exe = os.path.join(ROOT, "cuda-kernel-qwen3-8b-awq_amd", "qwen3_awq_infer")
     res = subprocess.run([exe], capture_output=True, text=True)
