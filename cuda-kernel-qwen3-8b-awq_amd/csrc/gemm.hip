@@ -343,7 +343,7 @@ __device__ __forceinline__ void static_for(F&& f) {
 // assembly: the compiler then knows that the LDS reads before it are complete)
 constexpr int waitcnt_vm_lgkm0(int n) { return (n & 15) | (7 << 4) | ((n >> 4) << 14); }
 
-// 17..64 tokens, 4096 rows, k of 2048 or 4096 (the model's attention output matrix): one workgroup of eight
+// 17..64 (and 129..192) tokens, 4096 rows, k of 2048 or 4096 (the model's attention output matrix): one workgroup of eight
 // wavefronts per compute unit takes one 16-row group, all of k and ALL tokens.  Whichever way the rows are cut,
 // every compute unit has to read every token (512 KB at 64 tokens), and what a compute unit has requested comes
 // back in the order of the requests: a token piece out of L2 queued behind weights out of memory arrives with
@@ -370,26 +370,12 @@ __global__ __launch_bounds__(512) void gemm_shared_kernel(GemmParams p, int n_rg
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int q = lane >> 4, r = lane & 15;
   const int rg0 = blockIdx.x * RG;
-  // token tile requests: instruction i of this wavefront brings token rows 2 (wave TT + i) and + 1, 1 KB
-  const half_t* src[TT];
-#pragma unroll
-  for (int i = 0; i < TT; ++i) {
-    const int row = 2 * (wave * TT + i) + (lane >> 5);
-    const int piece = (lane & 31) ^ (row & 15);
-    src[i] = p.x + (int64_t)min(row, p.M - 1) * p.k + piece * 8;
-  }
   // The workgroups of a die (those whose indices agree mod 8) take the steps in different rotations: in step
   // with each other they would all ask the same few channels of the die's L2 for the same 512-byte columns of
   // the tokens.
-  const int first = ((blockIdx.x >> 3) & 31) * NS >> 5;
-  auto step_at = [&](int s) __attribute__((always_inline)) { return (s + first) & (NS - 1); };
+  const int first_step = ((blockIdx.x >> 3) & 31) * NS >> 5;
+  auto step_at = [&](int s) __attribute__((always_inline)) { return (s + first_step) & (NS - 1); };
   static_assert((NS & (NS - 1)) == 0, "the rotation wraps with a mask");
-  auto request = [&](int s) __attribute__((always_inline)) {
-    half_t* const tile = tiles + (s & 3) * kTile + wave * TT * 512;
-#pragma unroll
-    for (int i = 0; i < TT; ++i)
-      __builtin_amdgcn_global_load_lds((gptr_t)(src[i] + step_at(s) * 256), (lptr_t)(tile + i * 512), 16, 0, 0);
-  };
   // Requests return in the order they are made: the scales, three tiles out of L2, then the weights.  Those into
   // registers are issued by hand and waited for by the counts at the barriers: the compiler, which counts them
   // together with the requests into LDS, would wait for everything in flight at the first use of any of them.
@@ -402,99 +388,129 @@ __global__ __launch_bounds__(512) void gemm_shared_kernel(GemmParams p, int n_rg
     asm volatile("global_load_ushort %0, %1, off" : "=v"(sc_raw[i]) : "v"(p.scale + gi) : "memory");
     asm volatile("global_load_ushort %0, %1, off" : "=v"(zz_raw[i]) : "v"(p.zp + gi) : "memory");
   }
-  request(0);
-  request(1);
-  request(2);
-  asm volatile("" ::: "memory");
-#pragma unroll
-  for (int s = 0; s < NS; ++s)
-#pragma unroll
-    for (int i = 0; i < RG; ++i) {
-      const int rg = min(rg0 + i, n_rg - 1);
-      const uint32_t* at = p.wq + (((int64_t)rg * p.nblk + wave + 8 * step_at(s)) * 16 + r) * 4 + q;
-      asm volatile("global_load_dword %0, %1, off nt" : "=v"(w[s][i]) : "v"(at) : "memory");
-    }
-  float4_t acc[RG][TT];
-#pragma unroll
-  for (int i = 0; i < RG; ++i)
-#pragma unroll
-    for (int t = 0; t < TT; ++t) acc[i][t] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+  half_t sc[RG], zz[RG];
   // the operand of token tile t: row 16 t + r, piece 4 wave + q of the step
   const int xoff = r * 256 + (((4 * wave + q) ^ r) << 3);
-  half8_t xr[2][TT], wop[2][RG];
-  // Bare barriers: __syncthreads() would wait for every request in flight.  The counts say how many of this
-  // wavefront's requests may still be out: a tile complete here is complete for everybody behind the barrier.
-  __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0((NS - 1) * RG));  // the scales, tiles 0 to 2, the first weights
-  __builtin_amdgcn_s_barrier();
-  asm volatile("" ::: "memory");
-  half_t sc[RG], zz[RG];
+  // More than 16 TT tokens: one slab of 16 TT tokens after the other against the same weights, which stay in
+  // their registers.  Only the first slab has weights in flight next to its tiles.
+  auto slab = [&](auto FIRST, int t0) __attribute__((always_inline)) {
+    constexpr bool first = decltype(FIRST)::value;
+    // token tile requests: instruction i of this wavefront brings token rows 2 (wave TT + i) and + 1, 1 KB
+    const half_t* src[TT];
 #pragma unroll
-  for (int i = 0; i < RG; ++i) {
-    asm volatile("" : "+v"(sc_raw[i]), "+v"(zz_raw[i]), "+v"(w[0][i]));  // not read before the wait above
-    sc[i] = __builtin_bit_cast(half_t, (unsigned short)sc_raw[i]);
-    zz[i] = __builtin_bit_cast(half_t, (unsigned short)zz_raw[i]);
-  }
+    for (int i = 0; i < TT; ++i) {
+      const int row = 2 * (wave * TT + i) + (lane >> 5);
+      const int piece = (lane & 31) ^ (row & 15);
+      src[i] = p.x + (int64_t)min(t0 + row, p.M - 1) * p.k + piece * 8;
+    }
+    auto request = [&](int s) __attribute__((always_inline)) {
+      half_t* const tile = tiles + (s & 3) * kTile + wave * TT * 512;
 #pragma unroll
-  for (int t = 0; t < TT; ++t) xr[0][t] = *reinterpret_cast<const half8_t*>(tiles + t * 16 * 256 + xoff);
+      for (int i = 0; i < TT; ++i)
+        __builtin_amdgcn_global_load_lds((gptr_t)(src[i] + step_at(s) * 256), (lptr_t)(tile + i * 512), 16, 0, 0);
+    };
+    request(0);
+    request(1);
+    request(2);
+    asm volatile("" ::: "memory");
+    if constexpr (first) {
 #pragma unroll
-  for (int i = 0; i < RG; ++i) wop[0][i] = dequant8<ZINT, false>(w[0][i], sc[i], zz[i]);
-  // A step reads the operands of the next one out of LDS and dequantises the next one's weights while the
-  // matrix cores work on its own.
-  static_for<NS>([&](auto S) __attribute__((always_inline)) {
-    constexpr int s = decltype(S)::value, c = s & 1, n = c ^ 1;
-    // the weights of step s + 1 and tile s + 1 (tiles 1 and 2 were requested ahead of the weights, tile 3 and
-    // later behind all of them: tile s + 2, if there is one, may be out), and this wavefront's operand reads of tile s are done:
-    // tile s - 1 can be replaced
-    __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(s < 2 ? (NS - 2 - s) * RG + s * TT : (s + 2 < NS ? TT : 0)));
+      for (int s = 0; s < NS; ++s)
+#pragma unroll
+        for (int i = 0; i < RG; ++i) {
+          const int rg = min(rg0 + i, n_rg - 1);
+          const uint32_t* at = p.wq + (((int64_t)rg * p.nblk + wave + 8 * step_at(s)) * 16 + r) * 4 + q;
+          asm volatile("global_load_dword %0, %1, off nt" : "=v"(w[s][i]) : "v"(at) : "memory");
+        }
+    }
+    float4_t acc[RG][TT];
+#pragma unroll
+    for (int i = 0; i < RG; ++i)
+#pragma unroll
+      for (int t = 0; t < TT; ++t) acc[i][t] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    half8_t xr[2][TT], wop[2][RG];
+    // Bare barriers: __syncthreads() would wait for every request in flight.  The counts say how many of this
+    // wavefront's requests may still be out: a tile complete here is complete for everybody behind the barrier.
+    // The scales, tiles 0 to 2 and the first weights; a later slab: tile 0.
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(first ? (NS - 1) * RG : 2 * TT));
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    if constexpr (s + 1 < NS) {
-#pragma unroll
-      for (int i = 0; i < RG; ++i) asm volatile("" : "+v"(w[s + 1][i]));  // not read before the wait above
-    }
-    // (what this step multiplies is not touched before the barrier: its products would wait for the reads there)
-#pragma unroll
-    for (int t = 0; t < TT; ++t) asm volatile("" : "+v"(xr[c][t]));
-#pragma unroll
-    for (int i = 0; i < RG; ++i) asm volatile("" : "+v"(wop[c][i]));
-    if constexpr (s + 3 < NS) request(s + 3);
-    if constexpr (s + 1 < NS) {
-#pragma unroll
-      for (int t = 0; t < TT; ++t)
-        xr[n][t] = *reinterpret_cast<const half8_t*>(tiles + ((s + 1) & 3) * kTile + t * 16 * 256 + xoff);
-    }
 #pragma unroll
     for (int i = 0; i < RG; ++i) {
-      if constexpr (s + 1 < NS) wop[n][i] = dequant8<ZINT, false>(w[s + 1][i], sc[i], zz[i]);
-#pragma unroll
-      for (int t = 0; t < TT; ++t) acc[i][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xr[c][t], wop[c][i], acc[i][t], 0, 0, 0);
-    }
-  });
-  __syncthreads();  // every wavefront has read its operands: the tiles make room for the sums
-  float* red = reinterpret_cast<float*>(shared_lds);  // [8 wavefronts][RG][TT][64 lanes][4]
-#pragma unroll
-  for (int i = 0; i < RG; ++i)
-#pragma unroll
-    for (int t = 0; t < TT; ++t) *reinterpret_cast<float4_t*>(red + (((wave * RG + i) * TT + t) * 64 + lane) * 4) = acc[i][t];
-  __syncthreads();
-  // D[token 4 (lane / 16) + e][row lane % 16] sits in element e of the lane; thread (i, t, token, row), rows fastest
-  with_epilogue(p, [&](auto E) {
-#pragma unroll
-    for (int i = 0; i < RG; ++i) {
-      if (rg0 + i >= n_rg) continue;
-      const float scf = (float)sc[i];
-#pragma unroll
-      for (int idx = tid; idx < TT * 256; idx += 512) {
-        const int t = idx >> 8, row = idx & 15, e = (idx >> 4) & 3, q4 = (idx >> 6) & 3;
-        const int tok = 16 * t + 4 * q4 + e;
-        const float* first = red + ((i * TT + t) * 64 + q4 * 16 + row) * 4 + e;
-        float v = first[0];
-#pragma unroll
-        for (int wv = 1; wv < 8; ++wv) v += first[wv * (RG * TT * 256)];
-        if (tok < p.M) store_out<decltype(E)::value, true>(p, tok, (rg0 + i) * 16 + row, v * scf);
+      asm volatile("" : "+v"(w[0][i]));  // not read before the wait above
+      if constexpr (first) {
+        asm volatile("" : "+v"(sc_raw[i]), "+v"(zz_raw[i]));
+        sc[i] = __builtin_bit_cast(half_t, (unsigned short)sc_raw[i]);
+        zz[i] = __builtin_bit_cast(half_t, (unsigned short)zz_raw[i]);
       }
     }
-  });
+#pragma unroll
+    for (int t = 0; t < TT; ++t) xr[0][t] = *reinterpret_cast<const half8_t*>(tiles + t * 16 * 256 + xoff);
+#pragma unroll
+    for (int i = 0; i < RG; ++i) wop[0][i] = dequant8<ZINT, false>(w[0][i], sc[i], zz[i]);
+    // A step reads the operands of the next one out of LDS and dequantises the next one's weights while the
+    // matrix cores work on its own.
+    static_for<NS>([&](auto S) __attribute__((always_inline)) {
+      constexpr int s = decltype(S)::value, c = s & 1, n = c ^ 1;
+      // the weights of step s + 1 and tile s + 1 (in the first slab tiles 1 and 2 were requested ahead of the
+      // weights, tile 3 and later behind all of them: tile s + 2, if there is one, may be out), and this
+      // wavefront's operand reads of tile s are done: tile s - 1 can be replaced
+      __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(first && s < 2 ? (NS - 2 - s) * RG + s * TT : (s + 2 < NS ? TT : 0)));
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+      if constexpr (s + 1 < NS) {
+#pragma unroll
+        for (int i = 0; i < RG; ++i) asm volatile("" : "+v"(w[s + 1][i]));  // not read before the wait above
+      }
+      // (what this step multiplies is not touched before the barrier: its products would wait for the reads there)
+#pragma unroll
+      for (int t = 0; t < TT; ++t) asm volatile("" : "+v"(xr[c][t]));
+#pragma unroll
+      for (int i = 0; i < RG; ++i) asm volatile("" : "+v"(wop[c][i]));
+      if constexpr (s + 3 < NS) request(s + 3);
+      if constexpr (s + 1 < NS) {
+#pragma unroll
+        for (int t = 0; t < TT; ++t)
+          xr[n][t] = *reinterpret_cast<const half8_t*>(tiles + ((s + 1) & 3) * kTile + t * 16 * 256 + xoff);
+      }
+#pragma unroll
+      for (int i = 0; i < RG; ++i) {
+        if constexpr (s + 1 < NS) wop[n][i] = dequant8<ZINT, false>(w[s + 1][i], sc[i], zz[i]);
+#pragma unroll
+        for (int t = 0; t < TT; ++t) acc[i][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xr[c][t], wop[c][i], acc[i][t], 0, 0, 0);
+      }
+    });
+    __syncthreads();  // every wavefront has read its operands: the tiles make room for the sums
+    float* red = reinterpret_cast<float*>(shared_lds);  // [8 wavefronts][RG][TT][64 lanes][4]
+#pragma unroll
+    for (int i = 0; i < RG; ++i)
+#pragma unroll
+      for (int t = 0; t < TT; ++t) *reinterpret_cast<float4_t*>(red + (((wave * RG + i) * TT + t) * 64 + lane) * 4) = acc[i][t];
+    __syncthreads();
+    // D[token 4 (lane / 16) + e][row lane % 16] sits in element e of the lane; thread (i, t, token, row), rows fastest
+    with_epilogue(p, [&](auto E) {
+#pragma unroll
+      for (int i = 0; i < RG; ++i) {
+        if (rg0 + i >= n_rg) continue;
+        const float scf = (float)sc[i];
+#pragma unroll
+        for (int idx = tid; idx < TT * 256; idx += 512) {
+          const int t = idx >> 8, row = idx & 15, e = (idx >> 4) & 3, q4 = (idx >> 6) & 3;
+          const int tok = t0 + 16 * t + 4 * q4 + e;
+          const float* part = red + ((i * TT + t) * 64 + q4 * 16 + row) * 4 + e;
+          float v = part[0];
+#pragma unroll
+          for (int wv = 1; wv < 8; ++wv) v += part[wv * (RG * TT * 256)];
+          if (tok < p.M) store_out<decltype(E)::value, true>(p, tok, (rg0 + i) * 16 + row, v * scf);
+        }
+      }
+    });
+  };
+  slab(std::true_type{}, 0);
+  for (int t0 = 16 * TT; t0 < p.M; t0 += 16 * TT) {
+    __syncthreads();  // the sums of the slab before have been read: its place takes tiles again
+    slab(std::false_type{}, t0);
+  }
 }
 
 // Many tokens: a wavefront owns 64 weight rows x 128 tokens as 2 x 4 accumulator
@@ -1282,10 +1298,13 @@ int mid_row_groups(int64_t m, int64_t k, int64_t M) {
   return rg;
 }
 
-// 17..64 tokens on 4096 rows and k of 2048 or 4096: gemm_shared_kernel, one 16-row group per compute unit
-// (4096 x 4096: 6.4-6.8 us at 17..32 tokens, 8.6-9.4 us at 48..64, against 9.1-9.2 and 10.3-10.5 us of the k-split
-// workgroups)
-bool shared_takes(int64_t m, int64_t k, int64_t M) { return M >= 17 && M <= 64 && (k == 2048 || k == 4096) && m == 4096; }
+// 17..64 and 129..192 tokens on 4096 rows and k of 2048 or 4096: gemm_shared_kernel, one 16-row group per compute
+// unit (4096 x 4096: 6.4-6.8 us at 17..32 tokens, 8.6-9.4 us at 48..64, against 9.1-9.2 and 10.3-10.5 us of the
+// k-split workgroups; in slabs of 64 tokens 19.2 against 22.1 us at 192, level with them at 65..128 -- 13.4-14.2 --
+// and behind at 256, 24.3 against 22.7)
+bool shared_takes(int64_t m, int64_t k, int64_t M) {
+  return ((M >= 17 && M <= 64) || (M >= 129 && M <= 192)) && (k == 2048 || k == 4096) && m == 4096;
+}
 template <int TT, int NS>
 int launch_shared(const GemmParams& p, bool zint, hipStream_t st) {
   auto kern = zint ? gemm_shared_kernel<TT, 1, NS, true> : gemm_shared_kernel<TT, 1, NS, false>;
@@ -1375,7 +1394,7 @@ static WidePlan plan_wide(int64_t m, int64_t k, int64_t M, bool has_workspace) {
 // room for a header and the partial sums of a product whose work is cut over workgroups (0: never cut)
 // the shape awq_gemm takes for a product (diagnostics and tests): 0 few tokens, 1 k split, 2 rows split
 // with a tile per workgroup, 3 rows split with 64 tokens per workgroup, 4 rows split with the work cut evenly,
-// 5 up to 16 tokens with several row groups per workgroup, 6 17..64 tokens on 4096 rows with the tokens shared
+// 5 up to 16 tokens with several row groups per workgroup, 6 17..64 and 129..192 tokens on 4096 rows with the tokens shared
 // through LDS, 7 17..256 tokens on 10240..16384 rows the same way with 64 rows per workgroup, 8 the same with k
 // cut over four workgroups (4096 x 12288 at 128..320 tokens)
 int gemm_plan(int64_t m, int64_t k, int64_t M, int has_workspace) {

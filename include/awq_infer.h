@@ -301,7 +301,7 @@ int64_t awq_gemm_workspace_bytes(int64_t m, int64_t k, int64_t M);
  * wavefronts of a 64-row workgroup, 2 rows split with a 256 x 128 tile per workgroup, 3 rows split
  * with 64 tokens per workgroup, 4 rows split with the work cut evenly and FP32 sums handed over
  * (needs the workspace), 5 two to sixteen tokens on a k that is a multiple of 4096 (up to 16384):
- * 16 wavefronts share up to three 16-row groups and split k, 6 17..64 tokens on 4096 rows and a k of
+ * 16 wavefronts share up to three 16-row groups and split k, 6 17..64 and 129..192 tokens on 4096 rows and a k of
  * 2048 or 4096: one 16-row group per workgroup, all weights requested at the start, the tokens
  * streamed through LDS, 7 17 to 256 tokens on 10240 to 16384 rows the same way: 64 rows per
  * workgroup on the 32 x 32 x 16 matrix instruction, 64 tokens after the other against weights

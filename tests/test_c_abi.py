@@ -203,6 +203,6 @@ def test_gemm_plan_for_the_model_matrices(lib):
     assert [plan(wo, M) for M in (17, 32, 33, 64)] == [6] * 4           # tokens shared through LDS
     assert plan((4096, 2048), 40) == 6 and plan((4096, 8192), 40) == K_SPLIT and plan((8192, 4096), 40) == K_SPLIT
     assert lib.awq_gemm_workspace_bytes(4096, 4096, 40) == 0
-    assert [plan(wo, M) for M in (65, 128, 512)] == [K_SPLIT] * 3
+    assert [plan(wo, M) for M in (65, 128, 193, 512)] == [K_SPLIT] * 4 and [plan(wo, M) for M in (129, 192)] == [6] * 2
     assert [plan(wo, M) for M in (576, 1024, 1280)] == [ROWS_64] * 3
     assert plan(wo, 2048) == ROWS and plan(wo, 2560) == ROWS_64 and plan(wo, 4096) == ROWS

@@ -722,6 +722,7 @@ def test_fused_qkv_attention_launch_against_the_two_launches_and_the_oracle(awq,
                                           # and four 16-token tiles, k of 16 and of 8 steps
                                           (4096, 4096, 17, True), (4096, 4096, 32, False), (4096, 4096, 33, True),
                                           (4096, 4096, 64, False), (4096, 2048, 20, True), (4096, 2048, 49, False),
+                                          (4096, 4096, 130, True), (4096, 4096, 192, False), (4096, 2048, 150, True),
                                           (12288, 4096, 33, True), (8192, 4096, 49, False),
                                           (12288, 4096, 20, False), (12288, 2048, 40, True), (10240, 2048, 31, False),
                                           # ... and 64 tokens after the other: two slabs, a ragged third, four
