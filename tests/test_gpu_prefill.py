@@ -47,13 +47,14 @@ def oracle_run(oracle, model, prompt, n_new):
 # up to 16 tokens (k a multiple of 4096) with its residual and GeLU endings, one and two slices of k
 WIDE = dict(n_layers=2, hidden=4096, inter=8192, vocab=1024, max_pos=64)
 # the reference's widths: a prompt of 17..64 tokens takes the kernels that share the token tiles through LDS, with
-# their store, residual and GeLU endings (16 and 64 rows per workgroup, one token tile and two)
-FULLW = dict(n_layers=2, hidden=4096, inter=12288, vocab=1024, max_pos=96)
+# their store, residual and GeLU endings (16 and 64 rows per workgroup, one token tile and two); one of 150 tokens
+# takes them 64 tokens at a time, and the 4096 x 12288 product with k cut over four workgroups
+FULLW = dict(n_layers=2, hidden=4096, inter=12288, vocab=1024, max_pos=192)
 
 
 @pytest.mark.parametrize("shape,n_prompt", [(SMALL, 1), (SMALL, 2), (SMALL, 5), (SMALL, 37), (SMALL, 100),
                                             (WIDE, 3), (WIDE, 12), (WIDE, 16), (WIDE, 20), (WIDE, 40),
-                                            (FULLW, 24), (FULLW, 50)],
+                                            (FULLW, 24), (FULLW, 50), (FULLW, 150)],
                          ids=lambda v: ("hidden%d-inter%d" % (v["hidden"], v["inter"])) if isinstance(v, dict) else str(v))
 def test_small_model_batched_prompt_matches_sequential(awq, oracle, torch_gpu, shape, n_prompt):
     cfg = awq.make_config(**shape)
